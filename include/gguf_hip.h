@@ -1,0 +1,102 @@
+/*
+ * C ABI of the MI355X (gfx950) GGUF quantized-matmul library, libgguf_hip.so.
+ *
+ * Every entry point is the native half of one operator of the reference plugin's
+ * extension module `_C_gguf` (vllm_gguf_plugin/csrc/torch_bindings.cpp:22-53); the
+ * reference file:line each one replaces is cited next to it.  The ABI carries
+ * plain pointers and sizes only: no torch types, no exceptions, no host
+ * synchronisation and no allocation.  The caller owns every buffer, including the
+ * activation-quantisation workspace, and passes the HIP stream to launch on.
+ *
+ * Conventions
+ *   - all pointers are device pointers valid on the current HIP device;
+ *   - W is the packed GGUF tensor, row-major, `K / block_elems * block_bytes`
+ *     bytes per row, rows contiguous (what the reference receives as a uint8
+ *     tensor);
+ *   - X and Y are row-major and share one dtype, given as a GGUF_DTYPE_* code;
+ *   - `type` is the ggml type id (2,3,6,7,8,10-14,16-23,29);
+ *   - return value: 0 on success, a negative GGUF_ERR_* code otherwise.  On error
+ *     nothing has been launched.  The reference's native ops do no validation at
+ *     all (an unknown type returns zeros or calls a null pointer,
+ *     gguf_kernel.cu:97-98,119-217); this library rejects such calls instead.
+ */
+#ifndef GGUF_HIP_H
+#define GGUF_HIP_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define GGUF_DTYPE_F32 0
+#define GGUF_DTYPE_F16 1
+#define GGUF_DTYPE_BF16 2
+
+#define GGUF_OK 0
+#define GGUF_ERR_TYPE (-1)   /* ggml type id not supported by this entry point */
+#define GGUF_ERR_DTYPE (-2)  /* dtype code not one of GGUF_DTYPE_* */
+#define GGUF_ERR_SHAPE (-3)  /* K not a multiple of the block size, negative size, ... */
+#define GGUF_ERR_NULL (-4)   /* required pointer is null */
+#define GGUF_ERR_LAUNCH (-5) /* hipLaunchKernel reported an error */
+
+typedef void* gguf_stream_t; /* a hipStream_t */
+
+/* Library version and the code-object architecture it was built for ("gfx950"). */
+const char* gguf_hip_version(void);
+
+/* Elements and bytes of one block of a ggml type; 0 if the type is unknown.
+ * Replaces gguf.GGML_QUANT_SIZES as used at quantization/linear.py:51. */
+int gguf_block_elems(int type);
+int gguf_block_bytes(int type);
+
+/* Bytes of activation workspace per row of X for inner dimension K.
+ * The reference sizes its workspace as int32[M, roundup(K,512)/32*9]
+ * (gguf_kernel.cu:114-115); this library's private layout needs 44 bytes per 32
+ * values instead of 36, so callers must size the workspace with this function. */
+int64_t gguf_q8_1_row_bytes(int64_t K);
+
+/* q8_1 activation quantizer: M rows of K values -> workspace.
+ * Replaces quantize_q8_1 / quantize_row_q8_1_cuda (gguf_kernel.cu:32-85). */
+int gguf_quantize_q8_1(const void* x, int xdtype, void* q8_workspace, int64_t M, int64_t K, gguf_stream_t stream);
+
+/* Read back the reference-visible content of a workspace row set (test hook):
+ * int8 quants [M, Kp] and (d, sum) as float pairs [M, Kp/32, 2], Kp = roundup(K,512). */
+int gguf_q8_1_unpack(const void* q8_workspace, int8_t* q, float* ds, int64_t M, int64_t K, gguf_stream_t stream);
+
+/* Dense values of `nelem` packed weights in element order.
+ * Replaces ggml_dequantize (gguf_kernel.cu:87-102, dequantize.cuh:527-571). */
+int gguf_dequantize(const void* W, int type, void* Y, int ydtype, int64_t nelem, gguf_stream_t stream);
+
+/* Y[M,N] = q8_1(X[M,K]) . W[N,K]^T, decode GEMV path.
+ * Replaces ggml_mul_mat_vec_a8 (gguf_kernel.cu:104-218, mmvq.cuh:2-212). */
+int gguf_mmvq(const void* W, const void* x, int xdtype, void* q8_workspace, void* Y, int type, int64_t N, int64_t K,
+              int64_t M, gguf_stream_t stream);
+
+/* Same contraction, prefill path on int8 MFMA.
+ * Replaces ggml_mul_mat_a8 (gguf_kernel.cu:220-290, mmq.cuh:2-610). */
+int gguf_mmq(const void* W, const void* x, int xdtype, void* q8_workspace, void* Y, int type, int64_t N, int64_t K,
+             int64_t M, gguf_stream_t stream);
+
+/* Grouped (MoE) variant: for every sorted slot s with p = sorted_token_ids[s] < tokens*top_k,
+ * Y[p,:] = q8_1(X[p / top_k,:]) . W[expert_ids[s / block],:,:]^T.  Rows of Y that no slot names are zero.
+ * Replaces ggml_moe_a8 (gguf_kernel.cu:292-393, moe.cuh:5-739).  `block` must equal
+ * gguf_moe_block_size(type). */
+int gguf_moe_mmq(const void* X, int xdtype, void* q8_workspace, const void* W, int64_t expert_stride_bytes,
+                 const int32_t* sorted_token_ids, const int32_t* expert_ids, const int32_t* num_tokens_post_padded,
+                 int64_t num_sorted, void* Y, int type, int64_t N, int64_t K, int64_t top_k, int64_t tokens,
+                 gguf_stream_t stream);
+
+/* Per-pair MoE GEMV: Y[z,:] = q8_1(X[z / top_k,:]) . W[topk_ids[z],:,:]^T for z < tokens*top_k.
+ * Replaces ggml_moe_a8_vec (gguf_kernel.cu:395-530, moe_vec.cuh:3-338).  Experts are densely packed. */
+int gguf_moe_vec(const void* X, int xdtype, void* q8_workspace, const void* W, const int32_t* topk_ids, void* Y, int type,
+                 int64_t N, int64_t K, int64_t top_k, int64_t tokens, gguf_stream_t stream);
+
+/* Token-tile size that moe_align_block_size must pad expert groups to; 0 for unknown types.
+ * Replaces ggml_moe_get_block_size (gguf_kernel.cu:532-566). */
+int gguf_moe_block_size(int type);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* GGUF_HIP_H */

@@ -1,0 +1,68 @@
+"""ctypes binding of libgguf_hip.so (the C ABI declared in include/gguf_hip.h)."""
+from __future__ import annotations
+
+import ctypes
+import os
+from pathlib import Path
+
+_PKG = Path(__file__).resolve().parent
+LIB_PATH = _PKG / "libgguf_hip.so"
+
+ERRORS = {
+    -1: "ggml type not supported by this entry point",
+    -2: "unsupported dtype (need float32, float16 or bfloat16)",
+    -3: "bad shape (K must be a positive multiple of the block size; sizes must be non-negative)",
+    -4: "null pointer",
+    -5: "kernel launch failed",
+}
+
+_lib = None
+
+_c = ctypes
+_SIGNATURES = {
+    "gguf_hip_version": (_c.c_char_p, []),
+    "gguf_block_elems": (_c.c_int, [_c.c_int]),
+    "gguf_block_bytes": (_c.c_int, [_c.c_int]),
+    "gguf_q8_1_row_bytes": (_c.c_int64, [_c.c_int64]),
+    "gguf_quantize_q8_1": (_c.c_int, [_c.c_void_p, _c.c_int, _c.c_void_p, _c.c_int64, _c.c_int64, _c.c_void_p]),
+    "gguf_q8_1_unpack": (_c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int64, _c.c_int64, _c.c_void_p]),
+    "gguf_dequantize": (_c.c_int, [_c.c_void_p, _c.c_int, _c.c_void_p, _c.c_int, _c.c_int64, _c.c_void_p]),
+    "gguf_mmvq": (_c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_int, _c.c_void_p, _c.c_void_p, _c.c_int, _c.c_int64,
+                             _c.c_int64, _c.c_int64, _c.c_void_p]),
+    "gguf_mmq": (_c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_int, _c.c_void_p, _c.c_void_p, _c.c_int, _c.c_int64,
+                            _c.c_int64, _c.c_int64, _c.c_void_p]),
+    "gguf_moe_mmq": (_c.c_int, [_c.c_void_p, _c.c_int, _c.c_void_p, _c.c_void_p, _c.c_int64, _c.c_void_p, _c.c_void_p,
+                                _c.c_void_p, _c.c_int64, _c.c_void_p, _c.c_int, _c.c_int64, _c.c_int64, _c.c_int64,
+                                _c.c_int64, _c.c_void_p]),
+    "gguf_moe_vec": (_c.c_int, [_c.c_void_p, _c.c_int, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int,
+                                _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_void_p]),
+    "gguf_moe_block_size": (_c.c_int, [_c.c_int]),
+}
+EXPORTS = tuple(_SIGNATURES)
+
+
+def lib() -> ctypes.CDLL:
+    """Load the HIP library; there is no fallback path, a missing library is an error."""
+    global _lib
+    if _lib is None:
+        path = os.environ.get("GGUF_HIP_LIBRARY", str(LIB_PATH))
+        if not os.path.exists(path):
+            raise RuntimeError(
+                f"{path} is missing: build it with `python -m vllm_gguf_plugin_prism_amd.build` "
+                "(hipcc, gfx950).  This package has no non-HIP implementation."
+            )
+        handle = ctypes.CDLL(path)
+        for name, (res, args) in _SIGNATURES.items():
+            fn = getattr(handle, name)
+            fn.restype = res
+            fn.argtypes = args
+        _lib = handle
+    return _lib
+
+
+def check(rc: int, what: str) -> None:
+    if rc != 0:
+        msg = ERRORS.get(rc, f"error {rc}")
+        if rc == -1:
+            raise NotImplementedError(f"{what}: {msg}")
+        raise ValueError(f"{what}: {msg}")

@@ -1,0 +1,60 @@
+"""Build libgguf_hip.so (HIP kernels + C ABI) for gfx950 with hipcc, in-tree.
+
+``python -m vllm_gguf_plugin_prism_amd.build`` compiles every ``csrc/*.hip`` and
+links them into ``vllm_gguf_plugin_prism_amd/libgguf_hip.so``.  hipcc cross-compiles,
+so no GPU is needed.  The grid-code header is regenerated from ``tables/`` first.
+"""
+from __future__ import annotations
+
+import concurrent.futures
+import os
+import subprocess
+import sys
+from pathlib import Path
+
+PKG = Path(__file__).resolve().parent
+CSRC = PKG / "csrc"
+LIB = PKG / "libgguf_hip.so"
+HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+FLAGS = [
+    "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
+    # packed fp32 VALU forms are kept out of the generated code on purpose
+    "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    "-Wno-unused-command-line-argument",
+]
+
+
+def _compile(src: Path, obj: Path) -> None:
+    cmd = [HIPCC, *FLAGS, "-c", str(src), "-o", str(obj)]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    err = "\n".join(l for l in res.stderr.splitlines() if "is not a recognized feature" not in l)
+    if res.returncode != 0:
+        raise RuntimeError(f"hipcc failed on {src.name}:\n{err}")
+
+
+def build(verbose: bool = True) -> Path:
+    from .tables import grids
+
+    header = CSRC / "grid_codes.h"
+    text = grids.emit_c_header()
+    if not header.exists() or header.read_text() != text:
+        header.write_text(text)
+    objdir = PKG / "build"
+    objdir.mkdir(exist_ok=True)
+    srcs = sorted(CSRC.glob("*.hip"))
+    objs = [objdir / (s.stem + ".o") for s in srcs]
+    with concurrent.futures.ThreadPoolExecutor(max_workers=min(8, len(srcs))) as pool:
+        list(pool.map(_compile, srcs, objs))
+    tmp = LIB.with_suffix(".so.tmp")
+    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", *map(str, objs), "-o", str(tmp)]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("link failed:\n" + res.stderr)
+    os.replace(tmp, LIB)
+    if verbose:
+        print(f"built {LIB} from {len(srcs)} sources", file=sys.stderr)
+    return LIB
+
+
+if __name__ == "__main__":
+    build()

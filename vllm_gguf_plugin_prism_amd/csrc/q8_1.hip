@@ -1,0 +1,153 @@
+// q8_1 activation quantizer for gfx950.
+//
+// Semantics follow the reference's quantize_q8_1 (csrc/gguf/gguf_kernel.cu:32-69):
+// per 32 values, amax and sum are reduced by an xor butterfly over lane masks
+// 16, 8, 4, 2, 1; d = amax / 127 in fp32; q = roundf(x / d) (0 when amax == 0);
+// d and sum are stored rounded to half; columns [K, roundup(K, 512)) count as 0.
+//
+// Layout here: four lanes own one block, eight consecutive values each, so
+// lane^2 / lane^1 are the butterfly partners for masks 16 / 8 (DPP quad
+// permutes) and masks 4, 2, 1 are in-register.  The fp32 addition tree is
+// therefore the same tree the reference evaluates.
+#include "gguf_common.h"
+
+namespace gguf {
+
+template <typename T>
+__device__ __forceinline__ void load8(const T* p, float (&v)[8]);
+template <>
+__device__ __forceinline__ void load8<float>(const float* p, float (&v)[8]) {
+  const float4 a = *(const float4*)p, b = *(const float4*)(p + 4);
+  v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+}
+template <>
+__device__ __forceinline__ void load8<_Float16>(const _Float16* p, float (&v)[8]) {
+  typedef _Float16 h8 __attribute__((ext_vector_type(8)));
+  const h8 a = *(const h8*)p;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) v[i] = (float)a[i];
+}
+template <>
+__device__ __forceinline__ void load8<bf16_t>(const bf16_t* p, float (&v)[8]) {
+  const uint4 a = *(const uint4*)p;
+  const uint32_t w[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    v[2 * i] = __builtin_bit_cast(float, w[i] << 16);
+    v[2 * i + 1] = __builtin_bit_cast(float, w[i] & 0xFFFF0000u);
+  }
+}
+
+template <int CTRL>
+__device__ __forceinline__ int dpp_mov_i(int v) {
+  return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, true);
+}
+
+template <typename T>
+__global__ __launch_bounds__(256) void quantize_q8_1_kernel(const T* __restrict__ x, char* __restrict__ ws, int K,
+                                                           int Kp, int64_t row_bytes) {
+  const int t = blockIdx.x * 256 + threadIdx.x;  // one thread per 8 values of the padded row
+  if (t * 8 >= Kp) return;
+  const int64_t m = blockIdx.y;
+  const int e0 = t * 8;
+  float v[8];
+  if (e0 < K) {
+    load8<T>(x + m * (int64_t)K + e0, v);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = 0.0f;
+  }
+  float amax = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(v[i]));
+  amax = fmaxf(amax, dpp_mov<0x4E>(amax));
+  amax = fmaxf(amax, dpp_mov<0xB1>(amax));
+
+  float s[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) s[i] = v[i] + dpp_mov<0x4E>(v[i]);  // mask 16: lane ^ 2
+#pragma unroll
+  for (int i = 0; i < 8; ++i) s[i] = s[i] + dpp_mov<0xB1>(s[i]);  // mask 8:  lane ^ 1
+  const float t0 = s[0] + s[4], t1 = s[1] + s[5], t2 = s[2] + s[6], t3 = s[3] + s[7];  // mask 4
+  const float u0 = t0 + t2, u1 = t1 + t3;                                             // mask 2
+  const float sum = u0 + u1;                                                          // mask 1
+
+  const float d = amax / 127.0f;
+  int q[8];
+  int isum = 0;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    q[i] = amax == 0.0f ? 0 : (int)roundf(v[i] / d);
+    isum += q[i];
+  }
+  isum += dpp_mov_i<0x4E>(isum);
+  isum += dpp_mov_i<0xB1>(isum);
+
+  char* row = ws + m * row_bytes;
+  uint2 packed;
+  packed.x = (q[0] & 0xFF) | ((q[1] & 0xFF) << 8) | ((q[2] & 0xFF) << 16) | ((uint32_t)(q[3] & 0xFF) << 24);
+  packed.y = (q[4] & 0xFF) | ((q[5] & 0xFF) << 8) | ((q[6] & 0xFF) << 16) | ((uint32_t)(q[7] & 0xFF) << 24);
+  *(uint2*)(row + e0) = packed;
+  if ((t & 3) == 0) {
+    const int b = t >> 2;
+    const int nb = Kp / 32;
+    float* fd = (float*)(row + Kp);
+    const float dh = (float)(_Float16)d;
+    fd[b] = dh;
+    fd[nb + b] = (float)(_Float16)sum;
+    fd[2 * nb + b] = dh * (float)isum;
+  }
+}
+
+__global__ void q8_1_unpack_kernel(const char* __restrict__ ws, int8_t* __restrict__ q, float* __restrict__ ds, int Kp,
+                                   int64_t row_bytes) {
+  const int64_t m = blockIdx.y;
+  const int i = blockIdx.x * 256 + threadIdx.x;
+  if (i >= Kp) return;
+  const char* row = ws + m * row_bytes;
+  q[m * Kp + i] = ((const int8_t*)row)[i];
+  if ((i & 31) == 0) {
+    const float* fd = (const float*)(row + Kp);
+    const int nb = Kp / 32, b = i >> 5;
+    ds[(m * nb + b) * 2] = fd[b];
+    ds[(m * nb + b) * 2 + 1] = fd[nb + b];
+  }
+}
+
+int quantize_q8_1(const void* x, int xdtype, void* ws, int64_t M, int64_t K, hipStream_t stream) {
+  if (M == 0) return GGUF_OK;
+  const int Kp = (int)q8_kp(K);
+  const int64_t rb = q8_row_bytes(K);
+  const int gx = (Kp / 8 + 255) / 256;
+  for (int64_t off = 0; off < M; off += 65535) {
+    const int rows = (int)((M - off) < 65535 ? (M - off) : 65535);
+    GGUF_DISPATCH_DTYPE(xdtype, hipLaunchKernelGGL(quantize_q8_1_kernel<scalar_t>, dim3(gx, rows), dim3(256), 0, stream,
+                                                   (const scalar_t*)x + off * K, (char*)ws + off * rb, (int)K, Kp, rb));
+  }
+  return launch_status();
+}
+
+}  // namespace gguf
+
+extern "C" int64_t gguf_q8_1_row_bytes(int64_t K) { return K < 0 ? 0 : gguf::q8_row_bytes(K); }
+
+extern "C" int gguf_quantize_q8_1(const void* x, int xdtype, void* ws, int64_t M, int64_t K, gguf_stream_t stream) {
+  if (M < 0 || K <= 0 || K % 32 != 0) return GGUF_ERR_SHAPE;
+  if (M > 0 && (!x || !ws)) return GGUF_ERR_NULL;
+  if (xdtype < 0 || xdtype > 2) return GGUF_ERR_DTYPE;
+  return gguf::quantize_q8_1(x, xdtype, ws, M, K, (hipStream_t)stream);
+}
+
+extern "C" int gguf_q8_1_unpack(const void* ws, int8_t* q, float* ds, int64_t M, int64_t K, gguf_stream_t stream) {
+  if (M < 0 || K <= 0 || K % 32 != 0) return GGUF_ERR_SHAPE;
+  if (M == 0) return GGUF_OK;
+  if (!ws || !q || !ds) return GGUF_ERR_NULL;
+  const int Kp = (int)gguf::q8_kp(K);
+  for (int64_t off = 0; off < M; off += 65535) {
+    const int rows = (int)((M - off) < 65535 ? (M - off) : 65535);
+    hipLaunchKernelGGL(gguf::q8_1_unpack_kernel, dim3((Kp + 255) / 256, rows), dim3(256), 0, (hipStream_t)stream,
+                       (const char*)ws + off * gguf::q8_row_bytes(K), q + off * Kp, ds + off * (Kp / 32) * 2, Kp,
+                       gguf::q8_row_bytes(K));
+  }
+  return gguf::launch_status();
+}

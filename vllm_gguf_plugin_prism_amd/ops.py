@@ -1,0 +1,165 @@
+"""Operator façade, drop-in for ``vllm_gguf_plugin/ops.py:181-286`` of the reference.
+
+Same function names, positional orders, output shapes and dtypes.  Every call
+lands in the hand-written gfx950 kernels of ``libgguf_hip.so`` through its C ABI;
+there is no Triton or other fallback, so a ggml type a kernel does not cover
+raises ``NotImplementedError`` instead of silently taking another path.
+
+Outputs and the activation workspace are allocated with torch, and kernels are
+launched on torch's current HIP stream, so calls are asynchronous and
+graph-capturable like the reference's (``csrc/gguf/gguf_kernel.cu:24-29,104-118``).
+"""
+from __future__ import annotations
+
+import torch
+
+from . import _lib
+
+_DTYPE_CODE = {torch.float32: 0, torch.float16: 1, torch.bfloat16: 2}
+
+
+def _code(dtype: torch.dtype) -> int:
+    try:
+        return _DTYPE_CODE[dtype]
+    except KeyError:
+        raise ValueError(f"unsupported dtype {dtype}; need float32, float16 or bfloat16") from None
+
+
+def _stream(t: torch.Tensor) -> int:
+    return torch.cuda.current_stream(t.device).cuda_stream
+
+
+def _check_inputs(*tensors: torch.Tensor) -> None:
+    for t in tensors:
+        if not t.is_cuda:
+            raise ValueError("GGUF ops need tensors on the GPU")
+        if not t.is_contiguous():
+            raise ValueError("GGUF ops need contiguous tensors")
+
+
+def _workspace(x: torch.Tensor, rows: int, k: int) -> torch.Tensor:
+    nbytes = rows * _lib.lib().gguf_q8_1_row_bytes(k)
+    return torch.empty(max(nbytes, 16), dtype=torch.uint8, device=x.device)
+
+
+def quant_sizes(quant_type: int) -> tuple[int, int]:
+    """(elements, bytes) of one block; stands in for ``gguf.GGML_QUANT_SIZES`` (quantization/linear.py:51)."""
+    L = _lib.lib()
+    qk, bs = L.gguf_block_elems(int(quant_type)), L.gguf_block_bytes(int(quant_type))
+    if qk == 0:
+        raise NotImplementedError(f"Unsupported GGUF quantization type: {quant_type}")
+    return qk, bs
+
+
+def ggml_dequantize(W: torch.Tensor, quant_type: int, m: int, n: int, dtype: torch.dtype | None) -> torch.Tensor:
+    """Dense ``[m, n]`` values of the packed tensor ``W`` (reference: gguf_kernel.cu:87-102)."""
+    _check_inputs(W)
+    out_dtype = dtype or torch.float16
+    with torch.cuda.device(W.device):
+        out = torch.empty((m, n), dtype=out_dtype, device=W.device)
+        rc = _lib.lib().gguf_dequantize(W.data_ptr(), int(quant_type), out.data_ptr(), _code(out_dtype), m * n, _stream(W))
+    _lib.check(rc, "ggml_dequantize")
+    return out
+
+
+def _mul_mat(entry: str, W: torch.Tensor, X: torch.Tensor, quant_type: int, row: int) -> torch.Tensor:
+    _check_inputs(W, X)
+    vecs, col = X.shape
+    with torch.cuda.device(X.device):
+        out = torch.empty((vecs, row), dtype=X.dtype, device=W.device)
+        ws = _workspace(X, vecs, col)
+        fn = getattr(_lib.lib(), entry)
+        rc = fn(W.data_ptr(), X.data_ptr(), _code(X.dtype), ws.data_ptr(), out.data_ptr(), int(quant_type), row, col, vecs,
+                _stream(X))
+    _lib.check(rc, entry)
+    return out
+
+
+def ggml_mul_mat_vec_a8(W: torch.Tensor, X: torch.Tensor, quant_type: int, row: int) -> torch.Tensor:
+    """Decode GEMV ``q8_1(X) @ W^T`` -> ``[X.shape[0], row]`` (reference: gguf_kernel.cu:104-218)."""
+    return _mul_mat("gguf_mmvq", W, X, quant_type, row)
+
+
+def ggml_mul_mat_a8(W: torch.Tensor, X: torch.Tensor, quant_type: int, row: int) -> torch.Tensor:
+    """Prefill GEMM ``q8_1(X) @ W^T`` on int8 MFMA (reference: gguf_kernel.cu:220-290)."""
+    return _mul_mat("gguf_mmq", W, X, quant_type, row)
+
+
+def ggml_moe_a8(
+    X: torch.Tensor,
+    W: torch.Tensor,
+    sorted_token_ids: torch.Tensor,
+    expert_ids: torch.Tensor,
+    num_tokens_post_padded: torch.Tensor,
+    quant_type: int,
+    row: int,
+    top_k: int,
+    tokens: int,
+) -> torch.Tensor:
+    """Grouped MoE GEMM -> ``[tokens * top_k, row]`` (reference: gguf_kernel.cu:292-393)."""
+    _check_inputs(X, W, sorted_token_ids, expert_ids, num_tokens_post_padded)
+    for t in (sorted_token_ids, expert_ids, num_tokens_post_padded):
+        if t.dtype != torch.int32:
+            raise ValueError("MoE index tensors must be int32")
+    col = X.shape[1]
+    with torch.cuda.device(X.device):
+        out = torch.empty((tokens * top_k, row), dtype=X.dtype, device=W.device)
+        ws = _workspace(X, tokens, col)
+        rc = _lib.lib().gguf_moe_mmq(
+            X.data_ptr(), _code(X.dtype), ws.data_ptr(), W.data_ptr(), W.stride(0) * W.element_size(),
+            sorted_token_ids.data_ptr(), expert_ids.data_ptr(), num_tokens_post_padded.data_ptr(),
+            sorted_token_ids.shape[0], out.data_ptr(), int(quant_type), row, col, top_k, tokens, _stream(X))
+    _lib.check(rc, "ggml_moe_a8")
+    return out
+
+
+def ggml_moe_a8_vec(
+    X: torch.Tensor,
+    W: torch.Tensor,
+    topk_ids: torch.Tensor,
+    top_k: int,
+    quant_type: int,
+    row: int,
+    tokens: int,
+) -> torch.Tensor:
+    """Per-pair MoE GEMV -> ``[tokens * top_k, row]`` (reference: gguf_kernel.cu:395-530)."""
+    _check_inputs(X, W, topk_ids)
+    if topk_ids.dtype != torch.int32:
+        raise ValueError("topk_ids must be int32")
+    col = X.shape[1]
+    with torch.cuda.device(X.device):
+        out = torch.empty((tokens * top_k, row), dtype=X.dtype, device=W.device)
+        ws = _workspace(X, tokens, col)
+        rc = _lib.lib().gguf_moe_vec(X.data_ptr(), _code(X.dtype), ws.data_ptr(), W.data_ptr(), topk_ids.data_ptr(),
+                                     out.data_ptr(), int(quant_type), row, col, top_k, tokens, _stream(X))
+    _lib.check(rc, "ggml_moe_a8_vec")
+    return out
+
+
+def ggml_moe_get_block_size(quant_type: int) -> int:
+    """Token-tile size for ``moe_align_block_size`` (reference: gguf_kernel.cu:532-566)."""
+    return int(_lib.lib().gguf_moe_block_size(int(quant_type)))
+
+
+def moe_sum(input: torch.Tensor, output: torch.Tensor) -> None:
+    """``output[t, :] = sum_k input[t, k, :]`` (the reference forwards to vLLM's ``_moe_C.moe_sum``, ops.py:285-286)."""
+    torch.sum(input, dim=1, out=output)
+
+
+def quantize_q8_1(X: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
+    """The q8_1 activation quantizer on its own (reference: gguf_kernel.cu:32-85).
+
+    Returns ``(q, ds)``: int8 ``[M, Kp]`` quants and float32 ``[M, Kp/32, 2]`` (scale, sum) pairs holding the
+    half-rounded values, with ``Kp`` = K rounded up to 512.
+    """
+    _check_inputs(X)
+    m, k = X.shape
+    kp = (k + 511) // 512 * 512
+    with torch.cuda.device(X.device):
+        ws = _workspace(X, m, k)
+        q = torch.empty((m, kp), dtype=torch.int8, device=X.device)
+        ds = torch.empty((m, kp // 32, 2), dtype=torch.float32, device=X.device)
+        L = _lib.lib()
+        _lib.check(L.gguf_quantize_q8_1(X.data_ptr(), _code(X.dtype), ws.data_ptr(), m, k, _stream(X)), "quantize_q8_1")
+        _lib.check(L.gguf_q8_1_unpack(ws.data_ptr(), q.data_ptr(), ds.data_ptr(), m, k, _stream(X)), "q8_1_unpack")
+    return q, ds
