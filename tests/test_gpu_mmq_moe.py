@@ -1,0 +1,151 @@
+"""GPU parity: int8-MFMA MMQ, grouped MoE MMQ and per-pair MoE GEMV against the CPU oracle (C ABI path)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import gguf_oracle as o
+
+pytestmark = pytest.mark.gpu
+
+SIX = [o.Q4_0, o.Q8_0, o.Q4_K, o.Q6_K, o.IQ4_XS, o.IQ2_XXS]
+TORCH_DT = {"f16": torch.float16, "bf16": torch.bfloat16, "f32": torch.float32}
+
+
+def _ops():
+    from vllm_gguf_plugin_prism_amd import ops
+    return ops
+
+
+def _dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def _x(rng, m, k, dt):
+    t = torch.from_numpy(rng.standard_normal((m, k)).astype(np.float32)).to(TORCH_DT[dt])
+    return t.cuda(), t.to(torch.float32).numpy()
+
+
+@pytest.mark.parametrize("qtype", SIX)
+@pytest.mark.parametrize("m", [7, 83, 128, 200])
+def test_mmq_matches_a8_oracle_fp32(qtype, m):
+    ops = _ops()
+    rng = np.random.default_rng(400 + qtype * 16 + m)
+    qk = o.QUANT_SIZES[qtype][0]
+    for n, k in [(256, 1024), (77, 768), (130, 736 if qk == 32 else 1280)]:
+        w = o.make_weights(rng, qtype, n, k)
+        xd, xv = _x(rng, m, k, "f32")
+        y = ops.ggml_mul_mat_a8(_dev(w), xd, qtype, n)
+        assert y.shape == (m, n) and y.dtype == torch.float32
+        exp = o.mul_mat_a8(w, xv, qtype, n, "mmq")
+        err = o.rel_l2(y.cpu().numpy(), exp)
+        assert err <= 1e-5, (o.TYPE_NAMES[qtype], m, n, k, err)
+
+
+@pytest.mark.parametrize("dt", ["f16", "bf16"])
+@pytest.mark.parametrize("qtype", SIX)
+def test_mmq_half_outputs_within_tolerance(qtype, dt):
+    # stated tolerance vs the a8 oracle: rel-L2 <= 1e-3 for fp16 outputs, 4e-3 for bf16 (8-bit significand)
+    ops = _ops()
+    rng = np.random.default_rng(500 + qtype)
+    n, k, m = 384, 2048, 160
+    w = o.make_weights(rng, qtype, n, k)
+    xd, xv = _x(rng, m, k, dt)
+    y = ops.ggml_mul_mat_a8(_dev(w), xd, qtype, n).to(torch.float32).cpu().numpy()
+    assert o.rel_l2(y, o.mul_mat_a8(w, xv, qtype, n, "mmq")) <= (1e-3 if dt == "f16" else 4e-3)
+    assert o.rel_l2(y, o.mul_mat_f32(w, xv, qtype, n)) <= 2e-2
+
+
+def test_mmq_and_mmvq_agree():
+    # same contraction through both paths; Q4_K differs only by which block sum the offset term uses
+    ops = _ops()
+    rng = np.random.default_rng(600)
+    for qtype in SIX:
+        w = _dev(o.make_weights(rng, qtype, 128, 1024))
+        xd, _ = _x(rng, 5, 1024, "f32")
+        a = ops.ggml_mul_mat_a8(w, xd, qtype, 128).cpu().numpy()
+        b = ops.ggml_mul_mat_vec_a8(w, xd, qtype, 128).cpu().numpy()
+        assert o.rel_l2(a, b) <= (2e-2 if qtype == o.Q4_K else 1e-5), o.TYPE_NAMES[qtype]
+
+
+@pytest.mark.parametrize("m", [128, 512])
+def test_config3_q6_k_qwen_mlp_slices(m):
+    # Qwen2.5-7B MLP shapes at full K; N is cut to 1024 rows so the fp64 oracle stays in seconds
+    ops = _ops()
+    rng = np.random.default_rng(3)
+    for n, k in [(1024, 3584), (1024, 18944)]:
+        w = o.make_weights(rng, o.Q6_K, n, k)
+        xd, xv = _x(rng, m, k, "f16")
+        y = ops.ggml_mul_mat_a8(_dev(w), xd, o.Q6_K, n).to(torch.float32).cpu().numpy()
+        assert o.rel_l2(y, o.mul_mat_a8(w, xv, o.Q6_K, n, "mmq")) <= 1e-3
+
+
+def _routing(rng, t, e, top_k):
+    logits = rng.standard_normal((t, e)).astype(np.float32)
+    ids = np.argsort(-logits, axis=1)[:, :top_k].astype(np.int32)
+    sel = np.take_along_axis(logits, ids.astype(np.int64), axis=1)
+    wts = np.exp(sel - sel.max(axis=1, keepdims=True))
+    return ids, (wts / wts.sum(axis=1, keepdims=True)).astype(np.float32)
+
+
+@pytest.mark.parametrize("qtype", [o.Q4_0, o.Q4_K, o.Q6_K, o.Q8_0])
+@pytest.mark.parametrize("t,top_k,e", [(7, 2, 8), (83, 4, 16), (128, 8, 64)])
+def test_moe_grouped_matches_oracle(qtype, t, top_k, e):
+    ops = _ops()
+    rng = np.random.default_rng(700 + qtype + t)
+    n, k = 160, 512
+    w = np.stack([o.make_weights(rng, qtype, n, k) for _ in range(e)])
+    xd, xv = _x(rng, t, k, "f32")
+    ids, _ = _routing(rng, t, e, top_k)
+    blk = ops.ggml_moe_get_block_size(qtype)
+    assert blk > 0
+    s, eids, npost = o.moe_align_block_size(ids, blk, e)
+    y = ops.ggml_moe_a8(xd, _dev(w), _dev(s), _dev(eids), _dev(npost), qtype, n, top_k, t)
+    assert y.shape == (t * top_k, n)
+    exp = o.moe_a8(xv, w, s, eids, npost, qtype, n, top_k, t, blk)
+    assert o.rel_l2(y.cpu().numpy(), exp) <= 1e-5
+    # second stage of the pipeline: top_k = 1 over tokens * top_k rows, same sorted ids
+    x2d, x2v = _x(rng, t * top_k, k, "f32")
+    y2 = ops.ggml_moe_a8(x2d, _dev(w), _dev(s), _dev(eids), _dev(npost), qtype, n, 1, t * top_k)
+    exp2 = o.moe_a8(x2v, w, s, eids, npost, qtype, n, 1, t * top_k, blk)
+    assert o.rel_l2(y2.cpu().numpy(), exp2) <= 1e-5
+
+
+def test_moe_grouped_padding_and_bad_experts_write_nothing():
+    ops = _ops()
+    rng = np.random.default_rng(800)
+    t, top_k, e, n, k, qtype = 20, 2, 6, 64, 256, o.Q4_0
+    w = np.stack([o.make_weights(rng, qtype, n, k) for _ in range(e)])
+    xd, xv = _x(rng, t, k, "f32")
+    ids, _ = _routing(rng, t, e, top_k)
+    blk = ops.ggml_moe_get_block_size(qtype)
+    s, eids, npost = o.moe_align_block_size(ids, blk, e)
+    eids2 = eids.copy()
+    eids2[0] = 300            # out-of-range expert: its block is skipped (moe.cuh:33)
+    y = ops.ggml_moe_a8(xd, _dev(w), _dev(s), _dev(eids2), _dev(npost), qtype, n, top_k, t).cpu().numpy()
+    exp = o.moe_a8(xv, w, s, eids2, npost, qtype, n, top_k, t, blk)
+    assert o.rel_l2(y, exp) <= 1e-5
+    skipped = s[:blk][s[:blk] < t * top_k]
+    assert len(skipped) > 0 and np.all(y[skipped] == 0)
+
+
+@pytest.mark.parametrize("qtype", SIX)
+def test_moe_vec_matches_oracle(qtype):
+    ops = _ops()
+    rng = np.random.default_rng(900 + qtype)
+    t, top_k, e, n, k = 9, 4, 8, 96, 512
+    w = np.stack([o.make_weights(rng, qtype, n, k) for _ in range(e)])
+    xd, xv = _x(rng, t, k, "f32")
+    ids, _ = _routing(rng, t, e, top_k)
+    y = ops.ggml_moe_a8_vec(xd, _dev(w), _dev(ids), top_k, qtype, n, t)
+    assert y.shape == (t * top_k, n)
+    assert o.rel_l2(y.cpu().numpy(), o.moe_a8_vec(xv, w, ids, top_k, qtype, n, t)) <= 1e-5
+
+
+def test_moe_sum_and_block_size():
+    ops = _ops()
+    x = torch.randn(5, 4, 32, device="cuda")
+    out = torch.empty(5, 32, device="cuda")
+    ops.moe_sum(x, out)
+    assert torch.allclose(out, x.sum(dim=1))
+    assert ops.ggml_moe_get_block_size(2) == ops.ggml_moe_get_block_size(14) > 0
+    assert ops.ggml_moe_get_block_size(99) == 0

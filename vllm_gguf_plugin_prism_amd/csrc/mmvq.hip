@@ -251,14 +251,24 @@ struct FmtIQ2_XXS {
 };
 
 // ------------------------------------------------------------------ kernel
-// EXPERT > 0 selects the MoE per-pair variant: blockIdx.y picks the (token, k) pair; see moe.hip.
-template <class F, int MT, int RPW, typename T>
+// MOE selects the per-pair variant (reference: csrc/gguf/moe_vec.cuh:3-53): blockIdx.y is the flat
+// (token, k) pair z; its expert topk_ids[z] picks the weight matrix (experts densely packed), its
+// token z / top_k picks the activation row, and the result goes to row z of Y.
+template <class F, int MT, int RPW, typename T, bool MOE>
 __global__ __launch_bounds__(256) void mmvq_kernel(const uint8_t* __restrict__ W, const char* __restrict__ ws,
                                                     T* __restrict__ Y, int N, int K, int kchunk, int64_t ws_row_bytes,
-                                                    int64_t y_vec_stride) {
+                                                    int64_t y_vec_stride, const int32_t* __restrict__ topk_ids,
+                                                    int top_k) {
   extern __shared__ __align__(16) char smem[];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int Kp = (int)q8_kp(K);
+  if (MOE) {
+    const int z = blockIdx.y;
+    const int e = topk_ids[z];
+    W += (int64_t)e * N * ((int64_t)(K / F::QK) * F::BS);
+    ws += (int64_t)(z / top_k) * ws_row_bytes;
+    Y += (int64_t)z * N;
+  }
   int8_t* lq = (int8_t*)smem;                         // [MT][kchunk]
   float* ldv = (float*)(smem + MT * kchunk);          // [MT][kchunk/32]
   float* lav = ldv + MT * (kchunk / 32);              // [MT][kchunk/32]
@@ -333,8 +343,35 @@ static void launch_mt(const void* W, const char* ws, T* Y, int N, int K, hipStre
   if (kchunk > kround) kchunk = kround;
   const size_t lds = (size_t)MT * kchunk + (size_t)MT * (kchunk / 32) * 4 * (F::AUX != AUX_NONE ? 2 : 1) + F::TABLE_BYTES;
   const int grid = (N + 4 * RPW - 1) / (4 * RPW);
-  hipLaunchKernelGGL((mmvq_kernel<F, MT, RPW, T>), dim3(grid), dim3(256), lds, stream, (const uint8_t*)W, ws, Y, N, K,
-                     kchunk, q8_row_bytes(K), (int64_t)N);
+  hipLaunchKernelGGL((mmvq_kernel<F, MT, RPW, T, false>), dim3(grid), dim3(256), lds, stream, (const uint8_t*)W, ws, Y, N,
+                     K, kchunk, q8_row_bytes(K), (int64_t)N, (const int32_t*)nullptr, 1);
+}
+
+template <class F, typename T>
+static int moe_vec_typed(const void* W, const char* ws, void* Y, int N, int K, const int32_t* topk_ids, int top_k,
+                         int pairs, hipStream_t stream) {
+  constexpr int RPW = 2;
+  int kchunk = kchunk_for(1);
+  const int kround = (K + 511) / 512 * 512;
+  if (kchunk > kround) kchunk = kround;
+  const size_t lds = (size_t)kchunk + (size_t)(kchunk / 32) * 4 * (F::AUX != AUX_NONE ? 2 : 1) + F::TABLE_BYTES;
+  const int grid = (N + 4 * RPW - 1) / (4 * RPW);
+  for (int z0 = 0; z0 < pairs; z0 += 65535) {
+    const int nz = pairs - z0 < 65535 ? pairs - z0 : 65535;
+    // the pair index is rebuilt from blockIdx.y, so later slabs shift the id and output bases by whole tokens
+    if (z0 % top_k != 0) return GGUF_ERR_SHAPE;
+    hipLaunchKernelGGL((mmvq_kernel<F, 1, RPW, T, true>), dim3(grid, nz), dim3(256), lds, stream, (const uint8_t*)W,
+                       ws + (int64_t)(z0 / top_k) * q8_row_bytes(K), (T*)Y + (int64_t)z0 * N, N, K, kchunk, q8_row_bytes(K),
+                       (int64_t)N, topk_ids + z0, top_k);
+  }
+  return launch_status();
+}
+
+template <class F>
+static int moe_vec_fmt(const void* W, const void* ws, void* Y, int dtype, int N, int K, const int32_t* ids, int top_k,
+                       int pairs, hipStream_t s) {
+  GGUF_DISPATCH_DTYPE(dtype, return (moe_vec_typed<F, scalar_t>(W, (const char*)ws, Y, N, K, ids, top_k, pairs, s)));
+  return GGUF_ERR_DTYPE;
 }
 
 template <class F, typename T>
@@ -386,6 +423,36 @@ extern "C" int gguf_mmvq(const void* W, const void* x, int xdtype, void* q8_work
     case T_Q6_K: return mmvq_fmt<FmtQ6_K>(W, q8_workspace, Y, xdtype, N, K, M, s);
     case T_IQ4_XS: return mmvq_fmt<FmtIQ4_XS>(W, q8_workspace, Y, xdtype, N, K, M, s);
     case T_IQ2_XXS: return mmvq_fmt<FmtIQ2_XXS>(W, q8_workspace, Y, xdtype, N, K, M, s);
+  }
+  return GGUF_ERR_TYPE;
+}
+
+extern "C" int gguf_moe_vec(const void* X, int xdtype, void* q8_workspace, const void* W, const int32_t* topk_ids, void* Y,
+                            int type, int64_t N, int64_t K, int64_t top_k, int64_t tokens, gguf_stream_t stream) {
+  using namespace gguf;
+  const int qk = block_elems(type);
+  if (qk == 0) return GGUF_ERR_TYPE;
+  if (N < 0 || tokens < 0 || top_k <= 0 || K <= 0 || K % qk != 0 || N > 0x7FFFFFF0LL || K > 0x7FFFFFF0LL ||
+      tokens * top_k > 0x7FFFFFF0LL)
+    return GGUF_ERR_SHAPE;
+  if (xdtype < 0 || xdtype > 2) return GGUF_ERR_DTYPE;
+  switch (type) {
+    case T_Q4_0: case T_Q8_0: case T_Q4_K: case T_Q6_K: case T_IQ4_XS: case T_IQ2_XXS: break;
+    default: return GGUF_ERR_TYPE;
+  }
+  if (N == 0 || tokens == 0) return GGUF_OK;
+  if (!X || !q8_workspace || !W || !topk_ids || !Y) return GGUF_ERR_NULL;
+  hipStream_t s = (hipStream_t)stream;
+  const int rc = quantize_q8_1(X, xdtype, q8_workspace, tokens, K, s);
+  if (rc != GGUF_OK) return rc;
+  const int pairs = (int)(tokens * top_k);
+  switch (type) {
+    case T_Q4_0: return moe_vec_fmt<FmtQ4_0>(W, q8_workspace, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
+    case T_Q8_0: return moe_vec_fmt<FmtQ8_0>(W, q8_workspace, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
+    case T_Q4_K: return moe_vec_fmt<FmtQ4_K>(W, q8_workspace, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
+    case T_Q6_K: return moe_vec_fmt<FmtQ6_K>(W, q8_workspace, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
+    case T_IQ4_XS: return moe_vec_fmt<FmtIQ4_XS>(W, q8_workspace, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
+    case T_IQ2_XXS: return moe_vec_fmt<FmtIQ2_XXS>(W, q8_workspace, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
   }
   return GGUF_ERR_TYPE;
 }
