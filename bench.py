@@ -1,0 +1,220 @@
+#!/usr/bin/env python3
+"""Headline benchmark of the GGUF quantized-matmul hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W]
+
+Prints ONE JSON line.  ``value`` is the whole-job throughput of the batch-1 Q4_K
+decode GEMV (BASELINE config 2) in algorithmic GB/s: one *step* runs
+``ops.ggml_mul_mat_vec_a8`` once on each of the three Llama-3-8B-like
+projections [4096,4096], [14336,4096], [4096,14336] (activation quantisation
+included), rotating over distinct weight copies that together exceed the 256 MB
+Infinity Cache, with every input resident in HBM before the clock starts.
+
+Beside it:
+  roofline      the GEMV kernel against the 8 TB/s HBM peak, timed per launch with HIP events
+  mmq           the second half of the metric: Q6_K int8-MFMA GEMM at M=512 (BASELINE config 3)
+                in TOPS against the 5.03 POPS dense int8 MFMA peak, with its own roofline
+  cpu_baseline  the reference's CPU path (block dequantize + fp32 matmul) restated in numpy/torch,
+                timed on this host's cores on a bounded sample of the same workload
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
+INT8_PEAK_TOPS = 5033.0        # dense int8 MFMA, K=32/64 shapes (256 CU x 8192 op/clk x 2.4 GHz)
+INT8_LEGACY_PEAK_TOPS = 2516.0  # legacy K=16 shapes run at half that rate
+Q4_K, Q6_K = 12, 14
+CFG2_SHAPES = [(4096, 4096), (14336, 4096), (4096, 14336)]
+CFG3_SHAPES = [(18944, 3584), (3584, 18944)]
+ROTATE_BYTES = 640 << 20       # distinct weight bytes walked per rotation (> 2x the 256 MB cache)
+
+
+def _events_ms(fn, iters):
+    """Average milliseconds per call of ``fn`` over ``iters`` back-to-back calls, by HIP events on torch's
+    current stream (the stream the kernels are launched on)."""
+    import torch
+
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    torch.cuda.synchronize()
+    start.record()
+    for i in range(iters):
+        fn(i)
+    stop.record()
+    stop.synchronize()
+    return start.elapsed_time(stop) / iters
+
+
+def _graph_ms(fn, calls, replays):
+    """Same, with the calls captured once into a HIP graph and replayed, so host launch cost is excluded."""
+    import torch
+
+    for i in range(min(calls, 3)):
+        fn(i)
+    torch.cuda.synchronize()
+    g = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(g):
+        for i in range(calls):
+            fn(i)
+    g.replay()
+    torch.cuda.synchronize()
+    start = torch.cuda.Event(enable_timing=True)
+    stop = torch.cuda.Event(enable_timing=True)
+    start.record()
+    for _ in range(replays):
+        g.replay()
+    stop.record()
+    stop.synchronize()
+    return start.elapsed_time(stop) / (replays * calls)
+
+
+def main() -> int:
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=200)
+    ap.add_argument("--warmup", type=int, default=20)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-mmq", action="store_true", help="skip the Q6_K MMQ leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (the operators shard by "
+              "rows/columns of W with no communication; see DESIGN.md). Run with --gpus 1.", file=sys.stderr)
+        return 2
+
+    import torch
+
+    from vllm_gguf_plugin_prism_amd import ops, synth
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU", file=sys.stderr)
+        return 3
+    dev = torch.device("cuda:0")
+    rng = np.random.default_rng(0)
+
+    # ---------------------------------------------------------------- config 2: Q4_K batch-1 GEMV
+    mats = []
+    total_copy_bytes = sum(n * (k // 256) * 144 for n, k in CFG2_SHAPES)
+    ncopies = max(2, -(-ROTATE_BYTES // total_copy_bytes))
+    host_w = {}
+    for n, k in CFG2_SHAPES:
+        w = np.concatenate([synth.make_weights(rng, Q4_K, min(2048, n - r), k) for r in range(0, n, 2048)], axis=0)
+        host_w[(n, k)] = w
+        base = torch.from_numpy(w).to(dev)
+        copies = [base] + [base.clone() for _ in range(ncopies - 1)]
+        x = torch.from_numpy(rng.standard_normal((1, k)).astype(np.float32)).to(torch.float16).to(dev)
+        mats.append((n, k, copies, x))
+    step_bytes = sum(n * (k // 256) * 144 + 2 * k + 2 * n for n, k in CFG2_SHAPES)
+
+    def step(i):
+        for n, k, copies, x in mats:
+            ops.ggml_mul_mat_vec_a8(copies[i % ncopies], x, Q4_K, n)
+
+    for i in range(args.warmup):
+        step(i)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        step(i)
+    torch.cuda.synchronize()
+    eager_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    # the same K steps as one HIP graph: host launch cost out of the timed region
+    graph_ms = _graph_ms(step, ncopies, max(1, args.steps // ncopies)) * 1.0
+    ms_per_step = min(eager_ms, graph_ms)
+    value = step_bytes / (ms_per_step * 1e-3) / 1e9
+
+    # per-launch duration of one matrix at a time (roofline of the dominant kernel)
+    per_shape = {}
+    for n, k, copies, x in mats:
+        ms = _graph_ms(lambda i, n=n, copies=copies, x=x: ops.ggml_mul_mat_vec_a8(copies[i % ncopies], x, Q4_K, n),
+                       ncopies * 4, 10)
+        b = n * (k // 256) * 144 + 2 * k + 2 * n
+        per_shape[f"{n}x{k}"] = {"us_per_call": ms * 1e3, "GBps": b / (ms * 1e-3) / 1e9, "bytes": b}
+    big = per_shape["14336x4096"]
+    roofline = {"bound": "hbm", "achieved": big["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": big["GBps"] / HBM_PEAK_GBS, "traffic": None,
+                "kernel": "mmvq Q4_K [14336,4096] bs1 (activation quantisation + GEMV per call)",
+                "per_shape": per_shape}
+
+    out = {
+        "metric": "Q4_K GEMV HBM GB/s (% peak) @bs1; Q6_K MMQ int8 TOPS (% peak) @M=512",
+        "value": value, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "int8 dot products, fp32 accumulate, fp16 in/out", "data": "synthetic (seeded N(0,0.02) weights quantized to Q4_K, N(0,1) fp16 activations)",
+        "config": {"workload": "BASELINE config 2: Q4_K batch-1 MMVQ over [4096,4096],[14336,4096],[4096,14336]",
+                   "weight_copies_rotated": ncopies, "rotated_bytes": ncopies * total_copy_bytes,
+                   "eager_ms_per_step": eager_ms, "graph_ms_per_step": graph_ms,
+                   "pct_of_hbm_peak": 100.0 * value / HBM_PEAK_GBS},
+        "roofline": roofline,
+    }
+
+    # ---------------------------------------------------------------- config 3: Q6_K MMQ at M=512
+    if not args.no_mmq:
+        mmq = {}
+        for n, k in CFG3_SHAPES:
+            w = np.concatenate([synth.make_weights(rng, Q6_K, min(2048, n - r), k) for r in range(0, n, 2048)], axis=0)
+            wd = torch.from_numpy(w).to(dev)
+            for m in (128, 512, 2048):
+                x = torch.from_numpy(rng.standard_normal((m, k)).astype(np.float32)).to(torch.float16).to(dev)
+                for _ in range(3):
+                    ops.ggml_mul_mat_a8(wd, x, Q6_K, n)
+                ms = _events_ms(lambda i: ops.ggml_mul_mat_a8(wd, x, Q6_K, n), 20)
+                tops = 2.0 * m * n * k / (ms * 1e-3) / 1e12
+                mmq[f"{n}x{k}@M{m}"] = {"ms": ms, "TOPS": tops, "frac_int8_peak": tops / INT8_PEAK_TOPS}
+            del wd
+        m512 = [v for key, v in mmq.items() if key.endswith("@M512")]
+        ops_total = sum(2.0 * 512 * n * k for n, k in CFG3_SHAPES)
+        t_total = sum(v["ms"] for v in m512) * 1e-3
+        tops512 = ops_total / t_total / 1e12
+        out["mmq"] = {
+            "metric": "Q6_K MMQ int8 TOPS @M=512", "value": tops512, "unit": "TOPS",
+            "roofline": {"bound": "mfma", "achieved": tops512, "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
+                         "frac": tops512 / INT8_PEAK_TOPS, "traffic": None,
+                         "denominator": "5.03 POPS dense int8 (v_mfma_i32_32x32x32_i8 rate); Q6_K uses the K=16 shape, "
+                                        f"whose own peak is {INT8_LEGACY_PEAK_TOPS} TOPS",
+                         "frac_of_legacy_k16_peak": tops512 / INT8_LEGACY_PEAK_TOPS},
+            "per_shape": mmq,
+            "note": "time per call = activation quantisation kernel + MMQ kernel",
+        }
+
+    # ---------------------------------------------------------------- CPU baseline (bounded sample)
+    if not args.no_cpu:
+        from oracle import gguf_oracle as oracle  # the checker, timed as the reference's CPU path
+
+        n, k = CFG2_SHAPES[0]
+        w = host_w[(n, k)]
+        x32 = torch.from_numpy(rng.standard_normal((1, k)).astype(np.float32))
+        best = None
+        t_end = time.perf_counter() + 20.0
+        reps = 0
+        while reps < 2 or (time.perf_counter() < t_end and reps < 8):
+            t0 = time.perf_counter()
+            wd = oracle.dequantize(w, Q4_K, "f32", flavour="f32").reshape(n, k)
+            t1 = time.perf_counter()
+            _ = x32 @ torch.from_numpy(wd).T
+            t2 = time.perf_counter()
+            if reps > 0 and (best is None or t2 - t0 < best[0]):
+                best = (t2 - t0, t1 - t0, t2 - t1)
+            reps += 1
+        qbytes = n * (k // 256) * 144
+        out["cpu_baseline"] = {
+            "value": qbytes / best[0] / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
+            "sample": f"Q4_K [{n},{k}] batch 1: numpy fp32 block dequantize ({best[1] * 1e3:.1f} ms) + torch fp32 matmul "
+                      f"({best[2] * 1e3:.1f} ms), best of {reps - 1} after 1 warm-up; os.cpu_count()={os.cpu_count()}",
+        }
+
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())
