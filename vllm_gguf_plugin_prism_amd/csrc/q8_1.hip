@@ -9,39 +9,9 @@
 // lane^2 / lane^1 are the butterfly partners for masks 16 / 8 (DPP quad
 // permutes) and masks 4, 2, 1 are in-register.  The fp32 addition tree is
 // therefore the same tree the reference evaluates.
-#include "gguf_common.h"
+#include "q8_1_device.h"
 
 namespace gguf {
-
-template <typename T>
-__device__ __forceinline__ void load8(const T* p, float (&v)[8]);
-template <>
-__device__ __forceinline__ void load8<float>(const float* p, float (&v)[8]) {
-  const float4 a = *(const float4*)p, b = *(const float4*)(p + 4);
-  v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
-}
-template <>
-__device__ __forceinline__ void load8<_Float16>(const _Float16* p, float (&v)[8]) {
-  typedef _Float16 h8 __attribute__((ext_vector_type(8)));
-  const h8 a = *(const h8*)p;
-#pragma unroll
-  for (int i = 0; i < 8; ++i) v[i] = (float)a[i];
-}
-template <>
-__device__ __forceinline__ void load8<bf16_t>(const bf16_t* p, float (&v)[8]) {
-  const uint4 a = *(const uint4*)p;
-  const uint32_t w[4] = {a.x, a.y, a.z, a.w};
-#pragma unroll
-  for (int i = 0; i < 4; ++i) {
-    v[2 * i] = __builtin_bit_cast(float, w[i] << 16);
-    v[2 * i + 1] = __builtin_bit_cast(float, w[i] & 0xFFFF0000u);
-  }
-}
-
-template <int CTRL>
-__device__ __forceinline__ int dpp_mov_i(int v) {
-  return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, true);
-}
 
 template <typename T>
 __global__ __launch_bounds__(256) void quantize_q8_1_kernel(const T* __restrict__ x, char* __restrict__ ws, int K,
@@ -57,45 +27,16 @@ __global__ __launch_bounds__(256) void quantize_q8_1_kernel(const T* __restrict_
 #pragma unroll
     for (int i = 0; i < 8; ++i) v[i] = 0.0f;
   }
-  float amax = 0.0f;
-#pragma unroll
-  for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(v[i]));
-  amax = fmaxf(amax, dpp_mov<0x4E>(amax));
-  amax = fmaxf(amax, dpp_mov<0xB1>(amax));
-
-  float s[8];
-#pragma unroll
-  for (int i = 0; i < 8; ++i) s[i] = v[i] + dpp_mov<0x4E>(v[i]);  // mask 16: lane ^ 2
-#pragma unroll
-  for (int i = 0; i < 8; ++i) s[i] = s[i] + dpp_mov<0xB1>(s[i]);  // mask 8:  lane ^ 1
-  const float t0 = s[0] + s[4], t1 = s[1] + s[5], t2 = s[2] + s[6], t3 = s[3] + s[7];  // mask 4
-  const float u0 = t0 + t2, u1 = t1 + t3;                                             // mask 2
-  const float sum = u0 + u1;                                                          // mask 1
-
-  const float d = amax / 127.0f;
-  int q[8];
-  int isum = 0;
-#pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    q[i] = amax == 0.0f ? 0 : (int)roundf(v[i] / d);
-    isum += q[i];
-  }
-  isum += dpp_mov_i<0x4E>(isum);
-  isum += dpp_mov_i<0xB1>(isum);
-
+  const Q8Quad r = q8_1_quantize8(v);
   char* row = ws + m * row_bytes;
-  uint2 packed;
-  packed.x = (q[0] & 0xFF) | ((q[1] & 0xFF) << 8) | ((q[2] & 0xFF) << 16) | ((uint32_t)(q[3] & 0xFF) << 24);
-  packed.y = (q[4] & 0xFF) | ((q[5] & 0xFF) << 8) | ((q[6] & 0xFF) << 16) | ((uint32_t)(q[7] & 0xFF) << 24);
-  *(uint2*)(row + e0) = packed;
+  *(uint2*)(row + e0) = r.q;
   if ((t & 3) == 0) {
     const int b = t >> 2;
     const int nb = Kp / 32;
     float* fd = (float*)(row + Kp);
-    const float dh = (float)(_Float16)d;
-    fd[b] = dh;
-    fd[nb + b] = (float)(_Float16)sum;
-    fd[2 * nb + b] = dh * (float)isum;
+    fd[b] = r.d;
+    fd[nb + b] = r.s;
+    fd[2 * nb + b] = r.du;
   }
 }
 

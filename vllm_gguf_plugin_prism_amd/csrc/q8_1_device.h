@@ -1,0 +1,118 @@
+// q8_1 quantisation of eight consecutive activation values per lane, four lanes (one DPP quad)
+// per 32-value block.  Shared by the stand-alone quantizer and by the GEMV prologue that
+// quantizes straight into LDS.
+//
+// Reference semantics (csrc/gguf/gguf_kernel.cu:32-69): amax and sum by an xor butterfly over
+// lane masks 16, 8, 4, 2, 1; d = amax / 127 (fp32, IEEE division); q = roundf(x / d), 0 when
+// amax == 0; d and sum stored rounded to half.  With eight values per lane, masks 16 and 8 are
+// the quad partners lane^2 and lane^1 and masks 4, 2, 1 are in-register, which evaluates the
+// same fp32 addition tree.
+#pragma once
+#include "gguf_common.h"
+
+namespace gguf {
+
+// Eight consecutive activation values: raw8<T>::load only issues the global load (so it can be hoisted
+// above other loads without forcing a wait), cvt widens to fp32.
+template <typename T> struct raw8;
+template <> struct raw8<float> {
+  float4 a, b;
+  __device__ __forceinline__ void load(const float* p) { a = *(const float4*)p; b = *(const float4*)(p + 4); }
+  __device__ __forceinline__ void cvt(float (&v)[8]) const {
+    v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
+  }
+};
+template <> struct raw8<_Float16> {
+  uint4 a;
+  __device__ __forceinline__ void load(const _Float16* p) { a = *(const uint4*)p; }
+  __device__ __forceinline__ void cvt(float (&v)[8]) const {
+    const uint32_t w[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      v[2 * i] = (float)__builtin_bit_cast(_Float16, (uint16_t)(w[i] & 0xFFFF));
+      v[2 * i + 1] = (float)__builtin_bit_cast(_Float16, (uint16_t)(w[i] >> 16));
+    }
+  }
+};
+template <> struct raw8<bf16_t> {
+  uint4 a;
+  __device__ __forceinline__ void load(const bf16_t* p) { a = *(const uint4*)p; }
+  __device__ __forceinline__ void cvt(float (&v)[8]) const {
+    const uint32_t w[4] = {a.x, a.y, a.z, a.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      v[2 * i] = __builtin_bit_cast(float, w[i] << 16);
+      v[2 * i + 1] = __builtin_bit_cast(float, w[i] & 0xFFFF0000u);
+    }
+  }
+};
+template <typename T>
+__device__ __forceinline__ void load8(const T* p, float (&v)[8]) {
+  raw8<T> r;
+  r.load(p);
+  r.cvt(v);
+}
+
+template <int CTRL>
+__device__ __forceinline__ int dpp_mov_i(int v) {
+  return __builtin_amdgcn_update_dpp(0, v, CTRL, 0xF, 0xF, true);
+}
+
+struct Q8Quad {
+  uint2 q;      // this lane's eight quants
+  float d;      // block scale, half-rounded           (same in all four lanes)
+  float s;      // block sum of the inputs, half-rounded
+  float du;     // d * sum of the block's quants
+};
+
+// All four lanes of a quad must call this together.
+__device__ __forceinline__ Q8Quad q8_1_quantize8(const float (&v)[8]) {
+  float amax = 0.0f;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) amax = fmaxf(amax, fabsf(v[i]));
+  amax = fmaxf(amax, dpp_mov<0x4E>(amax));
+  amax = fmaxf(amax, dpp_mov<0xB1>(amax));
+
+  float s[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) s[i] = v[i] + dpp_mov<0x4E>(v[i]);  // mask 16: lane ^ 2
+#pragma unroll
+  for (int i = 0; i < 8; ++i) s[i] = s[i] + dpp_mov<0xB1>(s[i]);  // mask 8:  lane ^ 1
+  const float t0 = s[0] + s[4], t1 = s[1] + s[5], t2 = s[2] + s[6], t3 = s[3] + s[7];  // mask 4
+  const float u0 = t0 + t2, u1 = t1 + t3;                                             // mask 2
+  const float sum = u0 + u1;                                                          // mask 1
+
+  const float d = amax / 127.0f;
+  const float dd = amax == 0.0f ? 1.0f : d;  // an all-zero block divides 0 by 1: q = 0 without a branch
+  // q = roundf(x / dd), ties away from zero, bit-for-bit what the IEEE quotient gives.  One reciprocal per
+  // lane replaces eight divisions: x * (1/dd) is within 127 * 2^-23 of the true quotient, so it rounds the
+  // same way unless the fraction lies within 2^-14 of a tie; only then is the exact quotient formed.
+  const float rd = 1.0f / dd;
+  int q[8];
+  int isum = 0;
+#pragma unroll
+  for (int i = 0; i < 8; ++i) {
+    float t = v[i] * rd;
+    float tr = truncf(t);
+    float fr = fabsf(t - tr);
+    if (fabsf(fr - 0.5f) < 6.1035156e-5f) {
+      t = v[i] / dd;
+      tr = truncf(t);
+      fr = fabsf(t - tr);
+    }
+    q[i] = (int)tr + (fr >= 0.5f ? (t < 0.0f ? -1 : 1) : 0);
+    isum += q[i];
+  }
+  isum += dpp_mov_i<0x4E>(isum);
+  isum += dpp_mov_i<0xB1>(isum);
+
+  Q8Quad r;
+  r.q.x = (q[0] & 0xFF) | ((q[1] & 0xFF) << 8) | ((q[2] & 0xFF) << 16) | ((uint32_t)(q[3] & 0xFF) << 24);
+  r.q.y = (q[4] & 0xFF) | ((q[5] & 0xFF) << 8) | ((q[6] & 0xFF) << 16) | ((uint32_t)(q[7] & 0xFF) << 24);
+  r.d = (float)(_Float16)d;
+  r.s = (float)(_Float16)sum;
+  r.du = r.d * (float)isum;
+  return r;
+}
+
+}  // namespace gguf
