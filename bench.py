@@ -85,7 +85,12 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-mmq", action="store_true", help="skip the Q6_K MMQ leg")
+    ap.add_argument("--profile", action="store_true",
+                    help="counter-collection mode: eager launches only (no HIP graph), no CPU leg, M=512 only for "
+                         "the MMQ leg, and one 256 MiB device copy at the end to calibrate byte counters")
     args = ap.parse_args()
+    if args.profile:
+        args.no_cpu = True
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (the operators shard by "
               "rows/columns of W with no communication; see DESIGN.md). Run with --gpus 1.", file=sys.stderr)
@@ -128,15 +133,15 @@ def main() -> int:
     torch.cuda.synchronize()
     eager_ms = (time.perf_counter() - t0) * 1e3 / args.steps
     # the same K steps as one HIP graph: host launch cost out of the timed region
-    graph_ms = _graph_ms(step, ncopies, max(1, args.steps // ncopies)) * 1.0
+    graph_ms = eager_ms if args.profile else _graph_ms(step, ncopies, max(1, args.steps // ncopies))
     ms_per_step = min(eager_ms, graph_ms)
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
 
     # per-launch duration of one matrix at a time (roofline of the dominant kernel)
     per_shape = {}
     for n, k, copies, x in mats:
-        ms = _graph_ms(lambda i, n=n, copies=copies, x=x: ops.ggml_mul_mat_vec_a8(copies[i % ncopies], x, Q4_K, n),
-                       ncopies * 4, 10)
+        one = lambda i, n=n, copies=copies, x=x: ops.ggml_mul_mat_vec_a8(copies[i % ncopies], x, Q4_K, n)  # noqa: E731
+        ms = _events_ms(one, ncopies * 4) if args.profile else _graph_ms(one, ncopies * 4, 10)
         b = n * (k // 256) * 144 + 2 * k + 2 * n
         per_shape[f"{n}x{k}"] = {"us_per_call": ms * 1e3, "GBps": b / (ms * 1e-3) / 1e9, "bytes": b}
     big = per_shape["14336x4096"]
@@ -163,7 +168,7 @@ def main() -> int:
         for n, k in CFG3_SHAPES:
             w = np.concatenate([synth.make_weights(rng, Q6_K, min(2048, n - r), k) for r in range(0, n, 2048)], axis=0)
             wd = torch.from_numpy(w).to(dev)
-            for m in (128, 512, 2048):
+            for m in ((512,) if args.profile else (128, 512, 2048)):
                 x = torch.from_numpy(rng.standard_normal((m, k)).astype(np.float32)).to(torch.float16).to(dev)
                 for _ in range(3):
                     ops.ggml_mul_mat_a8(wd, x, Q6_K, n)
@@ -211,6 +216,15 @@ def main() -> int:
             "sample": f"Q4_K [{n},{k}] batch 1: numpy fp32 block dequantize ({best[1] * 1e3:.1f} ms) + torch fp32 matmul "
                       f"({best[2] * 1e3:.1f} ms), best of {reps - 1} after 1 warm-up; os.cpu_count()={os.cpu_count()}",
         }
+
+    if args.profile:
+        # one plain device-to-device copy of known size: its FETCH_SIZE / WRITE_SIZE readings give the scale of
+        # those counters on this machine (268435456 bytes read, 268435456 bytes written)
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=dev)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        out["config"]["calibration_copy_bytes"] = 256 << 20
 
     print(json.dumps(out))
     return 0

@@ -1,0 +1,81 @@
+"""The C-ABI library loads without a GPU and exports exactly what include/gguf_hip.h declares."""
+import ctypes
+import re
+from pathlib import Path
+
+import pytest
+
+from vllm_gguf_plugin_prism_amd import _lib
+
+ROOT = Path(__file__).resolve().parent.parent
+HEADER = ROOT / "include" / "gguf_hip.h"
+
+# (elements, bytes) per block for every ggml type id of the reference's tables (triton/gemm/utils.py:28-47)
+BLOCK_SIZES = {
+    2: (32, 18), 3: (32, 20), 6: (32, 22), 7: (32, 24), 8: (32, 34),
+    10: (256, 84), 11: (256, 110), 12: (256, 144), 13: (256, 176), 14: (256, 210),
+    16: (256, 66), 17: (256, 74), 18: (256, 98), 19: (256, 50), 20: (32, 18), 21: (256, 110), 22: (256, 82),
+    23: (256, 136), 29: (256, 56),
+}
+
+
+def declared_symbols():
+    text = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
+    return sorted(set(re.findall(r"\b(gguf_[a-z0-9_]+)\s*\(", text)))
+
+
+@pytest.fixture(scope="module")
+def handle():
+    if not _lib.LIB_PATH.exists():
+        from vllm_gguf_plugin_prism_amd import build
+
+        build.build()
+    return _lib.lib()
+
+
+def test_header_declares_the_bound_entry_points():
+    assert declared_symbols() == sorted(_lib.EXPORTS)
+    assert len(declared_symbols()) == 12
+
+
+def test_every_declared_symbol_is_exported(handle):
+    raw = ctypes.CDLL(str(_lib.LIB_PATH))
+    for name in declared_symbols():
+        assert hasattr(raw, name), name
+
+
+def test_version_names_the_target(handle):
+    assert b"gfx950" in handle.gguf_hip_version()
+
+
+def test_block_sizes_match_the_format_table(handle):
+    for qt, (qk, nbytes) in BLOCK_SIZES.items():
+        assert (handle.gguf_block_elems(qt), handle.gguf_block_bytes(qt)) == (qk, nbytes), qt
+    for qt in (0, 1, 4, 5, 9, 15, 24, 30, 99, -3):
+        assert handle.gguf_block_elems(qt) == 0 and handle.gguf_block_bytes(qt) == 0
+
+
+def test_workspace_row_bytes(handle):
+    # 44 bytes per 32 values of K rounded up to 512 (int8 quants + three fp32 per block)
+    assert handle.gguf_q8_1_row_bytes(4096) == 4096 // 32 * 44
+    assert handle.gguf_q8_1_row_bytes(256) == 512 // 32 * 44
+    assert handle.gguf_q8_1_row_bytes(14336) == 14336 // 32 * 44
+    assert handle.gguf_q8_1_row_bytes(0) == 0
+
+
+def test_moe_block_size(handle):
+    for qt in (2, 8, 12, 14):
+        assert handle.gguf_moe_block_size(qt) == 32
+    assert handle.gguf_moe_block_size(99) == 0
+
+
+def test_argument_validation_needs_no_gpu(handle):
+    """Bad calls are rejected before any HIP call is made, so this runs on a machine without a GPU."""
+    assert handle.gguf_dequantize(None, 99, None, 1, 256, None) == -1      # unknown type
+    assert handle.gguf_dequantize(None, 12, None, 1, 100, None) == -3      # not a multiple of 256
+    assert handle.gguf_dequantize(None, 12, None, 7, 256, None) == -2      # dtype code
+    assert handle.gguf_dequantize(None, 12, None, 1, 256, None) == -4      # null pointers
+    assert handle.gguf_dequantize(None, 12, None, 1, 0, None) == 0         # empty is fine
+    assert handle.gguf_mmvq(None, None, 1, None, None, 99, 16, 256, 1, None) == -1
+    assert handle.gguf_mmvq(None, None, 1, None, None, 12, 16, 100, 1, None) == -3
+    assert handle.gguf_mmq(None, None, 1, None, None, 23, 16, 256, 1, None) in (-1, -4)

@@ -1,0 +1,81 @@
+"""The callers' layer on the GPU: dense dispatch, the two-stage MoE pipeline and embedding lookup,
+each checked against the numpy oracle (the in-tree definition of the MoE result is the per-token
+loop at quantization/fused_moe.py:119-132)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import gguf_oracle as o
+from vllm_gguf_plugin_prism_amd import dispatch as D
+from vllm_gguf_plugin_prism_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+
+def _moe_oracle(x, w1, w2, tw, ids, qt, qt2, path):
+    """Two-stage MoE in fp64 with the activations re-quantised to q8_1 before each GEMM, as the kernels see them.
+    The intermediate is rounded to fp16 where the device stores it."""
+    tokens, top_k = ids.shape
+    n1, n2 = w1.shape[1], w2.shape[1]
+    h = o.moe_a8_vec(x, w1, ids.reshape(-1), top_k, qt, n1, tokens) if path == "vec" else None
+    if h is None:
+        blk = 32
+        s, e, n = o.moe_align_block_size(ids, blk, w1.shape[0])
+        h = o.moe_a8(x, w1, s, e, n, qt, n1, top_k, tokens, blk)
+    h = h.astype(np.float16)
+    a = o.silu_and_mul(h.astype(np.float64)).astype(np.float16)
+    y = o.moe_a8_vec(a, w2, ids.reshape(-1), 1, qt2, n2, tokens * top_k).astype(np.float16).astype(np.float64)
+    y = y.reshape(tokens, top_k, n2) * tw.astype(np.float16).astype(np.float64)[:, :, None]
+    return y.astype(np.float16).astype(np.float64).sum(1)
+
+
+@pytest.mark.parametrize("tokens,expected_path", [(1, "vec"), (9, "vec"), (96, "grouped")])
+def test_fused_moe_pipeline_q4_0(tokens, expected_path):
+    """Reduced shape of the Q4_0 MoE config: 8 experts, hidden 512, intermediate 256, top-2."""
+    rng = np.random.default_rng(tokens)
+    E, H, I, top_k = 8, 512, 256, 2
+    w1 = np.stack([synth.make_weights(rng, o.Q4_0, 2 * I, H) for _ in range(E)])
+    w2 = np.stack([synth.make_weights(rng, o.Q4_0, H, I) for _ in range(E)])
+    # weights ~N(0,0.02) give tiny activations; scale x so intermediate values are O(1)
+    x = (rng.standard_normal((tokens, H)) * 4).astype(np.float16)
+    logits = rng.standard_normal((tokens, E))
+    ids = np.argsort(-logits, axis=1)[:, :top_k].astype(np.int32)
+    sel = np.take_along_axis(logits, ids, 1)
+    tw = (np.exp(sel) / np.exp(sel).sum(1, keepdims=True)).astype(np.float32)
+    assert D.select_moe_path(o.Q4_0, o.Q4_0, tokens) == expected_path
+    got = D.fused_moe_gguf(torch.from_numpy(x).cuda(), torch.from_numpy(w1).cuda(), torch.from_numpy(w2).cuda(),
+                           torch.from_numpy(tw).cuda().half(), torch.from_numpy(ids).cuda(), o.Q4_0, o.Q4_0, "silu")
+    torch.cuda.synchronize()
+    assert got.shape == (tokens, H) and got.dtype == torch.float16
+    want = _moe_oracle(x, w1, w2, tw, ids, o.Q4_0, o.Q4_0, expected_path)
+    # fp16 storage between stages and the re-quantisation of a slightly different intermediate bound the error
+    assert o.rel_l2(got.float().cpu().numpy(), want) <= 1e-2
+
+
+@pytest.mark.parametrize("qt,batch,rows,path", [(o.Q4_K, 2, 64, "mmvq"), (o.Q4_K, 7, 64, "mmq"),
+                                                (o.IQ4_XS, 3, 64, "mmvq"), (o.IQ4_XS, 40, 64, "dequant")])
+def test_fused_mul_mat_routes(qt, batch, rows, path):
+    rng = np.random.default_rng(rows + batch)
+    k = 512
+    w = synth.make_weights(rng, qt, rows, k)
+    x = rng.standard_normal((batch, k)).astype(np.float16)
+    assert D.select_mul_mat_path(qt, batch, rows) == path
+    got = D.fused_mul_mat_gguf(torch.from_numpy(x).cuda(), torch.from_numpy(w).cuda(), qt).float().cpu().numpy()
+    if path == "dequant":
+        want = o.mul_mat_f32(w, x, qt, rows)
+        assert o.rel_l2(got, want) <= 2e-3          # fp16 dense GEMM on exactly dequantised weights
+    else:
+        want = o.mul_mat_a8(w, x, qt, rows, path=path)
+        assert o.rel_l2(got, want) <= 1e-3
+
+
+@pytest.mark.parametrize("qt", [o.Q8_0, o.Q4_K, o.IQ2_XXS])
+def test_embedding_lookup_is_gather_of_exact_dequant(qt):
+    rng = np.random.default_rng(qt)
+    vocab, hidden = 50, 512
+    table = synth.make_weights(rng, qt, vocab, hidden)
+    ids = rng.integers(0, vocab, size=(3, 5))
+    got = D.apply_gguf_embedding(torch.from_numpy(ids).cuda(), torch.from_numpy(table).cuda(), qt, hidden, torch.float16)
+    assert got.shape == (3, 5, hidden)
+    dense = o.dequantize(table, qt, "f16").reshape(vocab, hidden)
+    assert np.array_equal(got.cpu().numpy().view(np.uint16), dense[ids].view(np.uint16))
