@@ -7,10 +7,13 @@
 // (csrc/gguf/mmq.cuh:2-104, vecdotq.cuh load_tiles_* / vec_dot_*_mul_mat).  Here S is
 // one v_mfma_i32_32x32x32_i8 per 32x32 output tile and 32-element block (two
 // v_mfma_i32_32x32x16_i8 for formats whose weight scale changes every 16 elements), and
-// the vector ALU only rescales: convert, multiply by the activation scale, fused
-// multiply-add with the weight scale into an fp32 accumulator.
+// the vector ALU only rescales: per result one fused multiply-add with the weight scale
+// (which also turns the int32 into fp32, see seeded_times) and one with the activation
+// scale into an fp32 accumulator, plus one for formats with an offset term.  On this
+// chip an MFMA and vector-ALU work of other waves on the same SIMD do not run at the
+// same time, so those two or three instructions per result, not the MFMA, set the pace.
 //
-// Work split: a workgroup of four waves owns an (M_T x N_T) output tile and walks K in
+// Work split: a workgroup of four or eight waves owns an (M_T x N_T) output tile and walks K in
 // steps of 128 elements.  Per step it stages the q8_1 activations (int8 + block scales)
 // and unpacks the GGUF blocks of its N_T weight rows to plain int8 + per-block fp32
 // scales in LDS; every wave then owns a (32*TM x 32*TN) sub-tile.  MFMA operands:
@@ -29,14 +32,53 @@ namespace gguf {
 typedef int v4i __attribute__((ext_vector_type(4)));
 typedef int v16i __attribute__((ext_vector_type(16)));
 
-// The element is taken by value first: a bit cast applied directly to a vector element expression reads
-// element 0 with this compiler.
-__device__ __forceinline__ float carrier_to_float(int bits) { return __int_as_float(bits) - 12582912.0f; }
+// int32 MFMA results reach fp32 without a convert instruction.  Every MFMA accumulates onto the bit pattern of
+// the float kSeed = 1.5 * 2^23, whose unit in the last place is 1: for |S| < 2^22 (32 products of int8 stay below
+// 2^19) the integer sum kSeedBits + S is the bit pattern of the float kSeed + S.  One fused multiply-add then gives
+//   fma(kSeed + S, dw, -kSeed * dw) = RN(S * dw)
+// exactly, because kSeed * dw is exact in fp32 whenever dw has at most 22 significant bits, and every weight scale
+// here is an fp16 value times an integer of at most 8 bits.  v_cvt_f32_i32 issues at half the rate of v_fma_f32.
+constexpr float kSeed = 12582912.0f;
+constexpr int kSeedBits = 0x4B400000;
+// Takes the MFMA element by value: a bit cast applied directly to a vector element expression reads element 0
+// with this compiler.
+__device__ __forceinline__ float seeded_times(int bits, float dw, float neg_seed_dw) {
+  return __builtin_fmaf(__int_as_float(bits), dw, neg_seed_dw);
+}
 
-constexpr int KS = 128;     // K elements per step
+// acc += v[lane (l & ~3) + T] * c : a fused multiply-add whose first factor is taken from lane T of the caller's
+// quad by DPP.  In the 32x32 MFMA result layout register r of lane l is row 8*(r/4) + 4*(l/32) + r%4, so when lane l
+// holds a per-row factor for row 8*g + 4*(l/32) + l%4, the factor of register 4*g + T sits in lane T of every quad:
+// four registers hold what sixteen would, and they cost four 4-byte LDS reads instead of four 16-byte ones.
+// The factor registers are written by LDS loads only, so no VALU-write-to-DPP-read wait states are needed.
+template <int T>
+__device__ __forceinline__ void fmac_quad(float& acc, float v, float c) {
+  static_assert(T >= 0 && T < 4, "lane within the quad");
+  if constexpr (T == 0) asm("v_fmac_f32_dpp %0, %1, %2 quad_perm:[0,0,0,0] row_mask:0xf bank_mask:0xf" : "+v"(acc) : "v"(v), "v"(c));
+  if constexpr (T == 1) asm("v_fmac_f32_dpp %0, %1, %2 quad_perm:[1,1,1,1] row_mask:0xf bank_mask:0xf" : "+v"(acc) : "v"(v), "v"(c));
+  if constexpr (T == 2) asm("v_fmac_f32_dpp %0, %1, %2 quad_perm:[2,2,2,2] row_mask:0xf bank_mask:0xf" : "+v"(acc) : "v"(v), "v"(c));
+  if constexpr (T == 3) asm("v_fmac_f32_dpp %0, %1, %2 quad_perm:[3,3,3,3] row_mask:0xf bank_mask:0xf" : "+v"(acc) : "v"(v), "v"(c));
+}
+template <int R>
+__device__ __forceinline__ void fmac_row(float& acc, const float (&v)[4], float c) { fmac_quad<R & 3>(acc, v[R >> 2], c); }
+
+// acc[r] += v[row of r] * c[r]  and  acc[r] += v[row of r] * c  over the 16 registers of one MFMA result
+__device__ __forceinline__ void rescale16(float (&acc)[16], const float (&v)[4], const float (&c)[16]) {
+  fmac_row<0>(acc[0], v, c[0]);    fmac_row<1>(acc[1], v, c[1]);    fmac_row<2>(acc[2], v, c[2]);    fmac_row<3>(acc[3], v, c[3]);
+  fmac_row<4>(acc[4], v, c[4]);    fmac_row<5>(acc[5], v, c[5]);    fmac_row<6>(acc[6], v, c[6]);    fmac_row<7>(acc[7], v, c[7]);
+  fmac_row<8>(acc[8], v, c[8]);    fmac_row<9>(acc[9], v, c[9]);    fmac_row<10>(acc[10], v, c[10]); fmac_row<11>(acc[11], v, c[11]);
+  fmac_row<12>(acc[12], v, c[12]); fmac_row<13>(acc[13], v, c[13]); fmac_row<14>(acc[14], v, c[14]); fmac_row<15>(acc[15], v, c[15]);
+}
+__device__ __forceinline__ void offset16(float (&acc)[16], const float (&v)[4], float c) {
+  fmac_row<0>(acc[0], v, c);   fmac_row<1>(acc[1], v, c);   fmac_row<2>(acc[2], v, c);   fmac_row<3>(acc[3], v, c);
+  fmac_row<4>(acc[4], v, c);   fmac_row<5>(acc[5], v, c);   fmac_row<6>(acc[6], v, c);   fmac_row<7>(acc[7], v, c);
+  fmac_row<8>(acc[8], v, c);   fmac_row<9>(acc[9], v, c);   fmac_row<10>(acc[10], v, c); fmac_row<11>(acc[11], v, c);
+  fmac_row<12>(acc[12], v, c); fmac_row<13>(acc[13], v, c); fmac_row<14>(acc[14], v, c); fmac_row<15>(acc[15], v, c);
+}
+
 // LDS row pitch in bytes.  K=32 operands are read 16 bytes per lane: a 16-byte skew (144) spreads 8 consecutive rows
 // over all banks.  K=16 operands are read 8 bytes per lane: an 8-byte skew (136) spreads 16 consecutive rows.
-template <int G> struct Pitch { static constexpr int value = G == 32 ? KS + 16 : KS + 8; };
+template <int G, int KS> struct Pitch { static constexpr int value = G == 32 ? KS + 16 : KS + 8; };
 
 // --------------------------------------------------------------------------------------------
 // Format policies: unpack one 32-element block of one weight row to int8 (8 dwords, element order)
@@ -48,6 +90,7 @@ template <int G> struct Pitch { static constexpr int value = G == 32 ? KS + 16 :
 struct MQ4_0 {  // vecdotq.cuh:46-66, 511-571
   static constexpr int QK = 32, BS = 18, G = 32;
   static constexpr bool HAS_MIN = true;
+  static constexpr bool LIGHT = true;  // packed block small enough to hold a step of them in registers
   struct Raw { uint16_t d; uint4 q; };
   static __device__ __forceinline__ Raw fetch(const uint8_t* row, int kb) {
     const uint8_t* b = row + (int64_t)kb * BS;
@@ -64,6 +107,7 @@ struct MQ4_0 {  // vecdotq.cuh:46-66, 511-571
 struct MQ8_0 {  // vecdotq.cuh:165-177, 869-921
   static constexpr int QK = 32, BS = 34, G = 32;
   static constexpr bool HAS_MIN = false;
+  static constexpr bool LIGHT = true;  // packed block small enough to hold a step of them in registers
   struct Raw { uint16_t d; uint4 q0, q1; };
   static __device__ __forceinline__ Raw fetch(const uint8_t* row, int kb) {
     const uint8_t* b = row + (int64_t)kb * BS;
@@ -78,6 +122,7 @@ struct MQ8_0 {  // vecdotq.cuh:165-177, 869-921
 struct MQ4_K {  // vecdotq.cuh:353-379, 1204-1277
   static constexpr int QK = 256, BS = 144, G = 32;
   static constexpr bool HAS_MIN = true;
+  static constexpr bool LIGHT = false;  // packed block small enough to hold a step of them in registers
   struct Raw { uint4 hdr, v0, v1; };
   static __device__ __forceinline__ Raw fetch(const uint8_t* row, int kb) {
     const int sb = kb >> 3, j = kb & 7;
@@ -108,6 +153,7 @@ struct MQ4_K {  // vecdotq.cuh:353-379, 1204-1277
 struct MQ6_K {  // vecdotq.cuh:467-491, 1443-1529: two int8 sub-scales per q8_1 block
   static constexpr int QK = 256, BS = 210, G = 16;
   static constexpr bool HAS_MIN = false;
+  static constexpr bool LIGHT = false;  // packed block small enough to hold a step of them in registers
   struct Raw { uint4 l0, l1, h0, h1; uint16_t sc, d; };
   static __device__ __forceinline__ Raw fetch(const uint8_t* row, int kb) {
     const int sb = kb >> 3, h = (kb >> 2) & 1, t = kb & 3;
@@ -149,6 +195,7 @@ __device__ __forceinline__ int lut16q(uint32_t idx) {  // kvalues_iq4nl lookup o
 struct MIQ4_XS {  // extension: the reference has no MMQ tiles for i-quants (gguf_kernel.cu:236-287)
   static constexpr int QK = 256, BS = 136, G = 32;
   static constexpr bool HAS_MIN = false;
+  static constexpr bool LIGHT = true;  // packed block small enough to hold a step of them in registers
   struct Raw { uint2 hdr; uint4 v; };
   static __device__ __forceinline__ Raw fetch(const uint8_t* row, int kb) {
     const int sb = kb >> 3, ib = kb & 7;
@@ -169,6 +216,7 @@ struct MIQ4_XS {  // extension: the reference has no MMQ tiles for i-quants (ggu
 struct MIQ2_XXS {  // extension, see MIQ4_XS
   static constexpr int QK = 256, BS = 66, G = 32;
   static constexpr bool HAS_MIN = false;
+  static constexpr bool LIGHT = false;  // packed block small enough to hold a step of them in registers
   struct Raw { uint16_t d; uint2 g; };
   static __device__ __forceinline__ Raw fetch(const uint8_t* row, int kb) {
     const int sb = kb >> 3, ib = kb & 7;
@@ -197,6 +245,14 @@ struct MIQ2_XXS {  // extension, see MIQ4_XS
 };
 
 // --------------------------------------------------------------------------------------------
+// LDS bytes of one group's tiles: int8 activations and weights, then their block scales (a multiple of 16).
+template <class F, int WM, int WN, int TM, int TN, int KS>
+__host__ __device__ constexpr size_t mmq_group_lds_bytes() {
+  constexpr int M_T = 32 * WM * TM, N_T = 32 * WN * TN, KB = KS / 32;
+  return (size_t)(M_T + N_T) * Pitch<F::G, KS>::value + (size_t)KB * M_T * 4 * (F::HAS_MIN ? 2 : 1) +
+         (size_t)(KS / F::G) * N_T * 4 + (F::HAS_MIN ? (size_t)KB * N_T * 4 : 0);
+}
+
 struct MoeArgs {
   const int32_t* sorted_token_ids;
   const int32_t* expert_ids;
@@ -206,28 +262,42 @@ struct MoeArgs {
   int num_pairs;          // tokens * top_k
 };
 
-template <class F, int WM, int WN, int TM, int TN, typename T, bool MOE>
-__global__ __launch_bounds__(64 * WM * WN, 2) void mmq_kernel(const uint8_t* __restrict__ W, const char* __restrict__ ws,
-                                                       T* __restrict__ Y, int M, int N, int K, int64_t ws_row_bytes,
-                                                       MoeArgs moe) {
-  constexpr int NT = 64 * WM * WN;       // threads per workgroup
-  constexpr int LDK = Pitch<F::G>::value;
+// MODE selects how staging and contraction overlap:
+//   MODE_PREFETCH  the next step's global loads are issued before this step's MFMA phase and held in registers;
+//   MODE_PLAIN     load, stage, contract in turn; latency is covered only by other workgroups on the CU;
+//   MODE_PINGPONG  the workgroup is two groups of WM*WN waves with private LDS tiles, side by side in N.  The
+//                  groups run half a period apart, separated by workgroup barriers: while one waits for its
+//                  global loads and unpacks them, the other runs its MFMA + rescale phase, so the vector ALU
+//                  (the bound of this kernel) always has a group to work for.
+enum { MODE_PREFETCH = 0, MODE_PLAIN = 1, MODE_PINGPONG = 2 };
+
+template <class F, int WM, int WN, int TM, int TN, int KS, int OCC, int MODE, typename T, bool MOE>
+__global__ __launch_bounds__(64 * WM * WN * (MODE == MODE_PINGPONG ? 2 : 1), OCC) void mmq_kernel(const uint8_t* __restrict__ W, const char* __restrict__ ws,
+                                                         T* __restrict__ Y, int M, int N, int K, int64_t ws_row_bytes,
+                                                         MoeArgs moe) {
+  constexpr int NT = 64 * WM * WN;       // threads per group (the whole workgroup unless MODE_PINGPONG)
+  constexpr int KB = KS / 32;            // q8_1 blocks per step
+  constexpr int GR = KS / 16;            // 16-byte granules per activation row and step
+  constexpr int LDK = Pitch<F::G, KS>::value;
   constexpr int M_T = 32 * WM * TM, N_T = 32 * WN * TN;
   constexpr int NG = KS / F::G;          // weight scales per row per step
-  constexpr int AQ = (M_T * 8 + NT - 1) / NT;  // 8-byte/16-byte activation granules per thread and step
-  constexpr int AS = (M_T * 4 + NT - 1) / NT;  // activation block scales per thread and step
-  constexpr int WP = (N_T * 4 + NT - 1) / NT;  // (weight row, 32-block) pairs per thread and step
+  constexpr int AQ = (M_T * GR + NT - 1) / NT;  // activation granules per thread and step
+  constexpr int AS = (M_T * KB + NT - 1) / NT;  // activation block scales per thread and step
+  constexpr int WP = (N_T * KB + NT - 1) / NT;  // (weight row, 32-block) pairs per thread and step
+  static_assert(!(MOE && MODE == MODE_PINGPONG), "the grouped variant has no ping-pong form");
   extern __shared__ __align__(16) char smem[];
-  int8_t* xq = (int8_t*)smem;                       // [M_T][LDK]
+  const int group = MODE == MODE_PINGPONG ? (int)threadIdx.x / NT : 0;  // wave-uniform
+  int8_t* xq = (int8_t*)smem + (size_t)group * mmq_group_lds_bytes<F, WM, WN, TM, TN, KS>();  // [M_T][LDK]
   int8_t* wq = xq + M_T * LDK;                      // [N_T][LDK]
-  float* xd = (float*)(wq + N_T * LDK);             // [4][M_T]   q8_1 block scales
-  float* xa = xd + 4 * M_T;                         // [4][M_T]   q8_1 block sums (HAS_MIN)
-  float* wsc = xa + (F::HAS_MIN ? 4 * M_T : 0);     // [NG][N_T]
-  float* wmn = wsc + NG * N_T;                      // [4][N_T]   (HAS_MIN)
+  float* xd = (float*)(wq + N_T * LDK);             // [KB][M_T]  q8_1 block scales
+  float* xa = xd + KB * M_T;                        // [KB][M_T]  q8_1 block sums (HAS_MIN)
+  float* wsc = xa + (F::HAS_MIN ? KB * M_T : 0);    // [NG][N_T]
+  float* wmn = wsc + NG * N_T;                      // [KB][N_T]  (HAS_MIN)
 
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+  const int tid = (int)threadIdx.x - group * NT, wave = tid >> 6, lane = tid & 63;  // indices inside the group
   const int wm = wave / WN, wn = wave % WN;
-  const int m_base = blockIdx.y * M_T, n_base = blockIdx.x * N_T;
+  const int m_base = blockIdx.y * M_T;
+  const int n_base = MODE == MODE_PINGPONG ? (blockIdx.x * 2 + group) * N_T : blockIdx.x * N_T;
   const int Kp = (int)q8_kp(K);
   const int64_t rowbytes = (int64_t)(K / F::QK) * F::BS;
   const int nkb_total = K >> 5;
@@ -245,9 +315,9 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void mmq_kernel(const uint8_t* __r
   bool aq_ok[AQ];
 #pragma unroll
   for (int i = 0; i < AQ; ++i) {
-    const int p = tid + NT * i, m = min(p >> 3, M_T - 1), g = p & 7;
+    const int p = tid + NT * i, m = min(p / GR, M_T - 1), g = p % GR;
     int src = m_base + m;
-    bool ok = p < M_T * 8;
+    bool ok = p < M_T * GR;
     if (MOE) {
       const int pair = moe.sorted_token_ids[src];
       ok = ok && pair < moe.num_pairs;
@@ -262,9 +332,9 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void mmq_kernel(const uint8_t* __r
   bool as_ok[AS];
 #pragma unroll
   for (int i = 0; i < AS; ++i) {
-    const int p = tid + NT * i, m = min(p >> 2, M_T - 1), kb = p & 3;
+    const int p = tid + NT * i, m = min(p / KB, M_T - 1), kb = p % KB;
     int src = m_base + m;
-    bool ok = p < M_T * 4;
+    bool ok = p < M_T * KB;
     if (MOE) {
       const int pair = moe.sorted_token_ids[src];
       ok = ok && pair < moe.num_pairs;
@@ -278,7 +348,7 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void mmq_kernel(const uint8_t* __r
   const uint8_t* w_src[WP];
 #pragma unroll
   for (int i = 0; i < WP; ++i) {
-    const int p = tid + NT * i, n = min(p >> 2, N_T - 1);
+    const int p = tid + NT * i, n = min(p / KB, N_T - 1);
     w_src[i] = W + (int64_t)min(n_base + n, N - 1) * rowbytes;
   }
 
@@ -287,6 +357,9 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void mmq_kernel(const uint8_t* __r
   typename F::Raw r_w[WP];
 
   auto fetch = [&](int k0) {
+#ifdef GGUF_DBG_NOFETCH
+    if (k0 > 0 && K > 0) return;
+#endif
     const int kb0 = k0 >> 5;
 #pragma unroll
     for (int i = 0; i < AQ; ++i) r_aq[i] = *(const uint4*)(aq_src[i] + k0);  // q8 rows are padded to 512, always readable
@@ -297,16 +370,19 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void mmq_kernel(const uint8_t* __r
     }
 #pragma unroll
     for (int i = 0; i < WP; ++i) {
-      const int kb = min(kb0 + ((tid + NT * i) & 3), nkb_total - 1);  // clamped: a step past K re-reads the last block
+      const int kb = min(kb0 + ((tid + NT * i) % KB), nkb_total - 1);  // clamped: a step past K re-reads the last block
       r_w[i] = F::fetch(w_src[i], kb);
     }
   };
   auto stash = [&](int k0) {
+#ifdef GGUF_DBG_NOSTASH
+    if (k0 > 0 && K > 0) return;
+#endif
     const int kb0 = k0 >> 5;
 #pragma unroll
     for (int i = 0; i < AQ; ++i) {
-      const int p = tid + NT * i, m = p >> 3, g = p & 7;
-      if (p < M_T * 8) {
+      const int p = tid + NT * i, m = p / GR, g = p % GR;
+      if (p < M_T * GR) {
         const bool ok = aq_ok[i] && kb0 + (g >> 1) < nkb_total;
         const uint4 v = ok ? r_aq[i] : make_uint4(0, 0, 0, 0);
         if (LDK % 16 == 0) {
@@ -319,8 +395,8 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void mmq_kernel(const uint8_t* __r
     }
 #pragma unroll
     for (int i = 0; i < AS; ++i) {
-      const int p = tid + NT * i, m = p >> 2, kb = p & 3;
-      if (p < M_T * 4) {
+      const int p = tid + NT * i, m = p / KB, kb = p % KB;
+      if (p < M_T * KB) {
         const bool ok = as_ok[i] && kb0 + kb < nkb_total;
         xd[kb * M_T + m] = ok ? r_ad[i] : 0.0f;
         if (F::HAS_MIN) xa[kb * M_T + m] = ok ? r_aa[i] : 0.0f;
@@ -328,8 +404,8 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void mmq_kernel(const uint8_t* __r
     }
 #pragma unroll
     for (int i = 0; i < WP; ++i) {
-      const int p = tid + NT * i, n = p >> 2, kb = p & 3;
-      if (p >= N_T * 4) continue;
+      const int p = tid + NT * i, n = p / KB, kb = p % KB;
+      if (p >= N_T * KB) continue;
       uint32_t q[8];
       float s0, s1, mn;
       F::unpack(r_w[i], kb0 + kb, q, s0, s1, mn);
@@ -365,97 +441,110 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void mmq_kernel(const uint8_t* __r
 
   const int lrow = lane & 31, lhalf = lane >> 5;
 
-  // int32 -> fp32 without a convert: the MFMA accumulates onto 0x4B400000 in every element, so the integer
-  // result S (|S| < 2^22 for 32 products of int8) comes out as the bit pattern of the float 12582912 + S,
-  // and one exact fp32 subtraction recovers S.  v_cvt_f32_i32 issues at half the rate of v_sub_f32 here.
-  v16i carrier;
+  v16i seed;
 #pragma unroll
-  for (int r = 0; r < 16; ++r) carrier[r] = 0x4B400000;
+  for (int r = 0; r < 16; ++r) seed[r] = kSeedBits;
 
-  fetch(0);
-  stash(0);
-  __syncthreads();
-
-  for (int k0 = 0; k0 < K; k0 += KS) {
-    const bool more = k0 + KS < K;
-#ifdef GGUF_DBG_NOFETCH
-    if (more && K < 0) fetch(k0 + KS);
-#else
-    if (more) fetch(k0 + KS);  // next step's global loads fly during this step's MFMA phase
-#endif
-
-    // ---- contract this step from LDS
-#ifdef GGUF_DBG_NOCOMPUTE
-    if (K < 0)
-#endif
-#pragma unroll 1
-    for (int kb = 0; kb < 4; ++kb) {
-      float d8[TM][16];
-      float a8[TM][16];
-      v4i af[TM];
+  // one 32-element block of the step in LDS -> accumulators
+  auto contract = [&](int kb) {
+    float d8[TM][4];   // q8_1 scale of row 8*g + 4*lhalf + lane%4 of tile j, one register per g (see fmac_quad)
+    float a8[TM][4];   // q8_1 stored sum, same arrangement
+    v4i af[TM];
 #pragma unroll
-      for (int j = 0; j < TM; ++j) {
-        const int mrow = 32 * (wm * TM + j);
-        if (F::G == 32) af[j] = *(const v4i*)(xq + (mrow + lrow) * LDK + 32 * kb + 16 * lhalf);
+    for (int j = 0; j < TM; ++j) {
+      const int mrow = 32 * (wm * TM + j);
+      if (F::G == 32) af[j] = *(const v4i*)(xq + (mrow + lrow) * LDK + 32 * kb + 16 * lhalf);
 #pragma unroll
-        for (int g = 0; g < 4; ++g) {
-          const float4 v = *(const float4*)(xd + kb * M_T + mrow + 8 * g + 4 * lhalf);
-          d8[j][4 * g] = v.x; d8[j][4 * g + 1] = v.y; d8[j][4 * g + 2] = v.z; d8[j][4 * g + 3] = v.w;
-          if (F::HAS_MIN) {
-            const float4 u = *(const float4*)(xa + kb * M_T + mrow + 8 * g + 4 * lhalf);
-            a8[j][4 * g] = u.x; a8[j][4 * g + 1] = u.y; a8[j][4 * g + 2] = u.z; a8[j][4 * g + 3] = u.w;
-          }
-        }
+      for (int g = 0; g < 4; ++g) {
+        d8[j][g] = xd[kb * M_T + mrow + 8 * g + 4 * lhalf + (lane & 3)];
+        if (F::HAS_MIN) a8[j][g] = xa[kb * M_T + mrow + 8 * g + 4 * lhalf + (lane & 3)];
       }
+    }
 #pragma unroll
-      for (int i = 0; i < TN; ++i) {
-        const int ncol = 32 * (wn * TN + i) + lrow;
-        if (F::G == 32) {
-          const v4i bf = *(const v4i*)(wq + ncol * LDK + 32 * kb + 16 * lhalf);
-          const float dw = wsc[kb * N_T + ncol];
-          const float mw = F::HAS_MIN ? wmn[kb * N_T + ncol] : 0.0f;
+    for (int i = 0; i < TN; ++i) {
+      const int ncol = 32 * (wn * TN + i) + lrow;
+      if (F::G == 32) {
+        const v4i bf = *(const v4i*)(wq + ncol * LDK + 32 * kb + 16 * lhalf);
+        const float dw = wsc[kb * N_T + ncol];
+        const float neg_mw = F::HAS_MIN ? -wmn[kb * N_T + ncol] : 0.0f;
+        const float neg_seed_dw = -kSeed * dw;
 #pragma unroll
-          for (int j = 0; j < TM; ++j) {
-            const v16i s = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[j], bf, carrier, 0, 0, 0);
+        for (int j = 0; j < TM; ++j) {
+          const v16i s = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[j], bf, seed, 0, 0, 0);
+          float c[16];
 #pragma unroll
-            for (int r = 0; r < 16; ++r) {
-              const float f = carrier_to_float(s[r]);  // exact int -> float
-              acc[j][i][r] = __builtin_fmaf(f * dw, d8[j][r], acc[j][i][r]);
-              if (F::HAS_MIN) acc[j][i][r] = __builtin_fmaf(-a8[j][r], mw, acc[j][i][r]);
-            }
+          for (int r = 0; r < 16; ++r) c[r] = seeded_times(s[r], dw, neg_seed_dw);  // = RN(S * dw)
+          rescale16(acc[j][i], d8[j], c);
+          if (F::HAS_MIN) offset16(acc[j][i], a8[j], neg_mw);
+        }
+      } else {
+        // weight scale changes every 16 elements: one K=16 MFMA per half block.  In the 16-byte operand a lane
+        // already holds, half h of the block is bytes [8h, 8h+8) of lane half 0 and of lane half 1; the K=16
+        // shape wants 8 consecutive k per lane half, so the operands are re-read with that addressing.
+        const float dwa = wsc[(2 * kb) * N_T + ncol], dwb = wsc[(2 * kb + 1) * N_T + ncol];
+        const float neg_seed_dwa = -kSeed * dwa, neg_seed_dwb = -kSeed * dwb;
+        const long b0 = *(const long*)(wq + ncol * LDK + 32 * kb + 8 * lhalf);
+        const long b1 = *(const long*)(wq + ncol * LDK + 32 * kb + 16 + 8 * lhalf);
+#pragma unroll
+        for (int j = 0; j < TM; ++j) {
+          const int mrow = 32 * (wm * TM + j);
+          const long a0 = *(const long*)(xq + (mrow + lrow) * LDK + 32 * kb + 8 * lhalf);
+          const long a1 = *(const long*)(xq + (mrow + lrow) * LDK + 32 * kb + 16 + 8 * lhalf);
+          const v16i sa = __builtin_amdgcn_mfma_i32_32x32x16_i8(a0, b0, seed, 0, 0, 0);
+          const v16i sb2 = __builtin_amdgcn_mfma_i32_32x32x16_i8(a1, b1, seed, 0, 0, 0);
+          float ca[16], cb[16];
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            ca[r] = seeded_times(sa[r], dwa, neg_seed_dwa);
+            cb[r] = seeded_times(sb2[r], dwb, neg_seed_dwb);
           }
-        } else {
-          // weight scale changes every 16 elements: one K=16 MFMA per half block.  In the 16-byte operand a lane
-          // already holds, half h of the block is bytes [8h, 8h+8) of lane half 0 and of lane half 1; the K=16
-          // shape wants 8 consecutive k per lane half, so the operands are re-read with that addressing.
-          const float dwa = wsc[(2 * kb) * N_T + ncol], dwb = wsc[(2 * kb + 1) * N_T + ncol];
-          const long b0 = *(const long*)(wq + ncol * LDK + 32 * kb + 8 * lhalf);
-          const long b1 = *(const long*)(wq + ncol * LDK + 32 * kb + 16 + 8 * lhalf);
-#pragma unroll
-          for (int j = 0; j < TM; ++j) {
-            const int mrow = 32 * (wm * TM + j);
-            const long a0 = *(const long*)(xq + (mrow + lrow) * LDK + 32 * kb + 8 * lhalf);
-            const long a1 = *(const long*)(xq + (mrow + lrow) * LDK + 32 * kb + 16 + 8 * lhalf);
-            const v16i sa = __builtin_amdgcn_mfma_i32_32x32x16_i8(a0, b0, carrier, 0, 0, 0);
-            const v16i sb2 = __builtin_amdgcn_mfma_i32_32x32x16_i8(a1, b1, carrier, 0, 0, 0);
-#pragma unroll
-            for (int r = 0; r < 16; ++r) {
-              const float fa = carrier_to_float(sa[r]);
-              const float fb = carrier_to_float(sb2[r]);
-              const float t = __builtin_fmaf(fb, dwb, fa * dwa);
-              acc[j][i][r] = __builtin_fmaf(t, d8[j][r], acc[j][i][r]);
-            }
-          }
+          rescale16(acc[j][i], d8[j], ca);
+          rescale16(acc[j][i], d8[j], cb);
         }
       }
     }
+  };
+
+  if constexpr (MODE == MODE_PREFETCH) {
+    fetch(0);
+    stash(0);
     __syncthreads();
-#ifdef GGUF_DBG_NOSTASH
-    if (more && K < 0) {
-#else
-    if (more) {
-#endif
-      stash(k0 + KS);
+    for (int k0 = 0; k0 < K; k0 += KS) {
+      const bool more = k0 + KS < K;
+      if (more) fetch(k0 + KS);
+#pragma unroll 1
+      for (int kb = 0; kb < KB; ++kb) contract(kb);
+      __syncthreads();
+      if (more) {
+        stash(k0 + KS);
+        __syncthreads();
+      }
+    }
+  } else if constexpr (MODE == MODE_PLAIN) {
+    for (int k0 = 0; k0 < K; k0 += KS) {
+      fetch(k0);
+      stash(k0);
+      __syncthreads();
+#pragma unroll 1
+      for (int kb = 0; kb < KB; ++kb) contract(kb);
+      __syncthreads();
+    }
+  } else {
+    // phase p: group g stages step (p-g)/2 when p-g is even and contracts step (p-g-1)/2 when it is odd.  A group's
+    // tile is written and read only by that group, in alternating phases, so one barrier per phase orders both.
+    const int nsteps = (K + KS - 1) / KS;
+#pragma unroll 1
+    for (int p = 0; p <= 2 * nsteps; ++p) {
+      const int q = p - group;
+      if (q >= 0 && q < 2 * nsteps) {
+        if ((q & 1) == 0) {
+          fetch((q >> 1) * KS);
+          stash((q >> 1) * KS);
+        } else {
+#pragma unroll 1
+          for (int kb = 0; kb < KB; ++kb) contract(kb);
+        }
+      }
       __syncthreads();
     }
   }
@@ -485,51 +574,80 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void mmq_kernel(const uint8_t* __r
   }
 }
 
-template <class F, int WM, int WN, int TM, int TN, bool MOE>
-static constexpr size_t mmq_lds_bytes() {
-  constexpr int M_T = 32 * WM * TM, N_T = 32 * WN * TN;
-  return (size_t)(M_T + N_T) * Pitch<F::G>::value + (size_t)4 * M_T * 4 * (F::HAS_MIN ? 2 : 1) +
-         (size_t)(KS / F::G) * N_T * 4 + (F::HAS_MIN ? (size_t)4 * N_T * 4 : 0);
-}
 
-template <class F, int WM, int WN, int TM, int TN, typename T, bool MOE>
+template <class F, int WM, int WN, int TM, int TN, int KS, int OCC, int MODE, typename T, bool MOE>
 static void launch_mmq(const void* W, const void* ws, void* Y, int M, int N, int K, int m_tiles, const MoeArgs& moe,
                        hipStream_t stream) {
-  constexpr int N_T = 32 * WN * TN;
-  constexpr size_t lds = mmq_lds_bytes<F, WM, WN, TM, TN, MOE>();
-  auto kern = mmq_kernel<F, WM, WN, TM, TN, T, MOE>;
-  static bool configured = false;  // opt in to > 64 KB of dynamic LDS once per instantiation
-  if (!configured) {
-    (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-    configured = true;
+  constexpr int G = MODE == MODE_PINGPONG ? 2 : 1;
+  constexpr int N_T = 32 * WN * TN * G;
+  constexpr size_t lds = mmq_group_lds_bytes<F, WM, WN, TM, TN, KS>() * G;
+  static_assert(mmq_group_lds_bytes<F, WM, WN, TM, TN, KS>() % 16 == 0, "group tiles keep 16-byte alignment");
+  auto kern = mmq_kernel<F, WM, WN, TM, TN, KS, OCC, MODE, T, MOE>;
+  if constexpr (lds > 65536) {
+    static bool configured = false;  // opt in to > 64 KB of dynamic LDS once per instantiation
+    if (!configured) {
+      (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+      configured = true;
+    }
   }
-  hipLaunchKernelGGL(kern, dim3((N + N_T - 1) / N_T, m_tiles), dim3(64 * WM * WN), lds, stream, (const uint8_t*)W, (const char*)ws,
+  hipLaunchKernelGGL(kern, dim3((N + N_T - 1) / N_T, m_tiles), dim3(64 * WM * WN * G), lds, stream, (const uint8_t*)W, (const char*)ws,
                      (T*)Y, M, N, K, q8_row_bytes(K), moe);
 }
 
 int quantize_q8_1(const void* x, int xdtype, void* ws, int64_t M, int64_t K, hipStream_t stream);
 
+#ifdef GGUF_MMQ_TUNE
+// tuning builds only: GGUF_MMQ_CFG in the environment forces one tile configuration (fp16 activations only)
+static int tune_cfg() {
+  static const int v = [] { const char* e = getenv("GGUF_MMQ_CFG"); return e ? atoi(e) : 0; }();
+  return v;
+}
+#endif
+
+// Tile choice.  The kernel is bound by vector-ALU issue, not by operand traffic, so small tiles cost little and what
+// matters is that every CU has several workgroups to overlap one group's load latency with another's arithmetic:
+//   large   128 x 128, 8 waves, two workgroups per CU      when that still gives every CU about two tiles
+//   small   64 x 64, 4 waves, four or more per CU          otherwise (few tokens, or a narrow N with a long K)
+// Formats whose packed block is small keep the next step's loads in registers across the MFMA phase (PREFETCH);
+// for the others that would push the kernel past 128 registers and halve the waves per SIMD.
 template <class F, typename T>
 static int mmq_typed(const void* W, const void* ws, void* Y, int M, int N, int K, hipStream_t stream) {
   MoeArgs none = {};
-  if (M <= 64) {
-    launch_mmq<F, 2, 2, 1, 2, T, false>(W, ws, Y, M, N, K, (M + 63) / 64, none, stream);      // 64 x 128
+  const int64_t large_tiles = (int64_t)((M + 127) / 128) * ((N + 127) / 128);
+#ifdef GGUF_MMQ_TUNE
+  switch (tune_cfg()) {
+    case 1: launch_mmq<F, 4, 1, 1, 2, 128, 4, MODE_PINGPONG, T, false>(W, ws, Y, M, N, K, (M + 127) / 128, none, stream); return launch_status();
+    case 3: launch_mmq<F, 2, 1, 1, 1, 128, 4, MODE_PINGPONG, T, false>(W, ws, Y, M, N, K, (M + 63) / 64, none, stream); return launch_status();
+    case 5: launch_mmq<F, 4, 2, 1, 2, 128, 4, MODE_PLAIN, T, false>(W, ws, Y, M, N, K, (M + 127) / 128, none, stream); return launch_status();
+    case 6: launch_mmq<F, 2, 2, 1, 1, 128, 4, MODE_PLAIN, T, false>(W, ws, Y, M, N, K, (M + 63) / 64, none, stream); return launch_status();
+    case 8: launch_mmq<F, 4, 2, 1, 2, 128, 4, MODE_PREFETCH, T, false>(W, ws, Y, M, N, K, (M + 127) / 128, none, stream); return launch_status();
+    default: break;
+  }
+#endif
+  if (large_tiles >= 400) {
+    constexpr int MODE = F::LIGHT ? MODE_PREFETCH : MODE_PLAIN;
+    launch_mmq<F, 4, 2, 1, 2, 128, 4, MODE, T, false>(W, ws, Y, M, N, K, (M + 127) / 128, none, stream);
   } else {
-    launch_mmq<F, 4, 2, 1, 2, T, false>(W, ws, Y, M, N, K, (M + 127) / 128, none, stream);    // 128 x 128, 8 waves
+    launch_mmq<F, 2, 2, 1, 1, 128, 4, MODE_PLAIN, T, false>(W, ws, Y, M, N, K, (M + 63) / 64, none, stream);
   }
   return launch_status();
 }
 
 template <class F>
 static int mmq_fmt(const void* W, const void* ws, void* Y, int dtype, int M, int N, int K, hipStream_t s) {
+#ifdef GGUF_MMQ_TUNE
+  if (dtype != GGUF_DTYPE_F16) return GGUF_ERR_DTYPE;
+  return mmq_typed<F, _Float16>(W, ws, Y, M, N, K, s);
+#else
   GGUF_DISPATCH_DTYPE(dtype, return (mmq_typed<F, scalar_t>(W, ws, Y, M, N, K, s)));
   return GGUF_ERR_DTYPE;
+#endif
 }
 
 template <class F, typename T>
 static int moe_typed(const void* W, const void* ws, void* Y, int N, int K, int num_sorted, const MoeArgs& moe,
                      hipStream_t stream) {
-  launch_mmq<F, 1, 4, 1, 2, T, true>(W, ws, Y, 0, N, K, num_sorted / 32, moe, stream);  // 32 slots x 256
+  launch_mmq<F, 1, 4, 1, 2, 128, 2, MODE_PREFETCH, T, true>(W, ws, Y, 0, N, K, num_sorted / 32, moe, stream);  // 32 slots x 256
   return launch_status();
 }
 
