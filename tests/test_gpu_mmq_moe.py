@@ -8,6 +8,8 @@ from oracle import gguf_oracle as o
 pytestmark = pytest.mark.gpu
 
 SIX = [o.Q4_0, o.Q8_0, o.Q4_K, o.Q6_K, o.IQ4_XS, o.IQ2_XXS]
+ALL = [o.Q4_0, o.Q4_1, o.Q5_0, o.Q5_1, o.Q8_0, o.Q2_K, o.Q3_K, o.Q4_K, o.Q5_K, o.Q6_K, o.IQ2_XXS, o.IQ2_XS, o.IQ3_XXS,
+       o.IQ1_S, o.IQ4_NL, o.IQ3_S, o.IQ2_S, o.IQ4_XS, o.IQ1_M]
 TORCH_DT = {"f16": torch.float16, "bf16": torch.bfloat16, "f32": torch.float32}
 
 
@@ -128,7 +130,7 @@ def test_moe_grouped_padding_and_bad_experts_write_nothing():
     assert len(skipped) > 0 and np.all(y[skipped] == 0)
 
 
-@pytest.mark.parametrize("qtype", SIX)
+@pytest.mark.parametrize("qtype", ALL)
 def test_moe_vec_matches_oracle(qtype):
     ops = _ops()
     rng = np.random.default_rng(900 + qtype)

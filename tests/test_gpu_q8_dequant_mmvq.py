@@ -81,7 +81,7 @@ def test_dequantize_default_dtype_and_shape_label():
     assert np.array_equal(out.cpu().numpy().reshape(-1), o.dequantize(w, o.Q8_0, "f16"))
 
 
-@pytest.mark.parametrize("qtype", SIX)
+@pytest.mark.parametrize("qtype", ALL)
 @pytest.mark.parametrize("m", [1, 2, 3, 5, 8, 11])
 def test_mmvq_matches_a8_oracle(qtype, m):
     ops = _ops()
@@ -99,7 +99,7 @@ def test_mmvq_matches_a8_oracle(qtype, m):
 
 
 @pytest.mark.parametrize("dt", ["f16", "bf16"])
-@pytest.mark.parametrize("qtype", SIX)
+@pytest.mark.parametrize("qtype", ALL)
 def test_mmvq_half_outputs_within_tolerance(qtype, dt):
     # stated tolerance: rel-L2 <= 1e-3 for fp16 outputs (bf16: 4e-3, its rounding alone is 2^-9) vs the a8 oracle
     ops = _ops()

@@ -1,731 +1,38 @@
-// Decode-path GEMV on packed GGUF weights with q8_1 activations (gfx950).
-//
-//   Y[m, n] = sum over blocks of  dot(W block of row n, q8_1 block(s) of X[m])
-//
-// with the per-format block formulas of the reference's vec_dot_<fmt>_q8_1
-// functions (csrc/gguf/vecdotq.cuh; cited at each format below).  The work
-// split is not the reference's "one 64-lane wave per (row, vector)" grid
-// (csrc/gguf/mmvq.cuh:2-50): here
-//   * a workgroup of four waves owns 4*RPW consecutive rows, so its weight bytes
-//     are one contiguous span of HBM, and every lane pulls 16 bytes per load;
-//   * the quantized activations of up to eight vectors are staged once per
-//     workgroup in LDS (quants + block scales), and every weight byte loaded is
-//     used for all of them, so weights cross HBM once per call for M <= 8;
-//   * a "unit" is the 32 weights one lane turns into int8 dot products per step;
-//     partial sums stay in fp32 registers and are reduced with DPP at the end.
-#include <type_traits>
-
-#include "q8_1_device.h"
-#include "grid_codes.h"
+// C entry points of the decode-path GEMV and of the per-pair MoE GEMV.  The kernels live in mmvq_core.h and are
+// instantiated per group of formats in the mmvq_<group>.hip files; this file validates and routes by ggml type.
+#include "gguf_common.h"
 
 namespace gguf {
 
-enum { AUX_NONE = 0, AUX_S8 = 1, AUX_DU = 2 };
+int mmvq_group_std_a(int type, const void* W, const void* x, void* ws, void* Y, int dtype, int64_t N, int64_t K, int64_t M,
+                   hipStream_t s);
+int mmvq_group_std_b(int type, const void* W, const void* x, void* ws, void* Y, int dtype, int64_t N, int64_t K, int64_t M,
+                   hipStream_t s);
+int mmvq_group_k_a(int type, const void* W, const void* x, void* ws, void* Y, int dtype, int64_t N, int64_t K, int64_t M,
+                   hipStream_t s);
+int mmvq_group_k_b(int type, const void* W, const void* x, void* ws, void* Y, int dtype, int64_t N, int64_t K, int64_t M,
+                   hipStream_t s);
+int mmvq_group_iq_a(int type, const void* W, const void* x, void* ws, void* Y, int dtype, int64_t N, int64_t K, int64_t M,
+                   hipStream_t s);
+int mmvq_group_iq_b(int type, const void* W, const void* x, void* ws, void* Y, int dtype, int64_t N, int64_t K, int64_t M,
+                   hipStream_t s);
+int mmvq_group_iq_c(int type, const void* W, const void* x, void* ws, void* Y, int dtype, int64_t N, int64_t K, int64_t M,
+                   hipStream_t s);
 
-struct Act {            // LDS views of one staged activation vector
-  const int8_t* q;      // [kc]
-  const float* d;       // [kc/32] block scales
-  const float* a;       // [kc/32] block sums (AUX_S8) or d*sum(q) (AUX_DU)
-  const char* tab;      // format lookup tables in LDS (i-quants)
-};
-
-// Every format splits its work in two: load() only issues global loads into raw registers (no use of
-// the loaded values, so consecutive loads stay in flight together), dot() decodes and multiplies.
-__device__ __forceinline__ float h2f(uint32_t bits) { return (float)__builtin_bit_cast(_Float16, (uint16_t)bits); }
-
-// ------------------------------------------------------------------ Q4_0 (vecdotq.cuh:46-66,493-509)
-struct FmtQ4_0 {
-  static constexpr int QK = 32, BS = 18, AUX = AUX_S8, TABLE_BYTES = 0;
-  struct Regs { uint16_t d; uint4 q; };
-  static __device__ __forceinline__ void init_tables(char*) {}
-  static __device__ __forceinline__ Regs load(const uint8_t* row, int u0, int u, const char*) {
-    const uint8_t* b = row + (int64_t)(u0 + u) * BS;
-    Regs r; r.d = ld<uint16_t>(b); r.q = ld<uint4>(b + 2); return r;
-  }
-  struct ActRegs { int4 lo, hi; float d, a; };
-  static __device__ __forceinline__ ActRegs load_act(const Act& x, int u) {
-    ActRegs a; a.lo = *(const int4*)(x.q + 32 * u); a.hi = *(const int4*)(x.q + 32 * u + 16); a.d = x.d[u]; a.a = x.a[u];
-    return a;
-  }
-  static __device__ __forceinline__ float dot(const Regs& r, const ActRegs& x, int u) {
-    const uint32_t q[4] = {r.q.x, r.q.y, r.q.z, r.q.w};
-    const int al[4] = {x.lo.x, x.lo.y, x.lo.z, x.lo.w}, ah[4] = {x.hi.x, x.hi.y, x.hi.z, x.hi.w};
-    int s = 0;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      s = dot4((int)(q[i] & 0x0F0F0F0Fu), al[i], s);
-      s = dot4((int)((q[i] >> 4) & 0x0F0F0F0Fu), ah[i], s);
-    }
-    return h2f(r.d) * ((float)s * x.d - 8.0f * x.a);
-  }
-  static __device__ __forceinline__ float dot(const Regs& r, const Act& x, int u, int lane) {
-    return dot(r, load_act(x, u), u);
-  }
-};
-
-// ------------------------------------------------------------------ Q8_0 (vecdotq.cuh:165-177,852-867)
-struct FmtQ8_0 {
-  static constexpr int QK = 32, BS = 34, AUX = AUX_NONE, TABLE_BYTES = 0;
-  struct Regs { uint16_t d; uint4 q0, q1; };
-  static __device__ __forceinline__ void init_tables(char*) {}
-  static __device__ __forceinline__ Regs load(const uint8_t* row, int u0, int u, const char*) {
-    const uint8_t* b = row + (int64_t)(u0 + u) * BS;
-    Regs r; r.d = ld<uint16_t>(b); r.q0 = ld<uint4>(b + 2); r.q1 = ld<uint4>(b + 18); return r;
-  }
-  struct ActRegs { int4 a0, a1; float d; };
-  static __device__ __forceinline__ ActRegs load_act(const Act& x, int u) {
-    ActRegs a; a.a0 = *(const int4*)(x.q + 32 * u); a.a1 = *(const int4*)(x.q + 32 * u + 16); a.d = x.d[u];
-    return a;
-  }
-  static __device__ __forceinline__ float dot(const Regs& r, const ActRegs& x, int u) {
-    int s = 0;
-    s = dot4((int)r.q0.x, x.a0.x, s); s = dot4((int)r.q0.y, x.a0.y, s); s = dot4((int)r.q0.z, x.a0.z, s); s = dot4((int)r.q0.w, x.a0.w, s);
-    s = dot4((int)r.q1.x, x.a1.x, s); s = dot4((int)r.q1.y, x.a1.y, s); s = dot4((int)r.q1.z, x.a1.z, s); s = dot4((int)r.q1.w, x.a1.w, s);
-    return h2f(r.d) * x.d * (float)s;
-  }
-  static __device__ __forceinline__ float dot(const Regs& r, const Act& x, int u, int lane) {
-    return dot(r, load_act(x, u), u);
-  }
-};
-
-// ------------------------------------------------------------------ Q4_K (vecdotq.cuh:328-351,1159-1202)
-// unit c of a super-block: 16 bytes of qs = 16 low nibbles of sub-block 2g and 16 high nibbles of 2g+1
-struct FmtQ4_K {
-  static constexpr int QK = 256, BS = 144, AUX = AUX_DU, TABLE_BYTES = 0;
-  struct Regs { uint4 hdr, q; };
-  static __device__ __forceinline__ void init_tables(char*) {}
-  static __device__ __forceinline__ Regs load(const uint8_t* row, int u0, int u, const char*) {
-    const int uu = u0 + u, sb = uu >> 3, c = uu & 7;
-    const uint8_t* b = row + (int64_t)sb * BS;
-    Regs r; r.hdr = ld<uint4>(b); r.q = ld<uint4>(b + 16 + 16 * c); return r;
-  }
-  struct ActRegs { int4 lo, hi; float2 d8, du; };
-  static __device__ __forceinline__ ActRegs load_act(const Act& x, int u) {
-    const int sb = u >> 3, c = u & 7, g = c >> 1, h = c & 1;
-    const int8_t* qa = x.q + 256 * sb + 64 * g + 16 * h;
-    ActRegs a;
-    a.lo = *(const int4*)qa; a.hi = *(const int4*)(qa + 32);
-    a.d8 = *(const float2*)(x.d + 8 * sb + 2 * g);
-    a.du = *(const float2*)(x.a + 8 * sb + 2 * g);
-    if (h) a.du = make_float2(0.0f, 0.0f);  // the offset term of a sub-block pair is added once, by its first unit
-    return a;
-  }
-  static __device__ __forceinline__ float dot(const Regs& r, const ActRegs& x, int u) {
-    const int g = (u & 7) >> 1;
-    // 6-bit scales and mins of sub-blocks 2g and 2g+1 (dequantize.cuh:156-163 in 16-bit lanes)
-    const int sh = 16 * (g & 1);
-    const uint32_t A = (r.hdr.y >> sh) & 0xFFFF, B = (r.hdr.z >> sh) & 0xFFFF, C = (r.hdr.w >> sh) & 0xFFFF;
-    uint32_t a0, a1;
-    if (g < 2) {
-      a0 = A & 0x3F3F; a1 = B & 0x3F3F;
-    } else {
-      a0 = (C & 0x0F0F) | ((A & 0xC0C0) >> 2);
-      a1 = ((C >> 4) & 0x0F0F) | ((B & 0xC0C0) >> 2);
-    }
-    const uint32_t q[4] = {r.q.x, r.q.y, r.q.z, r.q.w};
-    const int al[4] = {x.lo.x, x.lo.y, x.lo.z, x.lo.w}, ah[4] = {x.hi.x, x.hi.y, x.hi.z, x.hi.w};
-    int s0 = 0, s1 = 0;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      s0 = dot4((int)(q[i] & 0x0F0F0F0Fu), al[i], s0);
-      s1 = dot4((int)((q[i] >> 4) & 0x0F0F0F0Fu), ah[i], s1);
-    }
-    const float pos = x.d8.x * (float)(s0 * (int)(a0 & 0xFF)) + x.d8.y * (float)(s1 * (int)(a0 >> 8));
-    const float neg = x.du.x * (float)(a1 & 0xFF) + x.du.y * (float)(a1 >> 8);
-    return h2f(r.hdr.x & 0xFFFF) * pos - h2f(r.hdr.x >> 16) * neg;
-  }
-  static __device__ __forceinline__ float dot(const Regs& r, const Act& x, int u, int lane) {
-    return dot(r, load_act(x, u), u);
-  }
-};
-
-// ------------------------------------------------------------------ Q6_K (vecdotq.cuh:447-465,1417-1441)
-// unit c of a super-block: half h = c>>2, columns l in [8*(c&3), +8) of that half; covers elements
-// 128h + 32t + l for t = 0..3, i.e. eight values in each of four q8_1 blocks.
-struct FmtQ6_K {
-  static constexpr int QK = 256, BS = 210, AUX = AUX_NONE, TABLE_BYTES = 0;
-  struct Regs { uint2 qla, qlb, qh, sc; uint16_t d; };
-  static __device__ __forceinline__ void init_tables(char*) {}
-  static __device__ __forceinline__ Regs load(const uint8_t* row, int u0, int u, const char*) {
-    const int uu = u0 + u, sb = uu >> 3, c = uu & 7, h = c >> 2, cc = c & 3;
-    const uint8_t* b = row + (int64_t)sb * BS;
-    Regs r;
-    r.qla = ld<uint2>(b + 64 * h + 8 * cc);
-    r.qlb = ld<uint2>(b + 64 * h + 32 + 8 * cc);
-    r.qh = ld<uint2>(b + 128 + 32 * h + 8 * cc);
-    r.sc = ld<uint2>(b + 192 + 8 * h);
-    r.d = ld<uint16_t>(b + 208);
-    return r;
-  }
-  struct ActRegs { int2 a[4]; float d8[4]; int ones[4]; };
-  static __device__ __forceinline__ ActRegs load_act(const Act& x, int u) {
-    const int sb = u >> 3, c = u & 7, h = c >> 2, cc = c & 3;
-    const int8_t* qa = x.q + 256 * sb + 128 * h + 8 * cc;
-    ActRegs a;
-#pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      a.a[t] = *(const int2*)(qa + 32 * t);
-      a.d8[t] = x.d[8 * sb + 4 * h + t];
-      a.ones[t] = dot4(0x01010101, a.a[t].x, dot4(0x01010101, a.a[t].y, 0));  // for the -32 offset of the codes
-    }
-    return a;
-  }
-  static __device__ __forceinline__ float dot(const Regs& r, const ActRegs& x, int u) {
-    const int cc = u & 3;
-    const uint64_t sw = ((uint64_t)r.sc.y << 32) | r.sc.x;
-    const int so = 8 * (cc >> 1);
-    float acc = 0.0f;
-#pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      const uint2 ql = (t & 1) ? r.qlb : r.qla;
-      const int shl = (t >> 1) ? 4 : 0;
-      const int vx = (int)(((ql.x >> shl) & 0x0F0F0F0Fu) | (((r.qh.x >> (2 * t)) & 0x03030303u) << 4));
-      const int vy = (int)(((ql.y >> shl) & 0x0F0F0F0Fu) | (((r.qh.y >> (2 * t)) & 0x03030303u) << 4));
-      const int s = dot4(vx, x.a[t].x, dot4(vy, x.a[t].y, 0));
-      const int sc = (int)(int8_t)(sw >> (16 * t + so));
-      acc += x.d8[t] * (float)(sc * (s - 32 * x.ones[t]));
-    }
-    return h2f(r.d) * acc;
-  }
-  static __device__ __forceinline__ float dot(const Regs& r, const Act& x, int u, int lane) {
-    return dot(r, load_act(x, u), u);
-  }
-};
-
-// 16-entry signed byte table lookup of four 4-bit indices held one per byte
-__device__ __forceinline__ int lut16(uint32_t idx, uint32_t t0, uint32_t t1, uint32_t t2, uint32_t t3) {
-  const uint32_t sel = idx & 0x07070707u;
-  const uint32_t lo = __builtin_amdgcn_perm(t1, t0, sel);
-  const uint32_t hi = __builtin_amdgcn_perm(t3, t2, sel);
-  const uint32_t m = ((idx >> 3) & 0x01010101u) * 0xFFu;
-  return (int)((hi & m) | (lo & ~m));
-}
-
-// ------------------------------------------------------------------ IQ4_XS (vecdotq.cuh:1791-1811)
-struct FmtIQ4_XS {
-  static constexpr int QK = 256, BS = 136, AUX = AUX_NONE, TABLE_BYTES = 0;
-  struct Regs { uint2 hdr; uint4 q; };
-  static __device__ __forceinline__ void init_tables(char*) {}
-  static __device__ __forceinline__ Regs load(const uint8_t* row, int u0, int u, const char*) {
-    const int uu = u0 + u, sb = uu >> 3, ib = uu & 7;
-    const uint8_t* b = row + (int64_t)sb * BS;
-    Regs r; r.hdr = ld<uint2>(b); r.q = ld<uint4>(b + 8 + 16 * ib); return r;
-  }
-  struct ActRegs { int4 lo, hi; float d; };
-  static __device__ __forceinline__ ActRegs load_act(const Act& x, int u) {
-    ActRegs a; a.lo = *(const int4*)(x.q + 32 * u); a.hi = *(const int4*)(x.q + 32 * u + 16); a.d = x.d[u];
-    return a;
-  }
-  static __device__ __forceinline__ float dot(const Regs& r, const ActRegs& x, int u) {
-    const int ib = u & 7;
-    const int ls = (int)(((r.hdr.y >> (4 * ib)) & 0xF) | ((((r.hdr.x >> 16) >> (2 * ib)) & 3) << 4));
-    const float dl = h2f(r.hdr.x & 0xFFFF) * (float)(ls - 32);
-    // kvalues_iq4nl as four little-endian words
-    constexpr uint32_t T0 = 0xBFAD9881u, T1 = 0xF6EADDCFu, T2 = 0x26190D01u, T3 = 0x71594535u;
-    const uint32_t qq[4] = {r.q.x, r.q.y, r.q.z, r.q.w};
-    const int al[4] = {x.lo.x, x.lo.y, x.lo.z, x.lo.w}, ah[4] = {x.hi.x, x.hi.y, x.hi.z, x.hi.w};
-    int s = 0;
-#pragma unroll
-    for (int i = 0; i < 4; ++i) {
-      s = dot4(lut16(qq[i] & 0x0F0F0F0Fu, T0, T1, T2, T3), al[i], s);
-      s = dot4(lut16((qq[i] >> 4) & 0x0F0F0F0Fu, T0, T1, T2, T3), ah[i], s);
-    }
-    return dl * x.d * (float)s;
-  }
-  static __device__ __forceinline__ float dot(const Regs& r, const Act& x, int u, int lane) {
-    return dot(r, load_act(x, u), u);
-  }
-};
-
-// ------------------------------------------------------------------ IQ2_XXS (vecdotq.cuh:1531-1552)
-// LDS tables: the 256-entry grid expanded to 8 magnitudes per entry, and the 128 sign patterns as byte masks.
-struct FmtIQ2_XXS {
-  static constexpr int QK = 256, BS = 66, AUX = AUX_NONE, TABLE_BYTES = 256 * 8 + 128 * 8;
-  struct Regs { uint16_t d; uint2 g; };
-  static __device__ __forceinline__ void init_tables(char* tab) {
-    uint2* grid = (uint2*)tab;
-    uint2* sgn = grid + 256;
-    for (int t = threadIdx.x; t < 256; t += blockDim.x) {
-      const uint32_t code = k_iq2xxs_grid_codes[t];
-      uint32_t w[2] = {0, 0};
-#pragma unroll
-      for (int j = 0; j < 8; ++j) {
-        const uint32_t c = (code >> (2 * j)) & 3;
-        w[j >> 2] |= (8 + 17 * c + (c >> 1)) << (8 * (j & 3));
-      }
-      grid[t] = make_uint2(w[0], w[1]);
-      if (t < 128) {
-        const uint32_t sg = t | ((__builtin_popcount(t) & 1) << 7);
-        uint32_t m[2] = {0, 0};
-#pragma unroll
-        for (int j = 0; j < 8; ++j) m[j >> 2] |= ((sg >> j) & 1 ? 0xFFu : 0u) << (8 * (j & 3));
-        sgn[t] = make_uint2(m[0], m[1]);
-      }
-    }
-  }
-  static __device__ __forceinline__ Regs load(const uint8_t* row, int u0, int u, const char*) {
-    const int uu = u0 + u, sb = uu >> 3, ib = uu & 7;
-    const uint8_t* b = row + (int64_t)sb * BS;
-    Regs r; r.d = ld<uint16_t>(b); r.g = ld<uint2>(b + 2 + 8 * ib); return r;
-  }
-  struct ActRegs { int2 a[4]; float d; const char* tab; };
-  static __device__ __forceinline__ ActRegs load_act(const Act& x, int u) {
-    ActRegs a;
-#pragma unroll
-    for (int l = 0; l < 4; ++l) a.a[l] = *(const int2*)(x.q + 32 * u + 8 * l);
-    a.d = x.d[u]; a.tab = x.tab;
-    return a;
-  }
-  static __device__ __forceinline__ float dot(const Regs& r, const ActRegs& x, int u) {
-    const uint2* grid = (const uint2*)x.tab;
-    const uint2* sgn = grid + 256;
-    const float dl = h2f(r.d) * (0.5f + (float)(r.g.y >> 28)) * 0.25f;
-    int s = 0;
-#pragma unroll
-    for (int l = 0; l < 4; ++l) {
-      const uint2 mag = grid[(r.g.x >> (8 * l)) & 0xFF];
-      const uint2 m = sgn[(r.g.y >> (7 * l)) & 127];
-      s = dot4((int)neg_bytes(mag.x, m.x), x.a[l].x, s);
-      s = dot4((int)neg_bytes(mag.y, m.y), x.a[l].y, s);
-    }
-    return dl * x.d * (float)s;
-  }
-  static __device__ __forceinline__ float dot(const Regs& r, const Act& x, int u, int lane) {
-    return dot(r, load_act(x, u), u);
-  }
-};
-
-// ------------------------------------------------------------------ kernel
-// MOE selects the per-pair variant (reference: csrc/gguf/moe_vec.cuh:3-53): blockIdx.y is the flat
-// (token, k) pair z; its expert topk_ids[z] picks the weight matrix (experts densely packed), its
-// token z / top_k picks the activation row, and the result goes to row z of Y.
-//
-// FUSEQ: `xsrc` is the raw activation matrix (dtype T, row pitch K) and every workgroup quantizes
-// the vectors it needs straight into LDS, so a call is one launch and no workspace is touched;
-// otherwise `xsrc` is the q8_1 workspace written by the stand-alone quantizer.
-//
-// The first weight loads of a chunk are issued before the activations are staged, and the loop
-// keeps one step of loads in flight ahead of the dot products.
-template <class F, int MT, int RPW, typename T, bool MOE, bool FUSEQ>
-__global__ __launch_bounds__(256) void mmvq_kernel(const uint8_t* __restrict__ W, const char* __restrict__ xsrc,
-                                                    T* __restrict__ Y, int N, int K, int kchunk, int64_t x_row_bytes,
-                                                    int64_t y_vec_stride, const int32_t* __restrict__ topk_ids,
-                                                    int top_k) {
-  extern __shared__ __align__(16) char smem[];
-  const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-  const int Kp = (int)q8_kp(K);
-  if (MOE) {
-    const int z = blockIdx.y;
-    const int e = topk_ids[z];
-    W += (int64_t)e * N * ((int64_t)(K / F::QK) * F::BS);
-    xsrc += (int64_t)(z / top_k) * x_row_bytes;
-    Y += (int64_t)z * N;
-  }
-  int8_t* lq = (int8_t*)smem;                         // [MT][kchunk]
-  float* ldv = (float*)(smem + MT * kchunk);          // [MT][kchunk/32]
-  float* lav = ldv + MT * (kchunk / 32);              // [MT][kchunk/32]
-  char* tab = (char*)(lav + (F::AUX != AUX_NONE ? MT * (kchunk / 32) : 0));
-  F::init_tables(tab);
-  if (F::TABLE_BYTES > 0) __syncthreads();
-
-  const int row0 = (blockIdx.x * 4 + wave) * RPW;
-  const int64_t rowbytes = (int64_t)(K / F::QK) * F::BS;
-  const uint8_t* rows[RPW];
-#pragma unroll
-  for (int r = 0; r < RPW; ++r) rows[r] = W + (int64_t)min(row0 + r, N - 1) * rowbytes;
-
-  float acc[RPW][MT];
-#pragma unroll
-  for (int r = 0; r < RPW; ++r)
-#pragma unroll
-    for (int m = 0; m < MT; ++m) acc[r][m] = 0.0f;
-
-  for (int k0 = 0; k0 < K; k0 += kchunk) {
-    const int kc = min(kchunk, K - k0);
-    const int nb = kc >> 5;
-    const int u0 = k0 >> 5;  // first unit of this chunk within the row
-
-    // weights of the first step: in flight while the activations are staged
-    int u = lane;
-    bool have = u < nb;
-    typename F::Regs cur[RPW];
-    if (have) {
-#pragma unroll
-      for (int r = 0; r < RPW; ++r) cur[r] = F::load(rows[r], u0, u, tab);
-    }
-
-    if (k0 > 0) __syncthreads();
-    if (FUSEQ) {
-      // four lanes quantize one 32-value block; kc/8 is a multiple of 4, so quads stay whole
-      const int g8 = kc >> 3;
-      for (int i = tid; i < MT * g8; i += 256) {
-        const int m = i / g8, j = i - m * g8;
-        float v[8];
-        load8<T>((const T*)(xsrc + m * x_row_bytes) + k0 + 8 * j, v);
-        const Q8Quad qq = q8_1_quantize8(v);
-        *(uint2*)(lq + m * kchunk + 8 * j) = qq.q;
-        if ((j & 3) == 0) {
-          ldv[m * (kchunk / 32) + (j >> 2)] = qq.d;
-          if (F::AUX == AUX_S8) lav[m * (kchunk / 32) + (j >> 2)] = qq.s;
-          if (F::AUX == AUX_DU) lav[m * (kchunk / 32) + (j >> 2)] = qq.du;
-        }
-      }
-    } else {
-      // copy quants (16-byte granules) and block scales of the MT vectors from the workspace
-      const int g16 = kc >> 4;
-      for (int i = tid; i < MT * g16; i += 256) {
-        const int m = i / g16, j = i - m * g16;
-        *(uint4*)(lq + m * kchunk + 16 * j) = *(const uint4*)(xsrc + m * x_row_bytes + k0 + 16 * j);
-      }
-      for (int i = tid; i < MT * nb; i += 256) {
-        const int m = i / nb, j = i - m * nb;
-        const float* fd = (const float*)(xsrc + m * x_row_bytes + Kp) + u0 + j;
-        ldv[m * (kchunk / 32) + j] = fd[0];
-        if (F::AUX == AUX_S8) lav[m * (kchunk / 32) + j] = fd[Kp / 32];
-        if (F::AUX == AUX_DU) lav[m * (kchunk / 32) + j] = fd[2 * (Kp / 32)];
-      }
-    }
-    __syncthreads();
-
-    while (have) {
-      const int un = u + 64;
-      const bool hn = un < nb;
-      typename F::Regs nxt[RPW];
-      if (hn) {
-#pragma unroll
-        for (int r = 0; r < RPW; ++r) nxt[r] = F::load(rows[r], u0, un, tab);
-      }
-#pragma unroll
-      for (int m = 0; m < MT; ++m) {
-        Act x;
-        x.q = lq + m * kchunk;
-        x.d = ldv + m * (kchunk / 32);
-        x.a = lav + m * (kchunk / 32);
-        x.tab = tab;
-#pragma unroll
-        for (int r = 0; r < RPW; ++r) acc[r][m] += F::dot(cur[r], x, u, lane);
-      }
-#pragma unroll
-      for (int r = 0; r < RPW; ++r) cur[r] = nxt[r];
-      u = un;
-      have = hn;
-    }
-  }
-
-#pragma unroll
-  for (int r = 0; r < RPW; ++r) {
-#pragma unroll
-    for (int m = 0; m < MT; ++m) {
-      const float v = wave_sum(acc[r][m]);
-      if (lane == 0 && row0 + r < N) Y[m * y_vec_stride + row0 + r] = from_f32<T>(v);
-    }
-  }
-}
-
-// ------------------------------------------------------------------ streaming kernel (M <= 4)
-// The decode case is one pass over a few tens of MB, i.e. a handful of HBM latencies long, so the
-// whole game is to have every weight byte requested in the first microsecond and nothing else on
-// the critical path.
-//   * One fat workgroup (NW waves) per CU owns a contiguous band of rows.  A row of K/32 units needs
-//     S = ceil(K/2048) waves; the workgroup runs NW/S rows side by side ("slots"), and a lane keeps
-//     the same unit column for its whole life.
-//   * Every wave first requests the activation values it will quantize, then the weights of its first
-//     D rows, and only then does arithmetic: the workgroup quantizes the MT activation vectors into LDS
-//     (q8_1_device.h) once, while the weights fly.  A call is a single launch, no workspace traffic.
-//   * After one barrier each lane pulls the quantized activations of its column into registers, so the
-//     row loop touches no LDS except for one partial sum per (row, wave), and refills the load slot it
-//     has just consumed: D row-loads stay in flight per wave.
-//   * Row totals are summed from the per-wave partials in a fixed order.
-#ifndef GGUF_MMVQ_NW
-#define GGUF_MMVQ_NW 16
-#endif
-#ifndef GGUF_MMVQ_DEPTH
-#define GGUF_MMVQ_DEPTH 4
-#endif
-#ifndef GGUF_MMVQ_WG_PER_CU
-#define GGUF_MMVQ_WG_PER_CU 1
-#endif
-
-template <class F, int MT, int NW, int D, typename T>
-__global__ __launch_bounds__(64 * NW) void mmvq_stream_kernel(const uint8_t* __restrict__ W, const T* __restrict__ X,
-                                                               T* __restrict__ Y, int N, int K, int rows_per_wg) {
-  extern __shared__ __align__(16) char smem[];
-  const int tid = threadIdx.x, lane = tid & 63;
-  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: row arithmetic stays on the scalar unit
-  const int nb = K >> 5;                       // 32-weight units per row
-  const int S = (nb + 63) >> 6;                // waves per row
-  const int slots = NW / S;                    // rows in flight side by side (>= 1, checked by the host)
-  int8_t* lq = (int8_t*)smem;                  // [MT][K]
-  float* ldv = (float*)(smem + (size_t)MT * K);  // [MT][nb]
-  float* lav = ldv + MT * nb;                  // [MT][nb]
-  char* tab = (char*)(lav + (F::AUX != AUX_NONE ? MT * nb : 0));
-  float* part = (float*)(tab + F::TABLE_BYTES);  // [rows_per_wg][S][MT]
-
-  const int r_begin = blockIdx.x * rows_per_wg;
-  const int r_end = min(N, r_begin + rows_per_wg);
-  if (r_begin >= r_end) return;
-  const int nrows = r_end - r_begin;
-  const int64_t rowbytes = (int64_t)(K / F::QK) * F::BS;
-
-  // this wave: slot (which of the side-by-side rows) and step (which 64-unit stretch of the row)
-  const int slot = wave / S, step = wave - slot * S;
-  const bool wave_on = slot < slots;           // NW - slots*S waves have no weights to fetch; they still quantize
-  const int u_raw = step * 64 + lane;
-  const bool lane_on = wave_on && u_raw < nb;
-  const int u = min(u_raw, nb - 1);
-  const int my_rows = wave_on && nrows > slot ? (nrows - slot + slots - 1) / slots : 0;  // rows slot, slot+slots, ...
-  const int max_rows = (nrows + slots - 1) / slots;  // trip count of the row loop, same for every wave
-
-  if (F::TABLE_BYTES > 0) {
-    F::init_tables(tab);
-    __syncthreads();
-  }
-
-  // Loads are issued unconditionally (row index clamped into the band) so that every iteration issues the
-  // same number of loads and the hardware load counter can be waited on exactly, slot by slot.
-  const uint8_t* wbase = W + (int64_t)r_begin * rowbytes;
-  auto load_row = [&](int i) {
-    const int row = min(slot + slots * i, nrows - 1);
-    return F::load(wbase + (int64_t)row * rowbytes, 0, u, tab);
-  };
-
-  // Prologue, in one basic block per variant: request this thread's first QG groups of activation values,
-  // then the weights of the first D rows, then quantize the activations into LDS (four lanes per 32-value
-  // block) while the weights fly.  The activation loads go first so that waiting for them does not also
-  // wait for the weight loads behind them.  Groups past the end are clamped and their stores predicated.
-  constexpr int NT = 64 * NW;
-  const int g8 = K >> 3;
-  const int qtotal = MT * g8;  // a multiple of 4, so quads stay whole
-  typename F::Regs pre[D];
-  auto quantize_group = [&](const raw8<T>& raw, int q) {
-    const int qc = min(q, qtotal - 1);
-    const int m = qc / g8, j = qc - m * g8;
-    float xv[8];
-    raw.cvt(xv);
-#ifdef GGUF_DBG_NOQUANT
-    Q8Quad qq; qq.q = make_uint2(__builtin_bit_cast(uint32_t, xv[0]), __builtin_bit_cast(uint32_t, xv[7])); qq.d = xv[1]; qq.s = xv[2]; qq.du = xv[3];
-#else
-    const Q8Quad qq = q8_1_quantize8(xv);
-#endif
-    if (q < qtotal) {
-      *(uint2*)(lq + (size_t)m * K + 8 * j) = qq.q;
-      if ((j & 3) == 0) {
-        ldv[m * nb + (j >> 2)] = qq.d;
-        if (F::AUX == AUX_S8) lav[m * nb + (j >> 2)] = qq.s;
-        if (F::AUX == AUX_DU) lav[m * nb + (j >> 2)] = qq.du;
-      }
-    }
-  };
-  auto prologue = [&](auto qg_tag) {
-    constexpr int QG = decltype(qg_tag)::value;
-    raw8<T> xraw[QG];
-#pragma unroll
-    for (int g = 0; g < QG; ++g) {
-      const int qc = min(tid + g * NT, qtotal - 1);
-      const int m = qc / g8, j = qc - m * g8;
-      xraw[g].load(X + (int64_t)m * K + 8 * j);
-    }
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int d = 0; d < D; ++d) pre[d] = load_row(d);
-    __builtin_amdgcn_sched_barrier(0);
-#pragma unroll
-    for (int g = 0; g < QG; ++g) quantize_group(xraw[g], tid + g * NT);
-  };
-  if (qtotal <= NT) prologue(std::integral_constant<int, 1>{});
-  else if (qtotal <= 2 * NT) prologue(std::integral_constant<int, 2>{});
-  else prologue(std::integral_constant<int, 4>{});
-  for (int q = tid + 4 * NT; q - tid < qtotal; q += NT) {  // uniform trip count; only for K * MT > 32 * NT
-    const int qc = min(q, qtotal - 1);
-    const int m2 = qc / g8, j2 = qc - m2 * g8;
-    raw8<T> r;
-    r.load(X + (int64_t)m2 * K + 8 * j2);
-    quantize_group(r, q);
-  }
-  __syncthreads();
-
-  // this lane's column of every activation vector, held in registers for the whole row loop
-  typename F::ActRegs act[MT];
-#pragma unroll
-  for (int m = 0; m < MT; ++m) {
-    Act x;
-    x.q = lq + (size_t)m * K;
-    x.d = ldv + m * nb;
-    x.a = lav + m * nb;
-    x.tab = tab;
-    act[m] = F::load_act(x, u);
-  }
-
-  for (int i0 = 0; i0 < max_rows; i0 += D) {
-#pragma unroll
-    for (int d = 0; d < D; ++d) {
-      const int i = i0 + d;
-      const bool row_ok = i < my_rows;
-      float acc[MT];
-#pragma unroll
-      for (int m = 0; m < MT; ++m) {
-#ifdef GGUF_DBG_NODOT
-        const float v = (float)(((const uint32_t*)&pre[d])[0] ^ ((const uint32_t*)&pre[d])[sizeof(typename F::Regs) / 4 - 1]);
-#else
-        const float v = F::dot(pre[d], act[m], u);
-#endif
-        acc[m] = lane_on ? v : 0.0f;
-      }
-      pre[d] = load_row(i + D);  // refill the slot: D - 1 other slots are still in flight
-#pragma unroll
-      for (int m = 0; m < MT; ++m) {
-        const float v = wave_sum(acc[m]);
-        if (lane == 0 && row_ok) part[((slot + slots * i) * S + step) * MT + m] = v;
-      }
-    }
-  }
-  __syncthreads();
-  for (int i = tid; i < nrows * MT; i += 64 * NW) {
-    const int row = i / MT, m = i - row * MT;
-    float v = 0.0f;
-    for (int st = 0; st < S; ++st) v += part[(row * S + st) * MT + m];
-    Y[(int64_t)m * N + r_begin + row] = from_f32<T>(v);
-  }
-}
-
-static int num_cus() {
-  static int n = 0;
-  if (n == 0) {
-    int dev = 0;
-    hipDeviceProp_t prop;
-    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) n = prop.multiProcessorCount;
-    if (n <= 0) n = 256;
-  }
-  return n;
-}
-
-template <class F, int MT, int D, typename T>
-static void launch_stream_d(const void* W, const T* X, T* Y, int N, int K, int rows_per_wg, int grid, size_t lds,
-                            hipStream_t stream) {
-  constexpr int NW = GGUF_MMVQ_NW;
-  auto kern = mmvq_stream_kernel<F, MT, NW, D, T>;
-  static bool big_lds = false;
-  if (lds > 64 * 1024 && !big_lds) {
-    (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
-    big_lds = true;
-  }
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * NW), lds, stream, (const uint8_t*)W, X, Y, N, K, rows_per_wg);
-}
-
-// Returns false when the shape does not fit the streaming kernel (a row longer than NW waves, or activations
-// that do not fit in LDS); the caller then takes the workspace path.
-template <class F, int MT, typename T>
-static bool launch_stream(const void* W, const T* X, T* Y, int N, int K, hipStream_t stream) {
-  constexpr int NW = GGUF_MMVQ_NW;
-  const int nb = K / 32, S = (nb + 63) / 64;
-  if (S > NW) return false;
-  const int slots = NW / S;
-  const int target = num_cus() * GGUF_MMVQ_WG_PER_CU;
-  int rows_per_wg = (N + target - 1) / target;
-  if (rows_per_wg < slots) rows_per_wg = slots;  // at least one row per slot
-  const int grid = (N + rows_per_wg - 1) / rows_per_wg;
-  const size_t lds = (size_t)MT * K + (size_t)MT * nb * 4 * (F::AUX != AUX_NONE ? 2 : 1) + F::TABLE_BYTES +
-                     (size_t)rows_per_wg * S * MT * 4;
-  if (lds > 150 * 1024) return false;
-  const int per_wave = (rows_per_wg + slots - 1) / slots;  // rows each wave walks; the pipeline depth never exceeds it
-  if (per_wave >= GGUF_MMVQ_DEPTH) launch_stream_d<F, MT, GGUF_MMVQ_DEPTH, T>(W, X, Y, N, K, rows_per_wg, grid, lds, stream);
-  else if (per_wave >= 2) launch_stream_d<F, MT, 2, T>(W, X, Y, N, K, rows_per_wg, grid, lds, stream);
-  else launch_stream_d<F, MT, 1, T>(W, X, Y, N, K, rows_per_wg, grid, lds, stream);
-  return true;
-}
-
-#ifndef GGUF_MMVQ_RPW
-#define GGUF_MMVQ_RPW 2
-#endif
-#ifndef GGUF_MMVQ_MAX_FUSED_M
-#define GGUF_MMVQ_MAX_FUSED_M 4
-#endif
-constexpr int MAX_FUSED_M = GGUF_MMVQ_MAX_FUSED_M;  // up to this many vectors are quantized inside the GEMV itself
-
-static inline int kchunk_for(int mt, int K) {
-  int kchunk = mt == 1 ? 32768 : mt == 2 ? 16384 : mt == 4 ? 8192 : 4096;
-  const int kround = (K + 511) / 512 * 512;
-  return kchunk > kround ? kround : kchunk;
-}
-template <class F, int MT>
-static inline size_t mmvq_lds(int kchunk) {
-  return (size_t)MT * kchunk + (size_t)MT * (kchunk / 32) * 4 * (F::AUX != AUX_NONE ? 2 : 1) + F::TABLE_BYTES;
-}
-
-template <class F, int MT, typename T, bool FUSEQ>
-static void launch_mt(const void* W, const char* xsrc, T* Y, int N, int K, hipStream_t stream) {
-  constexpr int RPW = GGUF_MMVQ_RPW;
-  const int kchunk = kchunk_for(MT, K);
-  const int grid = (N + 4 * RPW - 1) / (4 * RPW);
-  const int64_t xrb = FUSEQ ? (int64_t)K * (int64_t)sizeof(T) : q8_row_bytes(K);
-  const size_t lds = mmvq_lds<F, MT>(kchunk);
-  hipLaunchKernelGGL((mmvq_kernel<F, MT, RPW, T, false, FUSEQ>), dim3(grid), dim3(256), lds, stream,
-                     (const uint8_t*)W, xsrc, Y, N, K, kchunk, xrb, (int64_t)N, (const int32_t*)nullptr, 1);
-}
-
-int quantize_q8_1(const void* x, int xdtype, void* ws, int64_t M, int64_t K, hipStream_t stream);
-
-template <class F, typename T>
-static int mmvq_typed(const void* W, const void* x, void* ws, void* Y, int xdtype, int64_t N, int64_t K, int64_t M,
-                      hipStream_t stream) {
-  if (M <= MAX_FUSED_M) {
-    const T* xs = (const T*)x;
-    bool ok;
-    if (M == 1) ok = launch_stream<F, 1, T>(W, xs, (T*)Y, (int)N, (int)K, stream);
-    else if (M == 2) ok = launch_stream<F, 2, T>(W, xs, (T*)Y, (int)N, (int)K, stream);
-    else if (M == 4) ok = launch_stream<F, 4, T>(W, xs, (T*)Y, (int)N, (int)K, stream);
-    else ok = launch_stream<F, 2, T>(W, xs, (T*)Y, (int)N, (int)K, stream) &&
-              launch_stream<F, 1, T>(W, xs + 2 * K, (T*)Y + 2 * N, (int)N, (int)K, stream);
-    if (ok) return launch_status();
-  }
-  const int rc = quantize_q8_1(x, xdtype, ws, M, K, stream);
-  if (rc != GGUF_OK) return rc;
-  const int64_t rb = q8_row_bytes(K);
-  int64_t m0 = 0;
-  while (m0 < M) {
-    const int64_t left = M - m0;
-    const char* wsm = (const char*)ws + m0 * rb;
-    T* ym = (T*)Y + m0 * N;
-    if (left >= 8) { launch_mt<F, 8, T, false>(W, wsm, ym, (int)N, (int)K, stream); m0 += 8; }
-    else if (left >= 4) { launch_mt<F, 4, T, false>(W, wsm, ym, (int)N, (int)K, stream); m0 += 4; }
-    else if (left >= 2) { launch_mt<F, 2, T, false>(W, wsm, ym, (int)N, (int)K, stream); m0 += 2; }
-    else { launch_mt<F, 1, T, false>(W, wsm, ym, (int)N, (int)K, stream); m0 += 1; }
-  }
-  return launch_status();
-}
-
-template <class F, typename T>
-static int moe_vec_typed(const void* W, const char* x, void* Y, int N, int K, const int32_t* topk_ids, int top_k,
-                         int pairs, hipStream_t stream) {
-  constexpr int RPW = GGUF_MMVQ_RPW;
-  const int kchunk = kchunk_for(1, K);
-  const int grid = (N + 4 * RPW - 1) / (4 * RPW);
-  const int64_t xrb = (int64_t)K * (int64_t)sizeof(T);
-  const size_t lds = mmvq_lds<F, 1>(kchunk);
-  for (int z0 = 0; z0 < pairs; z0 += 65535) {
-    const int nz = pairs - z0 < 65535 ? pairs - z0 : 65535;
-    // the pair index is rebuilt from blockIdx.y, so later slabs shift the id and output bases by whole tokens
-    if (z0 % top_k != 0) return GGUF_ERR_SHAPE;
-    hipLaunchKernelGGL((mmvq_kernel<F, 1, RPW, T, true, true>), dim3(grid, nz), dim3(256), lds, stream,
-                       (const uint8_t*)W, x + (int64_t)(z0 / top_k) * xrb, (T*)Y + (int64_t)z0 * N, N, K, kchunk, xrb,
-                       (int64_t)N, topk_ids + z0, top_k);
-  }
-  return launch_status();
-}
-
-template <class F>
-static int moe_vec_fmt(const void* W, const void* x, void* Y, int dtype, int N, int K, const int32_t* ids, int top_k,
-                       int pairs, hipStream_t s) {
-  GGUF_DISPATCH_DTYPE(dtype, return (moe_vec_typed<F, scalar_t>(W, (const char*)x, Y, N, K, ids, top_k, pairs, s)));
-  return GGUF_ERR_DTYPE;
-}
-
-template <class F>
-static int mmvq_fmt(const void* W, const void* x, void* ws, void* Y, int dtype, int64_t N, int64_t K, int64_t M,
-                    hipStream_t s) {
-  GGUF_DISPATCH_DTYPE(dtype, return (mmvq_typed<F, scalar_t>(W, x, ws, Y, dtype, N, K, M, s)));
-  return GGUF_ERR_DTYPE;
-}
+int moe_vec_group_std_a(int type, const void* W, const void* x, void* Y, int dtype, int N, int K, const int32_t* ids, int top_k,
+                      int pairs, hipStream_t s);
+int moe_vec_group_std_b(int type, const void* W, const void* x, void* Y, int dtype, int N, int K, const int32_t* ids, int top_k,
+                      int pairs, hipStream_t s);
+int moe_vec_group_k_a(int type, const void* W, const void* x, void* Y, int dtype, int N, int K, const int32_t* ids, int top_k,
+                      int pairs, hipStream_t s);
+int moe_vec_group_k_b(int type, const void* W, const void* x, void* Y, int dtype, int N, int K, const int32_t* ids, int top_k,
+                      int pairs, hipStream_t s);
+int moe_vec_group_iq_a(int type, const void* W, const void* x, void* Y, int dtype, int N, int K, const int32_t* ids, int top_k,
+                      int pairs, hipStream_t s);
+int moe_vec_group_iq_b(int type, const void* W, const void* x, void* Y, int dtype, int N, int K, const int32_t* ids, int top_k,
+                      int pairs, hipStream_t s);
+int moe_vec_group_iq_c(int type, const void* W, const void* x, void* Y, int dtype, int N, int K, const int32_t* ids, int top_k,
+                      int pairs, hipStream_t s);
 
 }  // namespace gguf
 
@@ -740,16 +47,25 @@ extern "C" int gguf_mmvq(const void* W, const void* x, int xdtype, void* q8_work
   if (!W || !x || !q8_workspace || !Y) return GGUF_ERR_NULL;
   hipStream_t s = (hipStream_t)stream;
   switch (type) {
-    case T_Q4_0: case T_Q8_0: case T_Q4_K: case T_Q6_K: case T_IQ4_XS: case T_IQ2_XXS: break;
-    default: return GGUF_ERR_TYPE;
-  }
-  switch (type) {
-    case T_Q4_0: return mmvq_fmt<FmtQ4_0>(W, x, q8_workspace, Y, xdtype, N, K, M, s);
-    case T_Q8_0: return mmvq_fmt<FmtQ8_0>(W, x, q8_workspace, Y, xdtype, N, K, M, s);
-    case T_Q4_K: return mmvq_fmt<FmtQ4_K>(W, x, q8_workspace, Y, xdtype, N, K, M, s);
-    case T_Q6_K: return mmvq_fmt<FmtQ6_K>(W, x, q8_workspace, Y, xdtype, N, K, M, s);
-    case T_IQ4_XS: return mmvq_fmt<FmtIQ4_XS>(W, x, q8_workspace, Y, xdtype, N, K, M, s);
-    case T_IQ2_XXS: return mmvq_fmt<FmtIQ2_XXS>(W, x, q8_workspace, Y, xdtype, N, K, M, s);
+    case T_Q4_0: return mmvq_group_std_a(type, W, x, q8_workspace, Y, xdtype, N, K, M, s);
+    case T_Q4_1: return mmvq_group_std_a(type, W, x, q8_workspace, Y, xdtype, N, K, M, s);
+    case T_Q8_0: return mmvq_group_std_a(type, W, x, q8_workspace, Y, xdtype, N, K, M, s);
+    case T_Q5_0: return mmvq_group_std_b(type, W, x, q8_workspace, Y, xdtype, N, K, M, s);
+    case T_Q5_1: return mmvq_group_std_b(type, W, x, q8_workspace, Y, xdtype, N, K, M, s);
+    case T_IQ4_NL: return mmvq_group_std_b(type, W, x, q8_workspace, Y, xdtype, N, K, M, s);
+    case T_Q2_K: return mmvq_group_k_a(type, W, x, q8_workspace, Y, xdtype, N, K, M, s);
+    case T_Q3_K: return mmvq_group_k_a(type, W, x, q8_workspace, Y, xdtype, N, K, M, s);
+    case T_Q6_K: return mmvq_group_k_a(type, W, x, q8_workspace, Y, xdtype, N, K, M, s);
+    case T_Q4_K: return mmvq_group_k_b(type, W, x, q8_workspace, Y, xdtype, N, K, M, s);
+    case T_Q5_K: return mmvq_group_k_b(type, W, x, q8_workspace, Y, xdtype, N, K, M, s);
+    case T_IQ4_XS: return mmvq_group_iq_a(type, W, x, q8_workspace, Y, xdtype, N, K, M, s);
+    case T_IQ2_XXS: return mmvq_group_iq_a(type, W, x, q8_workspace, Y, xdtype, N, K, M, s);
+    case T_IQ3_XXS: return mmvq_group_iq_a(type, W, x, q8_workspace, Y, xdtype, N, K, M, s);
+    case T_IQ2_XS: return mmvq_group_iq_b(type, W, x, q8_workspace, Y, xdtype, N, K, M, s);
+    case T_IQ2_S: return mmvq_group_iq_b(type, W, x, q8_workspace, Y, xdtype, N, K, M, s);
+    case T_IQ3_S: return mmvq_group_iq_b(type, W, x, q8_workspace, Y, xdtype, N, K, M, s);
+    case T_IQ1_S: return mmvq_group_iq_c(type, W, x, q8_workspace, Y, xdtype, N, K, M, s);
+    case T_IQ1_M: return mmvq_group_iq_c(type, W, x, q8_workspace, Y, xdtype, N, K, M, s);
   }
   return GGUF_ERR_TYPE;
 }
@@ -763,21 +79,30 @@ extern "C" int gguf_moe_vec(const void* X, int xdtype, void* q8_workspace, const
       tokens * top_k > 0x7FFFFFF0LL)
     return GGUF_ERR_SHAPE;
   if (xdtype < 0 || xdtype > 2) return GGUF_ERR_DTYPE;
-  switch (type) {
-    case T_Q4_0: case T_Q8_0: case T_Q4_K: case T_Q6_K: case T_IQ4_XS: case T_IQ2_XXS: break;
-    default: return GGUF_ERR_TYPE;
-  }
   if (N == 0 || tokens == 0) return GGUF_OK;
   if (!X || !q8_workspace || !W || !topk_ids || !Y) return GGUF_ERR_NULL;
   hipStream_t s = (hipStream_t)stream;
   const int pairs = (int)(tokens * top_k);
   switch (type) {
-    case T_Q4_0: return moe_vec_fmt<FmtQ4_0>(W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
-    case T_Q8_0: return moe_vec_fmt<FmtQ8_0>(W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
-    case T_Q4_K: return moe_vec_fmt<FmtQ4_K>(W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
-    case T_Q6_K: return moe_vec_fmt<FmtQ6_K>(W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
-    case T_IQ4_XS: return moe_vec_fmt<FmtIQ4_XS>(W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
-    case T_IQ2_XXS: return moe_vec_fmt<FmtIQ2_XXS>(W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
+    case T_Q4_0: return moe_vec_group_std_a(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
+    case T_Q4_1: return moe_vec_group_std_a(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
+    case T_Q8_0: return moe_vec_group_std_a(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
+    case T_Q5_0: return moe_vec_group_std_b(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
+    case T_Q5_1: return moe_vec_group_std_b(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
+    case T_IQ4_NL: return moe_vec_group_std_b(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
+    case T_Q2_K: return moe_vec_group_k_a(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
+    case T_Q3_K: return moe_vec_group_k_a(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
+    case T_Q6_K: return moe_vec_group_k_a(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
+    case T_Q4_K: return moe_vec_group_k_b(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
+    case T_Q5_K: return moe_vec_group_k_b(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
+    case T_IQ4_XS: return moe_vec_group_iq_a(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
+    case T_IQ2_XXS: return moe_vec_group_iq_a(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
+    case T_IQ3_XXS: return moe_vec_group_iq_a(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
+    case T_IQ2_XS: return moe_vec_group_iq_b(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
+    case T_IQ2_S: return moe_vec_group_iq_b(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
+    case T_IQ3_S: return moe_vec_group_iq_b(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
+    case T_IQ1_S: return moe_vec_group_iq_c(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
+    case T_IQ1_M: return moe_vec_group_iq_c(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
   }
   return GGUF_ERR_TYPE;
 }

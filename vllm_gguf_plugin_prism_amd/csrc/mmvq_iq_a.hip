@@ -1,0 +1,27 @@
+// GEMV and per-pair MoE GEMV instantiations for IQ4_XS, IQ2_XXS, IQ3_XXS (one translation unit per group of formats so
+// that the groups compile in parallel).  Returns GGUF_ERR_TYPE for a type outside the group.
+#include "mmvq_core.h"
+
+namespace gguf {
+
+int mmvq_group_iq_a(int type, const void* W, const void* x, void* ws, void* Y, int dtype, int64_t N, int64_t K, int64_t M,
+                   hipStream_t s) {
+  switch (type) {
+    case T_IQ4_XS: return mmvq_fmt<FmtIQ4_XS>(W, x, ws, Y, dtype, N, K, M, s);
+    case T_IQ2_XXS: return mmvq_fmt<FmtIQ2_XXS>(W, x, ws, Y, dtype, N, K, M, s);
+    case T_IQ3_XXS: return mmvq_fmt<FmtIQ3_XXS>(W, x, ws, Y, dtype, N, K, M, s);
+    default: return GGUF_ERR_TYPE;
+  }
+}
+
+int moe_vec_group_iq_a(int type, const void* W, const void* x, void* Y, int dtype, int N, int K, const int32_t* ids, int top_k,
+                      int pairs, hipStream_t s) {
+  switch (type) {
+    case T_IQ4_XS: return moe_vec_fmt<FmtIQ4_XS>(W, x, Y, dtype, N, K, ids, top_k, pairs, s);
+    case T_IQ2_XXS: return moe_vec_fmt<FmtIQ2_XXS>(W, x, Y, dtype, N, K, ids, top_k, pairs, s);
+    case T_IQ3_XXS: return moe_vec_fmt<FmtIQ3_XXS>(W, x, Y, dtype, N, K, ids, top_k, pairs, s);
+    default: return GGUF_ERR_TYPE;
+  }
+}
+
+}  // namespace gguf

@@ -1,0 +1,27 @@
+// GEMV and per-pair MoE GEMV instantiations for IQ2_XS, IQ2_S, IQ3_S (one translation unit per group of formats so
+// that the groups compile in parallel).  Returns GGUF_ERR_TYPE for a type outside the group.
+#include "mmvq_core.h"
+
+namespace gguf {
+
+int mmvq_group_iq_b(int type, const void* W, const void* x, void* ws, void* Y, int dtype, int64_t N, int64_t K, int64_t M,
+                   hipStream_t s) {
+  switch (type) {
+    case T_IQ2_XS: return mmvq_fmt<FmtIQ2_XS>(W, x, ws, Y, dtype, N, K, M, s);
+    case T_IQ2_S: return mmvq_fmt<FmtIQ2_S>(W, x, ws, Y, dtype, N, K, M, s);
+    case T_IQ3_S: return mmvq_fmt<FmtIQ3_S>(W, x, ws, Y, dtype, N, K, M, s);
+    default: return GGUF_ERR_TYPE;
+  }
+}
+
+int moe_vec_group_iq_b(int type, const void* W, const void* x, void* Y, int dtype, int N, int K, const int32_t* ids, int top_k,
+                      int pairs, hipStream_t s) {
+  switch (type) {
+    case T_IQ2_XS: return moe_vec_fmt<FmtIQ2_XS>(W, x, Y, dtype, N, K, ids, top_k, pairs, s);
+    case T_IQ2_S: return moe_vec_fmt<FmtIQ2_S>(W, x, Y, dtype, N, K, ids, top_k, pairs, s);
+    case T_IQ3_S: return moe_vec_fmt<FmtIQ3_S>(W, x, Y, dtype, N, K, ids, top_k, pairs, s);
+    default: return GGUF_ERR_TYPE;
+  }
+}
+
+}  // namespace gguf
