@@ -8,6 +8,7 @@ from oracle import gguf_oracle as o
 pytestmark = pytest.mark.gpu
 
 SIX = [o.Q4_0, o.Q8_0, o.Q4_K, o.Q6_K, o.IQ4_XS, o.IQ2_XXS]
+MMQ_TYPES = [o.Q4_0, o.Q4_1, o.Q5_0, o.Q5_1, o.Q8_0, o.Q2_K, o.Q3_K, o.Q4_K, o.Q5_K, o.Q6_K, o.IQ4_XS, o.IQ2_XXS]
 ALL = [o.Q4_0, o.Q4_1, o.Q5_0, o.Q5_1, o.Q8_0, o.Q2_K, o.Q3_K, o.Q4_K, o.Q5_K, o.Q6_K, o.IQ2_XXS, o.IQ2_XS, o.IQ3_XXS,
        o.IQ1_S, o.IQ4_NL, o.IQ3_S, o.IQ2_S, o.IQ4_XS, o.IQ1_M]
 TORCH_DT = {"f16": torch.float16, "bf16": torch.bfloat16, "f32": torch.float32}
@@ -27,7 +28,7 @@ def _x(rng, m, k, dt):
     return t.cuda(), t.to(torch.float32).numpy()
 
 
-@pytest.mark.parametrize("qtype", SIX)
+@pytest.mark.parametrize("qtype", MMQ_TYPES)
 @pytest.mark.parametrize("m", [7, 83, 128, 200])
 def test_mmq_matches_a8_oracle_fp32(qtype, m):
     ops = _ops()
@@ -44,7 +45,7 @@ def test_mmq_matches_a8_oracle_fp32(qtype, m):
 
 
 @pytest.mark.parametrize("dt", ["f16", "bf16"])
-@pytest.mark.parametrize("qtype", SIX)
+@pytest.mark.parametrize("qtype", MMQ_TYPES)
 def test_mmq_half_outputs_within_tolerance(qtype, dt):
     # stated tolerance vs the a8 oracle: rel-L2 <= 1e-3 for fp16 outputs, 4e-3 for bf16 (8-bit significand)
     ops = _ops()
@@ -89,7 +90,7 @@ def _routing(rng, t, e, top_k):
     return ids, (wts / wts.sum(axis=1, keepdims=True)).astype(np.float32)
 
 
-@pytest.mark.parametrize("qtype", [o.Q4_0, o.Q4_K, o.Q6_K, o.Q8_0])
+@pytest.mark.parametrize("qtype", [o.Q4_0, o.Q4_1, o.Q5_0, o.Q5_1, o.Q8_0, o.Q2_K, o.Q3_K, o.Q4_K, o.Q5_K, o.Q6_K])
 @pytest.mark.parametrize("t,top_k,e", [(7, 2, 8), (83, 4, 16), (128, 8, 64)])
 def test_moe_grouped_matches_oracle(qtype, t, top_k, e):
     ops = _ops()

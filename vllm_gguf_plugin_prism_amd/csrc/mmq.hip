@@ -59,6 +59,15 @@ __device__ __forceinline__ void fmac_quad(float& acc, float v, float c) {
   if constexpr (T == 2) asm("v_fmac_f32_dpp %0, %1, %2 quad_perm:[2,2,2,2] row_mask:0xf bank_mask:0xf" : "+v"(acc) : "v"(v), "v"(c));
   if constexpr (T == 3) asm("v_fmac_f32_dpp %0, %1, %2 quad_perm:[3,3,3,3] row_mask:0xf bank_mask:0xf" : "+v"(acc) : "v"(v), "v"(c));
 }
+// v[lane (l & ~3) + T] as a value (a DPP move the compiler can see and schedule)
+template <int T>
+__device__ __forceinline__ float quad_get(float v) {
+  constexpr int ctrl = T | (T << 2) | (T << 4) | (T << 6);
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), ctrl, 0xF, 0xF, true));
+}
+template <int R>
+__device__ __forceinline__ float row_get(const float (&v)[4]) { return quad_get<R & 3>(v[R >> 2]); }
+
 template <int R>
 __device__ __forceinline__ void fmac_row(float& acc, const float (&v)[4], float c) { fmac_quad<R & 3>(acc, v[R >> 2], c); }
 
@@ -76,6 +85,43 @@ __device__ __forceinline__ void offset16(float (&acc)[16], const float (&v)[4], 
   fmac_row<12>(acc[12], v, c); fmac_row<13>(acc[13], v, c); fmac_row<14>(acc[14], v, c); fmac_row<15>(acc[15], v, c);
 }
 
+
+// Q4_1 / Q5_1 (reference: vec_dot_q8_1_q8_1_impl, vecdotq.cuh:179-198): acc += S * half(d * d8) + half(m * s8),
+// both scale products rounded to half precision as __hmul2 does; d, d8, m and s8 are fp16 values held in floats.
+template <int R>
+__device__ __forceinline__ void half_products1(float& acc, int bits, const float (&d8)[4], const float (&s8)[4], float d, float m) {
+  const _Float16 dd = (_Float16)d * (_Float16)row_get<R>(d8);
+  const _Float16 ms = (_Float16)m * (_Float16)row_get<R>(s8);
+  acc += (__int_as_float(bits) - kSeed) * (float)dd + (float)ms;
+}
+__device__ __forceinline__ void half_products16(float (&acc)[16], const v16i& s, const float (&d8)[4], const float (&s8)[4], float d, float m) {
+  half_products1<0>(acc[0], s[0], d8, s8, d, m);    half_products1<1>(acc[1], s[1], d8, s8, d, m);
+  half_products1<2>(acc[2], s[2], d8, s8, d, m);    half_products1<3>(acc[3], s[3], d8, s8, d, m);
+  half_products1<4>(acc[4], s[4], d8, s8, d, m);    half_products1<5>(acc[5], s[5], d8, s8, d, m);
+  half_products1<6>(acc[6], s[6], d8, s8, d, m);    half_products1<7>(acc[7], s[7], d8, s8, d, m);
+  half_products1<8>(acc[8], s[8], d8, s8, d, m);    half_products1<9>(acc[9], s[9], d8, s8, d, m);
+  half_products1<10>(acc[10], s[10], d8, s8, d, m); half_products1<11>(acc[11], s[11], d8, s8, d, m);
+  half_products1<12>(acc[12], s[12], d8, s8, d, m); half_products1<13>(acc[13], s[13], d8, s8, d, m);
+  half_products1<14>(acc[14], s[14], d8, s8, d, m); half_products1<15>(acc[15], s[15], d8, s8, d, m);
+}
+
+// Q2_K: acc[r] += d8[row] * (ua[row] * nma + ub[row] * nmb)
+template <int R>
+__device__ __forceinline__ void group_offsets1(float& acc, const float (&d8)[4], const float (&ua)[4], const float (&ub)[4], float nma, float nmb) {
+  const float t = __builtin_fmaf(row_get<R>(ub), nmb, row_get<R>(ua) * nma);
+  fmac_row<R>(acc, d8, t);
+}
+__device__ __forceinline__ void group_offsets16(float (&acc)[16], const float (&d8)[4], const float (&ua)[4], const float (&ub)[4], float nma, float nmb) {
+  group_offsets1<0>(acc[0], d8, ua, ub, nma, nmb);   group_offsets1<1>(acc[1], d8, ua, ub, nma, nmb);
+  group_offsets1<2>(acc[2], d8, ua, ub, nma, nmb);   group_offsets1<3>(acc[3], d8, ua, ub, nma, nmb);
+  group_offsets1<4>(acc[4], d8, ua, ub, nma, nmb);   group_offsets1<5>(acc[5], d8, ua, ub, nma, nmb);
+  group_offsets1<6>(acc[6], d8, ua, ub, nma, nmb);   group_offsets1<7>(acc[7], d8, ua, ub, nma, nmb);
+  group_offsets1<8>(acc[8], d8, ua, ub, nma, nmb);   group_offsets1<9>(acc[9], d8, ua, ub, nma, nmb);
+  group_offsets1<10>(acc[10], d8, ua, ub, nma, nmb); group_offsets1<11>(acc[11], d8, ua, ub, nma, nmb);
+  group_offsets1<12>(acc[12], d8, ua, ub, nma, nmb); group_offsets1<13>(acc[13], d8, ua, ub, nma, nmb);
+  group_offsets1<14>(acc[14], d8, ua, ub, nma, nmb); group_offsets1<15>(acc[15], d8, ua, ub, nma, nmb);
+}
+
 // LDS row pitch in bytes.  K=32 operands are read 16 bytes per lane: a 16-byte skew (144) spreads 8 consecutive rows
 // over all banks.  K=16 operands are read 8 bytes per lane: an 8-byte skew (136) spreads 16 consecutive rows.
 template <int G, int KS> struct Pitch { static constexpr int value = G == 32 ? KS + 16 : KS + 8; };
@@ -91,12 +137,13 @@ struct MQ4_0 {  // vecdotq.cuh:46-66, 511-571
   static constexpr int QK = 32, BS = 18, G = 32;
   static constexpr bool HAS_MIN = true;
   static constexpr bool LIGHT = true;  // packed block small enough to hold a step of them in registers
+  static constexpr bool HALFPROD = false, MIN16 = false;
   struct Raw { uint16_t d; uint4 q; };
   static __device__ __forceinline__ Raw fetch(const uint8_t* row, int kb) {
     const uint8_t* b = row + (int64_t)kb * BS;
     Raw r; r.d = ld<uint16_t>(b); r.q = ld<uint4>(b + 2); return r;
   }
-  static __device__ __forceinline__ void unpack(const Raw& r, int kb, uint32_t (&q)[8], float& s0, float& s1, float& mn) {
+  static __device__ __forceinline__ void unpack(const Raw& r, int kb, uint32_t (&q)[8], float& s0, float& s1, float& mn, float& mn1) {
     const uint32_t w[4] = {r.q.x, r.q.y, r.q.z, r.q.w};
 #pragma unroll
     for (int i = 0; i < 4; ++i) { q[i] = w[i] & 0x0F0F0F0Fu; q[4 + i] = (w[i] >> 4) & 0x0F0F0F0Fu; }
@@ -108,12 +155,13 @@ struct MQ8_0 {  // vecdotq.cuh:165-177, 869-921
   static constexpr int QK = 32, BS = 34, G = 32;
   static constexpr bool HAS_MIN = false;
   static constexpr bool LIGHT = true;  // packed block small enough to hold a step of them in registers
+  static constexpr bool HALFPROD = false, MIN16 = false;
   struct Raw { uint16_t d; uint4 q0, q1; };
   static __device__ __forceinline__ Raw fetch(const uint8_t* row, int kb) {
     const uint8_t* b = row + (int64_t)kb * BS;
     Raw r; r.d = ld<uint16_t>(b); r.q0 = ld<uint4>(b + 2); r.q1 = ld<uint4>(b + 18); return r;
   }
-  static __device__ __forceinline__ void unpack(const Raw& r, int kb, uint32_t (&q)[8], float& s0, float& s1, float& mn) {
+  static __device__ __forceinline__ void unpack(const Raw& r, int kb, uint32_t (&q)[8], float& s0, float& s1, float& mn, float& mn1) {
     q[0] = r.q0.x; q[1] = r.q0.y; q[2] = r.q0.z; q[3] = r.q0.w; q[4] = r.q1.x; q[5] = r.q1.y; q[6] = r.q1.z; q[7] = r.q1.w;
     s0 = (float)__builtin_bit_cast(_Float16, r.d); s1 = s0; mn = 0.0f;
   }
@@ -123,13 +171,14 @@ struct MQ4_K {  // vecdotq.cuh:353-379, 1204-1277
   static constexpr int QK = 256, BS = 144, G = 32;
   static constexpr bool HAS_MIN = true;
   static constexpr bool LIGHT = false;  // packed block small enough to hold a step of them in registers
+  static constexpr bool HALFPROD = false, MIN16 = false;
   struct Raw { uint4 hdr, v0, v1; };
   static __device__ __forceinline__ Raw fetch(const uint8_t* row, int kb) {
     const int sb = kb >> 3, j = kb & 7;
     const uint8_t* b = row + (int64_t)sb * BS;
     Raw r; r.hdr = ld<uint4>(b); r.v0 = ld<uint4>(b + 16 + 32 * (j >> 1)); r.v1 = ld<uint4>(b + 32 + 32 * (j >> 1)); return r;
   }
-  static __device__ __forceinline__ void unpack(const Raw& r, int kb, uint32_t (&q)[8], float& s0, float& s1, float& mn) {
+  static __device__ __forceinline__ void unpack(const Raw& r, int kb, uint32_t (&q)[8], float& s0, float& s1, float& mn, float& mn1) {
     const int j = kb & 7;
     const int sh = (j & 1) ? 4 : 0;
     const uint32_t w[8] = {r.v0.x, r.v0.y, r.v0.z, r.v0.w, r.v1.x, r.v1.y, r.v1.z, r.v1.w};
@@ -154,6 +203,7 @@ struct MQ6_K {  // vecdotq.cuh:467-491, 1443-1529: two int8 sub-scales per q8_1 
   static constexpr int QK = 256, BS = 210, G = 16;
   static constexpr bool HAS_MIN = false;
   static constexpr bool LIGHT = false;  // packed block small enough to hold a step of them in registers
+  static constexpr bool HALFPROD = false, MIN16 = false;
   struct Raw { uint4 l0, l1, h0, h1; uint16_t sc, d; };
   static __device__ __forceinline__ Raw fetch(const uint8_t* row, int kb) {
     const int sb = kb >> 3, h = (kb >> 2) & 1, t = kb & 3;
@@ -166,7 +216,7 @@ struct MQ6_K {  // vecdotq.cuh:467-491, 1443-1529: two int8 sub-scales per q8_1 
     r.d = ld<uint16_t>(b + 208);
     return r;
   }
-  static __device__ __forceinline__ void unpack(const Raw& r, int kb, uint32_t (&q)[8], float& s0, float& s1, float& mn) {
+  static __device__ __forceinline__ void unpack(const Raw& r, int kb, uint32_t (&q)[8], float& s0, float& s1, float& mn, float& mn1) {
     const int t = kb & 3;
     const uint32_t lw[8] = {r.l0.x, r.l0.y, r.l0.z, r.l0.w, r.l1.x, r.l1.y, r.l1.z, r.l1.w};
     const uint32_t hw[8] = {r.h0.x, r.h0.y, r.h0.z, r.h0.w, r.h1.x, r.h1.y, r.h1.z, r.h1.w};
@@ -183,6 +233,156 @@ struct MQ6_K {  // vecdotq.cuh:467-491, 1443-1529: two int8 sub-scales per q8_1 
   }
 };
 
+// bits 0..3 of b -> bit 0 of bytes 0..3
+__device__ __forceinline__ uint32_t spread4q(uint32_t b) { return ((b & 0xFu) * 0x00204081u) & 0x01010101u; }
+// every byte of v (each below 128) minus c, with no borrow between bytes
+__device__ __forceinline__ uint32_t sub_bytes(uint32_t v, uint32_t c4) { return ((v | 0x80808080u) - c4) ^ 0x80808080u; }
+
+// Q4_1 and Q5_1 keep the reference's half-precision scale products: S * half(d*d8) + half(m*s8)
+// (vecdotq.cuh:71-93, 179-198, 591-646, 771-850).
+struct MQ4_1 {
+  static constexpr int QK = 32, BS = 20, G = 32;
+  static constexpr bool HAS_MIN = true;
+  static constexpr bool LIGHT = false;
+  static constexpr bool HALFPROD = true, MIN16 = false;
+  struct Raw { uint32_t dm; uint4 q; };
+  static __device__ __forceinline__ Raw fetch(const uint8_t* row, int kb) {
+    const uint8_t* b = row + (int64_t)kb * BS;
+    Raw r; r.dm = ld<uint32_t>(b); r.q = ld<uint4>(b + 4); return r;
+  }
+  static __device__ __forceinline__ void unpack(const Raw& r, int kb, uint32_t (&q)[8], float& s0, float& s1, float& mn, float& mn1) {
+    const uint32_t w[4] = {r.q.x, r.q.y, r.q.z, r.q.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) { q[i] = w[i] & 0x0F0F0F0Fu; q[4 + i] = (w[i] >> 4) & 0x0F0F0F0Fu; }
+    s0 = (float)__builtin_bit_cast(_Float16, (uint16_t)(r.dm & 0xFFFF)); s1 = s0;
+    mn = (float)__builtin_bit_cast(_Float16, (uint16_t)(r.dm >> 16)); mn1 = mn;
+  }
+};
+
+template <bool HAS_M>
+struct MQ5 {  // Q5_0: signed codes, no offset term (vecdotq.cuh:668-749); Q5_1: as Q4_1 with a fifth bit
+  static constexpr int QK = 32, BS = HAS_M ? 24 : 22, G = 32;
+  static constexpr bool HAS_MIN = HAS_M;
+  static constexpr bool LIGHT = !HAS_M;
+  static constexpr bool HALFPROD = HAS_M, MIN16 = false;
+  struct Raw { uint32_t dm, qh; uint4 q; };
+  static __device__ __forceinline__ Raw fetch(const uint8_t* row, int kb) {
+    const uint8_t* b = row + (int64_t)kb * BS;
+    Raw r;
+    if (HAS_M) { r.dm = ld<uint32_t>(b); r.qh = ld<uint32_t>(b + 4); r.q = ld<uint4>(b + 8); }
+    else { r.dm = ld<uint16_t>(b); r.qh = ld<uint32_t>(b + 2); r.q = ld<uint4>(b + 6); }
+    return r;
+  }
+  static __device__ __forceinline__ void unpack(const Raw& r, int kb, uint32_t (&q)[8], float& s0, float& s1, float& mn, float& mn1) {
+    const uint32_t w[4] = {r.q.x, r.q.y, r.q.z, r.q.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      q[i] = (w[i] & 0x0F0F0F0Fu) | (spread4q(r.qh >> (4 * i)) << 4);
+      q[4 + i] = ((w[i] >> 4) & 0x0F0F0F0Fu) | (spread4q(r.qh >> (16 + 4 * i)) << 4);
+      if (!HAS_M) { q[i] = sub_bytes(q[i], 0x10101010u); q[4 + i] = sub_bytes(q[4 + i], 0x10101010u); }
+    }
+    s0 = (float)__builtin_bit_cast(_Float16, (uint16_t)(r.dm & 0xFFFF)); s1 = s0;
+    mn = HAS_M ? (float)__builtin_bit_cast(_Float16, (uint16_t)(r.dm >> 16)) : 0.0f; mn1 = mn;
+  }
+};
+typedef MQ5<false> MQ5_0;
+typedef MQ5<true> MQ5_1;
+
+struct MQ2_K {  // vecdotq.cuh:232-263, 946-1022: per 16 elements a 4-bit scale and a 4-bit min; the min term
+                // multiplies the sum of the activation quants of those 16 elements, not the stored block sum
+  static constexpr int QK = 256, BS = 84, G = 16;
+  static constexpr bool HAS_MIN = true;
+  static constexpr bool LIGHT = false;
+  static constexpr bool HALFPROD = false, MIN16 = true;
+  struct Raw { uint4 v0, v1; uint32_t dm; uint16_t sc; };
+  static __device__ __forceinline__ Raw fetch(const uint8_t* row, int kb) {
+    const int sb = kb >> 3, n = (kb >> 2) & 1, t = kb & 3;
+    const uint8_t* b = row + (int64_t)sb * BS;
+    Raw r;
+    r.v0 = ld<uint4>(b + 16 + 32 * n); r.v1 = ld<uint4>(b + 32 + 32 * n);
+    r.sc = ld<uint16_t>(b + 8 * n + 2 * t); r.dm = ld<uint32_t>(b + 80);
+    return r;
+  }
+  static __device__ __forceinline__ void unpack(const Raw& r, int kb, uint32_t (&q)[8], float& s0, float& s1, float& mn, float& mn1) {
+    const int t = kb & 3;
+    const uint32_t w[8] = {r.v0.x, r.v0.y, r.v0.z, r.v0.w, r.v1.x, r.v1.y, r.v1.z, r.v1.w};
+#pragma unroll
+    for (int i = 0; i < 8; ++i) q[i] = (w[i] >> (2 * t)) & 0x03030303u;
+    const float d = (float)__builtin_bit_cast(_Float16, (uint16_t)(r.dm & 0xFFFF));
+    const float dmin = (float)__builtin_bit_cast(_Float16, (uint16_t)(r.dm >> 16));
+    s0 = d * (float)(r.sc & 0xF); s1 = d * (float)((r.sc >> 8) & 0xF);
+    mn = dmin * (float)((r.sc >> 4) & 0xF); mn1 = dmin * (float)(r.sc >> 12);
+  }
+};
+
+struct MQ3_K {  // vecdotq.cuh:298-322, 1051-1157: codes -4..3, a signed 6-bit scale per 16 elements
+  static constexpr int QK = 256, BS = 110, G = 16;
+  static constexpr bool HAS_MIN = false;
+  static constexpr bool LIGHT = false;
+  static constexpr bool HALFPROD = false, MIN16 = false;
+  struct Raw { uint4 v0, v1, h0, h1; uint2 sc01; uint32_t sc2; uint16_t d; };
+  static __device__ __forceinline__ Raw fetch(const uint8_t* row, int kb) {
+    const int sb = kb >> 3, n = (kb >> 2) & 1;
+    const uint8_t* b = row + (int64_t)sb * BS;
+    Raw r;
+    r.v0 = ld<uint4>(b + 32 + 32 * n); r.v1 = ld<uint4>(b + 48 + 32 * n); r.h0 = ld<uint4>(b); r.h1 = ld<uint4>(b + 16);
+    r.sc01 = ld<uint2>(b + 96); r.sc2 = ld<uint32_t>(b + 104); r.d = ld<uint16_t>(b + 108);
+    return r;
+  }
+  static __device__ __forceinline__ void unpack(const Raw& r, int kb, uint32_t (&q)[8], float& s0, float& s1, float& mn, float& mn1) {
+    const int n = (kb >> 2) & 1, t = kb & 3;
+    const uint32_t w[8] = {r.v0.x, r.v0.y, r.v0.z, r.v0.w, r.v1.x, r.v1.y, r.v1.z, r.v1.w};
+    const uint32_t h[8] = {r.h0.x, r.h0.y, r.h0.z, r.h0.w, r.h1.x, r.h1.y, r.h1.z, r.h1.w};
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+      q[i] = sub_bytes(((w[i] >> (2 * t)) & 0x03030303u) | (((h[i] >> (4 * n + t)) & 0x01010101u) << 2), 0x04040404u);
+    const uint64_t lo64 = ((uint64_t)r.sc01.y << 32) | r.sc01.x;
+    const float d = (float)__builtin_bit_cast(_Float16, r.d);
+    int us[2];
+#pragma unroll
+    for (int e = 0; e < 2; ++e) {  // 6-bit scale of 16-element group is = 8n + 2t + e (dequantize.cuh:137-140)
+      const int g = 2 * t + e, is = 8 * n + g;
+      us[e] = (int)((lo64 >> (8 * g + 4 * n)) & 0xF) | (int)(((r.sc2 >> (8 * (is & 3) + 2 * (is >> 2))) & 3) << 4);
+    }
+    s0 = d * (float)(us[0] - 32); s1 = d * (float)(us[1] - 32); mn = 0.0f; mn1 = 0.0f;
+  }
+};
+
+struct MQ5_K {  // vecdotq.cuh:415-441, 1325-1415: Q4_K with a fifth bit, bit j of qh[l] for sub-block j
+  static constexpr int QK = 256, BS = 176, G = 32;
+  static constexpr bool HAS_MIN = true;
+  static constexpr bool LIGHT = false;
+  static constexpr bool HALFPROD = false, MIN16 = false;
+  struct Raw { uint4 hdr, v0, v1, h0, h1; };
+  static __device__ __forceinline__ Raw fetch(const uint8_t* row, int kb) {
+    const int sb = kb >> 3, j = kb & 7;
+    const uint8_t* b = row + (int64_t)sb * BS;
+    Raw r;
+    r.hdr = ld<uint4>(b); r.h0 = ld<uint4>(b + 16); r.h1 = ld<uint4>(b + 32);
+    r.v0 = ld<uint4>(b + 48 + 32 * (j >> 1)); r.v1 = ld<uint4>(b + 64 + 32 * (j >> 1));
+    return r;
+  }
+  static __device__ __forceinline__ void unpack(const Raw& r, int kb, uint32_t (&q)[8], float& s0, float& s1, float& mn, float& mn1) {
+    const int j = kb & 7;
+    const int sh = (j & 1) ? 4 : 0;
+    const uint32_t w[8] = {r.v0.x, r.v0.y, r.v0.z, r.v0.w, r.v1.x, r.v1.y, r.v1.z, r.v1.w};
+    const uint32_t h[8] = {r.h0.x, r.h0.y, r.h0.z, r.h0.w, r.h1.x, r.h1.y, r.h1.z, r.h1.w};
+#pragma unroll
+    for (int i = 0; i < 8; ++i) q[i] = ((w[i] >> sh) & 0x0F0F0F0Fu) | (((h[i] >> j) & 0x01010101u) << 4);
+    const uint64_t lo = ((uint64_t)r.hdr.z << 32) | r.hdr.y;
+    const uint32_t hi = r.hdr.w;
+    const int jj = j & 3;
+    const uint32_t b_lo = (uint32_t)(lo >> (8 * jj)) & 0xFF;
+    const uint32_t b_mid = (uint32_t)(lo >> (8 * jj + 32)) & 0xFF;
+    const uint32_t b_hi = (hi >> (8 * jj)) & 0xFF;
+    const int sc = j < 4 ? (int)(b_lo & 63) : (int)((b_hi & 0xF) | ((b_lo >> 6) << 4));
+    const int m = j < 4 ? (int)(b_mid & 63) : (int)((b_hi >> 4) | ((b_mid >> 6) << 4));
+    const float d = (float)__builtin_bit_cast(_Float16, (uint16_t)(r.hdr.x & 0xFFFF));
+    const float dmin = (float)__builtin_bit_cast(_Float16, (uint16_t)(r.hdr.x >> 16));
+    s0 = d * (float)sc; s1 = s0; mn = dmin * (float)m; mn1 = mn;
+  }
+};
+
 __device__ __forceinline__ int lut16q(uint32_t idx) {  // kvalues_iq4nl lookup of four indices, one per byte
   constexpr uint32_t T0 = 0xBFAD9881u, T1 = 0xF6EADDCFu, T2 = 0x26190D01u, T3 = 0x71594535u;
   const uint32_t sel = idx & 0x07070707u;
@@ -196,13 +396,14 @@ struct MIQ4_XS {  // extension: the reference has no MMQ tiles for i-quants (ggu
   static constexpr int QK = 256, BS = 136, G = 32;
   static constexpr bool HAS_MIN = false;
   static constexpr bool LIGHT = true;  // packed block small enough to hold a step of them in registers
+  static constexpr bool HALFPROD = false, MIN16 = false;
   struct Raw { uint2 hdr; uint4 v; };
   static __device__ __forceinline__ Raw fetch(const uint8_t* row, int kb) {
     const int sb = kb >> 3, ib = kb & 7;
     const uint8_t* b = row + (int64_t)sb * BS;
     Raw r; r.hdr = ld<uint2>(b); r.v = ld<uint4>(b + 8 + 16 * ib); return r;
   }
-  static __device__ __forceinline__ void unpack(const Raw& r, int kb, uint32_t (&q)[8], float& s0, float& s1, float& mn) {
+  static __device__ __forceinline__ void unpack(const Raw& r, int kb, uint32_t (&q)[8], float& s0, float& s1, float& mn, float& mn1) {
     const int ib = kb & 7;
     const uint32_t w[4] = {r.v.x, r.v.y, r.v.z, r.v.w};
 #pragma unroll
@@ -217,13 +418,14 @@ struct MIQ2_XXS {  // extension, see MIQ4_XS
   static constexpr int QK = 256, BS = 66, G = 32;
   static constexpr bool HAS_MIN = false;
   static constexpr bool LIGHT = false;  // packed block small enough to hold a step of them in registers
+  static constexpr bool HALFPROD = false, MIN16 = false;
   struct Raw { uint16_t d; uint2 g; };
   static __device__ __forceinline__ Raw fetch(const uint8_t* row, int kb) {
     const int sb = kb >> 3, ib = kb & 7;
     const uint8_t* b = row + (int64_t)sb * BS;
     Raw r; r.d = ld<uint16_t>(b); r.g = ld<uint2>(b + 2 + 8 * ib); return r;
   }
-  static __device__ __forceinline__ void unpack(const Raw& r, int kb, uint32_t (&q)[8], float& s0, float& s1, float& mn) {
+  static __device__ __forceinline__ void unpack(const Raw& r, int kb, uint32_t (&q)[8], float& s0, float& s1, float& mn, float& mn1) {
 #pragma unroll
     for (int l = 0; l < 4; ++l) {
       const uint32_t code = k_iq2xxs_grid_codes[(r.g.x >> (8 * l)) & 0xFF];
@@ -249,8 +451,9 @@ struct MIQ2_XXS {  // extension, see MIQ4_XS
 template <class F, int WM, int WN, int TM, int TN, int KS>
 __host__ __device__ constexpr size_t mmq_group_lds_bytes() {
   constexpr int M_T = 32 * WM * TM, N_T = 32 * WN * TN, KB = KS / 32;
-  return (size_t)(M_T + N_T) * Pitch<F::G, KS>::value + (size_t)KB * M_T * 4 * (F::HAS_MIN ? 2 : 1) +
-         (size_t)(KS / F::G) * N_T * 4 + (F::HAS_MIN ? (size_t)KB * N_T * 4 : 0);
+  constexpr int XA = !F::HAS_MIN ? 0 : F::MIN16 ? 2 * KB : KB;  // per-row offset factors: block sums, or 16-element quant sums
+  constexpr int WMN = !F::HAS_MIN ? 0 : F::MIN16 ? KS / F::G : KB;
+  return (size_t)(M_T + N_T) * Pitch<F::G, KS>::value + (size_t)(KB + XA) * M_T * 4 + (size_t)(KS / F::G + WMN) * N_T * 4;
 }
 
 struct MoeArgs {
@@ -290,8 +493,8 @@ __global__ __launch_bounds__(64 * WM * WN * (MODE == MODE_PINGPONG ? 2 : 1), OCC
   int8_t* xq = (int8_t*)smem + (size_t)group * mmq_group_lds_bytes<F, WM, WN, TM, TN, KS>();  // [M_T][LDK]
   int8_t* wq = xq + M_T * LDK;                      // [N_T][LDK]
   float* xd = (float*)(wq + N_T * LDK);             // [KB][M_T]  q8_1 block scales
-  float* xa = xd + KB * M_T;                        // [KB][M_T]  q8_1 block sums (HAS_MIN)
-  float* wsc = xa + (F::HAS_MIN ? KB * M_T : 0);    // [NG][N_T]
+  float* xa = xd + KB * M_T;                        // [KB][M_T] q8_1 block sums (HAS_MIN), or [2*KB][M_T] quant sums (MIN16)
+  float* wsc = xa + (!F::HAS_MIN ? 0 : F::MIN16 ? 2 * KB * M_T : KB * M_T);  // [NG][N_T]
   float* wmn = wsc + NG * N_T;                      // [KB][N_T]  (HAS_MIN)
 
   const int tid = (int)threadIdx.x - group * NT, wave = tid >> 6, lane = tid & 63;  // indices inside the group
@@ -366,7 +569,7 @@ __global__ __launch_bounds__(64 * WM * WN * (MODE == MODE_PINGPONG ? 2 : 1), OCC
 #pragma unroll
     for (int i = 0; i < AS; ++i) {
       r_ad[i] = as_src[i][kb0];
-      if (F::HAS_MIN) r_aa[i] = as_src[i][kb0 + Kp / 32];
+      if (F::HAS_MIN && !F::MIN16) r_aa[i] = as_src[i][kb0 + Kp / 32];
     }
 #pragma unroll
     for (int i = 0; i < WP; ++i) {
@@ -385,6 +588,8 @@ __global__ __launch_bounds__(64 * WM * WN * (MODE == MODE_PINGPONG ? 2 : 1), OCC
       if (p < M_T * GR) {
         const bool ok = aq_ok[i] && kb0 + (g >> 1) < nkb_total;
         const uint4 v = ok ? r_aq[i] : make_uint4(0, 0, 0, 0);
+        if (F::MIN16)  // this granule is one 16-element group: its quant sum, for the per-group offset term
+          xa[g * M_T + m] = (float)dot4(0x01010101, (int)v.x, dot4(0x01010101, (int)v.y, dot4(0x01010101, (int)v.z, dot4(0x01010101, (int)v.w, 0))));
         if (LDK % 16 == 0) {
           *(uint4*)(xq + m * LDK + 16 * g) = v;
         } else {
@@ -399,7 +604,7 @@ __global__ __launch_bounds__(64 * WM * WN * (MODE == MODE_PINGPONG ? 2 : 1), OCC
       if (p < M_T * KB) {
         const bool ok = as_ok[i] && kb0 + kb < nkb_total;
         xd[kb * M_T + m] = ok ? r_ad[i] : 0.0f;
-        if (F::HAS_MIN) xa[kb * M_T + m] = ok ? r_aa[i] : 0.0f;
+        if (F::HAS_MIN && !F::MIN16) xa[kb * M_T + m] = ok ? r_aa[i] : 0.0f;
       }
     }
 #pragma unroll
@@ -407,12 +612,12 @@ __global__ __launch_bounds__(64 * WM * WN * (MODE == MODE_PINGPONG ? 2 : 1), OCC
       const int p = tid + NT * i, n = p / KB, kb = p % KB;
       if (p >= N_T * KB) continue;
       uint32_t q[8];
-      float s0, s1, mn;
-      F::unpack(r_w[i], kb0 + kb, q, s0, s1, mn);
+      float s0, s1, mn, mn1;
+      F::unpack(r_w[i], kb0 + kb, q, s0, s1, mn, mn1);
       if (kb0 + kb >= nkb_total) {
 #pragma unroll
         for (int t = 0; t < 8; ++t) q[t] = 0;
-        s0 = s1 = mn = 0.0f;
+        s0 = s1 = mn = mn1 = 0.0f;
       }
       if (LDK % 16 == 0) {
         *(uint4*)(wq + n * LDK + 32 * kb) = make_uint4(q[0], q[1], q[2], q[3]);
@@ -427,7 +632,8 @@ __global__ __launch_bounds__(64 * WM * WN * (MODE == MODE_PINGPONG ? 2 : 1), OCC
         wsc[(2 * kb) * N_T + n] = s0;
         wsc[(2 * kb + 1) * N_T + n] = s1;
       }
-      if (F::HAS_MIN) wmn[kb * N_T + n] = mn;
+      if (F::HAS_MIN && !F::MIN16) wmn[kb * N_T + n] = mn;
+      if (F::MIN16) { wmn[(2 * kb) * N_T + n] = mn; wmn[(2 * kb + 1) * N_T + n] = mn1; }
     }
   };
 
@@ -457,7 +663,7 @@ __global__ __launch_bounds__(64 * WM * WN * (MODE == MODE_PINGPONG ? 2 : 1), OCC
 #pragma unroll
       for (int g = 0; g < 4; ++g) {
         d8[j][g] = xd[kb * M_T + mrow + 8 * g + 4 * lhalf + (lane & 3)];
-        if (F::HAS_MIN) a8[j][g] = xa[kb * M_T + mrow + 8 * g + 4 * lhalf + (lane & 3)];
+        if (F::HAS_MIN && !F::MIN16) a8[j][g] = xa[kb * M_T + mrow + 8 * g + 4 * lhalf + (lane & 3)];
       }
     }
 #pragma unroll
@@ -471,11 +677,15 @@ __global__ __launch_bounds__(64 * WM * WN * (MODE == MODE_PINGPONG ? 2 : 1), OCC
 #pragma unroll
         for (int j = 0; j < TM; ++j) {
           const v16i s = __builtin_amdgcn_mfma_i32_32x32x32_i8(af[j], bf, seed, 0, 0, 0);
-          float c[16];
+          if constexpr (F::HALFPROD) {
+            half_products16(acc[j][i], s, d8[j], a8[j], dw, -neg_mw);
+          } else {
+            float c[16];
 #pragma unroll
-          for (int r = 0; r < 16; ++r) c[r] = seeded_times(s[r], dw, neg_seed_dw);  // = RN(S * dw)
-          rescale16(acc[j][i], d8[j], c);
-          if (F::HAS_MIN) offset16(acc[j][i], a8[j], neg_mw);
+            for (int r = 0; r < 16; ++r) c[r] = seeded_times(s[r], dw, neg_seed_dw);  // = RN(S * dw)
+            rescale16(acc[j][i], d8[j], c);
+            if (F::HAS_MIN) offset16(acc[j][i], a8[j], neg_mw);
+          }
         }
       } else {
         // weight scale changes every 16 elements: one K=16 MFMA per half block.  In the 16-byte operand a lane
@@ -500,6 +710,17 @@ __global__ __launch_bounds__(64 * WM * WN * (MODE == MODE_PINGPONG ? 2 : 1), OCC
           }
           rescale16(acc[j][i], d8[j], ca);
           rescale16(acc[j][i], d8[j], cb);
+          if constexpr (F::MIN16) {
+            // offset term per 16-element group: d8 * (U_a * -min_a + U_b * -min_b), U = sum of the group's quants
+            float ua[4], ub[4];
+#pragma unroll
+            for (int g = 0; g < 4; ++g) {
+              ua[g] = xa[(2 * kb) * M_T + mrow + 8 * g + 4 * lhalf + (lane & 3)];
+              ub[g] = xa[(2 * kb + 1) * M_T + mrow + 8 * g + 4 * lhalf + (lane & 3)];
+            }
+            const float nma = -wmn[(2 * kb) * N_T + ncol], nmb = -wmn[(2 * kb + 1) * N_T + ncol];
+            group_offsets16(acc[j][i], d8[j], ua, ub, nma, nmb);
+          }
         }
       }
     }
@@ -665,7 +886,8 @@ __global__ void zero_rows_kernel(uint4* __restrict__ p, int64_t n16) {
 
 static bool mmq_type_ok(int type) {
   switch (type) {
-    case T_Q4_0: case T_Q8_0: case T_Q4_K: case T_Q6_K: case T_IQ4_XS: case T_IQ2_XXS: return true;
+    case T_Q4_0: case T_Q4_1: case T_Q5_0: case T_Q5_1: case T_Q8_0: case T_Q2_K: case T_Q3_K: case T_Q4_K: case T_Q5_K:
+    case T_Q6_K: case T_IQ4_XS: case T_IQ2_XXS: return true;
     default: return false;
   }
 }
@@ -686,6 +908,12 @@ extern "C" int gguf_mmq(const void* W, const void* x, int xdtype, void* q8_works
   if (rc != GGUF_OK) return rc;
   switch (type) {
     case T_Q4_0: return mmq_fmt<MQ4_0>(W, q8_workspace, Y, xdtype, (int)M, (int)N, (int)K, s);
+    case T_Q4_1: return mmq_fmt<MQ4_1>(W, q8_workspace, Y, xdtype, (int)M, (int)N, (int)K, s);
+    case T_Q5_0: return mmq_fmt<MQ5_0>(W, q8_workspace, Y, xdtype, (int)M, (int)N, (int)K, s);
+    case T_Q5_1: return mmq_fmt<MQ5_1>(W, q8_workspace, Y, xdtype, (int)M, (int)N, (int)K, s);
+    case T_Q2_K: return mmq_fmt<MQ2_K>(W, q8_workspace, Y, xdtype, (int)M, (int)N, (int)K, s);
+    case T_Q3_K: return mmq_fmt<MQ3_K>(W, q8_workspace, Y, xdtype, (int)M, (int)N, (int)K, s);
+    case T_Q5_K: return mmq_fmt<MQ5_K>(W, q8_workspace, Y, xdtype, (int)M, (int)N, (int)K, s);
     case T_Q8_0: return mmq_fmt<MQ8_0>(W, q8_workspace, Y, xdtype, (int)M, (int)N, (int)K, s);
     case T_Q4_K: return mmq_fmt<MQ4_K>(W, q8_workspace, Y, xdtype, (int)M, (int)N, (int)K, s);
     case T_Q6_K: return mmq_fmt<MQ6_K>(W, q8_workspace, Y, xdtype, (int)M, (int)N, (int)K, s);
@@ -723,6 +951,12 @@ extern "C" int gguf_moe_mmq(const void* X, int xdtype, void* q8_workspace, const
   if (ns == 0) return launch_status();
   switch (type) {
     case T_Q4_0: return moe_fmt<MQ4_0>(W, q8_workspace, Y, xdtype, (int)N, (int)K, ns, moe, s);
+    case T_Q4_1: return moe_fmt<MQ4_1>(W, q8_workspace, Y, xdtype, (int)N, (int)K, ns, moe, s);
+    case T_Q5_0: return moe_fmt<MQ5_0>(W, q8_workspace, Y, xdtype, (int)N, (int)K, ns, moe, s);
+    case T_Q5_1: return moe_fmt<MQ5_1>(W, q8_workspace, Y, xdtype, (int)N, (int)K, ns, moe, s);
+    case T_Q2_K: return moe_fmt<MQ2_K>(W, q8_workspace, Y, xdtype, (int)N, (int)K, ns, moe, s);
+    case T_Q3_K: return moe_fmt<MQ3_K>(W, q8_workspace, Y, xdtype, (int)N, (int)K, ns, moe, s);
+    case T_Q5_K: return moe_fmt<MQ5_K>(W, q8_workspace, Y, xdtype, (int)N, (int)K, ns, moe, s);
     case T_Q8_0: return moe_fmt<MQ8_0>(W, q8_workspace, Y, xdtype, (int)N, (int)K, ns, moe, s);
     case T_Q4_K: return moe_fmt<MQ4_K>(W, q8_workspace, Y, xdtype, (int)N, (int)K, ns, moe, s);
     case T_Q6_K: return moe_fmt<MQ6_K>(W, q8_workspace, Y, xdtype, (int)N, (int)K, ns, moe, s);
