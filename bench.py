@@ -37,6 +37,11 @@ Q4_K, Q6_K = 12, 14
 CFG2_SHAPES = [(4096, 4096), (14336, 4096), (4096, 14336)]
 CFG3_SHAPES = [(18944, 3584), (3584, 18944)]
 ROTATE_BYTES = 640 << 20       # distinct weight bytes walked per rotation (> 2x the 256 MB cache)
+# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of `bench.py --profile`, each counter scaled by
+# what it reads for a 256 MiB device copy (x2.000 and x1.000); summarised in profiles/bench_mmvq_q4_k_bs1_mmq_q6_k.txt.
+# Counters cannot be read from inside this process, so these are constants of the measured build, not live values.
+TRAFFIC_MMVQ_Q4_K_14336x4096 = 33.37e6 + 0.02e6
+TRAFFIC_MMQ_Q6_K_M512 = {"18944x3584": 245.5e6 + 19.4e6, "3584x18944": 144.4e6 + 3.67e6}
 
 
 def _events_ms(fn, iters):
@@ -146,7 +151,8 @@ def main() -> int:
         per_shape[f"{n}x{k}"] = {"us_per_call": ms * 1e3, "GBps": b / (ms * 1e-3) / 1e9, "bytes": b}
     big = per_shape["14336x4096"]
     roofline = {"bound": "hbm", "achieved": big["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": big["GBps"] / HBM_PEAK_GBS, "traffic": None,
+                "frac": big["GBps"] / HBM_PEAK_GBS, "traffic": TRAFFIC_MMVQ_Q4_K_14336x4096,
+                "algorithmic_bytes": big["bytes"],
                 "kernel": "mmvq Q4_K [14336,4096] bs1 (activation quantisation + GEMV per call)",
                 "per_shape": per_shape}
 
@@ -183,7 +189,7 @@ def main() -> int:
         out["mmq"] = {
             "metric": "Q6_K MMQ int8 TOPS @M=512", "value": tops512, "unit": "TOPS",
             "roofline": {"bound": "mfma", "achieved": tops512, "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
-                         "frac": tops512 / INT8_PEAK_TOPS, "traffic": None,
+                         "frac": tops512 / INT8_PEAK_TOPS, "traffic": TRAFFIC_MMQ_Q6_K_M512,
                          "denominator": "5.03 POPS dense int8 (v_mfma_i32_32x32x32_i8 rate); Q6_K uses the K=16 shape, "
                                         f"whose own peak is {INT8_LEGACY_PEAK_TOPS} TOPS",
                          "frac_of_legacy_k16_peak": tops512 / INT8_LEGACY_PEAK_TOPS},
