@@ -58,6 +58,21 @@ def test_mmq_half_outputs_within_tolerance(qtype, dt):
     assert o.rel_l2(y, o.mul_mat_f32(w, xv, qtype, n)) <= 2e-2
 
 
+@pytest.mark.parametrize("qtype", [o.Q4_0, o.Q4_K, o.Q6_K, o.Q2_K, o.Q5_1])
+@pytest.mark.parametrize("m,n", [(512, 12800), (128, 16640), (300, 200)])
+def test_mmq_every_tile_configuration(qtype, m, n):
+    """The launcher picks its tile by output-tile count: 128x128 (>= 400 large tiles), 64x64 (more than 512 small
+    tiles) or 64x64 with the step's blocks split over two wave sets.  One shape per regime, ragged edges included."""
+    ops = _ops()
+    rng = np.random.default_rng(1000 + qtype + m)
+    k = 256
+    w = o.make_weights(rng, qtype, n, k)
+    xd, xv = _x(rng, m, k, "f32")
+    y = ops.ggml_mul_mat_a8(_dev(w), xd, qtype, n)
+    exp = o.mul_mat_a8(w, xv, qtype, n, "mmq")
+    assert o.rel_l2(y.cpu().numpy(), exp) <= 1e-5
+
+
 def test_mmq_and_mmvq_agree():
     # same contraction through both paths; Q4_K differs only by which block sum the offset term uses
     ops = _ops()

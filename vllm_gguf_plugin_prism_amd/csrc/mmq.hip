@@ -472,13 +472,18 @@ struct MoeArgs {
 //                  groups run half a period apart, separated by workgroup barriers: while one waits for its
 //                  global loads and unpacks them, the other runs its MFMA + rescale phase, so the vector ALU
 //                  (the bound of this kernel) always has a group to work for.
-enum { MODE_PREFETCH = 0, MODE_PLAIN = 1, MODE_PINGPONG = 2 };
+//   MODE_KSPLIT    MODE_PLAIN with twice the waves: all of them stage the step together, then each half of the
+//                  workgroup contracts half of the step's 32-blocks for the same outputs, and the two partial tiles
+//                  are added through LDS at the end.  For shapes with too few output tiles to fill the chip.
+enum { MODE_PREFETCH = 0, MODE_PLAIN = 1, MODE_PINGPONG = 2, MODE_KSPLIT = 3 };
 
 template <class F, int WM, int WN, int TM, int TN, int KS, int OCC, int MODE, typename T, bool MOE>
-__global__ __launch_bounds__(64 * WM * WN * (MODE == MODE_PINGPONG ? 2 : 1), OCC) void mmq_kernel(const uint8_t* __restrict__ W, const char* __restrict__ ws,
+__global__ __launch_bounds__(64 * WM * WN * (MODE == MODE_PINGPONG || MODE == MODE_KSPLIT ? 2 : 1), OCC) void mmq_kernel(const uint8_t* __restrict__ W, const char* __restrict__ ws,
                                                          T* __restrict__ Y, int M, int N, int K, int64_t ws_row_bytes,
                                                          MoeArgs moe) {
-  constexpr int NT = 64 * WM * WN;       // threads per group (the whole workgroup unless MODE_PINGPONG)
+  constexpr int GW = WM * WN;            // waves that share one set of accumulators' tile
+  constexpr int KW = MODE == MODE_KSPLIT ? 2 : 1;  // wave sets splitting the 32-blocks of a step
+  constexpr int NT = 64 * GW * KW;       // threads that stage one tile (the whole workgroup unless MODE_PINGPONG)
   constexpr int KB = KS / 32;            // q8_1 blocks per step
   constexpr int GR = KS / 16;            // 16-byte granules per activation row and step
   constexpr int LDK = Pitch<F::G, KS>::value;
@@ -497,8 +502,10 @@ __global__ __launch_bounds__(64 * WM * WN * (MODE == MODE_PINGPONG ? 2 : 1), OCC
   float* wsc = xa + (!F::HAS_MIN ? 0 : F::MIN16 ? 2 * KB * M_T : KB * M_T);  // [NG][N_T]
   float* wmn = wsc + NG * N_T;                      // [KB][N_T]  (HAS_MIN)
 
-  const int tid = (int)threadIdx.x - group * NT, wave = tid >> 6, lane = tid & 63;  // indices inside the group
+  const int tid = (int)threadIdx.x - group * NT, lane = tid & 63;  // indices inside the group
+  const int kgrp = (tid >> 6) / GW, wave = (tid >> 6) % GW;         // wave-uniform
   const int wm = wave / WN, wn = wave % WN;
+  constexpr int KB_MINE = (KS / 32) / KW;                            // 32-blocks of a step this wave contracts
   const int m_base = blockIdx.y * M_T;
   const int n_base = MODE == MODE_PINGPONG ? (blockIdx.x * 2 + group) * N_T : blockIdx.x * N_T;
   const int Kp = (int)q8_kp(K);
@@ -741,14 +748,36 @@ __global__ __launch_bounds__(64 * WM * WN * (MODE == MODE_PINGPONG ? 2 : 1), OCC
         __syncthreads();
       }
     }
-  } else if constexpr (MODE == MODE_PLAIN) {
+  } else if constexpr (MODE == MODE_PLAIN || MODE == MODE_KSPLIT) {
     for (int k0 = 0; k0 < K; k0 += KS) {
       fetch(k0);
       stash(k0);
       __syncthreads();
 #pragma unroll 1
-      for (int kb = 0; kb < KB; ++kb) contract(kb);
+      for (int kb = kgrp * KB_MINE; kb < (kgrp + 1) * KB_MINE; ++kb) contract(kb);
       __syncthreads();
+    }
+    if constexpr (KW == 2) {
+      // add the second wave set's partial tile to the first's through LDS (the tiles are free after the last barrier)
+      float* red = (float*)smem;
+      static_assert((size_t)GW * TM * TN * 16 * 64 * 4 <= mmq_group_lds_bytes<F, WM, WN, TM, TN, KS>(), "partial tile fits the staging area");
+#pragma unroll
+      for (int j = 0; j < TM; ++j)
+#pragma unroll
+        for (int i = 0; i < TN; ++i)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) {
+            float* slot = red + ((((wave * TM + j) * TN + i) * 16 + r) * 64 + lane);
+            if (kgrp == 1) *slot = acc[j][i][r];
+          }
+      __syncthreads();
+      if (kgrp == 1) return;
+#pragma unroll
+      for (int j = 0; j < TM; ++j)
+#pragma unroll
+        for (int i = 0; i < TN; ++i)
+#pragma unroll
+          for (int r = 0; r < 16; ++r) acc[j][i][r] += red[(((wave * TM + j) * TN + i) * 16 + r) * 64 + lane];
     }
   } else {
     // phase p: group g stages step (p-g)/2 when p-g is even and contracts step (p-g-1)/2 when it is odd.  A group's
@@ -800,6 +829,7 @@ template <class F, int WM, int WN, int TM, int TN, int KS, int OCC, int MODE, ty
 static void launch_mmq(const void* W, const void* ws, void* Y, int M, int N, int K, int m_tiles, const MoeArgs& moe,
                        hipStream_t stream) {
   constexpr int G = MODE == MODE_PINGPONG ? 2 : 1;
+  constexpr int KW = MODE == MODE_KSPLIT ? 2 : 1;
   constexpr int N_T = 32 * WN * TN * G;
   constexpr size_t lds = mmq_group_lds_bytes<F, WM, WN, TM, TN, KS>() * G;
   static_assert(mmq_group_lds_bytes<F, WM, WN, TM, TN, KS>() % 16 == 0, "group tiles keep 16-byte alignment");
@@ -811,7 +841,7 @@ static void launch_mmq(const void* W, const void* ws, void* Y, int M, int N, int
       configured = true;
     }
   }
-  hipLaunchKernelGGL(kern, dim3((N + N_T - 1) / N_T, m_tiles), dim3(64 * WM * WN * G), lds, stream, (const uint8_t*)W, (const char*)ws,
+  hipLaunchKernelGGL(kern, dim3((N + N_T - 1) / N_T, m_tiles), dim3(64 * WM * WN * G * KW), lds, stream, (const uint8_t*)W, (const char*)ws,
                      (T*)Y, M, N, K, q8_row_bytes(K), moe);
 }
 
@@ -829,6 +859,7 @@ static int tune_cfg() {
 // matters is that every CU has several workgroups to overlap one group's load latency with another's arithmetic:
 //   large   128 x 128, 8 waves, two workgroups per CU      when that still gives every CU about two tiles
 //   small   64 x 64, 4 waves, four or more per CU          otherwise (few tokens, or a narrow N with a long K)
+//   split   64 x 64, 8 waves (MODE_KSPLIT)                 when even the small tiles leave CUs with two workgroups or fewer
 // Formats whose packed block is small keep the next step's loads in registers across the MFMA phase (PREFETCH);
 // for the others that would push the kernel past 128 registers and halve the waves per SIMD.
 template <class F, typename T>
@@ -841,15 +872,19 @@ static int mmq_typed(const void* W, const void* ws, void* Y, int M, int N, int K
     case 3: launch_mmq<F, 2, 1, 1, 1, 128, 4, MODE_PINGPONG, T, false>(W, ws, Y, M, N, K, (M + 63) / 64, none, stream); return launch_status();
     case 5: launch_mmq<F, 4, 2, 1, 2, 128, 4, MODE_PLAIN, T, false>(W, ws, Y, M, N, K, (M + 127) / 128, none, stream); return launch_status();
     case 6: launch_mmq<F, 2, 2, 1, 1, 128, 4, MODE_PLAIN, T, false>(W, ws, Y, M, N, K, (M + 63) / 64, none, stream); return launch_status();
+    case 9: launch_mmq<F, 2, 2, 1, 1, 128, 4, MODE_KSPLIT, T, false>(W, ws, Y, M, N, K, (M + 63) / 64, none, stream); return launch_status();
     case 8: launch_mmq<F, 4, 2, 1, 2, 128, 4, MODE_PREFETCH, T, false>(W, ws, Y, M, N, K, (M + 127) / 128, none, stream); return launch_status();
     default: break;
   }
 #endif
+  const int64_t small_tiles = (int64_t)((M + 63) / 64) * ((N + 63) / 64);
   if (large_tiles >= 400) {
     constexpr int MODE = F::LIGHT ? MODE_PREFETCH : MODE_PLAIN;
     launch_mmq<F, 4, 2, 1, 2, 128, 4, MODE, T, false>(W, ws, Y, M, N, K, (M + 127) / 128, none, stream);
-  } else {
+  } else if (small_tiles > 512) {
     launch_mmq<F, 2, 2, 1, 1, 128, 4, MODE_PLAIN, T, false>(W, ws, Y, M, N, K, (M + 63) / 64, none, stream);
+  } else {  // at most two workgroups per CU: double the waves of each by splitting the step's blocks
+    launch_mmq<F, 2, 2, 1, 1, 128, 4, MODE_KSPLIT, T, false>(W, ws, Y, M, N, K, (M + 63) / 64, none, stream);
   }
   return launch_status();
 }
