@@ -68,6 +68,12 @@ int gguf_q8_1_unpack(const void* q8_workspace, int8_t* q, float* ds, int64_t M, 
  * Replaces ggml_dequantize (gguf_kernel.cu:87-102, dequantize.cuh:527-571). */
 int gguf_dequantize(const void* W, int type, void* Y, int ydtype, int64_t nelem, gguf_stream_t stream);
 
+/* Row gather fused with dequantisation: Y[i,:] = dense values of row row_ids[i] of the packed table W[n_rows, K].
+ * Replaces torch.index_select followed by ggml_dequantize in the embedding path
+ * (quantization/vocal_embeds.py:90-96).  A row id outside [0, n_rows) yields a row of zeros. */
+int gguf_dequantize_rows(const void* W, int type, const int64_t* row_ids, int64_t n_ids, int64_t n_rows, int64_t K, void* Y,
+                         int ydtype, gguf_stream_t stream);
+
 /* Y[M,N] = q8_1(X[M,K]) . W[N,K]^T, decode GEMV path.
  * Replaces ggml_mul_mat_vec_a8 (gguf_kernel.cu:104-218, mmvq.cuh:2-212). */
 int gguf_mmvq(const void* W, const void* x, int xdtype, void* q8_workspace, void* Y, int type, int64_t N, int64_t K,
@@ -95,6 +101,20 @@ int gguf_moe_vec(const void* X, int xdtype, void* q8_workspace, const void* W, c
 /* Token-tile size that moe_align_block_size must pad expert groups to; 0 for unknown types.
  * Replaces ggml_moe_get_block_size (gguf_kernel.cu:532-566). */
 int gguf_moe_block_size(int type);
+
+/* Routing sort for the grouped kernel: pairs (flat index token*top_k + choice) grouped by expert in ascending index
+ * order, every expert's run padded to a multiple of `block` with the value `numel`; one expert id per block (-1 past
+ * the padded total); the padded total.  Capacities: sorted >= numel + num_experts*(block-1), experts >= that / block
+ * rounded up.  The reference takes this from vLLM (quantization/fused_moe.py:53-66, moe_align_block_size); the
+ * meaning of the three outputs is the one moe.cuh:20-45 consumes.  num_experts <= 1024. */
+int gguf_moe_align_block_size(const int32_t* topk_ids, int64_t numel, int64_t num_experts, int64_t block,
+                              int32_t* sorted_token_ids, int64_t sorted_capacity, int32_t* expert_ids,
+                              int64_t expert_capacity, int32_t* num_tokens_post_padded, gguf_stream_t stream);
+
+/* out[t,:] = sum over k of round(Y[t*top_k + k,:] * topk_weights[t,k]) with fp32 accumulation, one launch for
+ * out.mul_(topk_weights) followed by ops.moe_sum (quantization/fused_moe.py:87-95, ops.py:285-286). */
+int gguf_moe_weighted_sum(const void* Y, const float* topk_weights, void* out, int dtype, int64_t tokens, int64_t top_k,
+                          int64_t N, gguf_stream_t stream);
 
 #ifdef __cplusplus
 }

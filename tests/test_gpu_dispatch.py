@@ -69,7 +69,7 @@ def test_fused_mul_mat_routes(qt, batch, rows, path):
         assert o.rel_l2(got, want) <= 1e-3
 
 
-@pytest.mark.parametrize("qt", [o.Q8_0, o.Q4_K, o.IQ2_XXS])
+@pytest.mark.parametrize("qt", [o.Q8_0, o.Q4_K, o.IQ2_XXS, o.Q5_1, o.Q3_K, o.IQ1_M, o.IQ3_S])
 def test_embedding_lookup_is_gather_of_exact_dequant(qt):
     rng = np.random.default_rng(qt)
     vocab, hidden = 50, 512
@@ -79,3 +79,55 @@ def test_embedding_lookup_is_gather_of_exact_dequant(qt):
     assert got.shape == (3, 5, hidden)
     dense = o.dequantize(table, qt, "f16").reshape(vocab, hidden)
     assert np.array_equal(got.cpu().numpy().view(np.uint16), dense[ids].view(np.uint16))
+
+
+@pytest.mark.parametrize("tokens,top_k,experts,block", [(1, 8, 64, 32), (7, 2, 4, 32), (512, 8, 64, 32), (33, 3, 5, 4),
+                                                        (2000, 2, 300, 32), (5, 1, 3, 8)])
+def test_native_moe_align_block_size_matches_checker(tokens, top_k, experts, block):
+    from vllm_gguf_plugin_prism_amd import ops
+
+    rng = np.random.default_rng(tokens * 7 + experts)
+    ids = np.stack([rng.permutation(experts)[:top_k] for _ in range(tokens)]).astype(np.int32)
+    s, e, n = ops.moe_align_block_size(torch.from_numpy(ids).cuda(), block, experts)
+    so, eo, no = o.moe_align_block_size(ids, block, experts)
+    total = int(no[0])
+    assert int(n.item()) == total
+    s, e = s.cpu().numpy(), e.cpu().numpy()
+    assert len(s) == ids.size + experts * (block - 1)
+    assert np.array_equal(s[:total], so[:total])          # stable order: identical, slot by slot
+    assert (s[total:] == ids.size).all()
+    assert np.array_equal(e[: total // block], eo[: total // block])
+    assert (e[total // block:] == -1).all()
+    # the torch statement of the same sort agrees too
+    st, et, nt = D.moe_align_block_size(torch.from_numpy(ids), block, experts)
+    assert int(nt[0]) == total and np.array_equal(st.numpy()[:total], s[:total])
+
+
+@pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16, torch.float32])
+def test_moe_weighted_sum_matches_mul_then_sum(dt):
+    from vllm_gguf_plugin_prism_amd import ops
+
+    torch.manual_seed(3)
+    t, k, n = 37, 8, 520
+    y = torch.randn(t, k, n, device="cuda").to(dt)
+    w = torch.softmax(torch.randn(t, k, device="cuda"), dim=1)
+    out = torch.empty(t, n, device="cuda", dtype=dt)
+    ops.moe_weighted_sum(y, w, out)
+    ref = y.clone().mul_(w.view(t, k, 1))                # rounds every product to dt, as the reference's mul_ does
+    want = ref.float().sum(dim=1).to(dt)                 # fp32 accumulation, one rounding
+    # identical products; only the fp32 summation order may differ, so at most the last bit of dt moves
+    assert torch.allclose(out.float(), want.float(), rtol=2 ** -7 if dt == torch.bfloat16 else 2 ** -10, atol=1e-6)
+    if dt != torch.float32:  # in fp32 the summation order itself is visible in the last bit
+        assert (out == want).float().mean().item() > 0.95
+
+
+def test_embedding_rows_out_of_range_are_zero():
+    from vllm_gguf_plugin_prism_amd import ops
+
+    rng = np.random.default_rng(9)
+    table = synth.make_weights(rng, o.Q4_K, 10, 256)
+    ids = torch.tensor([0, 9, 10, -1, 3], device="cuda")
+    got = ops.ggml_dequantize_rows(torch.from_numpy(table).cuda(), o.Q4_K, ids, 256, torch.float32).cpu().numpy()
+    dense = o.dequantize(table, o.Q4_K, "f32").reshape(10, 256)
+    assert np.array_equal(got[[0, 1, 4]], dense[[0, 9, 3]])
+    assert (got[[2, 3]] == 0).all()

@@ -27,6 +27,8 @@ _SIGNATURES = {
     "gguf_quantize_q8_1": (_c.c_int, [_c.c_void_p, _c.c_int, _c.c_void_p, _c.c_int64, _c.c_int64, _c.c_void_p]),
     "gguf_q8_1_unpack": (_c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int64, _c.c_int64, _c.c_void_p]),
     "gguf_dequantize": (_c.c_int, [_c.c_void_p, _c.c_int, _c.c_void_p, _c.c_int, _c.c_int64, _c.c_void_p]),
+    "gguf_dequantize_rows": (_c.c_int, [_c.c_void_p, _c.c_int, _c.c_void_p, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_void_p,
+                                        _c.c_int, _c.c_void_p]),
     "gguf_mmvq": (_c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_int, _c.c_void_p, _c.c_void_p, _c.c_int, _c.c_int64,
                              _c.c_int64, _c.c_int64, _c.c_void_p]),
     "gguf_mmq": (_c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_int, _c.c_void_p, _c.c_void_p, _c.c_int, _c.c_int64,
@@ -37,6 +39,10 @@ _SIGNATURES = {
     "gguf_moe_vec": (_c.c_int, [_c.c_void_p, _c.c_int, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int,
                                 _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_void_p]),
     "gguf_moe_block_size": (_c.c_int, [_c.c_int]),
+    "gguf_moe_align_block_size": (_c.c_int, [_c.c_void_p, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_void_p, _c.c_int64,
+                                             _c.c_void_p, _c.c_int64, _c.c_void_p, _c.c_void_p]),
+    "gguf_moe_weighted_sum": (_c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int, _c.c_int64, _c.c_int64,
+                                         _c.c_int64, _c.c_void_p]),
 }
 EXPORTS = tuple(_SIGNATURES)
 

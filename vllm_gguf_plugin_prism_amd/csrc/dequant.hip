@@ -380,10 +380,9 @@ __device__ __forceinline__ void store8(OutT* __restrict__ y, const OutT (&v)[8])
   }
 }
 
+// eight dense values of packed elements [e0, e0 + 8) of `w`, stored at `dst`
 template <int TYPE, typename OutT>
-__global__ __launch_bounds__(256) void dequant_kernel(const uint8_t* __restrict__ w, OutT* __restrict__ y, int64_t nelem) {
-  const int64_t e0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 8;
-  if (e0 >= nelem) return;
+__device__ __forceinline__ void dequant8(const uint8_t* __restrict__ w, int64_t e0, OutT* __restrict__ dst) {
   alignas(16) OutT out[8];
   constexpr bool F32_MATH = TYPE == T_IQ4_XS || TYPE == T_IQ2_XXS || TYPE == T_IQ2_XS || TYPE == T_IQ2_S || TYPE == T_IQ3_XXS ||
                             TYPE == T_IQ3_S || TYPE == T_IQ1_S || TYPE == T_IQ1_M || TYPE == T_IQ4_NL;
@@ -415,7 +414,33 @@ __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t* __restrict_
 #pragma unroll
     for (int i = 0; i < 8; ++i) out[i] = from_half<OutT>(h[i]);
   }
-  store8<OutT>(y + e0, out);
+  store8<OutT>(dst, out);
+}
+
+template <int TYPE, typename OutT>
+__global__ __launch_bounds__(256) void dequant_kernel(const uint8_t* __restrict__ w, OutT* __restrict__ y, int64_t nelem) {
+  const int64_t e0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 8;
+  if (e0 >= nelem) return;
+  dequant8<TYPE, OutT>(w, e0, y + e0);
+}
+
+// Row gather fused with dequantisation: Y[i, :] = dense(W[ids[i], :]).  A row whose id is outside [0, n_rows) is
+// written as zeros.  blockIdx.y walks the requested rows, blockIdx.x the K / 2048 column chunks.
+template <int TYPE, typename OutT>
+__global__ __launch_bounds__(256) void dequant_rows_kernel(const uint8_t* __restrict__ w, const int64_t* __restrict__ ids,
+                                                            int64_t n_ids, int64_t n_rows, int64_t K, OutT* __restrict__ y) {
+  const int64_t c0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 8;
+  if (c0 >= K) return;
+  for (int64_t i = blockIdx.y; i < n_ids; i += gridDim.y) {
+    const int64_t row = ids[i];
+    OutT* dst = y + i * K + c0;
+    if (row < 0 || row >= n_rows) {
+      alignas(16) OutT zero[8] = {};
+      store8<OutT>(dst, zero);
+    } else {
+      dequant8<TYPE, OutT>(w, row * K + c0, dst);
+    }
+  }
 }
 
 template <int TYPE>
@@ -427,7 +452,50 @@ static int launch_dequant(const void* w, void* y, int ydtype, int64_t nelem, hip
   return launch_status();
 }
 
+template <int TYPE>
+static int launch_dequant_rows(const void* w, const int64_t* ids, int64_t n_ids, int64_t n_rows, int64_t K, void* y,
+                               int ydtype, hipStream_t stream) {
+  const dim3 grid((unsigned)((K / 8 + 255) / 256), (unsigned)(n_ids < 32768 ? n_ids : 32768));
+  GGUF_DISPATCH_DTYPE(ydtype, hipLaunchKernelGGL((dequant_rows_kernel<TYPE, scalar_t>), grid, dim3(256), 0, stream,
+                                                 (const uint8_t*)w, ids, n_ids, n_rows, K, (scalar_t*)y));
+  return launch_status();
+}
+
 }  // namespace gguf
+
+extern "C" int gguf_dequantize_rows(const void* W, int type, const int64_t* row_ids, int64_t n_ids, int64_t n_rows, int64_t K,
+                                    void* Y, int ydtype, gguf_stream_t stream) {
+  using namespace gguf;
+  const int qk = block_elems(type);
+  if (qk == 0) return GGUF_ERR_TYPE;
+  if (n_ids < 0 || n_rows < 0 || K <= 0 || K % qk != 0 || K / 8 / 256 > 0x7FFFFFFFLL) return GGUF_ERR_SHAPE;
+  if (ydtype < 0 || ydtype > 2) return GGUF_ERR_DTYPE;
+  if (n_ids == 0) return GGUF_OK;
+  if (!W || !row_ids || !Y) return GGUF_ERR_NULL;
+  hipStream_t s = (hipStream_t)stream;
+  switch (type) {
+    case T_Q4_0: return launch_dequant_rows<T_Q4_0>(W, row_ids, n_ids, n_rows, K, Y, ydtype, s);
+    case T_Q4_1: return launch_dequant_rows<T_Q4_1>(W, row_ids, n_ids, n_rows, K, Y, ydtype, s);
+    case T_Q5_0: return launch_dequant_rows<T_Q5_0>(W, row_ids, n_ids, n_rows, K, Y, ydtype, s);
+    case T_Q5_1: return launch_dequant_rows<T_Q5_1>(W, row_ids, n_ids, n_rows, K, Y, ydtype, s);
+    case T_Q8_0: return launch_dequant_rows<T_Q8_0>(W, row_ids, n_ids, n_rows, K, Y, ydtype, s);
+    case T_Q2_K: return launch_dequant_rows<T_Q2_K>(W, row_ids, n_ids, n_rows, K, Y, ydtype, s);
+    case T_Q3_K: return launch_dequant_rows<T_Q3_K>(W, row_ids, n_ids, n_rows, K, Y, ydtype, s);
+    case T_Q4_K: return launch_dequant_rows<T_Q4_K>(W, row_ids, n_ids, n_rows, K, Y, ydtype, s);
+    case T_Q5_K: return launch_dequant_rows<T_Q5_K>(W, row_ids, n_ids, n_rows, K, Y, ydtype, s);
+    case T_Q6_K: return launch_dequant_rows<T_Q6_K>(W, row_ids, n_ids, n_rows, K, Y, ydtype, s);
+    case T_IQ2_XXS: return launch_dequant_rows<T_IQ2_XXS>(W, row_ids, n_ids, n_rows, K, Y, ydtype, s);
+    case T_IQ2_XS: return launch_dequant_rows<T_IQ2_XS>(W, row_ids, n_ids, n_rows, K, Y, ydtype, s);
+    case T_IQ3_XXS: return launch_dequant_rows<T_IQ3_XXS>(W, row_ids, n_ids, n_rows, K, Y, ydtype, s);
+    case T_IQ1_S: return launch_dequant_rows<T_IQ1_S>(W, row_ids, n_ids, n_rows, K, Y, ydtype, s);
+    case T_IQ4_NL: return launch_dequant_rows<T_IQ4_NL>(W, row_ids, n_ids, n_rows, K, Y, ydtype, s);
+    case T_IQ3_S: return launch_dequant_rows<T_IQ3_S>(W, row_ids, n_ids, n_rows, K, Y, ydtype, s);
+    case T_IQ2_S: return launch_dequant_rows<T_IQ2_S>(W, row_ids, n_ids, n_rows, K, Y, ydtype, s);
+    case T_IQ4_XS: return launch_dequant_rows<T_IQ4_XS>(W, row_ids, n_ids, n_rows, K, Y, ydtype, s);
+    case T_IQ1_M: return launch_dequant_rows<T_IQ1_M>(W, row_ids, n_ids, n_rows, K, Y, ydtype, s);
+    default: return GGUF_ERR_TYPE;
+  }
+}
 
 extern "C" int gguf_dequantize(const void* W, int type, void* Y, int ydtype, int64_t nelem, gguf_stream_t stream) {
   using namespace gguf;

@@ -100,7 +100,9 @@ def _activation(name: str, inp):
 
 
 def moe_align_block_size(topk_ids, block_size: int, num_experts: int):
-    """Sort (token, choice) pairs by expert and pad every expert's run to a multiple of ``block_size``.
+    """Torch statement of the routing sort (device-agnostic; the GPU path uses ``ops.moe_align_block_size``).
+
+    Sort (token, choice) pairs by expert and pad every expert's run to a multiple of ``block_size``.
 
     Returns ``(sorted_token_ids, expert_ids, num_tokens_post_padded)`` with the meaning ``moe.cuh:20-45`` gives them:
     entries of ``sorted_token_ids`` are flat pair indices ``token * top_k + choice``, padding entries hold
@@ -142,7 +144,7 @@ def fused_moe_gguf(x, w1, w2, topk_weights, topk_ids, weight_type: int, weight_t
     if path == "grouped":
         experts, rows, _ = w1.shape
         block = ops.ggml_moe_get_block_size(weight_type)
-        sorted_ids, expert_ids, post_padded = moe_align_block_size(topk_ids, block, experts)
+        sorted_ids, expert_ids, post_padded = ops.moe_align_block_size(topk_ids, block, experts)
         out = ops.ggml_moe_a8(x, w1, sorted_ids, expert_ids, post_padded, weight_type, rows, top_k, tokens)
         out = _activation(activation, out).contiguous()
         out = ops.ggml_moe_a8(out, w2, sorted_ids, expert_ids, post_padded, weight_type2, w2.shape[1], 1, tokens * top_k)
@@ -161,13 +163,13 @@ def fused_moe_gguf(x, w1, w2, topk_weights, topk_ids, weight_type: int, weight_t
                 acc = cur if acc is None else acc.add_(cur)
             out_hidden[tok] = acc
         return out_hidden
-    out = out.reshape(tokens, top_k, w2.shape[1]).mul_(topk_weights.view(tokens, top_k, 1).to(out.dtype))
-    ops.moe_sum(out, out_hidden)
+    ops.moe_weighted_sum(out.reshape(tokens, top_k, w2.shape[1]), topk_weights, out_hidden)  # mul_ by weights + moe_sum
     return out_hidden
 
 
 def apply_gguf_embedding(x, weight, weight_type: int, hidden_size: int, dtype=None):
-    """Embedding lookup from a packed table: gather rows, then dequantize them (vocal_embeds.py:79-98)."""
+    """Embedding lookup from a packed table (vocal_embeds.py:79-98); the reference gathers the packed rows with
+    index_select and dequantizes the copy, here one kernel reads the rows in place."""
     import torch
 
     from . import ops
@@ -178,7 +180,6 @@ def apply_gguf_embedding(x, weight, weight_type: int, hidden_size: int, dtype=No
         block_size, type_size = ops.quant_sizes(weight_type)
         flat = x.flatten()
         assert hidden_size == weight.shape[1] // type_size * block_size
-        quant = torch.index_select(weight, 0, flat)
-        dense = ops.ggml_dequantize(quant, weight_type, hidden_size, flat.shape[0], dtype)
+        dense = ops.ggml_dequantize_rows(weight, weight_type, flat, hidden_size, dtype)  # gather + dequantize, one kernel
         return dense.view(*x.shape, hidden_size)
     raise NotImplementedError(f"Unsupported GGUF quantization type: {weight_type}")

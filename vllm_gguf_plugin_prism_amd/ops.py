@@ -62,6 +62,21 @@ def ggml_dequantize(W: torch.Tensor, quant_type: int, m: int, n: int, dtype: tor
     return out
 
 
+def ggml_dequantize_rows(W: torch.Tensor, quant_type: int, row_ids: torch.Tensor, hidden_size: int,
+                         dtype: torch.dtype | None) -> torch.Tensor:
+    """Dense ``[row_ids.numel(), hidden_size]`` values of the selected rows of the packed table ``W``: the embedding
+    lookup of quantization/vocal_embeds.py:90-96 (index_select, then ggml_dequantize) in one kernel."""
+    _check_inputs(W, row_ids)
+    out_dtype = dtype or torch.float16
+    ids = row_ids.reshape(-1).to(torch.int64)
+    with torch.cuda.device(W.device):
+        out = torch.empty((ids.numel(), hidden_size), dtype=out_dtype, device=W.device)
+        rc = _lib.lib().gguf_dequantize_rows(W.data_ptr(), int(quant_type), ids.data_ptr(), ids.numel(), W.shape[0],
+                                             hidden_size, out.data_ptr(), _code(out_dtype), _stream(W))
+    _lib.check(rc, "ggml_dequantize_rows")
+    return out
+
+
 def _mul_mat(entry: str, W: torch.Tensor, X: torch.Tensor, quant_type: int, row: int) -> torch.Tensor:
     _check_inputs(W, X)
     vecs, col = X.shape
@@ -163,3 +178,38 @@ def quantize_q8_1(X: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
         _lib.check(L.gguf_quantize_q8_1(X.data_ptr(), _code(X.dtype), ws.data_ptr(), m, k, _stream(X)), "quantize_q8_1")
         _lib.check(L.gguf_q8_1_unpack(ws.data_ptr(), q.data_ptr(), ds.data_ptr(), m, k, _stream(X)), "q8_1_unpack")
     return q, ds
+
+
+def moe_align_block_size(topk_ids: torch.Tensor, block_size: int, num_experts: int):
+    """``(sorted_token_ids, expert_ids, num_tokens_post_padded)`` for the grouped kernel, in one launch.
+
+    Same contract as vLLM's ``moe_align_block_size`` as the reference calls it (quantization/fused_moe.py:62-66):
+    int32 outputs, padding slots hold ``topk_ids.numel()``, the order inside an expert's run is ascending pair index."""
+    _check_inputs(topk_ids)
+    ids = topk_ids.reshape(-1)
+    if ids.dtype != torch.int32:
+        ids = ids.to(torch.int32)
+    numel = ids.numel()
+    capacity = numel + num_experts * (block_size - 1)
+    nblocks = (capacity + block_size - 1) // block_size
+    with torch.cuda.device(ids.device):
+        sorted_ids = torch.empty(capacity, dtype=torch.int32, device=ids.device)
+        expert_ids = torch.empty(nblocks, dtype=torch.int32, device=ids.device)
+        post = torch.empty(1, dtype=torch.int32, device=ids.device)
+        rc = _lib.lib().gguf_moe_align_block_size(ids.data_ptr(), numel, int(num_experts), int(block_size),
+                                                  sorted_ids.data_ptr(), capacity, expert_ids.data_ptr(), nblocks,
+                                                  post.data_ptr(), _stream(ids))
+    _lib.check(rc, "moe_align_block_size")
+    return sorted_ids, expert_ids, post
+
+
+def moe_weighted_sum(expert_out: torch.Tensor, topk_weights: torch.Tensor, output: torch.Tensor) -> None:
+    """``output[t] = sum_k expert_out[t, k] * topk_weights[t, k]``: the ``mul_`` by the routing weights and the
+    ``moe_sum`` that end the reference's MoE layer (quantization/fused_moe.py:87-95), fused."""
+    tokens, top_k, n = expert_out.shape
+    _check_inputs(expert_out, output)
+    w = topk_weights.reshape(tokens, top_k).to(torch.float32).contiguous()
+    with torch.cuda.device(expert_out.device):
+        rc = _lib.lib().gguf_moe_weighted_sum(expert_out.data_ptr(), w.data_ptr(), output.data_ptr(), _code(expert_out.dtype),
+                                              tokens, top_k, n, _stream(expert_out))
+    _lib.check(rc, "moe_weighted_sum")
