@@ -131,3 +131,25 @@ def test_embedding_rows_out_of_range_are_zero():
     dense = o.dequantize(table, o.Q4_K, "f32").reshape(10, 256)
     assert np.array_equal(got[[0, 1, 4]], dense[[0, 9, 3]])
     assert (got[[2, 3]] == 0).all()
+
+
+def test_gguf_file_to_gemv(tmp_path):
+    """A packed tensor read from a GGUF file goes straight into the operators."""
+    import struct
+
+    from test_gguf_file import Writer
+    from vllm_gguf_plugin_prism_amd import gguf_file
+
+    rng = np.random.default_rng(21)
+    w = synth.make_weights(rng, o.Q6_K, 48, 512)
+    wr = Writer()
+    wr.add_kv("general.architecture", 8, wr.s("test"))
+    wr.add_tensor("blk.0.ffn_down.weight", [512, 48], o.Q6_K, w.tobytes())
+    path = tmp_path / "m.gguf"
+    wr.write(path)
+    items = dict(gguf_file.quant_weights_iterator([str(path)]))
+    qt = int(items["blk.0.ffn_down.weight_type"])
+    wt = items["blk.0.ffn_down.weight"].cuda()
+    x = rng.standard_normal((2, 512)).astype(np.float16)
+    y = D.fused_mul_mat_gguf(torch.from_numpy(x).cuda(), wt, qt).float().cpu().numpy()
+    assert o.rel_l2(y, o.mul_mat_a8(w, x, o.Q6_K, 48)) <= 1e-3
