@@ -98,6 +98,17 @@ int gguf_moe_mmq(const void* X, int xdtype, void* q8_workspace, const void* W, i
 int gguf_moe_vec(const void* X, int xdtype, void* q8_workspace, const void* W, const int32_t* topk_ids, void* Y, int type,
                  int64_t N, int64_t K, int64_t top_k, int64_t tokens, gguf_stream_t stream);
 
+/* The two MoE entry points with the layer's gated activation folded into their activation quantisation: X has
+ * 2*K columns per row, [gate | up], and the kernels see act(gate) * up rounded to X's dtype exactly as a separate
+ * activation kernel would have stored it (quantization/fused_moe.py:44-51,80,92: act() between the two GEMMs).
+ * act: 0 = none (X has K columns, same as the plain entry points), 1 = SiLU, 2 = GELU (erf). */
+int gguf_moe_mmq_act(const void* X, int xdtype, void* q8_workspace, const void* W, int64_t expert_stride_bytes,
+                     const int32_t* sorted_token_ids, const int32_t* expert_ids, const int32_t* num_tokens_post_padded,
+                     int64_t num_sorted, void* Y, int type, int64_t N, int64_t K, int64_t top_k, int64_t tokens, int act,
+                     gguf_stream_t stream);
+int gguf_moe_vec_act(const void* X, int xdtype, void* q8_workspace, const void* W, const int32_t* topk_ids, void* Y, int type,
+                     int64_t N, int64_t K, int64_t top_k, int64_t tokens, int act, gguf_stream_t stream);
+
 /* Token-tile size that moe_align_block_size must pad expert groups to; 0 for unknown types.
  * Replaces ggml_moe_get_block_size (gguf_kernel.cu:532-566). */
 int gguf_moe_block_size(int type);

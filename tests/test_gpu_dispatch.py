@@ -153,3 +153,29 @@ def test_gguf_file_to_gemv(tmp_path):
     x = rng.standard_normal((2, 512)).astype(np.float16)
     y = D.fused_mul_mat_gguf(torch.from_numpy(x).cuda(), wt, qt).float().cpu().numpy()
     assert o.rel_l2(y, o.mul_mat_a8(w, x, o.Q6_K, 48)) <= 1e-3
+
+
+@pytest.mark.parametrize("act", ["silu", "gelu"])
+@pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16, torch.float32])
+def test_fused_activation_equals_separate_activation(act, dt):
+    """The gated activation folded into the quantisation of the second MoE GEMM sees the same dtype-rounded values a
+    separate activation kernel would have written, so both routes give the same output."""
+    from vllm_gguf_plugin_prism_amd import ops
+
+    rng = np.random.default_rng(17)
+    E, I, H, pairs = 4, 256, 96, 11
+    w2 = torch.from_numpy(np.stack([synth.make_weights(rng, o.Q4_0, H, I) for _ in range(E)])).cuda()
+    h = (torch.randn(pairs, 2 * I, device="cuda") * 2).to(dt)
+    ids = torch.from_numpy(rng.integers(0, E, size=pairs).astype(np.int32)).cuda()
+    fn = torch.nn.functional.silu if act == "silu" else torch.nn.functional.gelu
+    sep_in = (fn(h[:, :I]) * h[:, I:]).contiguous()
+    want = ops.ggml_moe_a8_vec(sep_in, w2, ids, 1, o.Q4_0, H, pairs)
+    got = ops.ggml_moe_a8_vec(h, w2, ids, 1, o.Q4_0, H, pairs, activation=act)
+    # torch's and the kernel's exp/erf may differ in the last bit of a few activations; that moves a quant by one step
+    # at most, far below the 1e-3 contract
+    assert o.rel_l2(got.float().cpu().numpy(), want.float().cpu().numpy()) <= (2e-3 if dt == torch.bfloat16 else 5e-4)
+    # grouped path, same check
+    s_, e_, n_ = ops.moe_align_block_size(ids.view(pairs, 1), 32, E)
+    want = ops.ggml_moe_a8(sep_in, w2, s_, e_, n_, o.Q4_0, H, 1, pairs)
+    got = ops.ggml_moe_a8(h, w2, s_, e_, n_, o.Q4_0, H, 1, pairs, activation=act)
+    assert o.rel_l2(got.float().cpu().numpy(), want.float().cpu().numpy()) <= (2e-3 if dt == torch.bfloat16 else 5e-4)

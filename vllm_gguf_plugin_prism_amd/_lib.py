@@ -38,6 +38,11 @@ _SIGNATURES = {
                                 _c.c_int64, _c.c_void_p]),
     "gguf_moe_vec": (_c.c_int, [_c.c_void_p, _c.c_int, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int,
                                 _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_void_p]),
+    "gguf_moe_mmq_act": (_c.c_int, [_c.c_void_p, _c.c_int, _c.c_void_p, _c.c_void_p, _c.c_int64, _c.c_void_p, _c.c_void_p,
+                                    _c.c_void_p, _c.c_int64, _c.c_void_p, _c.c_int, _c.c_int64, _c.c_int64, _c.c_int64,
+                                    _c.c_int64, _c.c_int, _c.c_void_p]),
+    "gguf_moe_vec_act": (_c.c_int, [_c.c_void_p, _c.c_int, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int,
+                                    _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int, _c.c_void_p]),
     "gguf_moe_block_size": (_c.c_int, [_c.c_int]),
     "gguf_moe_align_block_size": (_c.c_int, [_c.c_void_p, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_void_p, _c.c_int64,
                                              _c.c_void_p, _c.c_int64, _c.c_void_p, _c.c_void_p]),

@@ -845,7 +845,7 @@ static void launch_mmq(const void* W, const void* ws, void* Y, int M, int N, int
                      (T*)Y, M, N, K, q8_row_bytes(K), moe);
 }
 
-int quantize_q8_1(const void* x, int xdtype, void* ws, int64_t M, int64_t K, hipStream_t stream);
+int quantize_q8_1(const void* x, int xdtype, void* ws, int64_t M, int64_t K, hipStream_t stream, int act = 0);
 
 #ifdef GGUF_MMQ_TUNE
 // tuning builds only: GGUF_MMQ_CFG in the environment forces one tile configuration (fp16 activations only)
@@ -960,11 +960,25 @@ extern "C" int gguf_mmq(const void* W, const void* x, int xdtype, void* q8_works
 
 extern "C" int gguf_moe_block_size(int type) { return gguf::block_elems(type) ? 32 : 0; }
 
+extern "C" int gguf_moe_mmq_act(const void* X, int xdtype, void* q8_workspace, const void* W, int64_t expert_stride_bytes,
+                                const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                                const int32_t* num_tokens_post_padded, int64_t num_sorted, void* Y, int type, int64_t N,
+                                int64_t K, int64_t top_k, int64_t tokens, int act, gguf_stream_t stream);
+
 extern "C" int gguf_moe_mmq(const void* X, int xdtype, void* q8_workspace, const void* W, int64_t expert_stride_bytes,
                             const int32_t* sorted_token_ids, const int32_t* expert_ids,
                             const int32_t* num_tokens_post_padded, int64_t num_sorted, void* Y, int type, int64_t N,
                             int64_t K, int64_t top_k, int64_t tokens, gguf_stream_t stream) {
+  return gguf_moe_mmq_act(X, xdtype, q8_workspace, W, expert_stride_bytes, sorted_token_ids, expert_ids, num_tokens_post_padded,
+                          num_sorted, Y, type, N, K, top_k, tokens, 0, stream);
+}
+
+extern "C" int gguf_moe_mmq_act(const void* X, int xdtype, void* q8_workspace, const void* W, int64_t expert_stride_bytes,
+                                const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                                const int32_t* num_tokens_post_padded, int64_t num_sorted, void* Y, int type, int64_t N,
+                                int64_t K, int64_t top_k, int64_t tokens, int act, gguf_stream_t stream) {
   using namespace gguf;
+  if (act < 0 || act > 2) return GGUF_ERR_SHAPE;
   const int qk = block_elems(type);
   if (qk == 0 || !mmq_type_ok(type)) return GGUF_ERR_TYPE;
   if (N < 0 || tokens < 0 || top_k <= 0 || num_sorted < 0 || K <= 0 || K % qk != 0 || expert_stride_bytes < 0 ||
@@ -979,7 +993,7 @@ extern "C" int gguf_moe_mmq(const void* X, int xdtype, void* q8_workspace, const
   const int64_t n16 = ybytes / 16;
   if (ybytes % 16 != 0) return GGUF_ERR_SHAPE;
   hipLaunchKernelGGL(zero_rows_kernel, dim3((unsigned)((n16 + 255) / 256)), dim3(256), 0, s, (uint4*)Y, n16);
-  const int rc = quantize_q8_1(X, xdtype, q8_workspace, tokens, K, s);
+  const int rc = quantize_q8_1(X, xdtype, q8_workspace, tokens, K, s, act);
   if (rc != GGUF_OK) return rc;
   MoeArgs moe = {sorted_token_ids, expert_ids, num_tokens_post_padded, expert_stride_bytes, (int)top_k, (int)(tokens * top_k)};
   const int ns = (int)(num_sorted / 32 * 32);  // a trailing partial block is ignored, like the reference's integer division

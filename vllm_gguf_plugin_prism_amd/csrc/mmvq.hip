@@ -20,19 +20,19 @@ int mmvq_group_iq_c(int type, const void* W, const void* x, void* ws, void* Y, i
                    hipStream_t s);
 
 int moe_vec_group_std_a(int type, const void* W, const void* x, void* Y, int dtype, int N, int K, const int32_t* ids, int top_k,
-                      int pairs, hipStream_t s);
+                      int pairs, int act, hipStream_t s);
 int moe_vec_group_std_b(int type, const void* W, const void* x, void* Y, int dtype, int N, int K, const int32_t* ids, int top_k,
-                      int pairs, hipStream_t s);
+                      int pairs, int act, hipStream_t s);
 int moe_vec_group_k_a(int type, const void* W, const void* x, void* Y, int dtype, int N, int K, const int32_t* ids, int top_k,
-                      int pairs, hipStream_t s);
+                      int pairs, int act, hipStream_t s);
 int moe_vec_group_k_b(int type, const void* W, const void* x, void* Y, int dtype, int N, int K, const int32_t* ids, int top_k,
-                      int pairs, hipStream_t s);
+                      int pairs, int act, hipStream_t s);
 int moe_vec_group_iq_a(int type, const void* W, const void* x, void* Y, int dtype, int N, int K, const int32_t* ids, int top_k,
-                      int pairs, hipStream_t s);
+                      int pairs, int act, hipStream_t s);
 int moe_vec_group_iq_b(int type, const void* W, const void* x, void* Y, int dtype, int N, int K, const int32_t* ids, int top_k,
-                      int pairs, hipStream_t s);
+                      int pairs, int act, hipStream_t s);
 int moe_vec_group_iq_c(int type, const void* W, const void* x, void* Y, int dtype, int N, int K, const int32_t* ids, int top_k,
-                      int pairs, hipStream_t s);
+                      int pairs, int act, hipStream_t s);
 
 }  // namespace gguf
 
@@ -70,9 +70,20 @@ extern "C" int gguf_mmvq(const void* W, const void* x, int xdtype, void* q8_work
   return GGUF_ERR_TYPE;
 }
 
+extern "C" int gguf_moe_vec_act(const void* X, int xdtype, void* q8_workspace, const void* W, const int32_t* topk_ids,
+                                void* Y, int type, int64_t N, int64_t K, int64_t top_k, int64_t tokens, int act,
+                                gguf_stream_t stream);
+
 extern "C" int gguf_moe_vec(const void* X, int xdtype, void* q8_workspace, const void* W, const int32_t* topk_ids, void* Y,
                             int type, int64_t N, int64_t K, int64_t top_k, int64_t tokens, gguf_stream_t stream) {
+  return gguf_moe_vec_act(X, xdtype, q8_workspace, W, topk_ids, Y, type, N, K, top_k, tokens, 0, stream);
+}
+
+extern "C" int gguf_moe_vec_act(const void* X, int xdtype, void* q8_workspace, const void* W, const int32_t* topk_ids,
+                                void* Y, int type, int64_t N, int64_t K, int64_t top_k, int64_t tokens, int act,
+                                gguf_stream_t stream) {
   using namespace gguf;
+  if (act < 0 || act > 2) return GGUF_ERR_SHAPE;
   const int qk = block_elems(type);
   if (qk == 0) return GGUF_ERR_TYPE;
   if (N < 0 || tokens < 0 || top_k <= 0 || K <= 0 || K % qk != 0 || N > 0x7FFFFFF0LL || K > 0x7FFFFFF0LL ||
@@ -84,25 +95,25 @@ extern "C" int gguf_moe_vec(const void* X, int xdtype, void* q8_workspace, const
   hipStream_t s = (hipStream_t)stream;
   const int pairs = (int)(tokens * top_k);
   switch (type) {
-    case T_Q4_0: return moe_vec_group_std_a(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
-    case T_Q4_1: return moe_vec_group_std_a(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
-    case T_Q8_0: return moe_vec_group_std_a(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
-    case T_Q5_0: return moe_vec_group_std_b(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
-    case T_Q5_1: return moe_vec_group_std_b(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
-    case T_IQ4_NL: return moe_vec_group_std_b(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
-    case T_Q2_K: return moe_vec_group_k_a(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
-    case T_Q3_K: return moe_vec_group_k_a(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
-    case T_Q6_K: return moe_vec_group_k_a(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
-    case T_Q4_K: return moe_vec_group_k_b(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
-    case T_Q5_K: return moe_vec_group_k_b(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
-    case T_IQ4_XS: return moe_vec_group_iq_a(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
-    case T_IQ2_XXS: return moe_vec_group_iq_a(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
-    case T_IQ3_XXS: return moe_vec_group_iq_a(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
-    case T_IQ2_XS: return moe_vec_group_iq_b(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
-    case T_IQ2_S: return moe_vec_group_iq_b(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
-    case T_IQ3_S: return moe_vec_group_iq_b(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
-    case T_IQ1_S: return moe_vec_group_iq_c(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
-    case T_IQ1_M: return moe_vec_group_iq_c(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, s);
+    case T_Q4_0: return moe_vec_group_std_a(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, s);
+    case T_Q4_1: return moe_vec_group_std_a(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, s);
+    case T_Q8_0: return moe_vec_group_std_a(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, s);
+    case T_Q5_0: return moe_vec_group_std_b(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, s);
+    case T_Q5_1: return moe_vec_group_std_b(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, s);
+    case T_IQ4_NL: return moe_vec_group_std_b(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, s);
+    case T_Q2_K: return moe_vec_group_k_a(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, s);
+    case T_Q3_K: return moe_vec_group_k_a(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, s);
+    case T_Q6_K: return moe_vec_group_k_a(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, s);
+    case T_Q4_K: return moe_vec_group_k_b(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, s);
+    case T_Q5_K: return moe_vec_group_k_b(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, s);
+    case T_IQ4_XS: return moe_vec_group_iq_a(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, s);
+    case T_IQ2_XXS: return moe_vec_group_iq_a(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, s);
+    case T_IQ3_XXS: return moe_vec_group_iq_a(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, s);
+    case T_IQ2_XS: return moe_vec_group_iq_b(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, s);
+    case T_IQ2_S: return moe_vec_group_iq_b(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, s);
+    case T_IQ3_S: return moe_vec_group_iq_b(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, s);
+    case T_IQ1_S: return moe_vec_group_iq_c(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, s);
+    case T_IQ1_M: return moe_vec_group_iq_c(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, s);
   }
   return GGUF_ERR_TYPE;
 }

@@ -57,7 +57,7 @@ template <class F, int MT, int RPW, typename T, bool MOE, bool FUSEQ>
 __global__ __launch_bounds__(256) void mmvq_kernel(const uint8_t* __restrict__ W, const char* __restrict__ xsrc,
                                                     T* __restrict__ Y, int N, int K, int kchunk, int64_t x_row_bytes,
                                                     int64_t y_vec_stride, const int32_t* __restrict__ topk_ids,
-                                                    int top_k) {
+                                                    int top_k, int act) {
   extern __shared__ __align__(16) char smem[];
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int Kp = (int)q8_kp(K);
@@ -108,7 +108,9 @@ __global__ __launch_bounds__(256) void mmvq_kernel(const uint8_t* __restrict__ W
       for (int i = tid; i < MT * g8; i += 256) {
         const int m = i / g8, j = i - m * g8;
         float v[8];
-        load8<T>((const T*)(xsrc + m * x_row_bytes) + k0 + 8 * j, v);
+        const T* xrow = (const T*)(xsrc + m * x_row_bytes);
+        if (act == ACT_NONE) load8<T>(xrow + k0 + 8 * j, v);
+        else load8_gated<T>(xrow + k0 + 8 * j, xrow + K + k0 + 8 * j, act, v);  // rows are [gate | up], K values each
         const Q8Quad qq = q8_1_quantize8(v);
         *(uint2*)(lq + m * kchunk + 8 * j) = qq.q;
         if ((j & 3) == 0) {
@@ -407,10 +409,10 @@ static void launch_mt(const void* W, const char* xsrc, T* Y, int N, int K, hipSt
   const int64_t xrb = FUSEQ ? (int64_t)K * (int64_t)sizeof(T) : q8_row_bytes(K);
   const size_t lds = mmvq_lds<F, MT>(kchunk);
   hipLaunchKernelGGL((mmvq_kernel<F, MT, RPW, T, false, FUSEQ>), dim3(grid), dim3(256), lds, stream,
-                     (const uint8_t*)W, xsrc, Y, N, K, kchunk, xrb, (int64_t)N, (const int32_t*)nullptr, 1);
+                     (const uint8_t*)W, xsrc, Y, N, K, kchunk, xrb, (int64_t)N, (const int32_t*)nullptr, 1, (int)ACT_NONE);
 }
 
-int quantize_q8_1(const void* x, int xdtype, void* ws, int64_t M, int64_t K, hipStream_t stream);
+int quantize_q8_1(const void* x, int xdtype, void* ws, int64_t M, int64_t K, hipStream_t stream, int act = 0);
 
 template <class F, typename T>
 static int mmvq_typed(const void* W, const void* x, void* ws, void* Y, int xdtype, int64_t N, int64_t K, int64_t M,
@@ -443,11 +445,11 @@ static int mmvq_typed(const void* W, const void* x, void* ws, void* Y, int xdtyp
 
 template <class F, typename T>
 static int moe_vec_typed(const void* W, const char* x, void* Y, int N, int K, const int32_t* topk_ids, int top_k,
-                         int pairs, hipStream_t stream) {
+                         int pairs, int act, hipStream_t stream) {
   constexpr int RPW = GGUF_MMVQ_RPW;
   const int kchunk = kchunk_for(1, K);
   const int grid = (N + 4 * RPW - 1) / (4 * RPW);
-  const int64_t xrb = (int64_t)K * (int64_t)sizeof(T);
+  const int64_t xrb = (int64_t)K * (int64_t)sizeof(T) * (act == ACT_NONE ? 1 : 2);
   const size_t lds = mmvq_lds<F, 1>(kchunk);
   for (int z0 = 0; z0 < pairs; z0 += 65535) {
     const int nz = pairs - z0 < 65535 ? pairs - z0 : 65535;
@@ -455,15 +457,15 @@ static int moe_vec_typed(const void* W, const char* x, void* Y, int N, int K, co
     if (z0 % top_k != 0) return GGUF_ERR_SHAPE;
     hipLaunchKernelGGL((mmvq_kernel<F, 1, RPW, T, true, true>), dim3(grid, nz), dim3(256), lds, stream,
                        (const uint8_t*)W, x + (int64_t)(z0 / top_k) * xrb, (T*)Y + (int64_t)z0 * N, N, K, kchunk, xrb,
-                       (int64_t)N, topk_ids + z0, top_k);
+                       (int64_t)N, topk_ids + z0, top_k, act);
   }
   return launch_status();
 }
 
 template <class F>
 static int moe_vec_fmt(const void* W, const void* x, void* Y, int dtype, int N, int K, const int32_t* ids, int top_k,
-                       int pairs, hipStream_t s) {
-  GGUF_DISPATCH_DTYPE(dtype, return (moe_vec_typed<F, scalar_t>(W, (const char*)x, Y, N, K, ids, top_k, pairs, s)));
+                       int pairs, int act, hipStream_t s) {
+  GGUF_DISPATCH_DTYPE(dtype, return (moe_vec_typed<F, scalar_t>(W, (const char*)x, Y, N, K, ids, top_k, pairs, act, s)));
   return GGUF_ERR_DTYPE;
 }
 

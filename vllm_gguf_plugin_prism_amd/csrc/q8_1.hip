@@ -15,14 +15,15 @@ namespace gguf {
 
 template <typename T>
 __global__ __launch_bounds__(256) void quantize_q8_1_kernel(const T* __restrict__ x, char* __restrict__ ws, int K,
-                                                           int Kp, int64_t row_bytes) {
+                                                           int Kp, int64_t row_bytes, int act) {
   const int t = blockIdx.x * 256 + threadIdx.x;  // one thread per 8 values of the padded row
   if (t * 8 >= Kp) return;
   const int64_t m = blockIdx.y;
   const int e0 = t * 8;
   float v[8];
   if (e0 < K) {
-    load8<T>(x + m * (int64_t)K + e0, v);
+    if (act == ACT_NONE) load8<T>(x + m * (int64_t)K + e0, v);
+    else load8_gated<T>(x + m * (int64_t)(2 * K) + e0, x + m * (int64_t)(2 * K) + K + e0, act, v);  // rows are [gate | up]
   } else {
 #pragma unroll
     for (int i = 0; i < 8; ++i) v[i] = 0.0f;
@@ -55,7 +56,7 @@ __global__ void q8_1_unpack_kernel(const char* __restrict__ ws, int8_t* __restri
   }
 }
 
-int quantize_q8_1(const void* x, int xdtype, void* ws, int64_t M, int64_t K, hipStream_t stream) {
+int quantize_q8_1(const void* x, int xdtype, void* ws, int64_t M, int64_t K, hipStream_t stream, int act) {
   if (M == 0) return GGUF_OK;
   const int Kp = (int)q8_kp(K);
   const int64_t rb = q8_row_bytes(K);
@@ -63,7 +64,7 @@ int quantize_q8_1(const void* x, int xdtype, void* ws, int64_t M, int64_t K, hip
   for (int64_t off = 0; off < M; off += 65535) {
     const int rows = (int)((M - off) < 65535 ? (M - off) : 65535);
     GGUF_DISPATCH_DTYPE(xdtype, hipLaunchKernelGGL(quantize_q8_1_kernel<scalar_t>, dim3(gx, rows), dim3(256), 0, stream,
-                                                   (const scalar_t*)x + off * K, (char*)ws + off * rb, (int)K, Kp, rb));
+                                                   (const scalar_t*)x + off * K * (act == ACT_NONE ? 1 : 2), (char*)ws + off * rb, (int)K, Kp, rb, act));
   }
   return launch_status();
 }
@@ -76,7 +77,7 @@ extern "C" int gguf_quantize_q8_1(const void* x, int xdtype, void* ws, int64_t M
   if (M < 0 || K <= 0 || K % 32 != 0) return GGUF_ERR_SHAPE;
   if (M > 0 && (!x || !ws)) return GGUF_ERR_NULL;
   if (xdtype < 0 || xdtype > 2) return GGUF_ERR_DTYPE;
-  return gguf::quantize_q8_1(x, xdtype, ws, M, K, (hipStream_t)stream);
+  return gguf::quantize_q8_1(x, xdtype, ws, M, K, (hipStream_t)stream, gguf::ACT_NONE);
 }
 
 extern "C" int gguf_q8_1_unpack(const void* ws, int8_t* q, float* ds, int64_t M, int64_t K, gguf_stream_t stream) {

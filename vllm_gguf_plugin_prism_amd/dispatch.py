@@ -146,13 +146,13 @@ def fused_moe_gguf(x, w1, w2, topk_weights, topk_ids, weight_type: int, weight_t
         block = ops.ggml_moe_get_block_size(weight_type)
         sorted_ids, expert_ids, post_padded = ops.moe_align_block_size(topk_ids, block, experts)
         out = ops.ggml_moe_a8(x, w1, sorted_ids, expert_ids, post_padded, weight_type, rows, top_k, tokens)
-        out = _activation(activation, out).contiguous()
-        out = ops.ggml_moe_a8(out, w2, sorted_ids, expert_ids, post_padded, weight_type2, w2.shape[1], 1, tokens * top_k)
+        # act() of the reference is applied inside the second call, while its rows are quantized
+        out = ops.ggml_moe_a8(out, w2, sorted_ids, expert_ids, post_padded, weight_type2, w2.shape[1], 1, tokens * top_k,
+                              activation=activation)
     elif path == "vec":
         rows = w1.shape[1]
         out = ops.ggml_moe_a8_vec(x, w1, topk_ids, top_k, weight_type, rows, tokens)
-        out = _activation(activation, out).contiguous()
-        out = ops.ggml_moe_a8_vec(out, w2, topk_ids, 1, weight_type2, w2.shape[1], tokens * top_k)
+        out = ops.ggml_moe_a8_vec(out, w2, topk_ids, 1, weight_type2, w2.shape[1], tokens * top_k, activation=activation)
     else:
         for tok in range(tokens):
             inp = x[tok : tok + 1]

@@ -37,6 +37,16 @@ def _check_inputs(*tensors: torch.Tensor) -> None:
             raise ValueError("GGUF ops need contiguous tensors")
 
 
+_ACT_CODE = {None: 0, "silu": 1, "gelu": 2}
+
+
+def _act_code(name: str | None) -> int:
+    try:
+        return _ACT_CODE[name]
+    except KeyError:
+        raise ValueError(f"unsupported MoE activation {name!r}; need 'silu' or 'gelu'") from None
+
+
 def _workspace(x: torch.Tensor, rows: int, k: int) -> torch.Tensor:
     nbytes = rows * _lib.lib().gguf_q8_1_row_bytes(k)
     return torch.empty(max(nbytes, 16), dtype=torch.uint8, device=x.device)
@@ -110,20 +120,26 @@ def ggml_moe_a8(
     row: int,
     top_k: int,
     tokens: int,
+    *,
+    activation: str | None = None,
 ) -> torch.Tensor:
-    """Grouped MoE GEMM -> ``[tokens * top_k, row]`` (reference: gguf_kernel.cu:292-393)."""
+    """Grouped MoE GEMM -> ``[tokens * top_k, row]`` (reference: gguf_kernel.cu:292-393).
+
+    ``activation`` ("silu" / "gelu") is an extension: X then holds ``[gate | up]`` rows of twice the inner dimension and
+    the gated activation is applied while the rows are quantized, instead of by a separate kernel beforehand."""
     _check_inputs(X, W, sorted_token_ids, expert_ids, num_tokens_post_padded)
     for t in (sorted_token_ids, expert_ids, num_tokens_post_padded):
         if t.dtype != torch.int32:
             raise ValueError("MoE index tensors must be int32")
-    col = X.shape[1]
+    act = _act_code(activation)
+    col = X.shape[1] // 2 if act else X.shape[1]
     with torch.cuda.device(X.device):
         out = torch.empty((tokens * top_k, row), dtype=X.dtype, device=W.device)
         ws = _workspace(X, tokens, col)
-        rc = _lib.lib().gguf_moe_mmq(
+        rc = _lib.lib().gguf_moe_mmq_act(
             X.data_ptr(), _code(X.dtype), ws.data_ptr(), W.data_ptr(), W.stride(0) * W.element_size(),
             sorted_token_ids.data_ptr(), expert_ids.data_ptr(), num_tokens_post_padded.data_ptr(),
-            sorted_token_ids.shape[0], out.data_ptr(), int(quant_type), row, col, top_k, tokens, _stream(X))
+            sorted_token_ids.shape[0], out.data_ptr(), int(quant_type), row, col, top_k, tokens, act, _stream(X))
     _lib.check(rc, "ggml_moe_a8")
     return out
 
@@ -136,17 +152,21 @@ def ggml_moe_a8_vec(
     quant_type: int,
     row: int,
     tokens: int,
+    *,
+    activation: str | None = None,
 ) -> torch.Tensor:
-    """Per-pair MoE GEMV -> ``[tokens * top_k, row]`` (reference: gguf_kernel.cu:395-530)."""
+    """Per-pair MoE GEMV -> ``[tokens * top_k, row]`` (reference: gguf_kernel.cu:395-530).  ``activation``: see
+    :func:`ggml_moe_a8`."""
     _check_inputs(X, W, topk_ids)
     if topk_ids.dtype != torch.int32:
         raise ValueError("topk_ids must be int32")
-    col = X.shape[1]
+    act = _act_code(activation)
+    col = X.shape[1] // 2 if act else X.shape[1]
     with torch.cuda.device(X.device):
         out = torch.empty((tokens * top_k, row), dtype=X.dtype, device=W.device)
         ws = _workspace(X, tokens, col)
-        rc = _lib.lib().gguf_moe_vec(X.data_ptr(), _code(X.dtype), ws.data_ptr(), W.data_ptr(), topk_ids.data_ptr(),
-                                     out.data_ptr(), int(quant_type), row, col, top_k, tokens, _stream(X))
+        rc = _lib.lib().gguf_moe_vec_act(X.data_ptr(), _code(X.dtype), ws.data_ptr(), W.data_ptr(), topk_ids.data_ptr(),
+                                         out.data_ptr(), int(quant_type), row, col, top_k, tokens, act, _stream(X))
     _lib.check(rc, "ggml_moe_a8_vec")
     return out
 
