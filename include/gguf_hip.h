@@ -101,13 +101,20 @@ int gguf_moe_vec(const void* X, int xdtype, void* q8_workspace, const void* W, c
 /* The two MoE entry points with the layer's gated activation folded into their activation quantisation: X has
  * 2*K columns per row, [gate | up], and the kernels see act(gate) * up rounded to X's dtype exactly as a separate
  * activation kernel would have stored it (quantization/fused_moe.py:44-51,80,92: act() between the two GEMMs).
- * act: 0 = none (X has K columns, same as the plain entry points), 1 = SiLU, 2 = GELU (erf). */
+ * act: 0 = none (X has K columns, same as the plain entry points), 1 = SiLU, 2 = GELU (erf).
+ * gguf_moe_vec_act also takes the number of experts in W (0 = unknown) and the size of the workspace (0 = the
+ * minimum, tokens * gguf_q8_1_row_bytes(K)).  When tokens*top_k >= 2*num_experts and the workspace has room for the
+ * routing sort as well -- gguf_moe_vec_workspace_bytes() -- the pairs are sorted by expert, the activations quantized
+ * once, and four pairs of an expert share each pass over its weights, so a shared expert is read about once per call
+ * rather than once per pair (the reference's grid re-reads it per pair, moe_vec.cuh:3-53).  Same results either way. */
+int64_t gguf_moe_vec_workspace_bytes(int64_t tokens, int64_t top_k, int64_t K, int64_t num_experts);
 int gguf_moe_mmq_act(const void* X, int xdtype, void* q8_workspace, const void* W, int64_t expert_stride_bytes,
                      const int32_t* sorted_token_ids, const int32_t* expert_ids, const int32_t* num_tokens_post_padded,
                      int64_t num_sorted, void* Y, int type, int64_t N, int64_t K, int64_t top_k, int64_t tokens, int act,
                      gguf_stream_t stream);
 int gguf_moe_vec_act(const void* X, int xdtype, void* q8_workspace, const void* W, const int32_t* topk_ids, void* Y, int type,
-                     int64_t N, int64_t K, int64_t top_k, int64_t tokens, int act, gguf_stream_t stream);
+                     int64_t N, int64_t K, int64_t top_k, int64_t tokens, int act, int64_t num_experts, int64_t workspace_bytes,
+                     gguf_stream_t stream);
 
 /* Token-tile size that moe_align_block_size must pad expert groups to; 0 for unknown types.
  * Replaces ggml_moe_get_block_size (gguf_kernel.cu:532-566). */

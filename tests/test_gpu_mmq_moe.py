@@ -146,6 +146,21 @@ def test_moe_grouped_padding_and_bad_experts_write_nothing():
     assert len(skipped) > 0 and np.all(y[skipped] == 0)
 
 
+@pytest.mark.parametrize("t,top_k,e", [(2, 2, 8), (64, 8, 64), (33, 1, 3)])
+@pytest.mark.parametrize("qtype", [o.Q4_0, o.Q4_K, o.IQ2_XXS])
+def test_moe_vec_grouped_and_per_pair_grids(qtype, t, top_k, e):
+    """Few pairs per expert run one pair per workgroup row, many pairs are sorted by expert and run four at a time;
+    both must give the per-pair result, including ragged last groups and experts nobody picked."""
+    ops = _ops()
+    rng = np.random.default_rng(950 + qtype + t)
+    n, k = 72, 512
+    w = np.stack([o.make_weights(rng, qtype, n, k) for _ in range(e)])
+    xd, xv = _x(rng, t, k, "f32")
+    ids, _ = _routing(rng, t, e, top_k)
+    y = ops.ggml_moe_a8_vec(xd, _dev(w), _dev(ids), top_k, qtype, n, t)
+    assert o.rel_l2(y.cpu().numpy(), o.moe_a8_vec(xv, w, ids, top_k, qtype, n, t)) <= 1e-5
+
+
 @pytest.mark.parametrize("qtype", ALL)
 def test_moe_vec_matches_oracle(qtype):
     ops = _ops()

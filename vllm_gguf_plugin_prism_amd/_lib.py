@@ -42,7 +42,9 @@ _SIGNATURES = {
                                     _c.c_void_p, _c.c_int64, _c.c_void_p, _c.c_int, _c.c_int64, _c.c_int64, _c.c_int64,
                                     _c.c_int64, _c.c_int, _c.c_void_p]),
     "gguf_moe_vec_act": (_c.c_int, [_c.c_void_p, _c.c_int, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int,
-                                    _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int, _c.c_void_p]),
+                                    _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int, _c.c_int64, _c.c_int64,
+                                    _c.c_void_p]),
+    "gguf_moe_vec_workspace_bytes": (_c.c_int64, [_c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64]),
     "gguf_moe_block_size": (_c.c_int, [_c.c_int]),
     "gguf_moe_align_block_size": (_c.c_int, [_c.c_void_p, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_void_p, _c.c_int64,
                                              _c.c_void_p, _c.c_int64, _c.c_void_p, _c.c_void_p]),
@@ -52,7 +54,22 @@ _SIGNATURES = {
 EXPORTS = tuple(_SIGNATURES)
 
 
-def lib() -> ctypes.CDLL:
+class _Bound:
+    """The library's entry points as attributes."""
+
+
+def _exact_arity(fn, name: str, nargs: int):
+    # ctypes accepts surplus arguments silently; one too many would land in the stream parameter
+    def call(*args):
+        if len(args) != nargs:
+            raise TypeError(f"{name} takes {nargs} arguments, got {len(args)}")
+        return fn(*args)
+
+    call.__name__ = name
+    return call
+
+
+def lib() -> "_Bound":
     """Load the HIP library; there is no fallback path, a missing library is an error."""
     global _lib
     if _lib is None:
@@ -63,11 +80,14 @@ def lib() -> ctypes.CDLL:
                 "(hipcc, gfx950).  This package has no non-HIP implementation."
             )
         handle = ctypes.CDLL(path)
+        bound = _Bound()
         for name, (res, args) in _SIGNATURES.items():
             fn = getattr(handle, name)
             fn.restype = res
             fn.argtypes = args
-        _lib = handle
+            setattr(bound, name, _exact_arity(fn, name, len(args)))
+        bound._handle = handle
+        _lib = bound
     return _lib
 
 

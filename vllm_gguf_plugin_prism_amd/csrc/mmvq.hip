@@ -20,19 +20,19 @@ int mmvq_group_iq_c(int type, const void* W, const void* x, void* ws, void* Y, i
                    hipStream_t s);
 
 int moe_vec_group_std_a(int type, const void* W, const void* x, void* Y, int dtype, int N, int K, const int32_t* ids, int top_k,
-                      int pairs, int act, hipStream_t s);
+                      int pairs, int act, int num_experts, void* scratch, int64_t scratch_bytes, hipStream_t s);
 int moe_vec_group_std_b(int type, const void* W, const void* x, void* Y, int dtype, int N, int K, const int32_t* ids, int top_k,
-                      int pairs, int act, hipStream_t s);
+                      int pairs, int act, int num_experts, void* scratch, int64_t scratch_bytes, hipStream_t s);
 int moe_vec_group_k_a(int type, const void* W, const void* x, void* Y, int dtype, int N, int K, const int32_t* ids, int top_k,
-                      int pairs, int act, hipStream_t s);
+                      int pairs, int act, int num_experts, void* scratch, int64_t scratch_bytes, hipStream_t s);
 int moe_vec_group_k_b(int type, const void* W, const void* x, void* Y, int dtype, int N, int K, const int32_t* ids, int top_k,
-                      int pairs, int act, hipStream_t s);
+                      int pairs, int act, int num_experts, void* scratch, int64_t scratch_bytes, hipStream_t s);
 int moe_vec_group_iq_a(int type, const void* W, const void* x, void* Y, int dtype, int N, int K, const int32_t* ids, int top_k,
-                      int pairs, int act, hipStream_t s);
+                      int pairs, int act, int num_experts, void* scratch, int64_t scratch_bytes, hipStream_t s);
 int moe_vec_group_iq_b(int type, const void* W, const void* x, void* Y, int dtype, int N, int K, const int32_t* ids, int top_k,
-                      int pairs, int act, hipStream_t s);
+                      int pairs, int act, int num_experts, void* scratch, int64_t scratch_bytes, hipStream_t s);
 int moe_vec_group_iq_c(int type, const void* W, const void* x, void* Y, int dtype, int N, int K, const int32_t* ids, int top_k,
-                      int pairs, int act, hipStream_t s);
+                      int pairs, int act, int num_experts, void* scratch, int64_t scratch_bytes, hipStream_t s);
 
 }  // namespace gguf
 
@@ -72,16 +72,22 @@ extern "C" int gguf_mmvq(const void* W, const void* x, int xdtype, void* q8_work
 
 extern "C" int gguf_moe_vec_act(const void* X, int xdtype, void* q8_workspace, const void* W, const int32_t* topk_ids,
                                 void* Y, int type, int64_t N, int64_t K, int64_t top_k, int64_t tokens, int act,
-                                gguf_stream_t stream);
+                                int64_t num_experts, int64_t workspace_bytes, gguf_stream_t stream);
+
+extern "C" int64_t gguf_moe_vec_workspace_bytes(int64_t tokens, int64_t top_k, int64_t K, int64_t num_experts) {
+  if (tokens < 0 || top_k <= 0 || K <= 0 || num_experts < 0) return 0;
+  const int64_t sorted_cap = tokens * top_k + num_experts * 7;  // room for groups of up to eight pairs per expert block
+  return tokens * gguf::q8_row_bytes(K) + (sorted_cap + (sorted_cap + 3) / 4 + 1) * 4;
+}
 
 extern "C" int gguf_moe_vec(const void* X, int xdtype, void* q8_workspace, const void* W, const int32_t* topk_ids, void* Y,
                             int type, int64_t N, int64_t K, int64_t top_k, int64_t tokens, gguf_stream_t stream) {
-  return gguf_moe_vec_act(X, xdtype, q8_workspace, W, topk_ids, Y, type, N, K, top_k, tokens, 0, stream);
+  return gguf_moe_vec_act(X, xdtype, q8_workspace, W, topk_ids, Y, type, N, K, top_k, tokens, 0, 0, 0, stream);
 }
 
 extern "C" int gguf_moe_vec_act(const void* X, int xdtype, void* q8_workspace, const void* W, const int32_t* topk_ids,
                                 void* Y, int type, int64_t N, int64_t K, int64_t top_k, int64_t tokens, int act,
-                                gguf_stream_t stream) {
+                                int64_t num_experts, int64_t workspace_bytes, gguf_stream_t stream) {
   using namespace gguf;
   if (act < 0 || act > 2) return GGUF_ERR_SHAPE;
   const int qk = block_elems(type);
@@ -94,26 +100,29 @@ extern "C" int gguf_moe_vec_act(const void* X, int xdtype, void* q8_workspace, c
   if (!X || !q8_workspace || !W || !topk_ids || !Y) return GGUF_ERR_NULL;
   hipStream_t s = (hipStream_t)stream;
   const int pairs = (int)(tokens * top_k);
+  const int ne = num_experts > 0 && num_experts <= 1024 ? (int)num_experts : 0;
+  // the workspace holds at least the quantized activations; a caller that provides more says so
+  const int64_t scratch_bytes = workspace_bytes > tokens * q8_row_bytes(K) ? workspace_bytes : tokens * q8_row_bytes(K);
   switch (type) {
-    case T_Q4_0: return moe_vec_group_std_a(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, s);
-    case T_Q4_1: return moe_vec_group_std_a(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, s);
-    case T_Q8_0: return moe_vec_group_std_a(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, s);
-    case T_Q5_0: return moe_vec_group_std_b(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, s);
-    case T_Q5_1: return moe_vec_group_std_b(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, s);
-    case T_IQ4_NL: return moe_vec_group_std_b(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, s);
-    case T_Q2_K: return moe_vec_group_k_a(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, s);
-    case T_Q3_K: return moe_vec_group_k_a(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, s);
-    case T_Q6_K: return moe_vec_group_k_a(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, s);
-    case T_Q4_K: return moe_vec_group_k_b(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, s);
-    case T_Q5_K: return moe_vec_group_k_b(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, s);
-    case T_IQ4_XS: return moe_vec_group_iq_a(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, s);
-    case T_IQ2_XXS: return moe_vec_group_iq_a(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, s);
-    case T_IQ3_XXS: return moe_vec_group_iq_a(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, s);
-    case T_IQ2_XS: return moe_vec_group_iq_b(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, s);
-    case T_IQ2_S: return moe_vec_group_iq_b(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, s);
-    case T_IQ3_S: return moe_vec_group_iq_b(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, s);
-    case T_IQ1_S: return moe_vec_group_iq_c(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, s);
-    case T_IQ1_M: return moe_vec_group_iq_c(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, s);
+    case T_Q4_0: return moe_vec_group_std_a(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, ne, q8_workspace, scratch_bytes, s);
+    case T_Q4_1: return moe_vec_group_std_a(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, ne, q8_workspace, scratch_bytes, s);
+    case T_Q8_0: return moe_vec_group_std_a(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, ne, q8_workspace, scratch_bytes, s);
+    case T_Q5_0: return moe_vec_group_std_b(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, ne, q8_workspace, scratch_bytes, s);
+    case T_Q5_1: return moe_vec_group_std_b(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, ne, q8_workspace, scratch_bytes, s);
+    case T_IQ4_NL: return moe_vec_group_std_b(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, ne, q8_workspace, scratch_bytes, s);
+    case T_Q2_K: return moe_vec_group_k_a(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, ne, q8_workspace, scratch_bytes, s);
+    case T_Q3_K: return moe_vec_group_k_a(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, ne, q8_workspace, scratch_bytes, s);
+    case T_Q6_K: return moe_vec_group_k_a(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, ne, q8_workspace, scratch_bytes, s);
+    case T_Q4_K: return moe_vec_group_k_b(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, ne, q8_workspace, scratch_bytes, s);
+    case T_Q5_K: return moe_vec_group_k_b(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, ne, q8_workspace, scratch_bytes, s);
+    case T_IQ4_XS: return moe_vec_group_iq_a(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, ne, q8_workspace, scratch_bytes, s);
+    case T_IQ2_XXS: return moe_vec_group_iq_a(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, ne, q8_workspace, scratch_bytes, s);
+    case T_IQ3_XXS: return moe_vec_group_iq_a(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, ne, q8_workspace, scratch_bytes, s);
+    case T_IQ2_XS: return moe_vec_group_iq_b(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, ne, q8_workspace, scratch_bytes, s);
+    case T_IQ2_S: return moe_vec_group_iq_b(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, ne, q8_workspace, scratch_bytes, s);
+    case T_IQ3_S: return moe_vec_group_iq_b(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, ne, q8_workspace, scratch_bytes, s);
+    case T_IQ1_S: return moe_vec_group_iq_c(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, ne, q8_workspace, scratch_bytes, s);
+    case T_IQ1_M: return moe_vec_group_iq_c(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, ne, q8_workspace, scratch_bytes, s);
   }
   return GGUF_ERR_TYPE;
 }

@@ -46,6 +46,9 @@ namespace gguf {
 // MOE selects the per-pair variant (reference: csrc/gguf/moe_vec.cuh:3-53): blockIdx.y is the flat
 // (token, k) pair z; its expert topk_ids[z] picks the weight matrix (experts densely packed), its
 // token z / top_k picks the activation row, and the result goes to row z of Y.
+// With MoeVecArgs::sorted_ids set, blockIdx.y is instead a block of MT slots of one expert out of the routing sort
+// (moe_aux.hip): the MT pairs share every weight byte the workgroup loads, so an expert that serves many pairs
+// crosses HBM about once instead of once per pair.
 //
 // FUSEQ: `xsrc` is the raw activation matrix (dtype T, row pitch K) and every workgroup quantizes
 // the vectors it needs straight into LDS, so a call is one launch and no workspace is touched;
@@ -53,20 +56,40 @@ namespace gguf {
 //
 // The first weight loads of a chunk are issued before the activations are staged, and the loop
 // keeps one step of loads in flight ahead of the dot products.
+struct MoeVecArgs {
+  const int32_t* topk_ids;    // [pairs] expert of every pair
+  const int32_t* sorted_ids;  // routing sort in blocks of MT slots, or null for one pair per workgroup row
+  const int32_t* expert_ids;  // [blocks]
+  int top_k, pairs, act;
+};
+
 template <class F, int MT, int RPW, typename T, bool MOE, bool FUSEQ>
 __global__ __launch_bounds__(256) void mmvq_kernel(const uint8_t* __restrict__ W, const char* __restrict__ xsrc,
                                                     T* __restrict__ Y, int N, int K, int kchunk, int64_t x_row_bytes,
-                                                    int64_t y_vec_stride, const int32_t* __restrict__ topk_ids,
-                                                    int top_k, int act) {
+                                                    int64_t y_vec_stride, MoeVecArgs moe) {
   extern __shared__ __align__(16) char smem[];
+  __shared__ int s_xrow[MT], s_yrow[MT];  // activation row and output row of every staged vector (MOE)
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
   const int Kp = (int)q8_kp(K);
+  const int act = moe.act;
   if (MOE) {
-    const int z = blockIdx.y;
-    const int e = topk_ids[z];
+    int e;
+    if (moe.sorted_ids == nullptr) {
+      const int z = blockIdx.y;
+      e = moe.topk_ids[z];
+      if (tid < MT) { s_xrow[tid] = z / moe.top_k; s_yrow[tid] = tid == 0 ? z : -1; }
+    } else {
+      e = moe.expert_ids[blockIdx.y];
+      if (e < 0) return;  // past the padded total
+      if (tid < MT) {
+        const int p = moe.sorted_ids[blockIdx.y * MT + tid];
+        const bool ok = p < moe.pairs;
+        s_xrow[tid] = ok ? p / moe.top_k : 0;
+        s_yrow[tid] = ok ? p : -1;
+      }
+    }
     W += (int64_t)e * N * ((int64_t)(K / F::QK) * F::BS);
-    xsrc += (int64_t)(z / top_k) * x_row_bytes;
-    Y += (int64_t)z * N;
+    __syncthreads();
   }
   int8_t* lq = (int8_t*)smem;                         // [MT][kchunk]
   float* ldv = (float*)(smem + MT * kchunk);          // [MT][kchunk/32]
@@ -108,7 +131,7 @@ __global__ __launch_bounds__(256) void mmvq_kernel(const uint8_t* __restrict__ W
       for (int i = tid; i < MT * g8; i += 256) {
         const int m = i / g8, j = i - m * g8;
         float v[8];
-        const T* xrow = (const T*)(xsrc + m * x_row_bytes);
+        const T* xrow = (const T*)(xsrc + (int64_t)(MOE ? s_xrow[m] : m) * x_row_bytes);
         if (act == ACT_NONE) load8<T>(xrow + k0 + 8 * j, v);
         else load8_gated<T>(xrow + k0 + 8 * j, xrow + K + k0 + 8 * j, act, v);  // rows are [gate | up], K values each
         const Q8Quad qq = q8_1_quantize8(v);
@@ -124,11 +147,11 @@ __global__ __launch_bounds__(256) void mmvq_kernel(const uint8_t* __restrict__ W
       const int g16 = kc >> 4;
       for (int i = tid; i < MT * g16; i += 256) {
         const int m = i / g16, j = i - m * g16;
-        *(uint4*)(lq + m * kchunk + 16 * j) = *(const uint4*)(xsrc + m * x_row_bytes + k0 + 16 * j);
+        *(uint4*)(lq + m * kchunk + 16 * j) = *(const uint4*)(xsrc + (int64_t)(MOE ? s_xrow[m] : m) * x_row_bytes + k0 + 16 * j);
       }
       for (int i = tid; i < MT * nb; i += 256) {
         const int m = i / nb, j = i - m * nb;
-        const float* fd = (const float*)(xsrc + m * x_row_bytes + Kp) + u0 + j;
+        const float* fd = (const float*)(xsrc + (int64_t)(MOE ? s_xrow[m] : m) * x_row_bytes + Kp) + u0 + j;
         ldv[m * (kchunk / 32) + j] = fd[0];
         if (F::AUX == AUX_S8) lav[m * (kchunk / 32) + j] = fd[Kp / 32];
         if (F::AUX == AUX_DU) lav[m * (kchunk / 32) + j] = fd[2 * (Kp / 32)];
@@ -166,7 +189,8 @@ __global__ __launch_bounds__(256) void mmvq_kernel(const uint8_t* __restrict__ W
 #pragma unroll
     for (int m = 0; m < MT; ++m) {
       const float v = wave_sum(acc[r][m]);
-      if (lane == 0 && row0 + r < N) Y[m * y_vec_stride + row0 + r] = from_f32<T>(v);
+      const int yrow = MOE ? s_yrow[m] : m;
+      if (lane == 0 && row0 + r < N && yrow >= 0) Y[(int64_t)yrow * y_vec_stride + row0 + r] = from_f32<T>(v);
     }
   }
 }
@@ -409,7 +433,7 @@ static void launch_mt(const void* W, const char* xsrc, T* Y, int N, int K, hipSt
   const int64_t xrb = FUSEQ ? (int64_t)K * (int64_t)sizeof(T) : q8_row_bytes(K);
   const size_t lds = mmvq_lds<F, MT>(kchunk);
   hipLaunchKernelGGL((mmvq_kernel<F, MT, RPW, T, false, FUSEQ>), dim3(grid), dim3(256), lds, stream,
-                     (const uint8_t*)W, xsrc, Y, N, K, kchunk, xrb, (int64_t)N, (const int32_t*)nullptr, 1, (int)ACT_NONE);
+                     (const uint8_t*)W, xsrc, Y, N, K, kchunk, xrb, (int64_t)N, MoeVecArgs{nullptr, nullptr, nullptr, 1, 0, (int)ACT_NONE});
 }
 
 int quantize_q8_1(const void* x, int xdtype, void* ws, int64_t M, int64_t K, hipStream_t stream, int act = 0);
@@ -443,13 +467,53 @@ static int mmvq_typed(const void* W, const void* x, void* ws, void* Y, int xdtyp
   return launch_status();
 }
 
+extern "C" int gguf_moe_align_block_size(const int32_t* topk_ids, int64_t numel, int64_t num_experts, int64_t block,
+                                         int32_t* sorted_token_ids, int64_t sorted_capacity, int32_t* expert_ids,
+                                         int64_t expert_capacity, int32_t* num_tokens_post_padded, gguf_stream_t stream);
+
+#ifndef GGUF_MOE_VEC_GROUP_RPW
+#define GGUF_MOE_VEC_GROUP_RPW 2
+#endif
+#ifndef GGUF_MOE_VEC_GROUP
+#define GGUF_MOE_VEC_GROUP 4
+#endif
+constexpr int MOE_VEC_GROUP = GGUF_MOE_VEC_GROUP;  // pairs of one expert that share a pass over its weights
+
+// With the expert count known and a workspace large enough for the quantized activations plus the routing sort
+// (q8 rows first, then the three sort arrays), pairs are grouped by expert: the activations are quantized once by the
+// stand-alone kernel instead of once per workgroup, and MOE_VEC_GROUP pairs share each pass over an expert's rows.
+// Otherwise every pair gets its own workgroup row and quantizes its token itself (one launch, no workspace).
 template <class F, typename T>
-static int moe_vec_typed(const void* W, const char* x, void* Y, int N, int K, const int32_t* topk_ids, int top_k,
-                         int pairs, int act, hipStream_t stream) {
+static int moe_vec_typed(const void* W, const char* x, void* Y, int xdtype, int N, int K, const int32_t* topk_ids, int top_k,
+                         int pairs, int act, int num_experts, void* scratch, int64_t scratch_bytes, hipStream_t stream) {
   constexpr int RPW = GGUF_MMVQ_RPW;
-  const int kchunk = kchunk_for(1, K);
   const int grid = (N + 4 * RPW - 1) / (4 * RPW);
   const int64_t xrb = (int64_t)K * (int64_t)sizeof(T) * (act == ACT_NONE ? 1 : 2);
+  const int tokens = pairs / top_k;
+  const int64_t q8_bytes = (int64_t)tokens * q8_row_bytes(K);
+  const int64_t sorted_cap = (int64_t)pairs + (int64_t)num_experts * (MOE_VEC_GROUP - 1);
+  const int64_t block_cap = (sorted_cap + MOE_VEC_GROUP - 1) / MOE_VEC_GROUP;
+  const int64_t need = q8_bytes + (sorted_cap + block_cap + 1) * (int64_t)sizeof(int32_t);
+  // grouping pays once experts are shared: at least two pairs per expert on average
+  if (num_experts > 0 && num_experts <= 1024 && pairs >= 2 * num_experts && block_cap <= 65535 && need <= scratch_bytes) {
+    int rc = quantize_q8_1(x, xdtype, scratch, tokens, K, stream, act);
+    if (rc != GGUF_OK) return rc;
+    int32_t* sorted = (int32_t*)((char*)scratch + q8_bytes);  // q8 rows are a multiple of 4 bytes long
+    int32_t* experts = sorted + sorted_cap;
+    int32_t* post = experts + block_cap;
+    rc = gguf_moe_align_block_size(topk_ids, pairs, num_experts, MOE_VEC_GROUP, sorted, sorted_cap, experts, block_cap, post,
+                                   (gguf_stream_t)stream);
+    if (rc != GGUF_OK) return rc;
+    const int kchunk = kchunk_for(MOE_VEC_GROUP, K);
+    const size_t lds = mmvq_lds<F, MOE_VEC_GROUP>(kchunk);
+    constexpr int GRPW = GGUF_MOE_VEC_GROUP_RPW;  // rows per wave: more rows amortise the staging of the group's activations
+    const int ggrid = (N + 4 * GRPW - 1) / (4 * GRPW);
+    hipLaunchKernelGGL((mmvq_kernel<F, MOE_VEC_GROUP, GRPW, T, true, false>), dim3(ggrid, (unsigned)block_cap), dim3(256), lds, stream,
+                       (const uint8_t*)W, (const char*)scratch, (T*)Y, N, K, kchunk, q8_row_bytes(K), (int64_t)N,
+                       MoeVecArgs{topk_ids, sorted, experts, top_k, pairs, (int)ACT_NONE});
+    return launch_status();
+  }
+  const int kchunk = kchunk_for(1, K);
   const size_t lds = mmvq_lds<F, 1>(kchunk);
   for (int z0 = 0; z0 < pairs; z0 += 65535) {
     const int nz = pairs - z0 < 65535 ? pairs - z0 : 65535;
@@ -457,15 +521,16 @@ static int moe_vec_typed(const void* W, const char* x, void* Y, int N, int K, co
     if (z0 % top_k != 0) return GGUF_ERR_SHAPE;
     hipLaunchKernelGGL((mmvq_kernel<F, 1, RPW, T, true, true>), dim3(grid, nz), dim3(256), lds, stream,
                        (const uint8_t*)W, x + (int64_t)(z0 / top_k) * xrb, (T*)Y + (int64_t)z0 * N, N, K, kchunk, xrb,
-                       (int64_t)N, topk_ids + z0, top_k, act);
+                       (int64_t)N, MoeVecArgs{topk_ids + z0, nullptr, nullptr, top_k, nz, act});
   }
   return launch_status();
 }
 
 template <class F>
 static int moe_vec_fmt(const void* W, const void* x, void* Y, int dtype, int N, int K, const int32_t* ids, int top_k,
-                       int pairs, int act, hipStream_t s) {
-  GGUF_DISPATCH_DTYPE(dtype, return (moe_vec_typed<F, scalar_t>(W, (const char*)x, Y, N, K, ids, top_k, pairs, act, s)));
+                       int pairs, int act, int num_experts, void* scratch, int64_t scratch_bytes, hipStream_t s) {
+  GGUF_DISPATCH_DTYPE(dtype, return (moe_vec_typed<F, scalar_t>(W, (const char*)x, Y, dtype, N, K, ids, top_k, pairs, act,
+                                                                num_experts, scratch, scratch_bytes, s)));
   return GGUF_ERR_DTYPE;
 }
 

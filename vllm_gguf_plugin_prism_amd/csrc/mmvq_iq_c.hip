@@ -14,10 +14,10 @@ int mmvq_group_iq_c(int type, const void* W, const void* x, void* ws, void* Y, i
 }
 
 int moe_vec_group_iq_c(int type, const void* W, const void* x, void* Y, int dtype, int N, int K, const int32_t* ids, int top_k,
-                      int pairs, int act, hipStream_t s) {
+                      int pairs, int act, int num_experts, void* scratch, int64_t scratch_bytes, hipStream_t s) {
   switch (type) {
-    case T_IQ1_S: return moe_vec_fmt<FmtIQ1_S>(W, x, Y, dtype, N, K, ids, top_k, pairs, act, s);
-    case T_IQ1_M: return moe_vec_fmt<FmtIQ1_M>(W, x, Y, dtype, N, K, ids, top_k, pairs, act, s);
+    case T_IQ1_S: return moe_vec_fmt<FmtIQ1_S>(W, x, Y, dtype, N, K, ids, top_k, pairs, act, num_experts, scratch, scratch_bytes, s);
+    case T_IQ1_M: return moe_vec_fmt<FmtIQ1_M>(W, x, Y, dtype, N, K, ids, top_k, pairs, act, num_experts, scratch, scratch_bytes, s);
     default: return GGUF_ERR_TYPE;
   }
 }

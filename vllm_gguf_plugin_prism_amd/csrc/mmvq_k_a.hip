@@ -15,11 +15,11 @@ int mmvq_group_k_a(int type, const void* W, const void* x, void* ws, void* Y, in
 }
 
 int moe_vec_group_k_a(int type, const void* W, const void* x, void* Y, int dtype, int N, int K, const int32_t* ids, int top_k,
-                      int pairs, int act, hipStream_t s) {
+                      int pairs, int act, int num_experts, void* scratch, int64_t scratch_bytes, hipStream_t s) {
   switch (type) {
-    case T_Q2_K: return moe_vec_fmt<FmtQ2_K>(W, x, Y, dtype, N, K, ids, top_k, pairs, act, s);
-    case T_Q3_K: return moe_vec_fmt<FmtQ3_K>(W, x, Y, dtype, N, K, ids, top_k, pairs, act, s);
-    case T_Q6_K: return moe_vec_fmt<FmtQ6_K>(W, x, Y, dtype, N, K, ids, top_k, pairs, act, s);
+    case T_Q2_K: return moe_vec_fmt<FmtQ2_K>(W, x, Y, dtype, N, K, ids, top_k, pairs, act, num_experts, scratch, scratch_bytes, s);
+    case T_Q3_K: return moe_vec_fmt<FmtQ3_K>(W, x, Y, dtype, N, K, ids, top_k, pairs, act, num_experts, scratch, scratch_bytes, s);
+    case T_Q6_K: return moe_vec_fmt<FmtQ6_K>(W, x, Y, dtype, N, K, ids, top_k, pairs, act, num_experts, scratch, scratch_bytes, s);
     default: return GGUF_ERR_TYPE;
   }
 }

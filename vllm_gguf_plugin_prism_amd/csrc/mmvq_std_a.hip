@@ -15,11 +15,11 @@ int mmvq_group_std_a(int type, const void* W, const void* x, void* ws, void* Y, 
 }
 
 int moe_vec_group_std_a(int type, const void* W, const void* x, void* Y, int dtype, int N, int K, const int32_t* ids, int top_k,
-                      int pairs, int act, hipStream_t s) {
+                      int pairs, int act, int num_experts, void* scratch, int64_t scratch_bytes, hipStream_t s) {
   switch (type) {
-    case T_Q4_0: return moe_vec_fmt<FmtQ4_0>(W, x, Y, dtype, N, K, ids, top_k, pairs, act, s);
-    case T_Q4_1: return moe_vec_fmt<FmtQ4_1>(W, x, Y, dtype, N, K, ids, top_k, pairs, act, s);
-    case T_Q8_0: return moe_vec_fmt<FmtQ8_0>(W, x, Y, dtype, N, K, ids, top_k, pairs, act, s);
+    case T_Q4_0: return moe_vec_fmt<FmtQ4_0>(W, x, Y, dtype, N, K, ids, top_k, pairs, act, num_experts, scratch, scratch_bytes, s);
+    case T_Q4_1: return moe_vec_fmt<FmtQ4_1>(W, x, Y, dtype, N, K, ids, top_k, pairs, act, num_experts, scratch, scratch_bytes, s);
+    case T_Q8_0: return moe_vec_fmt<FmtQ8_0>(W, x, Y, dtype, N, K, ids, top_k, pairs, act, num_experts, scratch, scratch_bytes, s);
     default: return GGUF_ERR_TYPE;
   }
 }

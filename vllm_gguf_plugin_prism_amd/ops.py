@@ -162,11 +162,13 @@ def ggml_moe_a8_vec(
         raise ValueError("topk_ids must be int32")
     act = _act_code(activation)
     col = X.shape[1] // 2 if act else X.shape[1]
+    L = _lib.lib()
     with torch.cuda.device(X.device):
         out = torch.empty((tokens * top_k, row), dtype=X.dtype, device=W.device)
-        ws = _workspace(X, tokens, col)
-        rc = _lib.lib().gguf_moe_vec_act(X.data_ptr(), _code(X.dtype), ws.data_ptr(), W.data_ptr(), topk_ids.data_ptr(),
-                                         out.data_ptr(), int(quant_type), row, col, top_k, tokens, act, _stream(X))
+        nbytes = max(16, L.gguf_moe_vec_workspace_bytes(tokens, top_k, col, W.shape[0]))  # quantized rows + routing sort
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=X.device)
+        rc = L.gguf_moe_vec_act(X.data_ptr(), _code(X.dtype), ws.data_ptr(), W.data_ptr(), topk_ids.data_ptr(),
+                                out.data_ptr(), int(quant_type), row, col, top_k, tokens, act, W.shape[0], nbytes, _stream(X))
     _lib.check(rc, "ggml_moe_a8_vec")
     return out
 
