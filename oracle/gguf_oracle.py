@@ -26,7 +26,11 @@ Two dequantisation flavours exist because "bit-exact" depends on the arithmetic:
 How each function is pinned (see tests/test_oracle_*.py): table hashes against
 tests/golden/table_sha256.json; hand-built blocks with closed-form answers;
 exhaustive sweeps of index/sign/scale spaces against direct bit descriptions;
-q8_1 properties; fp64 brute force loops on tiny shapes for the matmuls and MoE.
+q8_1 properties; fp64 brute force loops on tiny shapes for the matmuls and MoE;
+for every format, thread-by-thread scalar restatements of the reference's
+dequantize kernel and of its vec_dot function (MMVQ and MMQ semantics), written
+without this module's helpers, that the vectorised code must match bit for bit
+(dequantize) or to fp64 round-off (dot products).
 Agreement with the third-party ``gguf.dequantize`` (gguf-py >= 0.17.0, absent
 here) and with vLLM's ``moe_align_block_size`` ordering is PARITY UNPINNED.
 """
