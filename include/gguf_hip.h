@@ -52,8 +52,10 @@ int gguf_block_bytes(int type);
 
 /* Bytes of activation workspace per row of X for inner dimension K.
  * The reference sizes its workspace as int32[M, roundup(K,512)/32*9]
- * (gguf_kernel.cu:114-115); this library's private layout needs 44 bytes per 32
- * values instead of 36, so callers must size the workspace with this function. */
+ * (gguf_kernel.cu:114-115); this library's private layout needs 108 bytes per 32
+ * values instead of 36 (the quantized rows, and room for their dequantized half-precision
+ * copy that the half-MFMA engine of gguf_mmq reads), so callers must size the workspace
+ * with this function. */
 int64_t gguf_q8_1_row_bytes(int64_t K);
 
 /* q8_1 activation quantizer: M rows of K values -> workspace.
@@ -83,6 +85,21 @@ int gguf_mmvq(const void* W, const void* x, int xdtype, void* q8_workspace, void
  * Replaces ggml_mul_mat_a8 (gguf_kernel.cu:220-290, mmq.cuh:2-610). */
 int gguf_mmq(const void* W, const void* x, int xdtype, void* q8_workspace, void* Y, int type, int64_t N, int64_t K,
              int64_t M, gguf_stream_t stream);
+
+/* gguf_mmq with the arithmetic engine chosen by the caller.  The reference has one engine (dp4a, mmq.cuh:2-104);
+ * this library has two and gguf_mmq picks between them:
+ *   GGUF_MMQ_INT8  int8 MFMA on the block codes, block scales applied in fp32: the reference's arithmetic, differing
+ *                  only in the order of the fp32 additions;
+ *   GGUF_MMQ_HALF  half-precision MFMA on operands that carry their scales (activation d8*q and weight d*q, each
+ *                  rounded to half): two to three times faster, relative deviation about 2e-4 in the l2 norm, below
+ *                  the rounding of a half or bfloat16 result.  Not for fp32 results; not for Q4_1 / Q5_1.
+ *   GGUF_MMQ_AUTO  HALF where it applies, INT8 otherwise.
+ * Both read the workspace layout sized by gguf_q8_1_row_bytes. */
+#define GGUF_MMQ_AUTO 0
+#define GGUF_MMQ_INT8 1
+#define GGUF_MMQ_HALF 2
+int gguf_mmq_engine(const void* W, const void* x, int xdtype, void* q8_workspace, void* Y, int type, int64_t N, int64_t K,
+                    int64_t M, int engine, gguf_stream_t stream);
 
 /* Grouped (MoE) variant: for every sorted slot s with p = sorted_token_ids[s] < tokens*top_k,
  * Y[p,:] = q8_1(X[p / top_k,:]) . W[expert_ids[s / block],:,:]^T.  Rows of Y that no slot names are zero.

@@ -35,7 +35,7 @@ def handle():
 
 def test_header_declares_the_bound_entry_points():
     assert declared_symbols() == sorted(_lib.EXPORTS)
-    assert len(declared_symbols()) == 18
+    assert len(declared_symbols()) == 19
 
 
 def test_every_declared_symbol_is_exported(handle):
@@ -56,10 +56,10 @@ def test_block_sizes_match_the_format_table(handle):
 
 
 def test_workspace_row_bytes(handle):
-    # 44 bytes per 32 values of K rounded up to 512 (int8 quants + three fp32 per block)
-    assert handle.gguf_q8_1_row_bytes(4096) == 4096 // 32 * 44
-    assert handle.gguf_q8_1_row_bytes(256) == 512 // 32 * 44
-    assert handle.gguf_q8_1_row_bytes(14336) == 14336 // 32 * 44
+    # per 32 values of K rounded up to 512: int8 quants + three fp32 (44 bytes), and the half-precision copy (64 bytes) plus 256 bytes of row padding
+    assert handle.gguf_q8_1_row_bytes(4096) == 4096 // 32 * 108 + 256
+    assert handle.gguf_q8_1_row_bytes(256) == 512 // 32 * 108 + 256
+    assert handle.gguf_q8_1_row_bytes(14336) == 14336 // 32 * 108 + 256
     assert handle.gguf_q8_1_row_bytes(0) == 0
 
 

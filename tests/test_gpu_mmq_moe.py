@@ -1,4 +1,5 @@
-"""GPU parity: int8-MFMA MMQ, grouped MoE MMQ and per-pair MoE GEMV against the CPU oracle (C ABI path)."""
+"""GPU parity: MMQ (int8-MFMA and half-MFMA engines), grouped MoE MMQ and per-pair MoE GEMV against the CPU oracle
+(C ABI path)."""
 import numpy as np
 import pytest
 import torch
@@ -11,6 +12,7 @@ SIX = [o.Q4_0, o.Q8_0, o.Q4_K, o.Q6_K, o.IQ4_XS, o.IQ2_XXS]
 MMQ_TYPES = [o.Q4_0, o.Q4_1, o.Q5_0, o.Q5_1, o.Q8_0, o.Q2_K, o.Q3_K, o.Q4_K, o.Q5_K, o.Q6_K, o.IQ4_XS, o.IQ2_XXS]
 ALL = [o.Q4_0, o.Q4_1, o.Q5_0, o.Q5_1, o.Q8_0, o.Q2_K, o.Q3_K, o.Q4_K, o.Q5_K, o.Q6_K, o.IQ2_XXS, o.IQ2_XS, o.IQ3_XXS,
        o.IQ1_S, o.IQ4_NL, o.IQ3_S, o.IQ2_S, o.IQ4_XS, o.IQ1_M]
+HALF_ENGINE_TYPES = [o.Q4_0, o.Q5_0, o.Q8_0, o.Q2_K, o.Q3_K, o.Q4_K, o.Q5_K, o.Q6_K, o.IQ4_XS, o.IQ2_XXS]
 TORCH_DT = {"f16": torch.float16, "bf16": torch.bfloat16, "f32": torch.float32}
 
 
@@ -44,18 +46,69 @@ def test_mmq_matches_a8_oracle_fp32(qtype, m):
         assert err <= 1e-5, (o.TYPE_NAMES[qtype], m, n, k, err)
 
 
+@pytest.mark.parametrize("engine", ["auto", "int8", "half"])
 @pytest.mark.parametrize("dt", ["f16", "bf16"])
 @pytest.mark.parametrize("qtype", MMQ_TYPES)
-def test_mmq_half_outputs_within_tolerance(qtype, dt):
-    # stated tolerance vs the a8 oracle: rel-L2 <= 1e-3 for fp16 outputs, 4e-3 for bf16 (8-bit significand)
+def test_mmq_half_outputs_within_tolerance(qtype, dt, engine):
+    # stated tolerance vs the a8 oracle: rel-L2 <= 1e-3 for fp16 outputs, 4e-3 for bf16 (8-bit significand); it holds
+    # for both arithmetic engines ("auto" is the half-MFMA engine wherever that one applies)
+    if engine == "half" and qtype not in HALF_ENGINE_TYPES:
+        pytest.skip("no half-MFMA engine for this format")
     ops = _ops()
     rng = np.random.default_rng(500 + qtype)
-    n, k, m = 384, 2048, 160
+    n, k = 384, 2048
     w = o.make_weights(rng, qtype, n, k)
-    xd, xv = _x(rng, m, k, dt)
-    y = ops.ggml_mul_mat_a8(_dev(w), xd, qtype, n).to(torch.float32).cpu().numpy()
-    assert o.rel_l2(y, o.mul_mat_a8(w, xv, qtype, n, "mmq")) <= (1e-3 if dt == "f16" else 4e-3)
-    assert o.rel_l2(y, o.mul_mat_f32(w, xv, qtype, n)) <= 2e-2
+    for m in (160, 7):
+        xd, xv = _x(rng, m, k, dt)
+        y = ops.ggml_mul_mat_a8(_dev(w), xd, qtype, n, engine=engine).to(torch.float32).cpu().numpy()
+        assert o.rel_l2(y, o.mul_mat_a8(w, xv, qtype, n, "mmq")) <= (1e-3 if dt == "f16" else 4e-3)
+        assert o.rel_l2(y, o.mul_mat_f32(w, xv, qtype, n)) <= 2e-2
+
+
+def test_mmq_engines_differ_only_by_operand_rounding():
+    # both engines against the same fp32-output run of the integer engine: the half engine adds the rounding of its
+    # two operands to half precision (about 3.5e-4) to the rounding of the fp16 result (2.1e-4) and nothing else
+    ops = _ops()
+    rng = np.random.default_rng(77)
+    for qtype in HALF_ENGINE_TYPES:
+        n, k, m = 320, 2048, 96
+        w = _dev(o.make_weights(rng, qtype, n, k))
+        xd, _ = _x(rng, m, k, "f16")
+        exact = ops.ggml_mul_mat_a8(w, xd.float(), qtype, n).double()
+        half = ops.ggml_mul_mat_a8(w, xd, qtype, n, engine="half").double()
+        int8 = ops.ggml_mul_mat_a8(w, xd, qtype, n, engine="int8").double()
+        e_half = float((half - exact).norm() / exact.norm()), float((int8 - exact).norm() / exact.norm())
+        assert e_half[1] <= 3e-4 and e_half[0] <= 6e-4, (o.TYPE_NAMES[qtype], e_half)
+
+
+@pytest.mark.parametrize("qtype", [o.Q6_K, o.Q4_K, o.Q4_0, o.Q2_K, o.Q8_0])
+@pytest.mark.parametrize("m,n", [(512, 12800), (256, 12800), (256, 6400), (300, 200)])
+def test_mmq_half_engine_every_tile_configuration(qtype, m, n):
+    """The half-MFMA launcher takes the largest of 256x128, 128x128, 128x64 and 64x64 tiles that still yields 180
+    workgroups.  One shape per regime with ragged M and N edges; K is not a multiple of the 64-element step for the
+    32-element formats, so the last step is half empty and the offset pass ends inside a group of eight blocks."""
+    ops = _ops()
+    rng = np.random.default_rng(1100 + qtype + m)
+    k = 256 if o.QUANT_SIZES[qtype][0] == 256 else 352
+    w = o.make_weights(rng, qtype, n - 3, k)
+    xd, xv = _x(rng, m - 5, k, "f16")
+    y = ops.ggml_mul_mat_a8(_dev(w), xd, qtype, n - 3, engine="half")
+    assert y.shape == (m - 5, n - 3) and y.dtype == torch.float16
+    assert o.rel_l2(y.float().cpu().numpy(), o.mul_mat_a8(w, xv, qtype, n - 3, "mmq")) <= 1e-3
+
+
+def test_mmq_engine_rejections():
+    ops = _ops()
+    rng = np.random.default_rng(5)
+    w = _dev(o.make_weights(rng, o.Q4_1, 64, 256))
+    x16, _ = _x(rng, 4, 256, "f16")
+    x32, _ = _x(rng, 4, 256, "f32")
+    with pytest.raises(NotImplementedError):
+        ops.ggml_mul_mat_a8(w, x16, o.Q4_1, 64, engine="half")       # Q4_1 keeps the reference's half-rounded scale products
+    w6 = _dev(o.make_weights(rng, o.Q6_K, 64, 256))
+    with pytest.raises(ValueError):
+        ops.ggml_mul_mat_a8(w6, x32, o.Q6_K, 64, engine="half")      # fp32 results stay on the integer engine
+    assert ops.ggml_mul_mat_a8(w6, x32, o.Q6_K, 64).dtype == torch.float32
 
 
 @pytest.mark.parametrize("qtype", [o.Q4_0, o.Q4_K, o.Q6_K, o.Q2_K, o.Q5_1])

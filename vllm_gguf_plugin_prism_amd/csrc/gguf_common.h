@@ -43,6 +43,10 @@ __host__ __device__ constexpr int block_bytes(int t) {
 // ---------------------------------------------------------------------------
 __host__ __device__ inline int64_t q8_kp(int64_t K) { return (K + 511) / 512 * 512; }
 __host__ __device__ inline int64_t q8_row_bytes(int64_t K) { return q8_kp(K) / 32 * 44; }
+// Behind the M quantized rows the half-MFMA GEMM keeps the dequantized rows in half precision, [M][q8_half_pitch(K)].
+// The pitch is not a multiple of 4096 bytes: a tile reads the same columns of many rows at once, and rows a power of
+// two apart would all fall into the same memory channel.
+__host__ __device__ inline int64_t q8_half_pitch(int64_t K) { return q8_kp(K) + 128; }
 
 struct Q8Row {
   const int8_t* qs;
@@ -139,6 +143,11 @@ template <> __device__ __forceinline__ bf16_t from_half<bf16_t>(_Float16 v) { re
     case GGUF_DTYPE_BF16: { using scalar_t = gguf::bf16_t; __VA_ARGS__; break; } \
     default: return GGUF_ERR_DTYPE;                                      \
   }
+
+// q8_1 quantisation of M rows into the workspace (q8_1.hip).  act: gated activation applied while loading (see
+// q8_1_device.h).  half_plane: if not null, also the dequantized rows in half precision, [M][q8_kp(K)].
+int quantize_q8_1(const void* x, int xdtype, void* ws, int64_t M, int64_t K, hipStream_t stream, int act = 0,
+                  void* half_plane = nullptr);
 
 inline int launch_status() { return hipGetLastError() == hipSuccess ? GGUF_OK : GGUF_ERR_LAUNCH; }
 

@@ -436,7 +436,6 @@ static void launch_mt(const void* W, const char* xsrc, T* Y, int N, int K, hipSt
                      (const uint8_t*)W, xsrc, Y, N, K, kchunk, xrb, (int64_t)N, MoeVecArgs{nullptr, nullptr, nullptr, 1, 0, (int)ACT_NONE});
 }
 
-int quantize_q8_1(const void* x, int xdtype, void* ws, int64_t M, int64_t K, hipStream_t stream, int act = 0);
 
 template <class F, typename T>
 static int mmvq_typed(const void* W, const void* x, void* ws, void* Y, int xdtype, int64_t N, int64_t K, int64_t M,

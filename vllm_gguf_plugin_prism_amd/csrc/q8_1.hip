@@ -15,7 +15,8 @@ namespace gguf {
 
 template <typename T>
 __global__ __launch_bounds__(256) void quantize_q8_1_kernel(const T* __restrict__ x, char* __restrict__ ws, int K,
-                                                           int Kp, int64_t row_bytes, int act) {
+                                                           int Kp, int64_t row_bytes, int act,
+                                                           _Float16* __restrict__ xh) {
   const int t = blockIdx.x * 256 + threadIdx.x;  // one thread per 8 values of the padded row
   if (t * 8 >= Kp) return;
   const int64_t m = blockIdx.y;
@@ -31,6 +32,17 @@ __global__ __launch_bounds__(256) void quantize_q8_1_kernel(const T* __restrict_
   const Q8Quad r = q8_1_quantize8(v);
   char* row = ws + m * row_bytes;
   *(uint2*)(row + e0) = r.q;
+  if (xh) {
+    // the dequantized row in half precision for the half-MFMA GEMM: RN16(d * q), d being the half-rounded scale.
+    // d * q is exact in fp32; magnitudes past the half range saturate (only reachable from bf16 / fp32 inputs).
+    union { _Float16 h[8]; uint4 v; } o;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int q = (int)(int8_t)((i < 4 ? r.q.x >> (8 * i) : r.q.y >> (8 * (i - 4))) & 0xFF);
+      o.h[i] = (_Float16)fminf(fmaxf(r.d * (float)q, -65504.0f), 65504.0f);
+    }
+    *(uint4*)(xh + m * (int64_t)(Kp + 128) + e0) = o.v;   // row pitch: q8_half_pitch
+  }
   if ((t & 3) == 0) {
     const int b = t >> 2;
     const int nb = Kp / 32;
@@ -56,7 +68,7 @@ __global__ void q8_1_unpack_kernel(const char* __restrict__ ws, int8_t* __restri
   }
 }
 
-int quantize_q8_1(const void* x, int xdtype, void* ws, int64_t M, int64_t K, hipStream_t stream, int act) {
+int quantize_q8_1(const void* x, int xdtype, void* ws, int64_t M, int64_t K, hipStream_t stream, int act, void* half_plane) {
   if (M == 0) return GGUF_OK;
   const int Kp = (int)q8_kp(K);
   const int64_t rb = q8_row_bytes(K);
@@ -64,20 +76,21 @@ int quantize_q8_1(const void* x, int xdtype, void* ws, int64_t M, int64_t K, hip
   for (int64_t off = 0; off < M; off += 65535) {
     const int rows = (int)((M - off) < 65535 ? (M - off) : 65535);
     GGUF_DISPATCH_DTYPE(xdtype, hipLaunchKernelGGL(quantize_q8_1_kernel<scalar_t>, dim3(gx, rows), dim3(256), 0, stream,
-                                                   (const scalar_t*)x + off * K * (act == ACT_NONE ? 1 : 2), (char*)ws + off * rb, (int)K, Kp, rb, act));
+                                                   (const scalar_t*)x + off * K * (act == ACT_NONE ? 1 : 2), (char*)ws + off * rb, (int)K, Kp, rb, act,
+                                                   half_plane ? (_Float16*)half_plane + off * q8_half_pitch(K) : (_Float16*)nullptr));
   }
   return launch_status();
 }
 
 }  // namespace gguf
 
-extern "C" int64_t gguf_q8_1_row_bytes(int64_t K) { return K < 0 ? 0 : gguf::q8_row_bytes(K); }
+extern "C" int64_t gguf_q8_1_row_bytes(int64_t K) { return K <= 0 ? 0 : gguf::q8_row_bytes(K) + 2 * gguf::q8_half_pitch(K); }
 
 extern "C" int gguf_quantize_q8_1(const void* x, int xdtype, void* ws, int64_t M, int64_t K, gguf_stream_t stream) {
   if (M < 0 || K <= 0 || K % 32 != 0) return GGUF_ERR_SHAPE;
   if (M > 0 && (!x || !ws)) return GGUF_ERR_NULL;
   if (xdtype < 0 || xdtype > 2) return GGUF_ERR_DTYPE;
-  return gguf::quantize_q8_1(x, xdtype, ws, M, K, (hipStream_t)stream, gguf::ACT_NONE);
+  return gguf::quantize_q8_1(x, xdtype, ws, M, K, (hipStream_t)stream, gguf::ACT_NONE, nullptr);
 }
 
 extern "C" int gguf_q8_1_unpack(const void* ws, int8_t* q, float* ds, int64_t M, int64_t K, gguf_stream_t stream) {
