@@ -94,12 +94,16 @@ int gguf_mmq(const void* W, const void* x, int xdtype, void* q8_workspace, void*
  *                  rounded to half): two to three times faster, relative deviation about 2e-4 in the l2 norm, below
  *                  the rounding of a half or bfloat16 result.  Not for fp32 results; not for Q4_1 / Q5_1.
  *   GGUF_MMQ_AUTO  HALF where it applies, INT8 otherwise.
- * Both read the workspace layout sized by gguf_q8_1_row_bytes. */
+ * workspace_bytes is the size of q8_workspace; 0 stands for the minimum, M * gguf_q8_1_row_bytes(K).  Given
+ * gguf_mmq_workspace_bytes(M, N, K) bytes, the half engine splits K over several workgroups per output tile when the
+ * output alone has too few tiles to occupy the chip (few tokens or a narrow N with a long K), keeping fp32 partial
+ * tiles behind the rows and adding them in a second launch.  The result does not depend on the run, only on the shape. */
 #define GGUF_MMQ_AUTO 0
 #define GGUF_MMQ_INT8 1
 #define GGUF_MMQ_HALF 2
+int64_t gguf_mmq_workspace_bytes(int64_t M, int64_t N, int64_t K);
 int gguf_mmq_engine(const void* W, const void* x, int xdtype, void* q8_workspace, void* Y, int type, int64_t N, int64_t K,
-                    int64_t M, int engine, gguf_stream_t stream);
+                    int64_t M, int engine, int64_t workspace_bytes, gguf_stream_t stream);
 
 /* Grouped (MoE) variant: for every sorted slot s with p = sorted_token_ids[s] < tokens*top_k,
  * Y[p,:] = q8_1(X[p / top_k,:]) . W[expert_ids[s / block],:,:]^T.  Rows of Y that no slot names are zero.

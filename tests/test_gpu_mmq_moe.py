@@ -97,6 +97,33 @@ def test_mmq_half_engine_every_tile_configuration(qtype, m, n):
     assert o.rel_l2(y.float().cpu().numpy(), o.mul_mat_a8(w, xv, qtype, n - 3, "mmq")) <= 1e-3
 
 
+@pytest.mark.parametrize("qtype", [o.Q6_K, o.Q4_K, o.Q4_0])
+@pytest.mark.parametrize("m", [200, 100])
+def test_mmq_half_engine_split_k(qtype, m):
+    """Few output tiles and a long K: the half engine splits K over several workgroups per tile (fp32 partial tiles in
+    the workspace, summed by a second launch) when the workspace is sized by gguf_mmq_workspace_bytes, and must not
+    when it has only the minimum.  Same tolerance either way; the offset pass belongs to the first split."""
+    from vllm_gguf_plugin_prism_amd import _lib
+    ops = _ops()
+    rng = np.random.default_rng(1300 + qtype + m)
+    n, k = 250, 4096
+    assert _lib.lib().gguf_mmq_workspace_bytes(m, n, k) > m * _lib.lib().gguf_q8_1_row_bytes(k) + 256   # room for partials
+    w = o.make_weights(rng, qtype, n, k)
+    xd, xv = _x(rng, m, k, "f16")
+    exp = o.mul_mat_a8(w, xv, qtype, n, "mmq")
+    y_split = ops.ggml_mul_mat_a8(_dev(w), xd, qtype, n, engine="half")
+    assert o.rel_l2(y_split.float().cpu().numpy(), exp) <= 1e-3
+    # the plain C entry point passes no workspace size: no split
+    ws = torch.empty(m * _lib.lib().gguf_q8_1_row_bytes(k), dtype=torch.uint8, device="cuda")
+    y_plain = torch.empty_like(y_split)
+    wd = _dev(w)
+    rc = _lib.lib().gguf_mmq(wd.data_ptr(), xd.data_ptr(), 1, ws.data_ptr(), y_plain.data_ptr(), qtype, n, k, m,
+                             torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    assert o.rel_l2(y_plain.float().cpu().numpy(), exp) <= 1e-3
+    assert o.rel_l2(y_plain.float().cpu().numpy(), y_split.float().cpu().numpy()) <= 5e-4   # fp32 sums in another order, rounded to half
+
+
 def test_mmq_engine_rejections():
     ops = _ops()
     rng = np.random.default_rng(5)

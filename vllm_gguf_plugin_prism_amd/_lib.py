@@ -33,8 +33,9 @@ _SIGNATURES = {
                              _c.c_int64, _c.c_int64, _c.c_void_p]),
     "gguf_mmq": (_c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_int, _c.c_void_p, _c.c_void_p, _c.c_int, _c.c_int64,
                             _c.c_int64, _c.c_int64, _c.c_void_p]),
+    "gguf_mmq_workspace_bytes": (_c.c_int64, [_c.c_int64, _c.c_int64, _c.c_int64]),
     "gguf_mmq_engine": (_c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_int, _c.c_void_p, _c.c_void_p, _c.c_int, _c.c_int64,
-                                   _c.c_int64, _c.c_int64, _c.c_int, _c.c_void_p]),
+                                   _c.c_int64, _c.c_int64, _c.c_int, _c.c_int64, _c.c_void_p]),
     "gguf_moe_mmq": (_c.c_int, [_c.c_void_p, _c.c_int, _c.c_void_p, _c.c_void_p, _c.c_int64, _c.c_void_p, _c.c_void_p,
                                 _c.c_void_p, _c.c_int64, _c.c_void_p, _c.c_int, _c.c_int64, _c.c_int64, _c.c_int64,
                                 _c.c_int64, _c.c_void_p]),

@@ -607,19 +607,31 @@ static bool mmq_type_ok(int type) {
 }
 
 
-int mmq_half(const void* W, const void* ws, void* Y, int dtype, int type, int M, int N, int K, hipStream_t s);  // mmq_h.hip
+// mmq_h.hip
+int mmq_half(const void* W, const void* ws, void* Y, int dtype, int type, int M, int N, int K, float* partial,
+             int64_t partial_bytes, hipStream_t s);
 bool mmq_half_supported(int type);
+int mmq_half_splits(int M, int N, int K);
 
 }  // namespace gguf
 
+// bytes of the quantized rows and their half-precision copy, rounded up so that what follows is aligned
+static int64_t mmq_rows_bytes(int64_t M, int64_t K) { return (M * (gguf::q8_row_bytes(K) + 2 * gguf::q8_half_pitch(K)) + 255) / 256 * 256; }
+
+extern "C" int64_t gguf_mmq_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+  if (M <= 0 || N <= 0 || K <= 0 || M > 0x7FFFFFF0LL || N > 0x7FFFFFF0LL || K > 0x7FFFFFF0LL) return 0;
+  const int splits = gguf::mmq_half_splits((int)M, (int)N, (int)K);
+  return mmq_rows_bytes(M, K) + (splits > 1 ? (int64_t)splits * M * N * 4 : 0);
+}
+
 extern "C" int gguf_mmq_engine(const void* W, const void* x, int xdtype, void* q8_workspace, void* Y, int type, int64_t N,
-                               int64_t K, int64_t M, int engine, gguf_stream_t stream) {
+                               int64_t K, int64_t M, int engine, int64_t workspace_bytes, gguf_stream_t stream) {
   using namespace gguf;
   const int qk = block_elems(type);
   if (qk == 0 || !mmq_type_ok(type)) return GGUF_ERR_TYPE;
   if (N < 0 || M < 0 || K <= 0 || K % qk != 0 || N > 0x7FFFFFF0LL || K > 0x7FFFFFF0LL || M > 0x7FFFFFF0LL) return GGUF_ERR_SHAPE;
   if (xdtype < 0 || xdtype > 2) return GGUF_ERR_DTYPE;
-  if (engine < GGUF_MMQ_AUTO || engine > GGUF_MMQ_HALF) return GGUF_ERR_SHAPE;
+  if (engine < GGUF_MMQ_AUTO || engine > GGUF_MMQ_HALF || workspace_bytes < 0) return GGUF_ERR_SHAPE;
   if (engine == GGUF_MMQ_HALF && !mmq_half_supported(type)) return GGUF_ERR_TYPE;
   if (engine == GGUF_MMQ_HALF && xdtype == GGUF_DTYPE_F32) return GGUF_ERR_DTYPE;
   if (N == 0 || M == 0) return GGUF_OK;
@@ -630,7 +642,9 @@ extern "C" int gguf_mmq_engine(const void* W, const void* x, int xdtype, void* q
     void* half_plane = (char*)q8_workspace + M * q8_row_bytes(K);
     const int rc = quantize_q8_1(x, xdtype, q8_workspace, M, K, s, 0, half_plane);
     if (rc != GGUF_OK) return rc;
-    return mmq_half(W, q8_workspace, Y, xdtype, type, (int)M, (int)N, (int)K, s);
+    float* partial = (float*)((char*)q8_workspace + mmq_rows_bytes(M, K));
+    const int64_t partial_bytes = workspace_bytes > mmq_rows_bytes(M, K) ? workspace_bytes - mmq_rows_bytes(M, K) : 0;
+    return mmq_half(W, q8_workspace, Y, xdtype, type, (int)M, (int)N, (int)K, partial, partial_bytes, s);
   }
   const int rc = quantize_q8_1(x, xdtype, q8_workspace, M, K, s);
   if (rc != GGUF_OK) return rc;
@@ -653,7 +667,7 @@ extern "C" int gguf_mmq_engine(const void* W, const void* x, int xdtype, void* q
 
 extern "C" int gguf_mmq(const void* W, const void* x, int xdtype, void* q8_workspace, void* Y, int type, int64_t N,
                         int64_t K, int64_t M, gguf_stream_t stream) {
-  return gguf_mmq_engine(W, x, xdtype, q8_workspace, Y, type, N, K, M, GGUF_MMQ_AUTO, stream);
+  return gguf_mmq_engine(W, x, xdtype, q8_workspace, Y, type, N, K, M, GGUF_MMQ_AUTO, 0, stream);
 }
 
 extern "C" int gguf_moe_block_size(int type) { return gguf::block_elems(type) ? 32 : 0; }

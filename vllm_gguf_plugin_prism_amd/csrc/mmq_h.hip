@@ -95,7 +95,8 @@ template <class F> struct NeedsSumPass { static constexpr bool value = F::HAS_MI
 template <class F, int WM, int WN, int TM, int TN, int OCC, typename T>
 __global__ __launch_bounds__(64 * WM * WN, OCC) void mmqh_kernel(const uint8_t* __restrict__ W, const _Float16* __restrict__ xh,
                                                                   const char* __restrict__ ws, int64_t ws_row_bytes,
-                                                                  T* __restrict__ Y, int M, int N, int K, int Kp, int dbg) {
+                                                                  T* __restrict__ Y, float* __restrict__ partial, int M, int N,
+                                                                  int K, int Kp, int dbg) {
 #ifndef GGUF_MMQ_TUNE
   (void)dbg;
 #define DBG_SKIP(bit, cond) false
@@ -219,26 +220,33 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void mmqh_kernel(const uint8_t* 
   // wave's turn, the weight block decoded from the registers loaded DG iterations ago -- issues the global loads that
   // refill those registers, and then contracts step s.  Waves whose turn it is not go straight to the matrix work, so
   // a SIMD always has one wave decoding and one multiplying.
-  fetch_a(0);
-  if (grp < nsteps) fetch_w(grp);
-  for (int s = -1; s < nsteps; ++s) {
+  // With gridDim.z > 1 the steps of K are split over that many workgroups per tile, each leaving its fp32 partial tile
+  // in `partial`; a second kernel adds them.  For shapes whose output has too few tiles to occupy the chip.
+  const int per_split = (nsteps + (int)gridDim.z - 1) / (int)gridDim.z;
+  const int t0 = (int)blockIdx.z * per_split, t1 = min(nsteps, t0 + per_split);
+  if (t0 < t1) {
+    fetch_a(t0);
+    const int first = t0 + ((grp - t0) % DG + DG) % DG;   // this group's first step
+    if (first < t1) fetch_w(first);
+  }
+  for (int s = t0 - 1; s < t1; ++s) {
     const int t = s + 1;
-    if (t < nsteps) {
+    if (t < t1) {
       write_a(t & 1);
-      if (t + 1 < nsteps) fetch_a(t + 1);
+      if (t + 1 < t1) fetch_a(t + 1);
       if (t % DG == grp) {
         decode(t, t & 1);
-        if (t + DG < nsteps) fetch_w(t + DG);
+        if (t + DG < t1) fetch_w(t + DG);
       }
     }
-    if (s >= 0) contract(s & 1, KS / 16);
+    if (s >= t0) contract(s & 1, KS / 16);
     __syncthreads();
   }
   _Float16* const xs = tiles;                // the offset pass below reuses the first buffer
   _Float16* const wt = tiles + M_T * LDH;
 
-  if constexpr (NeedsSumPass<F>::value) {
-    // Offset term.  The reference's MMQ semantics multiply the offset factor mn by the stored sum s8 of the block's
+  if constexpr (NeedsSumPass<F>::value) if (blockIdx.z == 0) {
+    // Offset term (the first split adds it).  The reference's MMQ semantics multiply the offset factor mn by the stored sum s8 of the block's
     // unquantized activations (vecdotq.cuh:61-64, 369-372) while the codes meet the quantized ones, whose sum times
     // d8 is du.  With the codes centred at C in the main loop,
     //   s * sum q x^ - mn * s8  =  s * sum (q - C) x^  +  C s (du - s8)  +  (C s - mn) s8,
@@ -297,7 +305,10 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void mmqh_kernel(const uint8_t* 
 #pragma unroll
       for (int i = 0; i < TN; ++i) {
         const int n = n_base + 32 * (wn * TN + i) + lrow;
-        if (mt < M && n < N) Y[(int64_t)mt * N + n] = from_f32<T>(acc[j][i][r] * HP_UNSCALE);
+        if (mt < M && n < N) {
+          if (partial) partial[((int64_t)blockIdx.z * M + mt) * N + n] = acc[j][i][r];
+          else Y[(int64_t)mt * N + n] = from_f32<T>(acc[j][i][r] * HP_UNSCALE);
+        }
       }
     }
   }
@@ -312,8 +323,19 @@ static int tune_dbg() {
 #endif
 }
 
+// Y = T(sum of the `splits` fp32 partial tiles / 16)
+template <typename T>
+__global__ __launch_bounds__(256) void mmqh_reduce_kernel(const float* __restrict__ partial, T* __restrict__ Y, int64_t mn, int splits) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+  if (i >= mn) return;
+  float acc = partial[i];
+  for (int z = 1; z < splits; ++z) acc += partial[z * mn + i];
+  Y[i] = from_f32<T>(acc * HP_UNSCALE);
+}
+
 template <class F, int WM, int WN, int TM, int TN, int OCC, typename T>
-static void launch_mmqh(const void* W, const void* ws, void* Y, int M, int N, int K, hipStream_t stream) {
+static void launch_mmqh(const void* W, const void* ws, void* Y, int M, int N, int K, hipStream_t stream, int splits = 1,
+                        float* partial = nullptr) {
   constexpr int M_T = 32 * WM * TM, N_T = 32 * WN * TN;
   constexpr size_t lds = (size_t)(M_T + N_T) * (64 + 8) * 2 * 2;
   auto kern = mmqh_kernel<F, WM, WN, TM, TN, OCC, T>;
@@ -325,8 +347,13 @@ static void launch_mmqh(const void* W, const void* ws, void* Y, int M, int N, in
     }
   }
   const _Float16* xh = (const _Float16*)((const char*)ws + (int64_t)M * q8_row_bytes(K));
-  hipLaunchKernelGGL(kern, dim3((N + N_T - 1) / N_T, (M + M_T - 1) / M_T), dim3(64 * WM * WN), lds, stream, (const uint8_t*)W, xh,
-                     (const char*)ws, q8_row_bytes(K), (T*)Y, M, N, K, (int)q8_kp(K), tune_dbg());
+  hipLaunchKernelGGL(kern, dim3((N + N_T - 1) / N_T, (M + M_T - 1) / M_T, splits), dim3(64 * WM * WN), lds, stream, (const uint8_t*)W,
+                     xh, (const char*)ws, q8_row_bytes(K), (T*)Y, splits > 1 ? partial : (float*)nullptr, M, N, K, (int)q8_kp(K),
+                     tune_dbg());
+  if (splits > 1) {
+    const int64_t mn = (int64_t)M * N;
+    hipLaunchKernelGGL(mmqh_reduce_kernel<T>, dim3((unsigned)((mn + 255) / 256)), dim3(256), 0, stream, partial, (T*)Y, mn, splits);
+  }
 }
 
 #ifdef GGUF_MMQ_TUNE
@@ -336,8 +363,22 @@ static int tune_cfg_h() {
 }
 #endif
 
+// Number of K splits the half engine would like for this shape (1 = none): enough to give every CU a workgroup of the
+// large tile, every split keeping at least 16 steps of 64 elements.
+int mmq_half_splits(int M, int N, int K) {
+  const int mt = M > 128 ? 256 : 128;
+  const int64_t tiles = (int64_t)((M + mt - 1) / mt) * ((N + 127) / 128);
+  if (tiles >= 180 || tiles == 0) return 1;
+  int s = (int)(256 / tiles);
+  const int by_k = (K / 64) / 16;
+  if (s > by_k) s = by_k;
+  if (s > 8) s = 8;
+  return s < 2 ? 1 : s;
+}
+
 template <class F, typename T>
-static int mmqh_typed(const void* W, const void* ws, void* Y, int M, int N, int K, hipStream_t stream) {
+static int mmqh_typed(const void* W, const void* ws, void* Y, int M, int N, int K, float* partial, int64_t partial_bytes,
+                      hipStream_t stream) {
 #ifdef GGUF_MMQ_TUNE
   switch (tune_cfg_h()) {
     case 1: launch_mmqh<F, 4, 2, 2, 2, 1, T>(W, ws, Y, M, N, K, stream); return launch_status();   // 256 x 128, 8 waves
@@ -353,8 +394,15 @@ static int mmqh_typed(const void* W, const void* ws, void* Y, int M, int N, int 
   }
 #endif
   // Tile choice: the largest tile that still gives most CUs a workgroup.  Large tiles decode each weight block for
-  // more token rows and read less LDS per MFMA; small ones fill the chip when M or N is small.
+  // more token rows and read less LDS per MFMA; small ones fill the chip when M or N is small.  When even they leave
+  // CUs idle and K is long, the large tile is kept and K is split instead, if the workspace has room for the partials.
   const auto tiles = [&](int mt, int nt) { return (int64_t)((M + mt - 1) / mt) * ((N + nt - 1) / nt); };
+  const int splits = mmq_half_splits(M, N, K);
+  if (splits > 1 && partial_bytes >= (int64_t)splits * M * N * 4) {
+    if (M > 128) launch_mmqh<F, 4, 2, 2, 2, 1, T>(W, ws, Y, M, N, K, stream, splits, partial);
+    else launch_mmqh<F, 4, 2, 1, 2, 2, T>(W, ws, Y, M, N, K, stream, splits, partial);
+    return launch_status();
+  }
   if (tiles(256, 128) >= 180) launch_mmqh<F, 4, 2, 2, 2, 1, T>(W, ws, Y, M, N, K, stream);        // 256 x 128, 8 waves
   else if (tiles(128, 128) >= 180) launch_mmqh<F, 4, 2, 1, 2, 2, T>(W, ws, Y, M, N, K, stream);   // 128 x 128, 8 waves
   else if (tiles(128, 64) >= 180) launch_mmqh<F, 2, 2, 2, 1, 2, T>(W, ws, Y, M, N, K, stream);    // 128 x 64, 4 waves
@@ -363,29 +411,31 @@ static int mmqh_typed(const void* W, const void* ws, void* Y, int M, int N, int 
 }
 
 template <class F>
-static int mmqh_fmt(const void* W, const void* ws, void* Y, int dtype, int M, int N, int K, hipStream_t s) {
-  if (dtype == GGUF_DTYPE_F16) return mmqh_typed<F, _Float16>(W, ws, Y, M, N, K, s);
+static int mmqh_fmt(const void* W, const void* ws, void* Y, int dtype, int M, int N, int K, float* partial, int64_t partial_bytes,
+                    hipStream_t s) {
+  if (dtype == GGUF_DTYPE_F16) return mmqh_typed<F, _Float16>(W, ws, Y, M, N, K, partial, partial_bytes, s);
 #ifndef GGUF_MMQ_TUNE
-  if (dtype == GGUF_DTYPE_BF16) return mmqh_typed<F, bf16_t>(W, ws, Y, M, N, K, s);
+  if (dtype == GGUF_DTYPE_BF16) return mmqh_typed<F, bf16_t>(W, ws, Y, M, N, K, partial, partial_bytes, s);
 #endif
   return GGUF_ERR_DTYPE;
 }
 
 // The half-MFMA engine for one call; the workspace already holds the quantized rows and, behind them, their half plane.
-int mmq_half(const void* W, const void* ws, void* Y, int dtype, int type, int M, int N, int K, hipStream_t s) {
+int mmq_half(const void* W, const void* ws, void* Y, int dtype, int type, int M, int N, int K, float* partial,
+             int64_t partial_bytes, hipStream_t s) {
   switch (type) {
 #ifndef GGUF_MMQ_TUNE
-    case T_Q4_0: return mmqh_fmt<MQ4_0>(W, ws, Y, dtype, M, N, K, s);
-    case T_Q5_0: return mmqh_fmt<MQ5_0>(W, ws, Y, dtype, M, N, K, s);
-    case T_Q8_0: return mmqh_fmt<MQ8_0>(W, ws, Y, dtype, M, N, K, s);
-    case T_Q2_K: return mmqh_fmt<MQ2_K>(W, ws, Y, dtype, M, N, K, s);
-    case T_Q3_K: return mmqh_fmt<MQ3_K>(W, ws, Y, dtype, M, N, K, s);
-    case T_Q4_K: return mmqh_fmt<MQ4_K>(W, ws, Y, dtype, M, N, K, s);
-    case T_Q5_K: return mmqh_fmt<MQ5_K>(W, ws, Y, dtype, M, N, K, s);
-    case T_IQ4_XS: return mmqh_fmt<MIQ4_XS>(W, ws, Y, dtype, M, N, K, s);
-    case T_IQ2_XXS: return mmqh_fmt<MIQ2_XXS>(W, ws, Y, dtype, M, N, K, s);
+    case T_Q4_0: return mmqh_fmt<MQ4_0>(W, ws, Y, dtype, M, N, K, partial, partial_bytes, s);
+    case T_Q5_0: return mmqh_fmt<MQ5_0>(W, ws, Y, dtype, M, N, K, partial, partial_bytes, s);
+    case T_Q8_0: return mmqh_fmt<MQ8_0>(W, ws, Y, dtype, M, N, K, partial, partial_bytes, s);
+    case T_Q2_K: return mmqh_fmt<MQ2_K>(W, ws, Y, dtype, M, N, K, partial, partial_bytes, s);
+    case T_Q3_K: return mmqh_fmt<MQ3_K>(W, ws, Y, dtype, M, N, K, partial, partial_bytes, s);
+    case T_Q4_K: return mmqh_fmt<MQ4_K>(W, ws, Y, dtype, M, N, K, partial, partial_bytes, s);
+    case T_Q5_K: return mmqh_fmt<MQ5_K>(W, ws, Y, dtype, M, N, K, partial, partial_bytes, s);
+    case T_IQ4_XS: return mmqh_fmt<MIQ4_XS>(W, ws, Y, dtype, M, N, K, partial, partial_bytes, s);
+    case T_IQ2_XXS: return mmqh_fmt<MIQ2_XXS>(W, ws, Y, dtype, M, N, K, partial, partial_bytes, s);
 #endif
-    case T_Q6_K: return mmqh_fmt<MQ6_K>(W, ws, Y, dtype, M, N, K, s);
+    case T_Q6_K: return mmqh_fmt<MQ6_K>(W, ws, Y, dtype, M, N, K, partial, partial_bytes, s);
   }
   return GGUF_ERR_TYPE;
 }

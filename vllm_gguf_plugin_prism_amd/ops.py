@@ -118,9 +118,10 @@ def ggml_mul_mat_a8(W: torch.Tensor, X: torch.Tensor, quant_type: int, row: int,
     vecs, col = X.shape
     with torch.cuda.device(X.device):
         out = torch.empty((vecs, row), dtype=X.dtype, device=W.device)
-        ws = _workspace(X, vecs, col)
+        nbytes = max(_lib.lib().gguf_mmq_workspace_bytes(vecs, row, col), vecs * _lib.lib().gguf_q8_1_row_bytes(col), 16)
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=X.device)
         rc = _lib.lib().gguf_mmq_engine(W.data_ptr(), X.data_ptr(), _code(X.dtype), ws.data_ptr(), out.data_ptr(),
-                                        int(quant_type), row, col, vecs, MMQ_ENGINES[engine], _stream(X))
+                                        int(quant_type), row, col, vecs, MMQ_ENGINES[engine], nbytes, _stream(X))
     _lib.check(rc, "ggml_mul_mat_a8")
     return out
 
