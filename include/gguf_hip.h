@@ -105,6 +105,16 @@ int64_t gguf_mmq_workspace_bytes(int64_t M, int64_t N, int64_t K);
 int gguf_mmq_engine(const void* W, const void* x, int xdtype, void* q8_workspace, void* Y, int type, int64_t N, int64_t K,
                     int64_t M, int engine, int64_t workspace_bytes, gguf_stream_t stream);
 
+/* Y[M,N] = X[M,K] . dequant(W[N,K])^T with the activations as they are (no q8_1 quantisation): one GEMM on
+ * half-precision MFMA that decodes the packed blocks on the fly instead of the reference's fallback for formats and
+ * batch sizes without an a8 kernel, ggml_dequantize followed by x @ weight.T (quantization/linear.py:50-58,
+ * diffusion_config.py:21-30), which writes and re-reads the dense weights.  The weights take the half-precision
+ * values the reference's dequantize kernels produce; X is converted to half.  X / Y dtype: fp16 or bf16.  Types: the
+ * twelve standard and K formats plus IQ4_XS and IQ2_XXS.  Workspace: gguf_mmq_workspace_bytes(M, N, K) (or at least
+ * M * gguf_q8_1_row_bytes(K), without the K split for small outputs). */
+int gguf_dequant_gemm(const void* W, const void* x, int xdtype, void* workspace, void* Y, int type, int64_t N, int64_t K,
+                      int64_t M, int64_t workspace_bytes, gguf_stream_t stream);
+
 /* Grouped (MoE) variant: for every sorted slot s with p = sorted_token_ids[s] < tokens*top_k,
  * Y[p,:] = q8_1(X[p / top_k,:]) . W[expert_ids[s / block],:,:]^T.  Rows of Y that no slot names are zero.
  * Replaces ggml_moe_a8 (gguf_kernel.cu:292-393, moe.cuh:5-739).  `block` must equal

@@ -124,6 +124,47 @@ def test_mmq_half_engine_split_k(qtype, m):
     assert o.rel_l2(y_plain.float().cpu().numpy(), y_split.float().cpu().numpy()) <= 5e-4   # fp32 sums in another order, rounded to half
 
 
+@pytest.mark.parametrize("dt", ["f16", "bf16"])
+@pytest.mark.parametrize("qtype", MMQ_TYPES)
+def test_dequant_gemm_is_the_dense_product(qtype, dt):
+    """ggml_dequant_gemm = x @ ggml_dequantize(W).T with unquantized activations (the reference's fallback path,
+    linear.py:50-58) in one kernel.  Against the product formed in fp32 from the library's own bit-exact half-precision
+    dequantization, what remains is the rounding of the result (2.1e-4 for fp16) and, for formats whose scale product the
+    kernel rounds before the code is applied, one more half rounding of the weight (bf16 activations add nothing: they
+    are half-representable in this range); against the fp32 oracle the half-precision weights show as well."""
+    ops = _ops()
+    rng = np.random.default_rng(1500 + qtype)
+    qk = o.QUANT_SIZES[qtype][0]
+    for m, n, k in [(160, 384, 2048), (7, 130, 736 if qk == 32 else 768), (300, 6400, 256 if qk == 256 else 352)]:
+        w = o.make_weights(rng, qtype, n, k)
+        wd = _dev(w)
+        xd, xv = _x(rng, m, k, dt)
+        y = ops.ggml_dequant_gemm(wd, xd, qtype, n)
+        assert y.shape == (m, n) and y.dtype == TORCH_DT[dt]
+        dense = ops.ggml_dequantize(wd, qtype, n, k, torch.float16).float()
+        ref = (xd.float() @ dense.T).cpu().numpy()
+        got = y.float().cpu().numpy()
+        assert o.rel_l2(got, ref) <= (6e-4 if dt == "f16" else 3e-3), (o.TYPE_NAMES[qtype], m, n, k, o.rel_l2(got, ref))
+        assert o.rel_l2(got, o.mul_mat_f32(w, xv, qtype, n)) <= (1e-3 if dt == "f16" else 4e-3)
+
+
+def test_dequant_gemm_split_k_and_rejections():
+    ops = _ops()
+    rng = np.random.default_rng(1600)
+    m, n, k = 200, 250, 4096                      # few tiles, long K: the K split engages
+    w = o.make_weights(rng, o.IQ2_XXS, n, k)
+    xd, xv = _x(rng, m, k, "f16")
+    y = ops.ggml_dequant_gemm(_dev(w), xd, o.IQ2_XXS, n)
+    assert o.rel_l2(y.float().cpu().numpy(), o.mul_mat_f32(w, xv, o.IQ2_XXS, n)) <= 1e-3
+    x32, _ = _x(rng, 4, 256, "f32")
+    w6 = _dev(o.make_weights(rng, o.Q6_K, 64, 256))
+    with pytest.raises(ValueError):
+        ops.ggml_dequant_gemm(w6, x32, o.Q6_K, 64)
+    wi = _dev(o.make_weights(rng, o.IQ3_S, 64, 256))
+    with pytest.raises(NotImplementedError):
+        ops.ggml_dequant_gemm(wi, xd[:4, :256].contiguous(), o.IQ3_S, 64)
+
+
 def test_mmq_engine_rejections():
     ops = _ops()
     rng = np.random.default_rng(5)

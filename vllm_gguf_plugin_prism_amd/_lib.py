@@ -36,6 +36,8 @@ _SIGNATURES = {
     "gguf_mmq_workspace_bytes": (_c.c_int64, [_c.c_int64, _c.c_int64, _c.c_int64]),
     "gguf_mmq_engine": (_c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_int, _c.c_void_p, _c.c_void_p, _c.c_int, _c.c_int64,
                                    _c.c_int64, _c.c_int64, _c.c_int, _c.c_int64, _c.c_void_p]),
+    "gguf_dequant_gemm": (_c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_int, _c.c_void_p, _c.c_void_p, _c.c_int, _c.c_int64,
+                                     _c.c_int64, _c.c_int64, _c.c_int64, _c.c_void_p]),
     "gguf_moe_mmq": (_c.c_int, [_c.c_void_p, _c.c_int, _c.c_void_p, _c.c_void_p, _c.c_int64, _c.c_void_p, _c.c_void_p,
                                 _c.c_void_p, _c.c_int64, _c.c_void_p, _c.c_int, _c.c_int64, _c.c_int64, _c.c_int64,
                                 _c.c_int64, _c.c_void_p]),

@@ -1,367 +1,8 @@
-// Prefill-path GEMM on packed GGUF weights with q8_1 activations, on gfx950 half-precision MFMA.
-//
-//   Y[m, n] = sum_k  xh[m, k] * wh[n, k]        xh = RN16(d8 * xq)   the q8_1 activations, dequantized
-//                                               wh = RN16(RN16(dw) * wq)   the GGUF weights, dequantized
-//
-// The int8 engine (mmq.hip) keeps the block scales out of the matrix product and pays two to four vector-ALU
-// instructions per result and 32-element block for it, which on this chip cannot overlap the MFMAs of the same
-// SIMD.  Here both operands carry their scales into the product, so the K loop is MFMA and LDS reads only; the
-// vector ALU decodes every weight block once per workgroup and step (about 2.5 instructions per weight), amortised
-// over the M_T token rows of the tile.  v_mfma_f32_32x32x16_f16 runs at half the int8 rate, yet the loop is more
-// than twice as fast because nothing else is left in it.
-//
-// Arithmetic: the products of half operands are exact in the MFMA's fp32 accumulation, so the only differences from
-// the int8 engine are the roundings of the two operands to half precision (relative 2^-12 each, 2^-11 for the
-// weights' two roundings).  That is below the rounding of a half or bfloat16 result; fp32 results stay on the int8 engine.
-// Weights are staged times 2^4 and the result scaled back, which keeps small weight scales out of the half
-// subnormals; weights of magnitude 4094 and more overflow.
-//
-// Offset terms: formats whose offset multiplies the sum of the activation quants (Q2_K) fold it into wh.  Formats
-// whose offset multiplies the stored block sum of the unquantized activations (Q4_0, Q4_K, Q5_K in the reference's
-// MMQ semantics, vecdotq.cuh:61-64,369-372) centre their codes and add the rest in a second, 16 times shorter loop
-// over the blocks (see there).
-#include "mmq_formats.h"
+// The a8 prefill GEMM on the half-precision MFMA engine: q8_1-quantized activations times GGUF weights, the
+// reference's ggml_mul_mat_a8 semantics (gguf_kernel.cu:220-290) to within the operand roundings.  Kernel: mmq_h_core.h.
+#include "mmq_h_core.h"
 
 namespace gguf {
-
-typedef _Float16 v8h __attribute__((ext_vector_type(8)));
-typedef _Float16 v2h __attribute__((ext_vector_type(2)));
-typedef float v16f __attribute__((ext_vector_type(16)));
-
-typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));   // a plain vector: stays in registers where HIP's uint4 struct may not
-typedef u32x4 __attribute__((address_space(1))) global_u32x4;  // a load through an integer address must name its address space
-
-constexpr float HP_SCALE = 16.0f, HP_UNSCALE = 0.0625f;
-
-// How a format's codes reach half precision.  A byte b becomes the half 1024 + b by placing it under the exponent
-// byte 0x64, and subtracting 1024 + BIAS leaves the code exactly: formats with unsigned codes (BIAS = the code's
-// zero point) skip their own recentring, signed int8 codes are flipped to b = code + 128 first.
-template <class F> struct HalfCodes {
-  static constexpr bool FLIP = true;
-  static constexpr int BIAS = 128;
-  static __device__ __forceinline__ void unpack(const typename F::Raw& r, int kb, uint32_t (&q)[8], float& s0, float& s1, float& mn, float& mn1) {
-    F::unpack(r, kb, q, s0, s1, mn, mn1);
-  }
-};
-template <class F, int B> struct UnsignedCodes {
-  static constexpr bool FLIP = false;
-  static constexpr int BIAS = B;
-  static __device__ __forceinline__ void unpack(const typename F::Raw& r, int kb, uint32_t (&q)[8], float& s0, float& s1, float& mn, float& mn1) {
-    F::unpack(r, kb, q, s0, s1, mn, mn1);
-  }
-};
-template <class F, int B> struct RecentredCodes {
-  static constexpr bool FLIP = false;
-  static constexpr int BIAS = B;
-  static __device__ __forceinline__ void unpack(const typename F::Raw& r, int kb, uint32_t (&q)[8], float& s0, float& s1, float& mn, float& mn1) {
-    F::template unpack<false>(r, kb, q, s0, s1, mn, mn1);
-  }
-};
-template <> struct HalfCodes<MQ4_0> : UnsignedCodes<MQ4_0, MQ4_0::CENTRE> {};   // codes centred; the offset pass adds what that leaves
-template <> struct HalfCodes<MQ4_K> : UnsignedCodes<MQ4_K, MQ4_K::CENTRE> {};
-template <> struct HalfCodes<MQ5_K> : UnsignedCodes<MQ5_K, MQ5_K::CENTRE> {};
-template <> struct HalfCodes<MQ2_K> : UnsignedCodes<MQ2_K, 0> {};
-template <> struct HalfCodes<MQ6_K> : RecentredCodes<MQ6_K, 32> {};
-template <> struct HalfCodes<MQ3_K> : RecentredCodes<MQ3_K, 4> {};
-template <> struct HalfCodes<MQ5_0> : RecentredCodes<MQ5_0, 16> {};
-
-// 32 codes (element order, four per dword) -> 32 halfs  (code - BIAS) * s - m, with s and m per 16 elements
-template <bool FLIP, int BIAS, bool WITH_MIN>
-__device__ __forceinline__ void codes_to_half(const uint32_t (&q)[8], float s0, float s1, float m0, float m1, uint4 (&out)[4]) {
-  const _Float16 h0 = (_Float16)(s0 * HP_SCALE), h1 = (_Float16)(s1 * HP_SCALE);
-  const _Float16 g0 = (_Float16)(m0 * HP_SCALE), g1 = (_Float16)(m1 * HP_SCALE);
-  const v2h bias = {(_Float16)(1024.0f + BIAS), (_Float16)(1024.0f + BIAS)};
-  uint32_t w[16];
-#pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const uint32_t u = FLIP ? q[i] ^ 0x80808080u : q[i];
-    const uint32_t lo = __builtin_amdgcn_perm(0x64646464u, u, 0x04010400u);
-    const uint32_t hi = __builtin_amdgcn_perm(0x64646464u, u, 0x04030402u);
-    const _Float16 s = i < 4 ? h0 : h1, m = i < 4 ? g0 : g1;
-    const v2h sc = {s, s}, mn = {m, m};
-    v2h a = __builtin_bit_cast(v2h, lo) - bias, b = __builtin_bit_cast(v2h, hi) - bias;
-    if (WITH_MIN) { a = a * sc - mn; b = b * sc - mn; }
-    else { a = a * sc; b = b * sc; }
-    w[2 * i] = __builtin_bit_cast(uint32_t, a);
-    w[2 * i + 1] = __builtin_bit_cast(uint32_t, b);
-  }
-#pragma unroll
-  for (int i = 0; i < 4; ++i) out[i] = make_uint4(w[4 * i], w[4 * i + 1], w[4 * i + 2], w[4 * i + 3]);
-}
-
-// whether the format's offset term needs the second loop
-template <class F> struct NeedsSumPass { static constexpr bool value = F::HAS_MIN && !F::MIN16; };
-
-template <class F, int WM, int WN, int TM, int TN, int OCC, typename T>
-__global__ __launch_bounds__(64 * WM * WN, OCC) void mmqh_kernel(const uint8_t* __restrict__ W, const _Float16* __restrict__ xh,
-                                                                  const char* __restrict__ ws, int64_t ws_row_bytes,
-                                                                  T* __restrict__ Y, float* __restrict__ partial, int M, int N,
-                                                                  int K, int Kp, int dbg) {
-#ifndef GGUF_MMQ_TUNE
-  (void)dbg;
-#define DBG_SKIP(bit, cond) false
-#else
-#define DBG_SKIP(bit, cond) ((dbg & (bit)) && (cond))
-#endif
-  constexpr int NT = 64 * WM * WN;
-  constexpr int KS = 64;                 // elements of K per step
-  constexpr int KB = KS / 32;            // 32-blocks per step
-  constexpr int GR = KS / 8;             // 16-byte granules (8 halfs) per activation row and step
-  constexpr int LDH = KS + 8;            // LDS row pitch in halfs: a 16-byte skew spreads 8 consecutive rows over all banks
-  constexpr int M_T = 32 * WM * TM, N_T = 32 * WN * TN;
-  constexpr int PAIRS = N_T * KB;        // (weight row, 32-block) pairs to decode per step, one thread each
-  static_assert(NT % PAIRS == 0 && (M_T * GR) % NT == 0, "tile and workgroup sizes must divide evenly");
-  constexpr int DG = NT / PAIRS;         // decode groups: group g decodes the steps t with t % DG == g
-  constexpr int AQ = M_T * GR / NT;      // activation granules per thread and step
-  constexpr int TILE = (M_T + N_T) * LDH;  // halfs per buffer
-  extern __shared__ __align__(16) char smem[];
-  _Float16* const tiles = (_Float16*)smem;   // two buffers of { activations [M_T][LDH], decoded weights [N_T][LDH] }
-
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int wm = wave / WN, wn = wave % WN;
-  const int lrow = lane & 31, lhalf = lane >> 5;
-  const int m_base = blockIdx.y * M_T, n_base = blockIdx.x * N_T;
-  const int64_t rowbytes = (int64_t)(K / F::QK) * F::BS;
-  const int nkb_total = K >> 5;
-  const int nsteps = (K + KS - 1) / KS;
-
-  const _Float16* aq_src[AQ];
-#pragma unroll
-  for (int i = 0; i < AQ; ++i) {
-    const int p = tid + NT * i, m = p / GR, g = p % GR;
-    aq_src[i] = xh + (int64_t)min(m_base + m, M - 1) * (Kp + 128) + 8 * g;   // rows past M repeat the last row; never stored
-  }
-  const int grp = tid / PAIRS, n_dec = (tid % PAIRS) / KB, kb_dec = tid % KB;
-  const uint8_t* const w_row = W + (int64_t)min(n_base + n_dec, N - 1) * rowbytes;
-
-  u32x4 r_aq[AQ];
-  typename F::Raw r_w;
-
-  auto fetch_a = [&](int t) {
-    if (DBG_SKIP(2, t > 0)) return;
-#pragma unroll
-    for (int i = 0; i < AQ; ++i) r_aq[i] = *(const u32x4*)(aq_src[i] + t * KS);  // rows are padded with zeros to a multiple of 512
-  };
-  auto write_a = [&](int buf) {
-    _Float16* xs = tiles + buf * TILE;
-#pragma unroll
-    for (int i = 0; i < AQ; ++i) {
-      const int p = tid + NT * i;
-      *(u32x4*)(xs + (p / GR) * LDH + 8 * (p % GR)) = r_aq[i];
-    }
-  };
-  auto fetch_w = [&](int t) {
-    if (DBG_SKIP(8, t >= DG)) return;
-    r_w = F::fetch(w_row, min(t * KB + kb_dec, nkb_total - 1));  // clamped: a block past K is re-read and decoded to zeros
-  };
-  auto decode = [&](int t, int buf) {
-    if (DBG_SKIP(4, t >= DG)) return;
-    _Float16* wt = tiles + buf * TILE + M_T * LDH;
-    const int kb = t * KB + kb_dec;
-    uint32_t q[8];
-    float s0, s1, mn = 0.0f, mn1 = 0.0f;
-    HalfCodes<F>::unpack(r_w, kb, q, s0, s1, mn, mn1);
-    if (kb >= nkb_total) s0 = s1 = mn = mn1 = 0.0f;
-    uint4 h[4];
-    codes_to_half<HalfCodes<F>::FLIP, HalfCodes<F>::BIAS, F::MIN16>(q, s0, s1, mn, mn1, h);
-#pragma unroll
-    for (int j = 0; j < 4; ++j) *(uint4*)(wt + n_dec * LDH + 32 * kb_dec + 8 * j) = h[j];
-  };
-
-  v16f acc[TM][TN];
-#pragma unroll
-  for (int j = 0; j < TM; ++j)
-#pragma unroll
-    for (int i = 0; i < TN; ++i)
-#pragma unroll
-      for (int r = 0; r < 16; ++r) acc[j][i][r] = 0.0f;
-
-  // One step of K from buffer `buf`.  All operand reads of the step are issued before its first MFMA: every wave then
-  // keeps the LDS pipe busy for the whole step, and the matrix work of one wave runs under the reads of the other
-  // wave on its SIMD.
-  auto contract = [&](int buf, int slices) {
-    if (DBG_SKIP(16, true)) return;
-    const _Float16* xs = tiles + buf * TILE;
-    const _Float16* wt = xs + M_T * LDH;
-    v8h af[KS / 16][TM], bf[KS / 16][TN];
-#pragma unroll
-    for (int kk = 0; kk < KS / 16; ++kk) {
-#pragma unroll
-      for (int j = 0; j < TM; ++j) af[kk][j] = *(const v8h*)(xs + (32 * (wm * TM + j) + lrow) * LDH + 16 * kk + 8 * lhalf);
-#pragma unroll
-      for (int i = 0; i < TN; ++i) bf[kk][i] = *(const v8h*)(wt + (32 * (wn * TN + i) + lrow) * LDH + 16 * kk + 8 * lhalf);
-    }
-#pragma unroll
-    for (int kk = 0; kk < KS / 16; ++kk) {
-      if (kk >= slices) break;
-#pragma unroll
-      for (int j = 0; j < TM; ++j)
-#pragma unroll
-        for (int i = 0; i < TN; ++i) {
-          acc[j][i] = __builtin_amdgcn_mfma_f32_32x32x16_f16(af[kk][j], bf[kk][i], acc[j][i], 0, 0, 0);
-        }
-    }
-    // Instruction order for the scheduler: the first slice's operand reads, then one operand read behind every MFMA
-    // until the reads run out.  An MFMA occupies the matrix unit for 32 cycles but issues in 4, so the reads of the
-    // coming slices issue and complete under the matrix work instead of in front of it.
-    if (slices == KS / 16) {
-      constexpr int READS = (KS / 16) * (TM + TN), MFMAS = (KS / 16) * TM * TN, LEAD = TM + TN;
-      __builtin_amdgcn_sched_group_barrier(0x100, LEAD, 0);          // DS reads
-#pragma unroll
-      for (int i = 0; i < MFMAS; ++i) {
-        __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);           // one MFMA
-        if (i < READS - LEAD) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-      }
-    }
-  };
-
-  // Software pipeline over the steps, two LDS buffers, one barrier per step.  In iteration s every wave first moves
-  // step s+1 into the other buffer -- the activations from the registers loaded one iteration ago, and, if it is this
-  // wave's turn, the weight block decoded from the registers loaded DG iterations ago -- issues the global loads that
-  // refill those registers, and then contracts step s.  Waves whose turn it is not go straight to the matrix work, so
-  // a SIMD always has one wave decoding and one multiplying.
-  // With gridDim.z > 1 the steps of K are split over that many workgroups per tile, each leaving its fp32 partial tile
-  // in `partial`; a second kernel adds them.  For shapes whose output has too few tiles to occupy the chip.
-  const int per_split = (nsteps + (int)gridDim.z - 1) / (int)gridDim.z;
-  const int t0 = (int)blockIdx.z * per_split, t1 = min(nsteps, t0 + per_split);
-  if (t0 < t1) {
-    fetch_a(t0);
-    const int first = t0 + ((grp - t0) % DG + DG) % DG;   // this group's first step
-    if (first < t1) fetch_w(first);
-  }
-  for (int s = t0 - 1; s < t1; ++s) {
-    const int t = s + 1;
-    if (t < t1) {
-      write_a(t & 1);
-      if (t + 1 < t1) fetch_a(t + 1);
-      if (t % DG == grp) {
-        decode(t, t & 1);
-        if (t + DG < t1) fetch_w(t + DG);
-      }
-    }
-    if (s >= t0) contract(s & 1, KS / 16);
-    __syncthreads();
-  }
-  _Float16* const xs = tiles;                // the offset pass below reuses the first buffer
-  _Float16* const wt = tiles + M_T * LDH;
-
-  if constexpr (NeedsSumPass<F>::value) if (blockIdx.z == 0) {
-    // Offset term (the first split adds it).  The reference's MMQ semantics multiply the offset factor mn by the stored sum s8 of the block's
-    // unquantized activations (vecdotq.cuh:61-64, 369-372) while the codes meet the quantized ones, whose sum times
-    // d8 is du.  With the codes centred at C in the main loop,
-    //   s * sum q x^ - mn * s8  =  s * sum (q - C) x^  +  C s (du - s8)  +  (C s - mn) s8,
-    // what remains is a short second product with two columns per 32-block: A = (du - s8, s8), B = (C s, C s - mn).
-    // du - s8 is the small rounding residue of the block and C s - mn is small for blocks spread about their centre,
-    // so the half-precision operands of this product cost far less accuracy than an uncentred main loop would.
-    constexpr int SB = KS / 2;                      // blocks per step of this loop
-    const float* as_src[AQ];
-#pragma unroll
-    for (int i = 0; i < AQ; ++i) {
-      const int p = tid + NT * i, m = p / GR, g = p % GR;
-      as_src[i] = (const float*)(ws + (int64_t)min(m_base + m, M - 1) * ws_row_bytes + Kp) + Kp / 32 + 4 * g;  // s8 plane; du follows
-    }
-    constexpr int UNITS = N_T * (SB / 8);           // (weight row, group of 8 blocks) pairs per step
-    constexpr int WB = (UNITS + NT - 1) / NT;
-    for (int b0 = 0; b0 < nkb_total; b0 += SB) {
-      __syncthreads();
-#pragma unroll
-      for (int i = 0; i < AQ; ++i) {
-        const int p = tid + NT * i, m = p / GR, g = p % GR;
-        v8h o;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          const bool in = b0 + 4 * g + e < nkb_total;
-          const float s8 = in ? as_src[i][b0 + e] : 0.0f, du = in ? as_src[i][b0 + e + Kp / 32] : 0.0f;
-          o[2 * e] = (_Float16)(du - s8);
-          o[2 * e + 1] = (_Float16)s8;
-        }
-        *(v8h*)(xs + m * LDH + 8 * g) = o;
-      }
-#pragma unroll
-      for (int i = 0; i < WB; ++i) {
-        const int p = tid + NT * i, n = p / (SB / 8), q = p % (SB / 8);
-        if (p >= UNITS) continue;
-        float cs[8], cm[8];
-        F::offs8(W + (int64_t)min(n_base + n, N - 1) * rowbytes, b0 / 8 + q, nkb_total, cs, cm);
-        v8h o0, o1;
-#pragma unroll
-        for (int e = 0; e < 4; ++e) {
-          o0[2 * e] = (_Float16)(cs[e] * HP_SCALE);     o0[2 * e + 1] = (_Float16)(cm[e] * HP_SCALE);
-          o1[2 * e] = (_Float16)(cs[4 + e] * HP_SCALE); o1[2 * e + 1] = (_Float16)(cm[4 + e] * HP_SCALE);
-        }
-        *(v8h*)(wt + n * LDH + 16 * q) = o0;
-        *(v8h*)(wt + n * LDH + 16 * q + 8) = o1;
-      }
-      __syncthreads();
-      contract(0, (2 * min(nkb_total - b0, SB) + 15) / 16);
-    }
-  }
-
-#pragma unroll
-  for (int j = 0; j < TM; ++j) {
-#pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const int mt = m_base + 32 * (wm * TM + j) + 8 * (r >> 2) + 4 * lhalf + (r & 3);
-#pragma unroll
-      for (int i = 0; i < TN; ++i) {
-        const int n = n_base + 32 * (wn * TN + i) + lrow;
-        if (mt < M && n < N) {
-          if (partial) partial[((int64_t)blockIdx.z * M + mt) * N + n] = acc[j][i][r];
-          else Y[(int64_t)mt * N + n] = from_f32<T>(acc[j][i][r] * HP_UNSCALE);
-        }
-      }
-    }
-  }
-}
-
-static int tune_dbg() {
-#ifdef GGUF_MMQ_TUNE
-  static const int v = [] { const char* e = getenv("GGUF_MMQH_DBG"); return e ? atoi(e) : 0; }();
-  return v;
-#else
-  return 0;
-#endif
-}
-
-// Y = T(sum of the `splits` fp32 partial tiles / 16)
-template <typename T>
-__global__ __launch_bounds__(256) void mmqh_reduce_kernel(const float* __restrict__ partial, T* __restrict__ Y, int64_t mn, int splits) {
-  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (i >= mn) return;
-  float acc = partial[i];
-  for (int z = 1; z < splits; ++z) acc += partial[z * mn + i];
-  Y[i] = from_f32<T>(acc * HP_UNSCALE);
-}
-
-template <class F, int WM, int WN, int TM, int TN, int OCC, typename T>
-static void launch_mmqh(const void* W, const void* ws, void* Y, int M, int N, int K, hipStream_t stream, int splits = 1,
-                        float* partial = nullptr) {
-  constexpr int M_T = 32 * WM * TM, N_T = 32 * WN * TN;
-  constexpr size_t lds = (size_t)(M_T + N_T) * (64 + 8) * 2 * 2;
-  auto kern = mmqh_kernel<F, WM, WN, TM, TN, OCC, T>;
-  if constexpr (lds > 65536) {
-    static bool configured = false;  // opt in to > 64 KB of dynamic LDS once per instantiation
-    if (!configured) {
-      (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-      configured = true;
-    }
-  }
-  const _Float16* xh = (const _Float16*)((const char*)ws + (int64_t)M * q8_row_bytes(K));
-  hipLaunchKernelGGL(kern, dim3((N + N_T - 1) / N_T, (M + M_T - 1) / M_T, splits), dim3(64 * WM * WN), lds, stream, (const uint8_t*)W,
-                     xh, (const char*)ws, q8_row_bytes(K), (T*)Y, splits > 1 ? partial : (float*)nullptr, M, N, K, (int)q8_kp(K),
-                     tune_dbg());
-  if (splits > 1) {
-    const int64_t mn = (int64_t)M * N;
-    hipLaunchKernelGGL(mmqh_reduce_kernel<T>, dim3((unsigned)((mn + 255) / 256)), dim3(256), 0, stream, partial, (T*)Y, mn, splits);
-  }
-}
-
-#ifdef GGUF_MMQ_TUNE
-static int tune_cfg_h() {
-  static const int v = [] { const char* e = getenv("GGUF_MMQH_CFG"); return e ? atoi(e) : 0; }();
-  return v;
-}
-#endif
 
 // Number of K splits the half engine would like for this shape (1 = none): enough to give every CU a workgroup of the
 // large tile, every split keeping at least 16 steps of 64 elements.
@@ -376,46 +17,12 @@ int mmq_half_splits(int M, int N, int K) {
   return s < 2 ? 1 : s;
 }
 
-template <class F, typename T>
-static int mmqh_typed(const void* W, const void* ws, void* Y, int M, int N, int K, float* partial, int64_t partial_bytes,
-                      hipStream_t stream) {
-#ifdef GGUF_MMQ_TUNE
-  switch (tune_cfg_h()) {
-    case 1: launch_mmqh<F, 4, 2, 2, 2, 1, T>(W, ws, Y, M, N, K, stream); return launch_status();   // 256 x 128, 8 waves
-    case 2: launch_mmqh<F, 2, 2, 2, 2, 1, T>(W, ws, Y, M, N, K, stream); return launch_status();   // 128 x 128, 4 waves
-    case 3: launch_mmqh<F, 2, 4, 2, 2, 1, T>(W, ws, Y, M, N, K, stream); return launch_status();   // 128 x 256, 8 waves
-    case 4: launch_mmqh<F, 2, 2, 4, 2, 1, T>(W, ws, Y, M, N, K, stream); return launch_status();   // 256 x 128, 4 waves
-    case 5: launch_mmqh<F, 2, 2, 2, 1, 2, T>(W, ws, Y, M, N, K, stream); return launch_status();   // 128 x 64, 4 waves
-    case 6: launch_mmqh<F, 2, 4, 2, 1, 2, T>(W, ws, Y, M, N, K, stream); return launch_status();   // 128 x 128, 8 waves (64 x 32 each)
-    case 7: launch_mmqh<F, 2, 2, 1, 1, 4, T>(W, ws, Y, M, N, K, stream); return launch_status();   // 64 x 64, 4 waves
-    case 8: launch_mmqh<F, 4, 2, 1, 2, 2, T>(W, ws, Y, M, N, K, stream); return launch_status();   // 128 x 128, 8 waves (32 x 64 each)
-    case 9: launch_mmqh<F, 4, 2, 2, 4, 1, T>(W, ws, Y, M, N, K, stream); return launch_status();   // 256 x 256, 8 waves
-    default: break;
-  }
-#endif
-  // Tile choice: the largest tile that still gives most CUs a workgroup.  Large tiles decode each weight block for
-  // more token rows and read less LDS per MFMA; small ones fill the chip when M or N is small.  When even they leave
-  // CUs idle and K is long, the large tile is kept and K is split instead, if the workspace has room for the partials.
-  const auto tiles = [&](int mt, int nt) { return (int64_t)((M + mt - 1) / mt) * ((N + nt - 1) / nt); };
-  const int splits = mmq_half_splits(M, N, K);
-  if (splits > 1 && partial_bytes >= (int64_t)splits * M * N * 4) {
-    if (M > 128) launch_mmqh<F, 4, 2, 2, 2, 1, T>(W, ws, Y, M, N, K, stream, splits, partial);
-    else launch_mmqh<F, 4, 2, 1, 2, 2, T>(W, ws, Y, M, N, K, stream, splits, partial);
-    return launch_status();
-  }
-  if (tiles(256, 128) >= 180) launch_mmqh<F, 4, 2, 2, 2, 1, T>(W, ws, Y, M, N, K, stream);        // 256 x 128, 8 waves
-  else if (tiles(128, 128) >= 180) launch_mmqh<F, 4, 2, 1, 2, 2, T>(W, ws, Y, M, N, K, stream);   // 128 x 128, 8 waves
-  else if (tiles(128, 64) >= 180) launch_mmqh<F, 2, 2, 2, 1, 2, T>(W, ws, Y, M, N, K, stream);    // 128 x 64, 4 waves
-  else launch_mmqh<F, 2, 2, 1, 1, 4, T>(W, ws, Y, M, N, K, stream);                               // 64 x 64, 4 waves
-  return launch_status();
-}
-
 template <class F>
 static int mmqh_fmt(const void* W, const void* ws, void* Y, int dtype, int M, int N, int K, float* partial, int64_t partial_bytes,
                     hipStream_t s) {
-  if (dtype == GGUF_DTYPE_F16) return mmqh_typed<F, _Float16>(W, ws, Y, M, N, K, partial, partial_bytes, s);
+  if (dtype == GGUF_DTYPE_F16) return mmqh_typed<A8Codes<F>, _Float16>(W, ws, Y, M, N, K, partial, partial_bytes, s);
 #ifndef GGUF_MMQ_TUNE
-  if (dtype == GGUF_DTYPE_BF16) return mmqh_typed<F, bf16_t>(W, ws, Y, M, N, K, partial, partial_bytes, s);
+  if (dtype == GGUF_DTYPE_BF16) return mmqh_typed<A8Codes<F>, bf16_t>(W, ws, Y, M, N, K, partial, partial_bytes, s);
 #endif
   return GGUF_ERR_DTYPE;
 }

@@ -126,6 +126,25 @@ def ggml_mul_mat_a8(W: torch.Tensor, X: torch.Tensor, quant_type: int, row: int,
     return out
 
 
+DEQUANT_GEMM_TYPES = frozenset({2, 3, 6, 7, 8, 10, 11, 12, 13, 14, 16, 23})
+
+
+def ggml_dequant_gemm(W: torch.Tensor, X: torch.Tensor, quant_type: int, row: int) -> torch.Tensor:
+    """``X @ dequant(W)^T`` -> ``[X.shape[0], row]`` in one kernel, activations not quantized: the reference's
+    ``ggml_dequantize`` + ``x @ weight.T`` fallback (quantization/linear.py:50-58) without the dense copy of W.
+    fp16 / bf16 only; raises ``NotImplementedError`` for types outside ``DEQUANT_GEMM_TYPES``."""
+    _check_inputs(W, X)
+    vecs, col = X.shape
+    with torch.cuda.device(X.device):
+        out = torch.empty((vecs, row), dtype=X.dtype, device=W.device)
+        nbytes = max(_lib.lib().gguf_mmq_workspace_bytes(vecs, row, col), vecs * _lib.lib().gguf_q8_1_row_bytes(col), 16)
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=X.device)
+        rc = _lib.lib().gguf_dequant_gemm(W.data_ptr(), X.data_ptr(), _code(X.dtype), ws.data_ptr(), out.data_ptr(),
+                                          int(quant_type), row, col, vecs, nbytes, _stream(X))
+    _lib.check(rc, "ggml_dequant_gemm")
+    return out
+
+
 def ggml_moe_a8(
     X: torch.Tensor,
     W: torch.Tensor,
