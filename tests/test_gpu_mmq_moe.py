@@ -165,6 +165,29 @@ def test_dequant_gemm_split_k_and_rejections():
         ops.ggml_dequant_gemm(wi, xd[:4, :256].contiguous(), o.IQ3_S, 64)
 
 
+def test_mmq_half_engine_splits_the_last_round():
+    """More tiles than the chip holds at once and a sparse last round (296 tiles of 256x128 on 256 CUs): the 40 tiles of
+    that round are split along K and summed from fp32 partial tiles; the other 256 are whole.  Both kinds must agree
+    with the integer engine, and the result must not depend on whether the workspace had room for the split."""
+    from vllm_gguf_plugin_prism_amd import _lib
+    ops = _ops()
+    rng = np.random.default_rng(1700)
+    m, n, k = 512, 18944, 1024
+    w = _dev(np.concatenate([o.make_weights(rng, o.Q6_K, 2368, k) for _ in range(8)], axis=0))
+    xd, _ = _x(rng, m, k, "f16")
+    assert _lib.lib().gguf_mmq_workspace_bytes(m, n, k) > m * _lib.lib().gguf_q8_1_row_bytes(k) + 256
+    y = ops.ggml_mul_mat_a8(w, xd, o.Q6_K, n, engine="half").float()
+    ref = ops.ggml_mul_mat_a8(w, xd.float(), o.Q6_K, n).double()          # integer engine, fp32 result
+    err = ((y.double() - ref).norm(dim=0) / ref.norm(dim=0))               # per output column: every tile is looked at
+    assert float(err.max()) <= 1.5e-3 and float((y.double() - ref).norm() / ref.norm()) <= 6e-4
+    ws = torch.empty(m * _lib.lib().gguf_q8_1_row_bytes(k), dtype=torch.uint8, device="cuda")
+    y_plain = torch.empty_like(y, dtype=torch.float16)
+    rc = _lib.lib().gguf_mmq(w.data_ptr(), xd.data_ptr(), 1, ws.data_ptr(), y_plain.data_ptr(), o.Q6_K, n, k, m,
+                             torch.cuda.current_stream().cuda_stream)
+    assert rc == 0
+    assert float((y_plain.double() - y.double()).norm() / ref.norm()) <= 4e-4
+
+
 def test_mmq_engine_rejections():
     ops = _ops()
     rng = np.random.default_rng(5)

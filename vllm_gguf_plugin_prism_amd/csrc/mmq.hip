@@ -611,7 +611,7 @@ static bool mmq_type_ok(int type) {
 int mmq_half(const void* W, const void* ws, void* Y, int dtype, int type, int M, int N, int K, float* partial,
              int64_t partial_bytes, hipStream_t s);
 bool mmq_half_supported(int type);
-int mmq_half_splits(int M, int N, int K);
+int64_t mmq_half_partial_bytes(int M, int N, int K);
 
 }  // namespace gguf
 
@@ -620,8 +620,7 @@ static int64_t mmq_rows_bytes(int64_t M, int64_t K) { return (M * (gguf::q8_row_
 
 extern "C" int64_t gguf_mmq_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   if (M <= 0 || N <= 0 || K <= 0 || M > 0x7FFFFFF0LL || N > 0x7FFFFFF0LL || K > 0x7FFFFFF0LL) return 0;
-  const int splits = gguf::mmq_half_splits((int)M, (int)N, (int)K);
-  return mmq_rows_bytes(M, K) + (splits > 1 ? (int64_t)splits * M * N * 4 : 0);
+  return mmq_rows_bytes(M, K) + gguf::mmq_half_partial_bytes((int)M, (int)N, (int)K);
 }
 
 extern "C" int gguf_mmq_engine(const void* W, const void* x, int xdtype, void* q8_workspace, void* Y, int type, int64_t N,

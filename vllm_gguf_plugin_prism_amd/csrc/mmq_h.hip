@@ -4,17 +4,46 @@
 
 namespace gguf {
 
-// Number of K splits the half engine would like for this shape (1 = none): enough to give every CU a workgroup of the
-// large tile, every split keeping at least 16 steps of 64 elements.
-int mmq_half_splits(int M, int N, int K) {
-  const int mt = M > 128 ? 256 : 128;
-  const int64_t tiles = (int64_t)((M + mt - 1) / mt) * ((N + 127) / 128);
-  if (tiles >= 180 || tiles == 0) return 1;
-  int s = (int)(256 / tiles);
-  const int by_k = (K / 64) / 16;
-  if (s > by_k) s = by_k;
-  if (s > 8) s = 8;
-  return s < 2 ? 1 : s;
+// Tile size and the hand-out of tiles to workgroups for one launch (see MmqhPlan).
+//   * The largest tile that still gives most CUs a workgroup: large tiles decode each weight block for more token
+//     rows and read less LDS per MFMA; small ones fill the chip when M or N is small.
+//   * When even the large tile leaves most CUs idle and K is long, the large tile is kept and every tile is split
+//     along K instead.
+//   * When the tiles fill the chip once or more but the last round of workgroups would be mostly empty, the tiles of
+//     that round are split along K, so that the round is short instead of sparse.
+// Splitting needs fp32 scratch in the workspace; without it the plan falls back to whole tiles.
+MmqhPlan mmq_half_plan(int M, int N, int K, int64_t avail) {
+  constexpr int CUS = 256;
+  static const int MT[4] = {256, 128, 128, 64}, NT[4] = {128, 128, 64, 64};
+  const auto tiles = [&](int c) { return (int64_t)((M + MT[c] - 1) / MT[c]) * ((N + NT[c] - 1) / NT[c]); };
+  const int nsteps = (K + 63) / 64;
+  const int big = M > 128 ? 0 : 1;
+  MmqhPlan p = {3, 0, 0, 1};
+  const int64_t tb = tiles(big);
+  if (tb < 180 && tb > 0) {                     // too few tiles: split them all
+    int s = (int)(CUS / tb);
+    if (s > nsteps / 16) s = nsteps / 16;
+    if (s > 8) s = 8;
+    p = MmqhPlan{big, 0, (int)tb, s};
+    if (s >= 2 && p.partial_bytes() <= avail) return p;
+  }
+  int cfg = 3;
+  for (int c = big; c < 4; ++c)
+    if (tiles(c) >= 180) { cfg = c; break; }
+  const int64_t t = tiles(cfg);
+  p = MmqhPlan{cfg, (int)t, 0, 1};
+  const int slots = cfg == 0 ? CUS : 2 * CUS;   // workgroups the chip holds at once: one 256x128 tile per CU, two of 128x128
+  if (cfg <= 1 && t > slots) {                  // look at the last round
+    const int rest = (int)(t % slots);
+    int s = rest ? slots / rest : 1;
+    if (s > nsteps / 8) s = nsteps / 8;
+    if (s > 8) s = 8;
+    if (s >= 2) {
+      const MmqhPlan q = {cfg, (int)(t - rest), rest, s};
+      if (q.partial_bytes() <= avail) return q;
+    }
+  }
+  return p;
 }
 
 template <class F>
@@ -46,6 +75,9 @@ int mmq_half(const void* W, const void* ws, void* Y, int dtype, int type, int M,
   }
   return GGUF_ERR_TYPE;
 }
+
+// fp32 scratch the plan for this shape would use, given all the room it wants
+int64_t mmq_half_partial_bytes(int M, int N, int K) { return mmq_half_plan(M, N, K, INT64_MAX).partial_bytes(); }
 
 bool mmq_half_supported(int type) {
   switch (type) {

@@ -135,7 +135,8 @@ template <class C, int WM, int WN, int TM, int TN, int OCC, typename T>
 __global__ __launch_bounds__(64 * WM * WN, OCC) void mmqh_kernel(const uint8_t* __restrict__ W, const _Float16* __restrict__ xh,
                                                                   const char* __restrict__ ws, int64_t ws_row_bytes,
                                                                   T* __restrict__ Y, float* __restrict__ partial, int M, int N,
-                                                                  int K, int Kp, int dbg) {
+                                                                  int K, int Kp, int tiles_x, int whole_tiles, int shared_tiles, int splits,
+                                                                  int dbg) {
 #ifndef GGUF_MMQ_TUNE
   (void)dbg;
 #define DBG_SKIP(bit, cond) false
@@ -160,7 +161,13 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void mmqh_kernel(const uint8_t* 
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int wm = wave / WN, wn = wave % WN;
   const int lrow = lane & 31, lhalf = lane >> 5;
-  const int m_base = blockIdx.y * M_T, n_base = blockIdx.x * N_T;
+  // Workgroup -> work: the first `whole_tiles` workgroups take one output tile each over all of K; behind them every
+  // further tile is shared by `splits` workgroups, each taking a stretch of K (see the loop below).
+  const int wg = blockIdx.x;
+  const int tile = wg < whole_tiles ? wg : whole_tiles + (wg - whole_tiles) % shared_tiles;   // neighbours in launch order walk
+  const int split = wg < whole_tiles ? 0 : (wg - whole_tiles) / shared_tiles;                  // the same stretch of K
+  const int nsplit = wg < whole_tiles ? 1 : splits;
+  const int m_base = (tile / tiles_x) * M_T, n_base = (tile % tiles_x) * N_T;
   const int64_t rowbytes = (int64_t)(K / F::QK) * F::BS;
   const int nkb_total = K >> 5;
   const int nsteps = (K + KS - 1) / KS;
@@ -261,10 +268,11 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void mmqh_kernel(const uint8_t* 
   // wave's turn, the weight block decoded from the registers loaded DG iterations ago -- issues the global loads that
   // refill those registers, and then contracts step s.  Waves whose turn it is not go straight to the matrix work, so
   // a SIMD always has one wave decoding and one multiplying.
-  // With gridDim.z > 1 the steps of K are split over that many workgroups per tile, each leaving its fp32 partial tile
-  // in `partial`; a second kernel adds them.  For shapes whose output has too few tiles to occupy the chip.
-  const int per_split = (nsteps + (int)gridDim.z - 1) / (int)gridDim.z;
-  const int t0 = (int)blockIdx.z * per_split, t1 = min(nsteps, t0 + per_split);
+  // A tile whose K is split leaves one fp32 partial tile per split in `partial`; a second kernel adds them.  Splitting
+  // serves shapes whose output has too few tiles to occupy the chip, and the last, partly filled round of workgroups
+  // of any shape: instead of a few CUs working through whole tiles while the rest idle, all CUs share those tiles.
+  const int per_split = (nsteps + nsplit - 1) / nsplit;
+  const int t0 = split * per_split, t1 = min(nsteps, t0 + per_split);
   if (t0 < t1) {
     fetch_a(t0);
     const int first = t0 + ((grp - t0) % DG + DG) % DG;   // this group's first step
@@ -286,7 +294,7 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void mmqh_kernel(const uint8_t* 
   _Float16* const xs = tiles;                // the offset pass below reuses the first buffer
   _Float16* const wt = tiles + M_T * LDH;
 
-  if constexpr (C::SUM_PASS) if (blockIdx.z == 0) {
+  if constexpr (C::SUM_PASS) if (split == 0) {
     // Offset term (the first split adds it).  The reference's MMQ semantics multiply the offset factor mn by the stored sum s8 of the block's
     // unquantized activations (vecdotq.cuh:61-64, 369-372) while the codes meet the quantized ones, whose sum times
     // d8 is du.  With the codes centred at C in the main loop,
@@ -338,18 +346,17 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void mmqh_kernel(const uint8_t* 
     }
   }
 
+  float* const my_partial = nsplit > 1 ? partial + ((int64_t)(tile - whole_tiles) * splits + split) * (M_T * N_T) : nullptr;
 #pragma unroll
   for (int j = 0; j < TM; ++j) {
 #pragma unroll
     for (int r = 0; r < 16; ++r) {
-      const int mt = m_base + 32 * (wm * TM + j) + 8 * (r >> 2) + 4 * lhalf + (r & 3);
+      const int ml = 32 * (wm * TM + j) + 8 * (r >> 2) + 4 * lhalf + (r & 3), mt = m_base + ml;
 #pragma unroll
       for (int i = 0; i < TN; ++i) {
-        const int n = n_base + 32 * (wn * TN + i) + lrow;
-        if (mt < M && n < N) {
-          if (partial) partial[((int64_t)blockIdx.z * M + mt) * N + n] = acc[j][i][r];
-          else Y[(int64_t)mt * N + n] = from_f32<T>(acc[j][i][r] * HP_UNSCALE);
-        }
+        const int nl = 32 * (wn * TN + i) + lrow, n = n_base + nl;
+        if (my_partial) my_partial[ml * N_T + nl] = acc[j][i][r];   // the whole tile, edges included: the adder masks them
+        else if (mt < M && n < N) Y[(int64_t)mt * N + n] = from_f32<T>(acc[j][i][r] * HP_UNSCALE);
       }
     }
   }
@@ -364,19 +371,43 @@ static int tune_dbg() {
 #endif
 }
 
-// Y = T(sum of the `splits` fp32 partial tiles / 16)
-template <typename T>
-__global__ __launch_bounds__(256) void mmqh_reduce_kernel(const float* __restrict__ partial, T* __restrict__ Y, int64_t mn, int splits) {
-  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
-  if (i >= mn) return;
-  float acc = partial[i];
-  for (int z = 1; z < splits; ++z) acc += partial[z * mn + i];
-  Y[i] = from_f32<T>(acc * HP_UNSCALE);
+// Y tile = T(sum of its `splits` fp32 partial tiles / 16), gridDim.y workgroups per split tile, fixed order of addition
+template <int M_T, int N_T, typename T>
+__global__ __launch_bounds__(256) void mmqh_reduce_kernel(const float* __restrict__ partial, T* __restrict__ Y, int M, int N,
+                                                          int tiles_x, int whole_tiles, int splits) {
+  const int tile = whole_tiles + blockIdx.x;
+  const int m_base = (tile / tiles_x) * M_T, n_base = (tile % tiles_x) * N_T;
+  const float* p = partial + (int64_t)blockIdx.x * splits * (M_T * N_T);
+  for (int i = (blockIdx.y * 256 + threadIdx.x) * 4; i < M_T * N_T; i += gridDim.y * 256 * 4) {
+    float4 acc = *(const float4*)(p + i);
+    for (int z = 1; z < splits; ++z) {
+      const float4 v = *(const float4*)(p + (int64_t)z * (M_T * N_T) + i);
+      acc.x += v.x; acc.y += v.y; acc.z += v.z; acc.w += v.w;
+    }
+    const int m = m_base + i / N_T, n = n_base + i % N_T;
+    if (m >= M) continue;
+    const float out[4] = {acc.x, acc.y, acc.z, acc.w};
+#pragma unroll
+    for (int e = 0; e < 4; ++e)
+      if (n + e < N) Y[(int64_t)m * N + n + e] = from_f32<T>(out[e] * HP_UNSCALE);
+  }
 }
 
+// How the tiles of one launch are handed out: `whole` tiles get a workgroup each, the remaining `shared` tiles are
+// split `splits` ways along K.  partial_bytes() is the fp32 scratch the shared tiles need.
+struct MmqhPlan {
+  int cfg;            // 0: 256x128, 1: 128x128, 2: 128x64, 3: 64x64
+  int whole, shared, splits;
+  int64_t partial_bytes() const {
+    static const int tile_elems[4] = {256 * 128, 128 * 128, 128 * 64, 64 * 64};
+    return (int64_t)shared * splits * tile_elems[cfg] * 4;
+  }
+};
+MmqhPlan mmq_half_plan(int M, int N, int K, int64_t partial_bytes_available);  // mmq_h.hip
+
 template <class C, int WM, int WN, int TM, int TN, int OCC, typename T>
-static void launch_mmqh(const void* W, const void* ws, void* Y, int M, int N, int K, hipStream_t stream, int splits = 1,
-                        float* partial = nullptr) {
+static void launch_mmqh(const void* W, const void* ws, void* Y, int M, int N, int K, hipStream_t stream, int whole = -1, int shared = 0,
+                        int splits = 1, float* partial = nullptr) {
   constexpr int M_T = 32 * WM * TM, N_T = 32 * WN * TN;
   constexpr size_t lds = (size_t)(M_T + N_T) * (64 + 8) * 2 * 2;
   auto kern = mmqh_kernel<C, WM, WN, TM, TN, OCC, T>;
@@ -387,14 +418,14 @@ static void launch_mmqh(const void* W, const void* ws, void* Y, int M, int N, in
       configured = true;
     }
   }
+  const int tiles_x = (N + N_T - 1) / N_T, tiles = tiles_x * ((M + M_T - 1) / M_T);
+  if (whole < 0) { whole = tiles; shared = 0; splits = 1; }
   const _Float16* xh = (const _Float16*)((const char*)ws + (int64_t)M * q8_row_bytes(K));
-  hipLaunchKernelGGL(kern, dim3((N + N_T - 1) / N_T, (M + M_T - 1) / M_T, splits), dim3(64 * WM * WN), lds, stream, (const uint8_t*)W,
-                     xh, (const char*)ws, q8_row_bytes(K), (T*)Y, splits > 1 ? partial : (float*)nullptr, M, N, K, (int)q8_kp(K),
-                     tune_dbg());
-  if (splits > 1) {
-    const int64_t mn = (int64_t)M * N;
-    hipLaunchKernelGGL(mmqh_reduce_kernel<T>, dim3((unsigned)((mn + 255) / 256)), dim3(256), 0, stream, partial, (T*)Y, mn, splits);
-  }
+  hipLaunchKernelGGL(kern, dim3(whole + shared * splits), dim3(64 * WM * WN), lds, stream, (const uint8_t*)W, xh, (const char*)ws,
+                     q8_row_bytes(K), (T*)Y, partial, M, N, K, (int)q8_kp(K), tiles_x, whole, shared > 0 ? shared : 1, splits, tune_dbg());
+  if (shared > 0)
+    hipLaunchKernelGGL((mmqh_reduce_kernel<M_T, N_T, T>), dim3(shared, M_T * N_T / 1024), dim3(256), 0, stream, partial, (T*)Y, M, N, tiles_x,
+                       whole, splits);
 }
 
 #ifdef GGUF_MMQ_TUNE
@@ -403,8 +434,6 @@ static int tune_cfg_h() {
   return v;
 }
 #endif
-
-int mmq_half_splits(int M, int N, int K);  // mmq_h.hip
 
 template <class C, typename T>
 static int mmqh_typed(const void* W, const void* ws, void* Y, int M, int N, int K, float* partial, int64_t partial_bytes,
@@ -423,20 +452,13 @@ static int mmqh_typed(const void* W, const void* ws, void* Y, int M, int N, int 
     default: break;
   }
 #endif
-  // Tile choice: the largest tile that still gives most CUs a workgroup.  Large tiles decode each weight block for
-  // more token rows and read less LDS per MFMA; small ones fill the chip when M or N is small.  When even they leave
-  // CUs idle and K is long, the large tile is kept and K is split instead, if the workspace has room for the partials.
-  const auto tiles = [&](int mt, int nt) { return (int64_t)((M + mt - 1) / mt) * ((N + nt - 1) / nt); };
-  const int splits = mmq_half_splits(M, N, K);
-  if (splits > 1 && partial_bytes >= (int64_t)splits * M * N * 4) {
-    if (M > 128) launch_mmqh<C, 4, 2, 2, 2, 1, T>(W, ws, Y, M, N, K, stream, splits, partial);
-    else launch_mmqh<C, 4, 2, 1, 2, 2, T>(W, ws, Y, M, N, K, stream, splits, partial);
-    return launch_status();
+  const MmqhPlan p = mmq_half_plan(M, N, K, partial_bytes);
+  switch (p.cfg) {
+    case 0: launch_mmqh<C, 4, 2, 2, 2, 1, T>(W, ws, Y, M, N, K, stream, p.whole, p.shared, p.splits, partial); break;  // 256 x 128, 8 waves
+    case 1: launch_mmqh<C, 4, 2, 1, 2, 2, T>(W, ws, Y, M, N, K, stream, p.whole, p.shared, p.splits, partial); break;  // 128 x 128, 8 waves
+    case 2: launch_mmqh<C, 2, 2, 2, 1, 2, T>(W, ws, Y, M, N, K, stream, p.whole, p.shared, p.splits, partial); break;  // 128 x 64, 4 waves
+    default: launch_mmqh<C, 2, 2, 1, 1, 4, T>(W, ws, Y, M, N, K, stream, p.whole, p.shared, p.splits, partial); break; // 64 x 64, 4 waves
   }
-  if (tiles(256, 128) >= 180) launch_mmqh<C, 4, 2, 2, 2, 1, T>(W, ws, Y, M, N, K, stream);        // 256 x 128, 8 waves
-  else if (tiles(128, 128) >= 180) launch_mmqh<C, 4, 2, 1, 2, 2, T>(W, ws, Y, M, N, K, stream);   // 128 x 128, 8 waves
-  else if (tiles(128, 64) >= 180) launch_mmqh<C, 2, 2, 2, 1, 2, T>(W, ws, Y, M, N, K, stream);    // 128 x 64, 4 waves
-  else launch_mmqh<C, 2, 2, 1, 1, 4, T>(W, ws, Y, M, N, K, stream);                               // 64 x 64, 4 waves
   return launch_status();
 }
 
