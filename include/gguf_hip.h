@@ -105,6 +105,21 @@ int64_t gguf_mmq_workspace_bytes(int64_t M, int64_t N, int64_t K);
 int gguf_mmq_engine(const void* W, const void* x, int xdtype, void* q8_workspace, void* Y, int type, int64_t N, int64_t K,
                     int64_t M, int engine, int64_t workspace_bytes, gguf_stream_t stream);
 
+/* The two a8 operators for one shard of a merged linear layer.  quantization/linear.py:229-262 keeps the shards of a
+ * fused layer (q/k/v, gate/up) in one uint8 tensor padded to the widest row; when their ggml types differ it copies
+ * every shard out with .contiguous() on each forward pass, multiplies, concatenates the results and adds the bias.
+ * These entry points read the shard where it lies and write where the result belongs:
+ *   W                  first row of the shard; rows are w_row_pitch_bytes apart (>= K / block * block_bytes);
+ *   Y                  first result column of the shard in the merged output; rows are y_row_pitch elements apart;
+ *   bias               null, or N values of Y's dtype (the shard's slice of the layer bias), added to every row after
+ *                      the product is rounded to Y's dtype, as out.add_(bias) does.
+ * gguf_mmvq / gguf_mmq / gguf_mmq_engine are these with dense rows, y_row_pitch = N and no bias. */
+int gguf_mmvq_linear(const void* W, int64_t w_row_pitch_bytes, const void* x, int xdtype, void* q8_workspace, void* Y,
+                     int64_t y_row_pitch, const void* bias, int type, int64_t N, int64_t K, int64_t M, gguf_stream_t stream);
+int gguf_mmq_linear(const void* W, int64_t w_row_pitch_bytes, const void* x, int xdtype, void* q8_workspace, void* Y,
+                    int64_t y_row_pitch, const void* bias, int type, int64_t N, int64_t K, int64_t M, int engine,
+                    int64_t workspace_bytes, gguf_stream_t stream);
+
 /* Y[M,N] = X[M,K] . dequant(W[N,K])^T with the activations as they are (no q8_1 quantisation): one GEMM on
  * half-precision MFMA that decodes the packed blocks on the fly instead of the reference's fallback for formats and
  * batch sizes without an a8 kernel, ggml_dequantize followed by x @ weight.T (quantization/linear.py:50-58,

@@ -179,3 +179,80 @@ def test_fused_activation_equals_separate_activation(act, dt):
     want = ops.ggml_moe_a8(sep_in, w2, s_, e_, n_, o.Q4_0, H, 1, pairs)
     got = ops.ggml_moe_a8(h, w2, s_, e_, n_, o.Q4_0, H, 1, pairs, activation=act)
     assert o.rel_l2(got.float().cpu().numpy(), want.float().cpu().numpy()) <= (2e-3 if dt == torch.bfloat16 else 5e-4)
+
+
+def _merged_layer(rng, shards, k):
+    """A padded merged tensor like quantization/linear.py:150-219 builds: shards stacked by rows, every row padded to
+    the widest shard's row bytes.  shards: list of (id, ggml type, rows)."""
+    parts, offsets, start = [], {}, 0
+    for sid, qt, rows in shards:
+        w = o.make_weights(rng, qt, rows, k)
+        parts.append(w)
+        offsets[sid] = (start, start + rows, w.shape[1])
+        start += rows
+    width = max(p.shape[1] for p in parts)
+    merged = np.full((start, width), 0xA5, dtype=np.uint8)   # padding bytes that would show if a kernel read them
+    for (sid, _, _), p in zip(shards, parts):
+        s, e, rb = offsets[sid]
+        merged[s:e, :rb] = p
+    return merged, offsets, parts
+
+
+@pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16, torch.float32])
+@pytest.mark.parametrize("m", [1, 3, 5, 40, 300])
+def test_apply_linear_mixed_type_shards_in_place(m, dt):
+    """q and k in Q4_K, v in Q6_K (what Q4_K_M checkpoints hold): the reference multiplies a .contiguous() copy of every
+    shard, concatenates and adds the bias (linear.py:247-262).  apply_linear must give the same bits while reading the
+    shards inside the padded tensor and writing into the merged result directly, for every path (GEMV, both MMQ
+    engines) the batch size selects."""
+    from vllm_gguf_plugin_prism_amd import ops
+    rng = np.random.default_rng(2000 + m)
+    k = 1024
+    shards = [("q", o.Q4_K, 512), ("k", o.Q4_K, 128), ("v", o.Q6_K, 130)]
+    merged, offsets, parts = _merged_layer(rng, shards, k)
+    wd = torch.from_numpy(merged).cuda()
+    x = torch.from_numpy(rng.standard_normal((m, k)).astype(np.float32)).to(dt).cuda()
+    bias = torch.from_numpy(rng.standard_normal(770).astype(np.float32)).to(dt).cuda()
+    types = {"q": o.Q4_K, "k": o.Q4_K, "v": o.Q6_K}
+    got = D.apply_linear(x, wd, o.Q4_K, shard_ids=["q", "k", "v"], shard_offset_map=offsets, shard_weight_types=types, bias=bias)
+    # the reference's sequence, with the same operators on contiguous copies
+    ref = torch.cat([D.fused_mul_mat_gguf(x, torch.from_numpy(p).cuda(), qt) for (_, qt, _), p in zip(shards, parts)], dim=1)
+    ref.add_(bias)
+    assert got.shape == (m, 770) and got.dtype == dt
+    assert torch.equal(got, ref)
+    # and against the oracle, so that "the same bits" is not two equal mistakes
+    xv = x.float().cpu().numpy()
+    path = D.select_mul_mat_path(o.Q4_K, m, 512)
+    exp = np.concatenate([o.mul_mat_a8(p, xv, qt, p.shape[0], path) for (_, qt, _), p in zip(shards, parts)], axis=1)
+    exp = exp + bias.float().cpu().numpy()
+    tol = {torch.float16: 2e-3, torch.bfloat16: 8e-3, torch.float32: 1e-5}[dt]
+    assert o.rel_l2(got.float().cpu().numpy(), exp) <= tol
+
+
+def test_apply_linear_single_type_and_plain_layers():
+    rng = np.random.default_rng(2100)
+    k = 512
+    merged, offsets, parts = _merged_layer(rng, [(0, o.Q8_0, 96), (1, o.Q8_0, 160)], k)
+    wd = torch.from_numpy(merged).cuda()
+    x = torch.from_numpy(rng.standard_normal((2, k)).astype(np.float32)).to(torch.float16).cuda()
+    bias = torch.from_numpy(rng.standard_normal(256).astype(np.float32)).to(torch.float16).cuda()
+    one = D.apply_linear(x, wd, o.Q8_0, shard_ids=[0, 1], shard_offset_map=offsets, bias=bias)
+    plain = D.apply_linear(x, wd, o.Q8_0, bias=bias)
+    ref = D.fused_mul_mat_gguf(x, wd, o.Q8_0)
+    ref.add_(bias)
+    assert torch.equal(one, ref) and torch.equal(plain, ref)
+
+
+def test_shard_operators_reject_bad_views():
+    from vllm_gguf_plugin_prism_amd import ops
+    rng = np.random.default_rng(2200)
+    w = torch.from_numpy(o.make_weights(rng, o.Q4_K, 64, 512)).cuda()
+    x = torch.randn(2, 512, dtype=torch.float16, device="cuda")
+    with pytest.raises(ValueError):
+        ops.ggml_mul_mat_vec_a8(w[:, :100], x, o.Q4_K, 64)                       # rows shorter than K needs
+    with pytest.raises(ValueError):
+        ops.ggml_mul_mat_vec_a8(w, x, o.Q4_K, 64, out=torch.empty(2, 63, dtype=torch.float16, device="cuda"))
+    with pytest.raises(ValueError):
+        ops.ggml_mul_mat_a8(w, x, o.Q4_K, 64, bias=torch.zeros(64, dtype=torch.float32, device="cuda"))
+    with pytest.raises(ValueError):
+        ops.ggml_mul_mat_a8(w.t(), x, o.Q4_K, 64)

@@ -33,6 +33,10 @@ _SIGNATURES = {
                              _c.c_int64, _c.c_int64, _c.c_void_p]),
     "gguf_mmq": (_c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_int, _c.c_void_p, _c.c_void_p, _c.c_int, _c.c_int64,
                             _c.c_int64, _c.c_int64, _c.c_void_p]),
+    "gguf_mmvq_linear": (_c.c_int, [_c.c_void_p, _c.c_int64, _c.c_void_p, _c.c_int, _c.c_void_p, _c.c_void_p, _c.c_int64,
+                                    _c.c_void_p, _c.c_int, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_void_p]),
+    "gguf_mmq_linear": (_c.c_int, [_c.c_void_p, _c.c_int64, _c.c_void_p, _c.c_int, _c.c_void_p, _c.c_void_p, _c.c_int64,
+                                   _c.c_void_p, _c.c_int, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int, _c.c_int64, _c.c_void_p]),
     "gguf_mmq_workspace_bytes": (_c.c_int64, [_c.c_int64, _c.c_int64, _c.c_int64]),
     "gguf_mmq_engine": (_c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_int, _c.c_void_p, _c.c_void_p, _c.c_int, _c.c_int64,
                                    _c.c_int64, _c.c_int64, _c.c_int, _c.c_int64, _c.c_void_p]),

@@ -144,6 +144,20 @@ template <> __device__ __forceinline__ bf16_t from_half<bf16_t>(_Float16 v) { re
     default: return GGUF_ERR_DTYPE;                                      \
   }
 
+// How one call addresses a shard of a merged linear layer (quantization/linear.py:229-262): the rows of W may sit in a
+// wider, padded tensor, the result may be a column range of a wider output, and the layer's bias may be added.
+struct LinearArgs {
+  int64_t w_pitch = 0;         // bytes between rows of W; 0 = rows are dense
+  int64_t ldy = 0;             // elements between rows of Y; 0 = N
+  const void* bias = nullptr;  // N values of Y's dtype, added to every row of the result after it is rounded; or null
+};
+// out = round(round(v) + bias): the reference rounds the product to the output dtype and then adds in that dtype
+template <typename T>
+__device__ __forceinline__ T finish(float v, const T* bias, int64_t n) {
+  const T r = from_f32<T>(v);
+  return bias ? from_f32<T>(to_f32<T>(r) + to_f32<T>(bias[n])) : r;
+}
+
 // q8_1 quantisation of M rows into the workspace (q8_1.hip).  act: gated activation applied while loading (see
 // q8_1_device.h).  half_plane: if not null, also the dequantized rows in half precision, [M][q8_kp(K)].
 int quantize_q8_1(const void* x, int xdtype, void* ws, int64_t M, int64_t K, hipStream_t stream, int act = 0,

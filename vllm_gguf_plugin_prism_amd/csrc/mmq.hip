@@ -160,7 +160,7 @@ enum { MODE_PREFETCH = 0, MODE_PLAIN = 1, MODE_PINGPONG = 2, MODE_KSPLIT = 3 };
 template <class F, int WM, int WN, int TM, int TN, int KS, int OCC, int MODE, typename T, bool MOE>
 __global__ __launch_bounds__(64 * WM * WN * (MODE == MODE_PINGPONG || MODE == MODE_KSPLIT ? 2 : 1), OCC) void mmq_kernel(const uint8_t* __restrict__ W, const char* __restrict__ ws,
                                                          T* __restrict__ Y, int M, int N, int K, int64_t ws_row_bytes,
-                                                         MoeArgs moe) {
+                                                         MoeArgs moe, int64_t w_pitch, int64_t ldy, const T* __restrict__ bias) {
   constexpr int GW = WM * WN;            // waves that share one set of accumulators' tile
   constexpr int KW = MODE == MODE_KSPLIT ? 2 : 1;  // wave sets splitting the 32-blocks of a step
   constexpr int NT = 64 * GW * KW;       // threads that stage one tile (the whole workgroup unless MODE_PINGPONG)
@@ -189,7 +189,7 @@ __global__ __launch_bounds__(64 * WM * WN * (MODE == MODE_PINGPONG || MODE == MO
   const int m_base = blockIdx.y * M_T;
   const int n_base = MODE == MODE_PINGPONG ? (blockIdx.x * 2 + group) * N_T : blockIdx.x * N_T;
   const int Kp = (int)q8_kp(K);
-  const int64_t rowbytes = (int64_t)(K / F::QK) * F::BS;
+  const int64_t rowbytes = w_pitch;   // bytes between rows of W: the dense row size unless the caller's tensor is padded
   const int nkb_total = K >> 5;
 
   if (MOE) {
@@ -498,7 +498,7 @@ __global__ __launch_bounds__(64 * WM * WN * (MODE == MODE_PINGPONG || MODE == MO
 #pragma unroll
       for (int i = 0; i < TN; ++i) {
         const int n = n_base + 32 * (wn * TN + i) + lrow;
-        if (ok && n < N) Y[dst * N + n] = from_f32<T>(acc[j][i][r]);
+        if (ok && n < N) Y[dst * ldy + n] = finish<T>(acc[j][i][r], bias, n);
       }
     }
   }
@@ -507,7 +507,7 @@ __global__ __launch_bounds__(64 * WM * WN * (MODE == MODE_PINGPONG || MODE == MO
 
 template <class F, int WM, int WN, int TM, int TN, int KS, int OCC, int MODE, typename T, bool MOE>
 static void launch_mmq(const void* W, const void* ws, void* Y, int M, int N, int K, int m_tiles, const MoeArgs& moe,
-                       hipStream_t stream) {
+                       hipStream_t stream, const LinearArgs& la = LinearArgs()) {
   constexpr int G = MODE == MODE_PINGPONG ? 2 : 1;
   constexpr int KW = MODE == MODE_KSPLIT ? 2 : 1;
   constexpr int N_T = 32 * WN * TN * G;
@@ -522,7 +522,8 @@ static void launch_mmq(const void* W, const void* ws, void* Y, int M, int N, int
     }
   }
   hipLaunchKernelGGL(kern, dim3((N + N_T - 1) / N_T, m_tiles), dim3(64 * WM * WN * G * KW), lds, stream, (const uint8_t*)W, (const char*)ws,
-                     (T*)Y, M, N, K, q8_row_bytes(K), moe);
+                     (T*)Y, M, N, K, q8_row_bytes(K), moe, la.w_pitch ? la.w_pitch : (int64_t)(K / F::QK) * F::BS,
+                     la.ldy ? la.ldy : (int64_t)N, (const T*)la.bias);
 }
 
 
@@ -542,39 +543,39 @@ static int tune_cfg() {
 // Formats whose packed block is small keep the next step's loads in registers across the MFMA phase (PREFETCH);
 // for the others that would push the kernel past 128 registers and halve the waves per SIMD.
 template <class F, typename T>
-static int mmq_typed(const void* W, const void* ws, void* Y, int M, int N, int K, hipStream_t stream) {
+static int mmq_typed(const void* W, const void* ws, void* Y, int M, int N, int K, hipStream_t stream, const LinearArgs& la) {
   MoeArgs none = {};
   const int64_t large_tiles = (int64_t)((M + 127) / 128) * ((N + 127) / 128);
 #ifdef GGUF_MMQ_TUNE
   switch (tune_cfg()) {
-    case 1: launch_mmq<F, 4, 1, 1, 2, 128, 4, MODE_PINGPONG, T, false>(W, ws, Y, M, N, K, (M + 127) / 128, none, stream); return launch_status();
-    case 3: launch_mmq<F, 2, 1, 1, 1, 128, 4, MODE_PINGPONG, T, false>(W, ws, Y, M, N, K, (M + 63) / 64, none, stream); return launch_status();
-    case 5: launch_mmq<F, 4, 2, 1, 2, 128, 4, MODE_PLAIN, T, false>(W, ws, Y, M, N, K, (M + 127) / 128, none, stream); return launch_status();
-    case 6: launch_mmq<F, 2, 2, 1, 1, 128, 4, MODE_PLAIN, T, false>(W, ws, Y, M, N, K, (M + 63) / 64, none, stream); return launch_status();
-    case 9: launch_mmq<F, 2, 2, 1, 1, 128, 4, MODE_KSPLIT, T, false>(W, ws, Y, M, N, K, (M + 63) / 64, none, stream); return launch_status();
-    case 8: launch_mmq<F, 4, 2, 1, 2, 128, 4, MODE_PREFETCH, T, false>(W, ws, Y, M, N, K, (M + 127) / 128, none, stream); return launch_status();
+    case 1: launch_mmq<F, 4, 1, 1, 2, 128, 4, MODE_PINGPONG, T, false>(W, ws, Y, M, N, K, (M + 127) / 128, none, stream, la); return launch_status();
+    case 3: launch_mmq<F, 2, 1, 1, 1, 128, 4, MODE_PINGPONG, T, false>(W, ws, Y, M, N, K, (M + 63) / 64, none, stream, la); return launch_status();
+    case 5: launch_mmq<F, 4, 2, 1, 2, 128, 4, MODE_PLAIN, T, false>(W, ws, Y, M, N, K, (M + 127) / 128, none, stream, la); return launch_status();
+    case 6: launch_mmq<F, 2, 2, 1, 1, 128, 4, MODE_PLAIN, T, false>(W, ws, Y, M, N, K, (M + 63) / 64, none, stream, la); return launch_status();
+    case 9: launch_mmq<F, 2, 2, 1, 1, 128, 4, MODE_KSPLIT, T, false>(W, ws, Y, M, N, K, (M + 63) / 64, none, stream, la); return launch_status();
+    case 8: launch_mmq<F, 4, 2, 1, 2, 128, 4, MODE_PREFETCH, T, false>(W, ws, Y, M, N, K, (M + 127) / 128, none, stream, la); return launch_status();
     default: break;
   }
 #endif
   const int64_t small_tiles = (int64_t)((M + 63) / 64) * ((N + 63) / 64);
   if (large_tiles >= 400) {
     constexpr int MODE = F::LIGHT ? MODE_PREFETCH : MODE_PLAIN;
-    launch_mmq<F, 4, 2, 1, 2, 128, 4, MODE, T, false>(W, ws, Y, M, N, K, (M + 127) / 128, none, stream);
+    launch_mmq<F, 4, 2, 1, 2, 128, 4, MODE, T, false>(W, ws, Y, M, N, K, (M + 127) / 128, none, stream, la);
   } else if (small_tiles > 512) {
-    launch_mmq<F, 2, 2, 1, 1, 128, 4, MODE_PLAIN, T, false>(W, ws, Y, M, N, K, (M + 63) / 64, none, stream);
+    launch_mmq<F, 2, 2, 1, 1, 128, 4, MODE_PLAIN, T, false>(W, ws, Y, M, N, K, (M + 63) / 64, none, stream, la);
   } else {  // at most two workgroups per CU: double the waves of each by splitting the step's blocks
-    launch_mmq<F, 2, 2, 1, 1, 128, 4, MODE_KSPLIT, T, false>(W, ws, Y, M, N, K, (M + 63) / 64, none, stream);
+    launch_mmq<F, 2, 2, 1, 1, 128, 4, MODE_KSPLIT, T, false>(W, ws, Y, M, N, K, (M + 63) / 64, none, stream, la);
   }
   return launch_status();
 }
 
 template <class F>
-static int mmq_fmt(const void* W, const void* ws, void* Y, int dtype, int M, int N, int K, hipStream_t s) {
+static int mmq_fmt(const void* W, const void* ws, void* Y, int dtype, int M, int N, int K, hipStream_t s, const LinearArgs& la) {
 #ifdef GGUF_MMQ_TUNE
   if (dtype != GGUF_DTYPE_F16) return GGUF_ERR_DTYPE;
-  return mmq_typed<F, _Float16>(W, ws, Y, M, N, K, s);
+  return mmq_typed<F, _Float16>(W, ws, Y, M, N, K, s, la);
 #else
-  GGUF_DISPATCH_DTYPE(dtype, return (mmq_typed<F, scalar_t>(W, ws, Y, M, N, K, s)));
+  GGUF_DISPATCH_DTYPE(dtype, return (mmq_typed<F, scalar_t>(W, ws, Y, M, N, K, s, la)));
   return GGUF_ERR_DTYPE;
 #endif
 }
@@ -609,7 +610,7 @@ static bool mmq_type_ok(int type) {
 
 // mmq_h.hip
 int mmq_half(const void* W, const void* ws, void* Y, int dtype, int type, int M, int N, int K, float* partial,
-             int64_t partial_bytes, hipStream_t s);
+             int64_t partial_bytes, hipStream_t s, const LinearArgs& la);
 bool mmq_half_supported(int type);
 int64_t mmq_half_partial_bytes(int M, int N, int K);
 
@@ -623,11 +624,17 @@ extern "C" int64_t gguf_mmq_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   return mmq_rows_bytes(M, K) + gguf::mmq_half_partial_bytes((int)M, (int)N, (int)K);
 }
 
-extern "C" int gguf_mmq_engine(const void* W, const void* x, int xdtype, void* q8_workspace, void* Y, int type, int64_t N,
-                               int64_t K, int64_t M, int engine, int64_t workspace_bytes, gguf_stream_t stream) {
+extern "C" int gguf_mmq_linear(const void* W, int64_t w_row_pitch_bytes, const void* x, int xdtype, void* q8_workspace, void* Y,
+                               int64_t y_row_pitch, const void* bias, int type, int64_t N, int64_t K, int64_t M, int engine,
+                               int64_t workspace_bytes, gguf_stream_t stream) {
   using namespace gguf;
   const int qk = block_elems(type);
   if (qk == 0 || !mmq_type_ok(type)) return GGUF_ERR_TYPE;
+  if (K > 0 && K % qk == 0 && (w_row_pitch_bytes < K / qk * block_bytes(type) || y_row_pitch < N)) return GGUF_ERR_SHAPE;
+  LinearArgs la;
+  la.w_pitch = w_row_pitch_bytes;
+  la.ldy = y_row_pitch;
+  la.bias = bias;
   if (N < 0 || M < 0 || K <= 0 || K % qk != 0 || N > 0x7FFFFFF0LL || K > 0x7FFFFFF0LL || M > 0x7FFFFFF0LL) return GGUF_ERR_SHAPE;
   if (xdtype < 0 || xdtype > 2) return GGUF_ERR_DTYPE;
   if (engine < GGUF_MMQ_AUTO || engine > GGUF_MMQ_HALF || workspace_bytes < 0) return GGUF_ERR_SHAPE;
@@ -643,25 +650,34 @@ extern "C" int gguf_mmq_engine(const void* W, const void* x, int xdtype, void* q
     if (rc != GGUF_OK) return rc;
     float* partial = (float*)((char*)q8_workspace + mmq_rows_bytes(M, K));
     const int64_t partial_bytes = workspace_bytes > mmq_rows_bytes(M, K) ? workspace_bytes - mmq_rows_bytes(M, K) : 0;
-    return mmq_half(W, q8_workspace, Y, xdtype, type, (int)M, (int)N, (int)K, partial, partial_bytes, s);
+    return mmq_half(W, q8_workspace, Y, xdtype, type, (int)M, (int)N, (int)K, partial, partial_bytes, s, la);
   }
   const int rc = quantize_q8_1(x, xdtype, q8_workspace, M, K, s);
   if (rc != GGUF_OK) return rc;
   switch (type) {
-    case T_Q4_0: return mmq_fmt<MQ4_0>(W, q8_workspace, Y, xdtype, (int)M, (int)N, (int)K, s);
-    case T_Q4_1: return mmq_fmt<MQ4_1>(W, q8_workspace, Y, xdtype, (int)M, (int)N, (int)K, s);
-    case T_Q5_0: return mmq_fmt<MQ5_0>(W, q8_workspace, Y, xdtype, (int)M, (int)N, (int)K, s);
-    case T_Q5_1: return mmq_fmt<MQ5_1>(W, q8_workspace, Y, xdtype, (int)M, (int)N, (int)K, s);
-    case T_Q2_K: return mmq_fmt<MQ2_K>(W, q8_workspace, Y, xdtype, (int)M, (int)N, (int)K, s);
-    case T_Q3_K: return mmq_fmt<MQ3_K>(W, q8_workspace, Y, xdtype, (int)M, (int)N, (int)K, s);
-    case T_Q5_K: return mmq_fmt<MQ5_K>(W, q8_workspace, Y, xdtype, (int)M, (int)N, (int)K, s);
-    case T_Q8_0: return mmq_fmt<MQ8_0>(W, q8_workspace, Y, xdtype, (int)M, (int)N, (int)K, s);
-    case T_Q4_K: return mmq_fmt<MQ4_K>(W, q8_workspace, Y, xdtype, (int)M, (int)N, (int)K, s);
-    case T_Q6_K: return mmq_fmt<MQ6_K>(W, q8_workspace, Y, xdtype, (int)M, (int)N, (int)K, s);
-    case T_IQ4_XS: return mmq_fmt<MIQ4_XS>(W, q8_workspace, Y, xdtype, (int)M, (int)N, (int)K, s);
-    case T_IQ2_XXS: return mmq_fmt<MIQ2_XXS>(W, q8_workspace, Y, xdtype, (int)M, (int)N, (int)K, s);
+    case T_Q4_0: return mmq_fmt<MQ4_0>(W, q8_workspace, Y, xdtype, (int)M, (int)N, (int)K, s, la);
+    case T_Q4_1: return mmq_fmt<MQ4_1>(W, q8_workspace, Y, xdtype, (int)M, (int)N, (int)K, s, la);
+    case T_Q5_0: return mmq_fmt<MQ5_0>(W, q8_workspace, Y, xdtype, (int)M, (int)N, (int)K, s, la);
+    case T_Q5_1: return mmq_fmt<MQ5_1>(W, q8_workspace, Y, xdtype, (int)M, (int)N, (int)K, s, la);
+    case T_Q2_K: return mmq_fmt<MQ2_K>(W, q8_workspace, Y, xdtype, (int)M, (int)N, (int)K, s, la);
+    case T_Q3_K: return mmq_fmt<MQ3_K>(W, q8_workspace, Y, xdtype, (int)M, (int)N, (int)K, s, la);
+    case T_Q5_K: return mmq_fmt<MQ5_K>(W, q8_workspace, Y, xdtype, (int)M, (int)N, (int)K, s, la);
+    case T_Q8_0: return mmq_fmt<MQ8_0>(W, q8_workspace, Y, xdtype, (int)M, (int)N, (int)K, s, la);
+    case T_Q4_K: return mmq_fmt<MQ4_K>(W, q8_workspace, Y, xdtype, (int)M, (int)N, (int)K, s, la);
+    case T_Q6_K: return mmq_fmt<MQ6_K>(W, q8_workspace, Y, xdtype, (int)M, (int)N, (int)K, s, la);
+    case T_IQ4_XS: return mmq_fmt<MIQ4_XS>(W, q8_workspace, Y, xdtype, (int)M, (int)N, (int)K, s, la);
+    case T_IQ2_XXS: return mmq_fmt<MIQ2_XXS>(W, q8_workspace, Y, xdtype, (int)M, (int)N, (int)K, s, la);
   }
   return GGUF_ERR_TYPE;
+}
+
+extern "C" int gguf_mmq_engine(const void* W, const void* x, int xdtype, void* q8_workspace, void* Y, int type, int64_t N,
+                               int64_t K, int64_t M, int engine, int64_t workspace_bytes, gguf_stream_t stream) {
+  const int qk = gguf::block_elems(type);
+  if (qk == 0) return GGUF_ERR_TYPE;
+  if (K <= 0 || K % qk != 0) return GGUF_ERR_SHAPE;
+  return gguf_mmq_linear(W, K / qk * gguf::block_bytes(type), x, xdtype, q8_workspace, Y, N, nullptr, type, N, K, M, engine,
+                         workspace_bytes, stream);
 }
 
 extern "C" int gguf_mmq(const void* W, const void* x, int xdtype, void* q8_workspace, void* Y, int type, int64_t N,

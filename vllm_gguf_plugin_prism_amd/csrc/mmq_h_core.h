@@ -136,7 +136,7 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void mmqh_kernel(const uint8_t* 
                                                                   const char* __restrict__ ws, int64_t ws_row_bytes,
                                                                   T* __restrict__ Y, float* __restrict__ partial, int M, int N,
                                                                   int K, int Kp, int tiles_x, int whole_tiles, int shared_tiles, int splits,
-                                                                  int dbg) {
+                                                                  int64_t w_pitch, int64_t ldy, const T* __restrict__ bias, int dbg) {
 #ifndef GGUF_MMQ_TUNE
   (void)dbg;
 #define DBG_SKIP(bit, cond) false
@@ -168,7 +168,7 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void mmqh_kernel(const uint8_t* 
   const int split = wg < whole_tiles ? 0 : (wg - whole_tiles) / shared_tiles;                  // the same stretch of K
   const int nsplit = wg < whole_tiles ? 1 : splits;
   const int m_base = (tile / tiles_x) * M_T, n_base = (tile % tiles_x) * N_T;
-  const int64_t rowbytes = (int64_t)(K / F::QK) * F::BS;
+  const int64_t rowbytes = w_pitch;   // bytes between rows of W: the dense row size unless the caller's tensor is padded
   const int nkb_total = K >> 5;
   const int nsteps = (K + KS - 1) / KS;
 
@@ -356,7 +356,7 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void mmqh_kernel(const uint8_t* 
       for (int i = 0; i < TN; ++i) {
         const int nl = 32 * (wn * TN + i) + lrow, n = n_base + nl;
         if (my_partial) my_partial[ml * N_T + nl] = acc[j][i][r];   // the whole tile, edges included: the adder masks them
-        else if (mt < M && n < N) Y[(int64_t)mt * N + n] = from_f32<T>(acc[j][i][r] * HP_UNSCALE);
+        else if (mt < M && n < N) Y[(int64_t)mt * ldy + n] = finish<T>(acc[j][i][r] * HP_UNSCALE, bias, n);
       }
     }
   }
@@ -374,7 +374,8 @@ static int tune_dbg() {
 // Y tile = T(sum of its `splits` fp32 partial tiles / 16), gridDim.y workgroups per split tile, fixed order of addition
 template <int M_T, int N_T, typename T>
 __global__ __launch_bounds__(256) void mmqh_reduce_kernel(const float* __restrict__ partial, T* __restrict__ Y, int M, int N,
-                                                          int tiles_x, int whole_tiles, int splits) {
+                                                          int tiles_x, int whole_tiles, int splits, int64_t ldy,
+                                                          const T* __restrict__ bias) {
   const int tile = whole_tiles + blockIdx.x;
   const int m_base = (tile / tiles_x) * M_T, n_base = (tile % tiles_x) * N_T;
   const float* p = partial + (int64_t)blockIdx.x * splits * (M_T * N_T);
@@ -389,7 +390,7 @@ __global__ __launch_bounds__(256) void mmqh_reduce_kernel(const float* __restric
     const float out[4] = {acc.x, acc.y, acc.z, acc.w};
 #pragma unroll
     for (int e = 0; e < 4; ++e)
-      if (n + e < N) Y[(int64_t)m * N + n + e] = from_f32<T>(out[e] * HP_UNSCALE);
+      if (n + e < N) Y[(int64_t)m * ldy + n + e] = finish<T>(out[e] * HP_UNSCALE, bias, n + e);
   }
 }
 
@@ -407,7 +408,9 @@ MmqhPlan mmq_half_plan(int M, int N, int K, int64_t partial_bytes_available);  /
 
 template <class C, int WM, int WN, int TM, int TN, int OCC, typename T>
 static void launch_mmqh(const void* W, const void* ws, void* Y, int M, int N, int K, hipStream_t stream, int whole = -1, int shared = 0,
-                        int splits = 1, float* partial = nullptr) {
+                        int splits = 1, float* partial = nullptr, const LinearArgs& la = LinearArgs()) {
+  using F = typename C::Fmt;
+  const int64_t w_pitch = la.w_pitch ? la.w_pitch : (int64_t)(K / F::QK) * F::BS, ldy = la.ldy ? la.ldy : (int64_t)N;
   constexpr int M_T = 32 * WM * TM, N_T = 32 * WN * TN;
   constexpr size_t lds = (size_t)(M_T + N_T) * (64 + 8) * 2 * 2;
   auto kern = mmqh_kernel<C, WM, WN, TM, TN, OCC, T>;
@@ -422,10 +425,11 @@ static void launch_mmqh(const void* W, const void* ws, void* Y, int M, int N, in
   if (whole < 0) { whole = tiles; shared = 0; splits = 1; }
   const _Float16* xh = (const _Float16*)((const char*)ws + (int64_t)M * q8_row_bytes(K));
   hipLaunchKernelGGL(kern, dim3(whole + shared * splits), dim3(64 * WM * WN), lds, stream, (const uint8_t*)W, xh, (const char*)ws,
-                     q8_row_bytes(K), (T*)Y, partial, M, N, K, (int)q8_kp(K), tiles_x, whole, shared > 0 ? shared : 1, splits, tune_dbg());
+                     q8_row_bytes(K), (T*)Y, partial, M, N, K, (int)q8_kp(K), tiles_x, whole, shared > 0 ? shared : 1, splits, w_pitch, ldy,
+                     (const T*)la.bias, tune_dbg());
   if (shared > 0)
     hipLaunchKernelGGL((mmqh_reduce_kernel<M_T, N_T, T>), dim3(shared, M_T * N_T / 1024), dim3(256), 0, stream, partial, (T*)Y, M, N, tiles_x,
-                       whole, splits);
+                       whole, splits, ldy, (const T*)la.bias);
 }
 
 #ifdef GGUF_MMQ_TUNE
@@ -437,7 +441,7 @@ static int tune_cfg_h() {
 
 template <class C, typename T>
 static int mmqh_typed(const void* W, const void* ws, void* Y, int M, int N, int K, float* partial, int64_t partial_bytes,
-                      hipStream_t stream) {
+                      hipStream_t stream, const LinearArgs& la = LinearArgs()) {
 #ifdef GGUF_MMQ_TUNE
   switch (tune_cfg_h()) {
     case 1: launch_mmqh<C, 4, 2, 2, 2, 1, T>(W, ws, Y, M, N, K, stream); return launch_status();   // 256 x 128, 8 waves
@@ -454,10 +458,10 @@ static int mmqh_typed(const void* W, const void* ws, void* Y, int M, int N, int 
 #endif
   const MmqhPlan p = mmq_half_plan(M, N, K, partial_bytes);
   switch (p.cfg) {
-    case 0: launch_mmqh<C, 4, 2, 2, 2, 1, T>(W, ws, Y, M, N, K, stream, p.whole, p.shared, p.splits, partial); break;  // 256 x 128, 8 waves
-    case 1: launch_mmqh<C, 4, 2, 1, 2, 2, T>(W, ws, Y, M, N, K, stream, p.whole, p.shared, p.splits, partial); break;  // 128 x 128, 8 waves
-    case 2: launch_mmqh<C, 2, 2, 2, 1, 2, T>(W, ws, Y, M, N, K, stream, p.whole, p.shared, p.splits, partial); break;  // 128 x 64, 4 waves
-    default: launch_mmqh<C, 2, 2, 1, 1, 4, T>(W, ws, Y, M, N, K, stream, p.whole, p.shared, p.splits, partial); break; // 64 x 64, 4 waves
+    case 0: launch_mmqh<C, 4, 2, 2, 2, 1, T>(W, ws, Y, M, N, K, stream, p.whole, p.shared, p.splits, partial, la); break;  // 256 x 128, 8 waves
+    case 1: launch_mmqh<C, 4, 2, 1, 2, 2, T>(W, ws, Y, M, N, K, stream, p.whole, p.shared, p.splits, partial, la); break;  // 128 x 128, 8 waves
+    case 2: launch_mmqh<C, 2, 2, 2, 1, 2, T>(W, ws, Y, M, N, K, stream, p.whole, p.shared, p.splits, partial, la); break;  // 128 x 64, 4 waves
+    default: launch_mmqh<C, 2, 2, 1, 1, 4, T>(W, ws, Y, M, N, K, stream, p.whole, p.shared, p.splits, partial, la); break; // 64 x 64, 4 waves
   }
   return launch_status();
 }

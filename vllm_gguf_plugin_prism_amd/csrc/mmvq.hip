@@ -5,19 +5,19 @@
 namespace gguf {
 
 int mmvq_group_std_a(int type, const void* W, const void* x, void* ws, void* Y, int dtype, int64_t N, int64_t K, int64_t M,
-                   hipStream_t s);
+                   hipStream_t s, const LinearArgs& la);
 int mmvq_group_std_b(int type, const void* W, const void* x, void* ws, void* Y, int dtype, int64_t N, int64_t K, int64_t M,
-                   hipStream_t s);
+                   hipStream_t s, const LinearArgs& la);
 int mmvq_group_k_a(int type, const void* W, const void* x, void* ws, void* Y, int dtype, int64_t N, int64_t K, int64_t M,
-                   hipStream_t s);
+                   hipStream_t s, const LinearArgs& la);
 int mmvq_group_k_b(int type, const void* W, const void* x, void* ws, void* Y, int dtype, int64_t N, int64_t K, int64_t M,
-                   hipStream_t s);
+                   hipStream_t s, const LinearArgs& la);
 int mmvq_group_iq_a(int type, const void* W, const void* x, void* ws, void* Y, int dtype, int64_t N, int64_t K, int64_t M,
-                   hipStream_t s);
+                   hipStream_t s, const LinearArgs& la);
 int mmvq_group_iq_b(int type, const void* W, const void* x, void* ws, void* Y, int dtype, int64_t N, int64_t K, int64_t M,
-                   hipStream_t s);
+                   hipStream_t s, const LinearArgs& la);
 int mmvq_group_iq_c(int type, const void* W, const void* x, void* ws, void* Y, int dtype, int64_t N, int64_t K, int64_t M,
-                   hipStream_t s);
+                   hipStream_t s, const LinearArgs& la);
 
 int moe_vec_group_std_a(int type, const void* W, const void* x, void* Y, int dtype, int N, int K, const int32_t* ids, int top_k,
                       int pairs, int act, int num_experts, void* scratch, int64_t scratch_bytes, hipStream_t s);
@@ -36,38 +36,52 @@ int moe_vec_group_iq_c(int type, const void* W, const void* x, void* Y, int dtyp
 
 }  // namespace gguf
 
-extern "C" int gguf_mmvq(const void* W, const void* x, int xdtype, void* q8_workspace, void* Y, int type, int64_t N,
-                         int64_t K, int64_t M, gguf_stream_t stream) {
+extern "C" int gguf_mmvq_linear(const void* W, int64_t w_row_pitch_bytes, const void* x, int xdtype, void* q8_workspace, void* Y,
+                                int64_t y_row_pitch, const void* bias, int type, int64_t N, int64_t K, int64_t M,
+                                gguf_stream_t stream) {
   using namespace gguf;
   const int qk = block_elems(type);
   if (qk == 0) return GGUF_ERR_TYPE;
   if (N < 0 || M < 0 || K <= 0 || K % qk != 0 || N > 0x7FFFFFF0LL || K > 0x7FFFFFF0LL) return GGUF_ERR_SHAPE;
+  if (w_row_pitch_bytes < K / qk * block_bytes(type) || y_row_pitch < N) return GGUF_ERR_SHAPE;
+  LinearArgs la;
+  la.w_pitch = w_row_pitch_bytes;
+  la.ldy = y_row_pitch;
+  la.bias = bias;
   if (xdtype < 0 || xdtype > 2) return GGUF_ERR_DTYPE;
   if (N == 0 || M == 0) return GGUF_OK;
   if (!W || !x || !q8_workspace || !Y) return GGUF_ERR_NULL;
   hipStream_t s = (hipStream_t)stream;
   switch (type) {
-    case T_Q4_0: return mmvq_group_std_a(type, W, x, q8_workspace, Y, xdtype, N, K, M, s);
-    case T_Q4_1: return mmvq_group_std_a(type, W, x, q8_workspace, Y, xdtype, N, K, M, s);
-    case T_Q8_0: return mmvq_group_std_a(type, W, x, q8_workspace, Y, xdtype, N, K, M, s);
-    case T_Q5_0: return mmvq_group_std_b(type, W, x, q8_workspace, Y, xdtype, N, K, M, s);
-    case T_Q5_1: return mmvq_group_std_b(type, W, x, q8_workspace, Y, xdtype, N, K, M, s);
-    case T_IQ4_NL: return mmvq_group_std_b(type, W, x, q8_workspace, Y, xdtype, N, K, M, s);
-    case T_Q2_K: return mmvq_group_k_a(type, W, x, q8_workspace, Y, xdtype, N, K, M, s);
-    case T_Q3_K: return mmvq_group_k_a(type, W, x, q8_workspace, Y, xdtype, N, K, M, s);
-    case T_Q6_K: return mmvq_group_k_a(type, W, x, q8_workspace, Y, xdtype, N, K, M, s);
-    case T_Q4_K: return mmvq_group_k_b(type, W, x, q8_workspace, Y, xdtype, N, K, M, s);
-    case T_Q5_K: return mmvq_group_k_b(type, W, x, q8_workspace, Y, xdtype, N, K, M, s);
-    case T_IQ4_XS: return mmvq_group_iq_a(type, W, x, q8_workspace, Y, xdtype, N, K, M, s);
-    case T_IQ2_XXS: return mmvq_group_iq_a(type, W, x, q8_workspace, Y, xdtype, N, K, M, s);
-    case T_IQ3_XXS: return mmvq_group_iq_a(type, W, x, q8_workspace, Y, xdtype, N, K, M, s);
-    case T_IQ2_XS: return mmvq_group_iq_b(type, W, x, q8_workspace, Y, xdtype, N, K, M, s);
-    case T_IQ2_S: return mmvq_group_iq_b(type, W, x, q8_workspace, Y, xdtype, N, K, M, s);
-    case T_IQ3_S: return mmvq_group_iq_b(type, W, x, q8_workspace, Y, xdtype, N, K, M, s);
-    case T_IQ1_S: return mmvq_group_iq_c(type, W, x, q8_workspace, Y, xdtype, N, K, M, s);
-    case T_IQ1_M: return mmvq_group_iq_c(type, W, x, q8_workspace, Y, xdtype, N, K, M, s);
+    case T_Q4_0: return mmvq_group_std_a(type, W, x, q8_workspace, Y, xdtype, N, K, M, s, la);
+    case T_Q4_1: return mmvq_group_std_a(type, W, x, q8_workspace, Y, xdtype, N, K, M, s, la);
+    case T_Q8_0: return mmvq_group_std_a(type, W, x, q8_workspace, Y, xdtype, N, K, M, s, la);
+    case T_Q5_0: return mmvq_group_std_b(type, W, x, q8_workspace, Y, xdtype, N, K, M, s, la);
+    case T_Q5_1: return mmvq_group_std_b(type, W, x, q8_workspace, Y, xdtype, N, K, M, s, la);
+    case T_IQ4_NL: return mmvq_group_std_b(type, W, x, q8_workspace, Y, xdtype, N, K, M, s, la);
+    case T_Q2_K: return mmvq_group_k_a(type, W, x, q8_workspace, Y, xdtype, N, K, M, s, la);
+    case T_Q3_K: return mmvq_group_k_a(type, W, x, q8_workspace, Y, xdtype, N, K, M, s, la);
+    case T_Q6_K: return mmvq_group_k_a(type, W, x, q8_workspace, Y, xdtype, N, K, M, s, la);
+    case T_Q4_K: return mmvq_group_k_b(type, W, x, q8_workspace, Y, xdtype, N, K, M, s, la);
+    case T_Q5_K: return mmvq_group_k_b(type, W, x, q8_workspace, Y, xdtype, N, K, M, s, la);
+    case T_IQ4_XS: return mmvq_group_iq_a(type, W, x, q8_workspace, Y, xdtype, N, K, M, s, la);
+    case T_IQ2_XXS: return mmvq_group_iq_a(type, W, x, q8_workspace, Y, xdtype, N, K, M, s, la);
+    case T_IQ3_XXS: return mmvq_group_iq_a(type, W, x, q8_workspace, Y, xdtype, N, K, M, s, la);
+    case T_IQ2_XS: return mmvq_group_iq_b(type, W, x, q8_workspace, Y, xdtype, N, K, M, s, la);
+    case T_IQ2_S: return mmvq_group_iq_b(type, W, x, q8_workspace, Y, xdtype, N, K, M, s, la);
+    case T_IQ3_S: return mmvq_group_iq_b(type, W, x, q8_workspace, Y, xdtype, N, K, M, s, la);
+    case T_IQ1_S: return mmvq_group_iq_c(type, W, x, q8_workspace, Y, xdtype, N, K, M, s, la);
+    case T_IQ1_M: return mmvq_group_iq_c(type, W, x, q8_workspace, Y, xdtype, N, K, M, s, la);
   }
   return GGUF_ERR_TYPE;
+}
+
+extern "C" int gguf_mmvq(const void* W, const void* x, int xdtype, void* q8_workspace, void* Y, int type, int64_t N,
+                         int64_t K, int64_t M, gguf_stream_t stream) {
+  const int qk = gguf::block_elems(type);
+  if (qk == 0) return GGUF_ERR_TYPE;
+  if (K <= 0 || K % qk != 0) return GGUF_ERR_SHAPE;
+  return gguf_mmvq_linear(W, K / qk * gguf::block_bytes(type), x, xdtype, q8_workspace, Y, N, nullptr, type, N, K, M, stream);
 }
 
 extern "C" int gguf_moe_vec_act(const void* X, int xdtype, void* q8_workspace, const void* W, const int32_t* topk_ids,

@@ -66,7 +66,7 @@ struct MoeVecArgs {
 template <class F, int MT, int RPW, typename T, bool MOE, bool FUSEQ>
 __global__ __launch_bounds__(256) void mmvq_kernel(const uint8_t* __restrict__ W, const char* __restrict__ xsrc,
                                                     T* __restrict__ Y, int N, int K, int kchunk, int64_t x_row_bytes,
-                                                    int64_t y_vec_stride, MoeVecArgs moe) {
+                                                    int64_t y_vec_stride, MoeVecArgs moe, int64_t w_pitch, const T* __restrict__ bias) {
   extern __shared__ __align__(16) char smem[];
   __shared__ int s_xrow[MT], s_yrow[MT];  // activation row and output row of every staged vector (MOE)
   const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
@@ -99,7 +99,7 @@ __global__ __launch_bounds__(256) void mmvq_kernel(const uint8_t* __restrict__ W
   if (F::TABLE_BYTES > 0) __syncthreads();
 
   const int row0 = (blockIdx.x * 4 + wave) * RPW;
-  const int64_t rowbytes = (int64_t)(K / F::QK) * F::BS;
+  const int64_t rowbytes = w_pitch;   // bytes between rows: the dense row size unless the caller's tensor is padded
   const uint8_t* rows[RPW];
 #pragma unroll
   for (int r = 0; r < RPW; ++r) rows[r] = W + (int64_t)min(row0 + r, N - 1) * rowbytes;
@@ -190,7 +190,7 @@ __global__ __launch_bounds__(256) void mmvq_kernel(const uint8_t* __restrict__ W
     for (int m = 0; m < MT; ++m) {
       const float v = wave_sum(acc[r][m]);
       const int yrow = MOE ? s_yrow[m] : m;
-      if (lane == 0 && row0 + r < N && yrow >= 0) Y[(int64_t)yrow * y_vec_stride + row0 + r] = from_f32<T>(v);
+      if (lane == 0 && row0 + r < N && yrow >= 0) Y[(int64_t)yrow * y_vec_stride + row0 + r] = finish<T>(v, bias, row0 + r);
     }
   }
 }
@@ -221,7 +221,8 @@ __global__ __launch_bounds__(256) void mmvq_kernel(const uint8_t* __restrict__ W
 
 template <class F, int MT, int NW, int D, typename T>
 __global__ __launch_bounds__(64 * NW) void mmvq_stream_kernel(const uint8_t* __restrict__ W, const T* __restrict__ X,
-                                                               T* __restrict__ Y, int N, int K, int rows_per_wg) {
+                                                               T* __restrict__ Y, int N, int K, int rows_per_wg, int64_t w_pitch,
+                                                               int64_t ldy, const T* __restrict__ bias) {
   extern __shared__ __align__(16) char smem[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: row arithmetic stays on the scalar unit
@@ -238,7 +239,7 @@ __global__ __launch_bounds__(64 * NW) void mmvq_stream_kernel(const uint8_t* __r
   const int r_end = min(N, r_begin + rows_per_wg);
   if (r_begin >= r_end) return;
   const int nrows = r_end - r_begin;
-  const int64_t rowbytes = (int64_t)(K / F::QK) * F::BS;
+  const int64_t rowbytes = w_pitch;   // bytes between rows: the dense row size unless the caller's tensor is padded
 
   // this wave: slot (which of the side-by-side rows) and step (which 64-unit stretch of the row)
   const int slot = wave / S, step = wave - slot * S;
@@ -357,7 +358,7 @@ __global__ __launch_bounds__(64 * NW) void mmvq_stream_kernel(const uint8_t* __r
     const int row = i / MT, m = i - row * MT;
     float v = 0.0f;
     for (int st = 0; st < S; ++st) v += part[(row * S + st) * MT + m];
-    Y[(int64_t)m * N + r_begin + row] = from_f32<T>(v);
+    Y[(int64_t)m * ldy + r_begin + row] = finish<T>(v, bias, r_begin + row);
   }
 }
 
@@ -373,7 +374,7 @@ static int num_cus() {
 }
 
 template <class F, int MT, int D, typename T>
-static void launch_stream_d(const void* W, const T* X, T* Y, int N, int K, int rows_per_wg, int grid, size_t lds,
+static void launch_stream_d(const void* W, const T* X, T* Y, int N, int K, int rows_per_wg, int grid, size_t lds, const LinearArgs& la,
                             hipStream_t stream) {
   constexpr int NW = GGUF_MMVQ_NW;
   auto kern = mmvq_stream_kernel<F, MT, NW, D, T>;
@@ -382,13 +383,14 @@ static void launch_stream_d(const void* W, const T* X, T* Y, int N, int K, int r
     (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
     big_lds = true;
   }
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * NW), lds, stream, (const uint8_t*)W, X, Y, N, K, rows_per_wg);
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * NW), lds, stream, (const uint8_t*)W, X, Y, N, K, rows_per_wg,
+                     la.w_pitch ? la.w_pitch : (int64_t)(K / F::QK) * F::BS, la.ldy ? la.ldy : (int64_t)N, (const T*)la.bias);
 }
 
 // Returns false when the shape does not fit the streaming kernel (a row longer than NW waves, or activations
 // that do not fit in LDS); the caller then takes the workspace path.
 template <class F, int MT, typename T>
-static bool launch_stream(const void* W, const T* X, T* Y, int N, int K, hipStream_t stream) {
+static bool launch_stream(const void* W, const T* X, T* Y, int N, int K, hipStream_t stream, const LinearArgs& la) {
   constexpr int NW = GGUF_MMVQ_NW;
   const int nb = K / 32, S = (nb + 63) / 64;
   if (S > NW) return false;
@@ -401,9 +403,9 @@ static bool launch_stream(const void* W, const T* X, T* Y, int N, int K, hipStre
                      (size_t)rows_per_wg * S * MT * 4;
   if (lds > 150 * 1024) return false;
   const int per_wave = (rows_per_wg + slots - 1) / slots;  // rows each wave walks; the pipeline depth never exceeds it
-  if (per_wave >= GGUF_MMVQ_DEPTH) launch_stream_d<F, MT, GGUF_MMVQ_DEPTH, T>(W, X, Y, N, K, rows_per_wg, grid, lds, stream);
-  else if (per_wave >= 2) launch_stream_d<F, MT, 2, T>(W, X, Y, N, K, rows_per_wg, grid, lds, stream);
-  else launch_stream_d<F, MT, 1, T>(W, X, Y, N, K, rows_per_wg, grid, lds, stream);
+  if (per_wave >= GGUF_MMVQ_DEPTH) launch_stream_d<F, MT, GGUF_MMVQ_DEPTH, T>(W, X, Y, N, K, rows_per_wg, grid, lds, la, stream);
+  else if (per_wave >= 2) launch_stream_d<F, MT, 2, T>(W, X, Y, N, K, rows_per_wg, grid, lds, la, stream);
+  else launch_stream_d<F, MT, 1, T>(W, X, Y, N, K, rows_per_wg, grid, lds, la, stream);
   return true;
 }
 
@@ -426,28 +428,31 @@ static inline size_t mmvq_lds(int kchunk) {
 }
 
 template <class F, int MT, typename T, bool FUSEQ>
-static void launch_mt(const void* W, const char* xsrc, T* Y, int N, int K, hipStream_t stream) {
+static void launch_mt(const void* W, const char* xsrc, T* Y, int N, int K, hipStream_t stream, const LinearArgs& la) {
   constexpr int RPW = GGUF_MMVQ_RPW;
   const int kchunk = kchunk_for(MT, K);
   const int grid = (N + 4 * RPW - 1) / (4 * RPW);
   const int64_t xrb = FUSEQ ? (int64_t)K * (int64_t)sizeof(T) : q8_row_bytes(K);
   const size_t lds = mmvq_lds<F, MT>(kchunk);
   hipLaunchKernelGGL((mmvq_kernel<F, MT, RPW, T, false, FUSEQ>), dim3(grid), dim3(256), lds, stream,
-                     (const uint8_t*)W, xsrc, Y, N, K, kchunk, xrb, (int64_t)N, MoeVecArgs{nullptr, nullptr, nullptr, 1, 0, (int)ACT_NONE});
+                     (const uint8_t*)W, xsrc, Y, N, K, kchunk, xrb, la.ldy ? la.ldy : (int64_t)N,
+                     MoeVecArgs{nullptr, nullptr, nullptr, 1, 0, (int)ACT_NONE}, la.w_pitch ? la.w_pitch : (int64_t)(K / F::QK) * F::BS,
+                     (const T*)la.bias);
 }
 
 
 template <class F, typename T>
 static int mmvq_typed(const void* W, const void* x, void* ws, void* Y, int xdtype, int64_t N, int64_t K, int64_t M,
-                      hipStream_t stream) {
+                      hipStream_t stream, const LinearArgs& la) {
+  const int64_t ldy = la.ldy ? la.ldy : N;
   if (M <= MAX_FUSED_M) {
     const T* xs = (const T*)x;
     bool ok;
-    if (M == 1) ok = launch_stream<F, 1, T>(W, xs, (T*)Y, (int)N, (int)K, stream);
-    else if (M == 2) ok = launch_stream<F, 2, T>(W, xs, (T*)Y, (int)N, (int)K, stream);
-    else if (M == 4) ok = launch_stream<F, 4, T>(W, xs, (T*)Y, (int)N, (int)K, stream);
-    else ok = launch_stream<F, 2, T>(W, xs, (T*)Y, (int)N, (int)K, stream) &&
-              launch_stream<F, 1, T>(W, xs + 2 * K, (T*)Y + 2 * N, (int)N, (int)K, stream);
+    if (M == 1) ok = launch_stream<F, 1, T>(W, xs, (T*)Y, (int)N, (int)K, stream, la);
+    else if (M == 2) ok = launch_stream<F, 2, T>(W, xs, (T*)Y, (int)N, (int)K, stream, la);
+    else if (M == 4) ok = launch_stream<F, 4, T>(W, xs, (T*)Y, (int)N, (int)K, stream, la);
+    else ok = launch_stream<F, 2, T>(W, xs, (T*)Y, (int)N, (int)K, stream, la) &&
+              launch_stream<F, 1, T>(W, xs + 2 * K, (T*)Y + 2 * ldy, (int)N, (int)K, stream, la);
     if (ok) return launch_status();
   }
   const int rc = quantize_q8_1(x, xdtype, ws, M, K, stream);
@@ -457,11 +462,11 @@ static int mmvq_typed(const void* W, const void* x, void* ws, void* Y, int xdtyp
   while (m0 < M) {
     const int64_t left = M - m0;
     const char* wsm = (const char*)ws + m0 * rb;
-    T* ym = (T*)Y + m0 * N;
-    if (left >= 8) { launch_mt<F, 8, T, false>(W, wsm, ym, (int)N, (int)K, stream); m0 += 8; }
-    else if (left >= 4) { launch_mt<F, 4, T, false>(W, wsm, ym, (int)N, (int)K, stream); m0 += 4; }
-    else if (left >= 2) { launch_mt<F, 2, T, false>(W, wsm, ym, (int)N, (int)K, stream); m0 += 2; }
-    else { launch_mt<F, 1, T, false>(W, wsm, ym, (int)N, (int)K, stream); m0 += 1; }
+    T* ym = (T*)Y + m0 * ldy;
+    if (left >= 8) { launch_mt<F, 8, T, false>(W, wsm, ym, (int)N, (int)K, stream, la); m0 += 8; }
+    else if (left >= 4) { launch_mt<F, 4, T, false>(W, wsm, ym, (int)N, (int)K, stream, la); m0 += 4; }
+    else if (left >= 2) { launch_mt<F, 2, T, false>(W, wsm, ym, (int)N, (int)K, stream, la); m0 += 2; }
+    else { launch_mt<F, 1, T, false>(W, wsm, ym, (int)N, (int)K, stream, la); m0 += 1; }
   }
   return launch_status();
 }
@@ -509,7 +514,7 @@ static int moe_vec_typed(const void* W, const char* x, void* Y, int xdtype, int 
     const int ggrid = (N + 4 * GRPW - 1) / (4 * GRPW);
     hipLaunchKernelGGL((mmvq_kernel<F, MOE_VEC_GROUP, GRPW, T, true, false>), dim3(ggrid, (unsigned)block_cap), dim3(256), lds, stream,
                        (const uint8_t*)W, (const char*)scratch, (T*)Y, N, K, kchunk, q8_row_bytes(K), (int64_t)N,
-                       MoeVecArgs{topk_ids, sorted, experts, top_k, pairs, (int)ACT_NONE});
+                       MoeVecArgs{topk_ids, sorted, experts, top_k, pairs, (int)ACT_NONE}, (int64_t)(K / F::QK) * F::BS, (const T*)nullptr);
     return launch_status();
   }
   const int kchunk = kchunk_for(1, K);
@@ -520,7 +525,7 @@ static int moe_vec_typed(const void* W, const char* x, void* Y, int xdtype, int 
     if (z0 % top_k != 0) return GGUF_ERR_SHAPE;
     hipLaunchKernelGGL((mmvq_kernel<F, 1, RPW, T, true, true>), dim3(grid, nz), dim3(256), lds, stream,
                        (const uint8_t*)W, x + (int64_t)(z0 / top_k) * xrb, (T*)Y + (int64_t)z0 * N, N, K, kchunk, xrb,
-                       (int64_t)N, MoeVecArgs{topk_ids + z0, nullptr, nullptr, top_k, nz, act});
+                       (int64_t)N, MoeVecArgs{topk_ids + z0, nullptr, nullptr, top_k, nz, act}, (int64_t)(K / F::QK) * F::BS, (const T*)nullptr);
   }
   return launch_status();
 }
@@ -535,8 +540,8 @@ static int moe_vec_fmt(const void* W, const void* x, void* Y, int dtype, int N, 
 
 template <class F>
 static int mmvq_fmt(const void* W, const void* x, void* ws, void* Y, int dtype, int64_t N, int64_t K, int64_t M,
-                    hipStream_t s) {
-  GGUF_DISPATCH_DTYPE(dtype, return (mmvq_typed<F, scalar_t>(W, x, ws, Y, dtype, N, K, M, s)));
+                    hipStream_t s, const LinearArgs& la) {
+  GGUF_DISPATCH_DTYPE(dtype, return (mmvq_typed<F, scalar_t>(W, x, ws, Y, dtype, N, K, M, s, la)));
   return GGUF_ERR_DTYPE;
 }
 

@@ -5,11 +5,11 @@
 namespace gguf {
 
 int mmvq_group_iq_b(int type, const void* W, const void* x, void* ws, void* Y, int dtype, int64_t N, int64_t K, int64_t M,
-                   hipStream_t s) {
+                   hipStream_t s, const LinearArgs& la) {
   switch (type) {
-    case T_IQ2_XS: return mmvq_fmt<FmtIQ2_XS>(W, x, ws, Y, dtype, N, K, M, s);
-    case T_IQ2_S: return mmvq_fmt<FmtIQ2_S>(W, x, ws, Y, dtype, N, K, M, s);
-    case T_IQ3_S: return mmvq_fmt<FmtIQ3_S>(W, x, ws, Y, dtype, N, K, M, s);
+    case T_IQ2_XS: return mmvq_fmt<FmtIQ2_XS>(W, x, ws, Y, dtype, N, K, M, s, la);
+    case T_IQ2_S: return mmvq_fmt<FmtIQ2_S>(W, x, ws, Y, dtype, N, K, M, s, la);
+    case T_IQ3_S: return mmvq_fmt<FmtIQ3_S>(W, x, ws, Y, dtype, N, K, M, s, la);
     default: return GGUF_ERR_TYPE;
   }
 }

@@ -5,10 +5,10 @@
 namespace gguf {
 
 int mmvq_group_iq_c(int type, const void* W, const void* x, void* ws, void* Y, int dtype, int64_t N, int64_t K, int64_t M,
-                   hipStream_t s) {
+                   hipStream_t s, const LinearArgs& la) {
   switch (type) {
-    case T_IQ1_S: return mmvq_fmt<FmtIQ1_S>(W, x, ws, Y, dtype, N, K, M, s);
-    case T_IQ1_M: return mmvq_fmt<FmtIQ1_M>(W, x, ws, Y, dtype, N, K, M, s);
+    case T_IQ1_S: return mmvq_fmt<FmtIQ1_S>(W, x, ws, Y, dtype, N, K, M, s, la);
+    case T_IQ1_M: return mmvq_fmt<FmtIQ1_M>(W, x, ws, Y, dtype, N, K, M, s, la);
     default: return GGUF_ERR_TYPE;
   }
 }

@@ -5,11 +5,11 @@
 namespace gguf {
 
 int mmvq_group_k_a(int type, const void* W, const void* x, void* ws, void* Y, int dtype, int64_t N, int64_t K, int64_t M,
-                   hipStream_t s) {
+                   hipStream_t s, const LinearArgs& la) {
   switch (type) {
-    case T_Q2_K: return mmvq_fmt<FmtQ2_K>(W, x, ws, Y, dtype, N, K, M, s);
-    case T_Q3_K: return mmvq_fmt<FmtQ3_K>(W, x, ws, Y, dtype, N, K, M, s);
-    case T_Q6_K: return mmvq_fmt<FmtQ6_K>(W, x, ws, Y, dtype, N, K, M, s);
+    case T_Q2_K: return mmvq_fmt<FmtQ2_K>(W, x, ws, Y, dtype, N, K, M, s, la);
+    case T_Q3_K: return mmvq_fmt<FmtQ3_K>(W, x, ws, Y, dtype, N, K, M, s, la);
+    case T_Q6_K: return mmvq_fmt<FmtQ6_K>(W, x, ws, Y, dtype, N, K, M, s, la);
     default: return GGUF_ERR_TYPE;
   }
 }

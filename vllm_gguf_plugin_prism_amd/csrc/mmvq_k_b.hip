@@ -5,10 +5,10 @@
 namespace gguf {
 
 int mmvq_group_k_b(int type, const void* W, const void* x, void* ws, void* Y, int dtype, int64_t N, int64_t K, int64_t M,
-                   hipStream_t s) {
+                   hipStream_t s, const LinearArgs& la) {
   switch (type) {
-    case T_Q4_K: return mmvq_fmt<FmtQ4_K>(W, x, ws, Y, dtype, N, K, M, s);
-    case T_Q5_K: return mmvq_fmt<FmtQ5_K>(W, x, ws, Y, dtype, N, K, M, s);
+    case T_Q4_K: return mmvq_fmt<FmtQ4_K>(W, x, ws, Y, dtype, N, K, M, s, la);
+    case T_Q5_K: return mmvq_fmt<FmtQ5_K>(W, x, ws, Y, dtype, N, K, M, s, la);
     default: return GGUF_ERR_TYPE;
   }
 }

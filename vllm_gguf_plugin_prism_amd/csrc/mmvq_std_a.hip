@@ -5,11 +5,11 @@
 namespace gguf {
 
 int mmvq_group_std_a(int type, const void* W, const void* x, void* ws, void* Y, int dtype, int64_t N, int64_t K, int64_t M,
-                   hipStream_t s) {
+                   hipStream_t s, const LinearArgs& la) {
   switch (type) {
-    case T_Q4_0: return mmvq_fmt<FmtQ4_0>(W, x, ws, Y, dtype, N, K, M, s);
-    case T_Q4_1: return mmvq_fmt<FmtQ4_1>(W, x, ws, Y, dtype, N, K, M, s);
-    case T_Q8_0: return mmvq_fmt<FmtQ8_0>(W, x, ws, Y, dtype, N, K, M, s);
+    case T_Q4_0: return mmvq_fmt<FmtQ4_0>(W, x, ws, Y, dtype, N, K, M, s, la);
+    case T_Q4_1: return mmvq_fmt<FmtQ4_1>(W, x, ws, Y, dtype, N, K, M, s, la);
+    case T_Q8_0: return mmvq_fmt<FmtQ8_0>(W, x, ws, Y, dtype, N, K, M, s, la);
     default: return GGUF_ERR_TYPE;
   }
 }

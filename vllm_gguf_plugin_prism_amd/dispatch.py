@@ -64,28 +64,68 @@ def select_moe_path(weight_type: int, weight_type2: int, tokens: int) -> str:
 # ---------------------------------------------------------------------------------------- tensor level
 
 
-def fused_mul_mat_gguf(x, weight, weight_type: int):
-    """``x @ dequant(weight).T`` through the path the reference would pick (linear.py:35-58)."""
+def fused_mul_mat_gguf(x, weight, weight_type: int, *, out=None, bias=None):
+    """``x @ dequant(weight).T`` through the path the reference would pick (linear.py:35-58).
+
+    ``weight`` may be a slice ``merged[start:end, :row_bytes]`` of a padded merged tensor, ``out`` a column slice of the
+    merged result and ``bias`` the matching slice of the layer bias: the a8 kernels address all three in place."""
     import torch
 
     from . import ops
 
     rows = weight.shape[0]
     path = select_mul_mat_path(int(weight_type), x.shape[0], rows)
-    if path == "empty":
-        return torch.empty(x.shape[0], rows, dtype=x.dtype, device=x.device)
-    if path == "unquantized":
-        return x @ weight.T
     if path == "mmvq":
-        return ops.ggml_mul_mat_vec_a8(weight, x, weight_type, rows)
+        return ops.ggml_mul_mat_vec_a8(weight, x, weight_type, rows, out=out, bias=bias)
     if path == "mmq":
-        return ops.ggml_mul_mat_a8(weight, x, weight_type, rows)
-    # ops.ggml_dequant_gemm forms the same product without the dense copy of the weights; measured on MI355X it is
-    # faster than the two steps below only for few tokens (IQ4_XS [5120,5120]: 40 vs 68 us at M=256, 213 vs 116 us at
-    # M=2048, where the library GEMM runs near 900 TFLOP/s), so the reference's two steps stay the default here.
-    block_size, type_size = ops.quant_sizes(weight_type)
-    dense = ops.ggml_dequantize(weight, weight_type, rows, weight.shape[1] // type_size * block_size, x.dtype)
-    return x @ dense.T
+        return ops.ggml_mul_mat_a8(weight, x, weight_type, rows, out=out, bias=bias)
+    if path == "empty":
+        y = torch.empty(x.shape[0], rows, dtype=x.dtype, device=x.device)
+    elif path == "unquantized":
+        y = x @ weight.T
+    else:
+        # ops.ggml_dequant_gemm forms the same product without the dense copy of the weights; measured on MI355X it is
+        # faster than the two steps below only for few tokens (IQ4_XS [5120,5120]: 40 vs 68 us at M=256, 213 vs 116 us
+        # at M=2048, where the library GEMM runs near 900 TFLOP/s), so the reference's two steps stay the default here.
+        block_size, type_size = ops.quant_sizes(weight_type)
+        packed = weight if weight.is_contiguous() else weight.contiguous()
+        dense = ops.ggml_dequantize(packed, weight_type, rows, packed.shape[1] // type_size * block_size, x.dtype)
+        y = x @ dense.T
+    if bias is not None:
+        y.add_(bias)
+    if out is not None:
+        out.copy_(y)
+        return out
+    return y
+
+
+def apply_linear(x, weight, weight_type: int, *, shard_ids=(), shard_offset_map=None, shard_weight_types=None, bias=None):
+    """The forward pass of a GGUF linear layer (quantization/linear.py:221-262).
+
+    ``weight`` is the layer's packed tensor.  For a merged layer (q/k/v, gate/up) ``shard_ids`` lists the shards in
+    output order, ``shard_offset_map[id] = (start_row, end_row, row_bytes)`` locates each one in the padded tensor and
+    ``shard_weight_types[id]`` gives its ggml type (default ``weight_type``).  Shards of one type are multiplied in one
+    call, as in the reference.  Shards of different types are multiplied one by one, but where the reference copies
+    every shard out of the padded tensor on every call and concatenates the results, each call here reads its rows in
+    place and writes its columns of the merged result, bias included."""
+    import torch
+
+    shard_ids = list(shard_ids)
+    if not shard_ids:
+        return fused_mul_mat_gguf(x, weight, weight_type, bias=bias)
+    shard_ids = ["q", "k", "v"] if "q" in shard_ids else shard_ids
+    types = [int((shard_weight_types or {}).get(i, weight_type)) for i in shard_ids]
+    if len(set(types)) == 1:
+        return fused_mul_mat_gguf(x, weight, types[0], bias=bias)
+    widths = [shard_offset_map[i][1] - shard_offset_map[i][0] for i in shard_ids]
+    out = torch.empty(x.shape[0], sum(widths), dtype=x.dtype, device=x.device)
+    col = 0
+    for i, t, w in zip(shard_ids, types, widths):
+        start, end, row_bytes = shard_offset_map[i]
+        fused_mul_mat_gguf(x, weight[start:end, :row_bytes], t, out=out[:, col:col + w],
+                           bias=None if bias is None else bias[col:col + w])
+        col += w
+    return out
 
 
 def _activation(name: str, inp):

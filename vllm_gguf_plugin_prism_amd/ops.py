@@ -87,41 +87,72 @@ def ggml_dequantize_rows(W: torch.Tensor, quant_type: int, row_ids: torch.Tensor
     return out
 
 
-def _mul_mat(entry: str, W: torch.Tensor, X: torch.Tensor, quant_type: int, row: int) -> torch.Tensor:
-    _check_inputs(W, X)
+def _shard_args(W: torch.Tensor, X: torch.Tensor, quant_type: int, row: int, out: torch.Tensor | None,
+                bias: torch.Tensor | None) -> tuple[torch.Tensor, int, int]:
+    """Validate one shard of a (possibly merged, padded) linear layer; returns (output, bytes between rows of W,
+    elements between rows of the output).  ``W`` may be a row/column slice of a wider uint8 tensor and ``out`` a column
+    slice of a wider result (quantization/linear.py:247-257 copies such slices with ``.contiguous()`` and concatenates
+    the results; here the kernels address them in place)."""
+    for t in (W, X) + ((out,) if out is not None else ()) + ((bias,) if bias is not None else ()):
+        if not t.is_cuda:
+            raise ValueError("GGUF ops need tensors on the GPU")
+    if not X.is_contiguous() or X.dim() != 2:
+        raise ValueError("GGUF ops need a contiguous 2-D activation tensor")
+    qk, bs = quant_sizes(quant_type)
+    vecs, col = X.shape
+    if col % qk:
+        raise ValueError(f"K = {col} is not a multiple of the block size {qk}")
+    if W.dim() != 2 or W.dtype != torch.uint8 or (W.shape[1] > 1 and W.stride(1) != 1):
+        raise ValueError("the packed weights must be a 2-D uint8 tensor with contiguous rows")
+    if W.shape[0] < row or W.shape[1] < col // qk * bs:
+        raise ValueError("the packed weights are smaller than [row, K / block * block_bytes]")
+    w_pitch = W.stride(0) if W.shape[0] > 1 else col // qk * bs
+    if out is None:
+        out = torch.empty((vecs, row), dtype=X.dtype, device=W.device)
+    elif out.shape != (vecs, row) or out.dtype != X.dtype or (row > 1 and out.stride(1) != 1):
+        raise ValueError("out must be [X.shape[0], row] of X's dtype with contiguous rows")
+    ldy = out.stride(0) if vecs > 1 else row
+    if bias is not None and (bias.shape != (row,) or bias.dtype != X.dtype or not bias.is_contiguous()):
+        raise ValueError("bias must be a contiguous [row] tensor of X's dtype")
+    return out, w_pitch, ldy
+
+
+def ggml_mul_mat_vec_a8(W: torch.Tensor, X: torch.Tensor, quant_type: int, row: int, *, out: torch.Tensor | None = None,
+                        bias: torch.Tensor | None = None) -> torch.Tensor:
+    """Decode GEMV ``q8_1(X) @ W^T`` -> ``[X.shape[0], row]`` (reference: gguf_kernel.cu:104-218).
+
+    ``W`` may be a slice of a wider tensor (rows any pitch apart), ``out`` a column slice of a wider result, and
+    ``bias`` is added the way ``out.add_(bias)`` would (quantization/linear.py:243-262)."""
+    out, w_pitch, ldy = _shard_args(W, X, quant_type, row, out, bias)
     vecs, col = X.shape
     with torch.cuda.device(X.device):
-        out = torch.empty((vecs, row), dtype=X.dtype, device=W.device)
         ws = _workspace(X, vecs, col)
-        fn = getattr(_lib.lib(), entry)
-        rc = fn(W.data_ptr(), X.data_ptr(), _code(X.dtype), ws.data_ptr(), out.data_ptr(), int(quant_type), row, col, vecs,
-                _stream(X))
-    _lib.check(rc, entry)
+        rc = _lib.lib().gguf_mmvq_linear(W.data_ptr(), w_pitch, X.data_ptr(), _code(X.dtype), ws.data_ptr(), out.data_ptr(), ldy,
+                                         bias.data_ptr() if bias is not None else None, int(quant_type), row, col, vecs,
+                                         _stream(X))
+    _lib.check(rc, "ggml_mul_mat_vec_a8")
     return out
-
-
-def ggml_mul_mat_vec_a8(W: torch.Tensor, X: torch.Tensor, quant_type: int, row: int) -> torch.Tensor:
-    """Decode GEMV ``q8_1(X) @ W^T`` -> ``[X.shape[0], row]`` (reference: gguf_kernel.cu:104-218)."""
-    return _mul_mat("gguf_mmvq", W, X, quant_type, row)
 
 
 MMQ_ENGINES = {"auto": 0, "int8": 1, "half": 2}
 
 
-def ggml_mul_mat_a8(W: torch.Tensor, X: torch.Tensor, quant_type: int, row: int, *, engine: str = "auto") -> torch.Tensor:
+def ggml_mul_mat_a8(W: torch.Tensor, X: torch.Tensor, quant_type: int, row: int, *, engine: str = "auto",
+                    out: torch.Tensor | None = None, bias: torch.Tensor | None = None) -> torch.Tensor:
     """Prefill GEMM ``q8_1(X) @ W^T`` on MFMA (reference: gguf_kernel.cu:220-290).
 
     ``engine``: ``"int8"`` keeps the reference's integer arithmetic (int8 MFMA, block scales in fp32); ``"half"``
     multiplies the dequantized operands on half-precision MFMA (faster, about 2e-4 relative deviation, half and
-    bfloat16 results only); ``"auto"`` takes ``"half"`` where it applies."""
-    _check_inputs(W, X)
+    bfloat16 results only); ``"auto"`` takes ``"half"`` where it applies.  ``out`` / ``bias`` / sliced ``W``: as for
+    :func:`ggml_mul_mat_vec_a8`."""
+    out, w_pitch, ldy = _shard_args(W, X, quant_type, row, out, bias)
     vecs, col = X.shape
     with torch.cuda.device(X.device):
-        out = torch.empty((vecs, row), dtype=X.dtype, device=W.device)
         nbytes = max(_lib.lib().gguf_mmq_workspace_bytes(vecs, row, col), vecs * _lib.lib().gguf_q8_1_row_bytes(col), 16)
         ws = torch.empty(nbytes, dtype=torch.uint8, device=X.device)
-        rc = _lib.lib().gguf_mmq_engine(W.data_ptr(), X.data_ptr(), _code(X.dtype), ws.data_ptr(), out.data_ptr(),
-                                        int(quant_type), row, col, vecs, MMQ_ENGINES[engine], nbytes, _stream(X))
+        rc = _lib.lib().gguf_mmq_linear(W.data_ptr(), w_pitch, X.data_ptr(), _code(X.dtype), ws.data_ptr(), out.data_ptr(), ldy,
+                                        bias.data_ptr() if bias is not None else None, int(quant_type), row, col, vecs,
+                                        MMQ_ENGINES[engine], nbytes, _stream(X))
     _lib.check(rc, "ggml_mul_mat_a8")
     return out
 
