@@ -19,6 +19,17 @@ MmqhPlan mmq_half_plan(int M, int N, int K, int64_t avail) {
   const int nsteps = (K + 63) / 64;
   const int big = M > 128 ? 0 : 1;
   MmqhPlan p = {3, 0, 0, 1};
+  if (M <= 64) {
+    // A handful of tokens: the weights are read once and little is computed, so what counts is how many independent
+    // streams of weight blocks are in flight.  Small tiles, four workgroups per CU, K split as far as that fills them.
+    const int64_t t = tiles(3);
+    int s = t > 0 ? (int)(4 * CUS / t) : 1;
+    if (s > nsteps / 4) s = nsteps / 4;
+    if (s > 8) s = 8;
+    p = MmqhPlan{3, 0, (int)t, s};
+    if (s >= 2 && p.partial_bytes() <= avail) return p;
+    return MmqhPlan{3, (int)t, 0, 1};
+  }
   const int64_t tb = tiles(big);
   if (tb < 180 && tb > 0) {                     // too few tiles: split them all
     int s = (int)(CUS / tb);
