@@ -1,0 +1,63 @@
+"""GPU: the operators are captured into HIP graphs and replayed (the reference's ops are graph-capturable,
+csrc/gguf/gguf_kernel.cu:24-29: caller's stream, no host synchronisation).  Every replay is compared with the eager
+result, with eager work and synchronisations between the replays."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import gguf_oracle as o
+
+pytestmark = pytest.mark.gpu
+
+
+def _dev(a):
+    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+
+
+def _capture(fn):
+    side = torch.cuda.Stream()
+    side.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(side):
+        for _ in range(2):
+            fn()                       # warm-up on the capture stream: library handles, LDS-size attributes
+    torch.cuda.current_stream().wait_stream(side)
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        out = fn()
+    return graph, out
+
+
+@pytest.mark.parametrize("case", ["mmvq", "mmq_half", "mmq_half_split", "mmq_int8", "dequant_gemm", "moe_vec_grouped"])
+def test_replays_match_eager(case):
+    from vllm_gguf_plugin_prism_amd import ops
+    rng = np.random.default_rng(abs(hash(case)) % 1000)
+    if case == "moe_vec_grouped":
+        e, t, top_k, n, k = 8, 16, 4, 256, 512
+        w = _dev(np.stack([o.make_weights(rng, o.Q4_0, n, k) for _ in range(e)]))
+        ids = _dev(np.stack([rng.choice(e, size=top_k, replace=False) for _ in range(t)]).astype(np.int32))
+        xs = [torch.randn(t, k, dtype=torch.float16, device="cuda") for _ in range(3)]
+        x = xs[0].clone()
+        fn = lambda: ops.ggml_moe_a8_vec(x, w, ids, top_k, o.Q4_0, n, t)
+    else:
+        qtype, m, n, k = {"mmvq": (o.Q4_K, 1, 512, 1024), "mmq_half": (o.Q6_K, 96, 384, 1024),
+                          "mmq_half_split": (o.Q4_K, 200, 250, 4096), "mmq_int8": (o.Q6_K, 96, 384, 1024),
+                          "dequant_gemm": (o.IQ4_XS, 64, 256, 1024)}[case]
+        w = _dev(o.make_weights(rng, qtype, n, k))
+        xs = [torch.randn(m, k, dtype=torch.float16, device="cuda") for _ in range(3)]
+        x = xs[0].clone()
+        if case == "mmvq":
+            fn = lambda: ops.ggml_mul_mat_vec_a8(w, x, qtype, n)
+        elif case == "dequant_gemm":
+            fn = lambda: ops.ggml_dequant_gemm(w, x, qtype, n)
+        else:
+            engine = "int8" if case == "mmq_int8" else "half"
+            fn = lambda: ops.ggml_mul_mat_a8(w, x, qtype, n, engine=engine)
+    graph, out = _capture(fn)
+    for xi in xs:
+        x.copy_(xi)
+        eager = fn().clone()            # eager work between the replays
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), case

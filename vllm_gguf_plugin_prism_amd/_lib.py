@@ -88,6 +88,12 @@ def lib() -> "_Bound":
                 f"{path} is missing: build it with `python -m vllm_gguf_plugin_prism_amd.build` "
                 "(hipcc, gfx950).  This package has no non-HIP implementation."
             )
+        # The process must hold one HIP runtime.  torch ships its own libamdhip64; if this library were loaded first it
+        # would bring in the system's copy, torch would later add its own, and kernels launched through the one on
+        # pointers and streams of the other fail to launch.  With torch's copy loaded first, this library's dependency
+        # on the same soname resolves to it.
+        import torch  # noqa: F401
+
         handle = ctypes.CDLL(path)
         bound = _Bound()
         for name, (res, args) in _SIGNATURES.items():
