@@ -152,6 +152,7 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void mmqh_kernel(const uint8_t* 
   constexpr int M_T = 32 * WM * TM, N_T = 32 * WN * TN;
   constexpr int PAIRS = N_T * KB;        // (weight row, 32-block) pairs to decode per step, one thread each
   static_assert(NT % PAIRS == 0 && (M_T * GR) % NT == 0, "tile and workgroup sizes must divide evenly");
+  static_assert(NT / PAIRS == 2, "the unrolled pipeline below assumes two decode groups");
   constexpr int DG = NT / PAIRS;         // decode groups: group g decodes the steps t with t % DG == g
   constexpr int AQ = M_T * GR / NT;      // activation granules per thread and step
   constexpr int TILE = (M_T + N_T) * LDH;  // halfs per buffer
@@ -181,33 +182,39 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void mmqh_kernel(const uint8_t* 
   const int grp = tid / PAIRS, n_dec = (tid % PAIRS) / KB, kb_dec = tid % KB;
   const uint8_t* const w_row = W + (int64_t)min(n_base + n_dec, N - 1) * rowbytes;
 
-  u32x4 r_aq[AQ];
-  typename F::Raw r_w;
+  // Global loads run two turns ahead of their use: two register stages for the activations (a turn = one step) and two
+  // for this thread's weight block (a turn = DG steps), indexed by compile-time constants so that they stay registers.
+  u32x4 r_aq[2][AQ];
+  typename F::Raw r_w[2];
 
-  auto fetch_a = [&](int t) {
+  auto fetch_a = [&](auto stage, int t) {
+    constexpr int S = decltype(stage)::value;
     if (DBG_SKIP(2, t > 0)) return;
 #pragma unroll
-    for (int i = 0; i < AQ; ++i) r_aq[i] = *(const u32x4*)(aq_src[i] + t * KS);  // rows are padded with zeros to a multiple of 512
+    for (int i = 0; i < AQ; ++i) r_aq[S][i] = *(const u32x4*)(aq_src[i] + t * KS);  // rows are padded with zeros to a multiple of 512
   };
-  auto write_a = [&](int buf) {
+  auto write_a = [&](auto stage, int buf) {
+    constexpr int S = decltype(stage)::value;
     _Float16* xs = tiles + buf * TILE;
 #pragma unroll
     for (int i = 0; i < AQ; ++i) {
       const int p = tid + NT * i;
-      *(u32x4*)(xs + (p / GR) * LDH + 8 * (p % GR)) = r_aq[i];
+      *(u32x4*)(xs + (p / GR) * LDH + 8 * (p % GR)) = r_aq[S][i];
     }
   };
-  auto fetch_w = [&](int t) {
+  auto fetch_w = [&](auto stage, int t) {
+    constexpr int S = decltype(stage)::value;
     if (DBG_SKIP(8, t >= DG)) return;
-    r_w = F::fetch(w_row, min(t * KB + kb_dec, nkb_total - 1));  // clamped: a block past K is re-read and decoded to zeros
+    r_w[S] = F::fetch(w_row, min(t * KB + kb_dec, nkb_total - 1));  // clamped: a block past K is re-read and decoded to zeros
   };
-  auto decode = [&](int t, int buf) {
+  auto decode = [&](auto stage, int t, int buf) {
+    constexpr int S = decltype(stage)::value;
     if (DBG_SKIP(4, t >= DG)) return;
     _Float16* wt = tiles + buf * TILE + M_T * LDH;
     const int kb = t * KB + kb_dec;
     uint32_t q[8];
     float s0, s1, mn = 0.0f, mn1 = 0.0f;
-    C::unpack(r_w, kb, q, s0, s1, mn, mn1);
+    C::unpack(r_w[S], kb, q, s0, s1, mn, mn1);
     if (!F::MIN16) mn1 = mn;   // one offset factor per 32-block unless the format has one per 16
     if (kb >= nkb_total) s0 = s1 = mn = mn1 = 0.0f;
     uint4 h[4];
@@ -273,23 +280,37 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void mmqh_kernel(const uint8_t* 
   // of any shape: instead of a few CUs working through whole tiles while the rest idle, all CUs share those tiles.
   const int per_split = (nsteps + nsplit - 1) / nsplit;
   const int t0 = split * per_split, t1 = min(nsteps, t0 + per_split);
-  if (t0 < t1) {
-    fetch_a(t0);
-    const int first = t0 + ((grp - t0) % DG + DG) % DG;   // this group's first step
-    if (first < t1) fetch_w(first);
-  }
-  for (int s = t0 - 1; s < t1; ++s) {
-    const int t = s + 1;
-    if (t < t1) {
-      write_a(t & 1);
-      if (t + 1 < t1) fetch_a(t + 1);
-      if (t % DG == grp) {
-        decode(t, t & 1);
-        if (t + DG < t1) fetch_w(t + DG);
+  const int n = t1 - t0;                               // steps of this workgroup; step j of them is step t0 + j of K
+  const int gpar = ((grp - t0) % DG + DG) % DG;         // this group decodes the steps j with j % DG == gpar
+  constexpr std::integral_constant<int, 0> S0{};
+  constexpr std::integral_constant<int, 1> S1{};
+  if (n > 0) fetch_a(S0, t0);
+  if (n > 1) fetch_a(S1, t0 + 1);
+  if (gpar < n) fetch_w(S0, t0 + gpar);
+  if (gpar + DG < n) fetch_w(S1, t0 + gpar + DG);
+  // turn j: stage step j (activation stage j % 2; weight stage (j / DG) % 2 if it is this group's turn), refill the
+  // stages just emptied with the loads of two turns ahead, contract step j - 1, barrier
+  auto turn = [&](auto jmod, int j) {
+    constexpr int J = decltype(jmod)::value;           // j % (2 * DG), so that every stage index is a constant
+    constexpr std::integral_constant<int, J & 1> sa{};
+    constexpr std::integral_constant<int, (J / DG) & 1> sw{};
+    if (j > n) return;
+    if (j < n) {
+      write_a(sa, j & 1);
+      if (j + 2 < n) fetch_a(sa, t0 + j + 2);
+      if (J % DG == gpar) {
+        decode(sw, t0 + j, j & 1);
+        if (j + 2 * DG < n) fetch_w(sw, t0 + j + 2 * DG);
       }
     }
-    if (s >= t0) contract(s & 1, KS / 16);
+    if (j >= 1) contract((j - 1) & 1, KS / 16);
     __syncthreads();
+  };
+  for (int j = 0; j <= n; j += 2 * DG) {
+    turn(std::integral_constant<int, 0>{}, j);
+    turn(std::integral_constant<int, 1>{}, j + 1);
+    turn(std::integral_constant<int, 2>{}, j + 2);
+    turn(std::integral_constant<int, 3>{}, j + 3);
   }
   _Float16* const xs = tiles;                // the offset pass below reuses the first buffer
   _Float16* const wt = tiles + M_T * LDH;
