@@ -466,14 +466,10 @@ static int mmqh_typed(const void* W, const void* ws, void* Y, int M, int N, int 
 #ifdef GGUF_MMQ_TUNE
   switch (tune_cfg_h()) {
     case 1: launch_mmqh<C, 4, 2, 2, 2, 1, T>(W, ws, Y, M, N, K, stream); return launch_status();   // 256 x 128, 8 waves
-    case 2: launch_mmqh<C, 2, 2, 2, 2, 1, T>(W, ws, Y, M, N, K, stream); return launch_status();   // 128 x 128, 4 waves
-    case 3: launch_mmqh<C, 2, 4, 2, 2, 1, T>(W, ws, Y, M, N, K, stream); return launch_status();   // 128 x 256, 8 waves
-    case 4: launch_mmqh<C, 2, 2, 4, 2, 1, T>(W, ws, Y, M, N, K, stream); return launch_status();   // 256 x 128, 4 waves
     case 5: launch_mmqh<C, 2, 2, 2, 1, 2, T>(W, ws, Y, M, N, K, stream); return launch_status();   // 128 x 64, 4 waves
     case 6: launch_mmqh<C, 2, 4, 2, 1, 2, T>(W, ws, Y, M, N, K, stream); return launch_status();   // 128 x 128, 8 waves (64 x 32 each)
     case 7: launch_mmqh<C, 2, 2, 1, 1, 4, T>(W, ws, Y, M, N, K, stream); return launch_status();   // 64 x 64, 4 waves
     case 8: launch_mmqh<C, 4, 2, 1, 2, 2, T>(W, ws, Y, M, N, K, stream); return launch_status();   // 128 x 128, 8 waves (32 x 64 each)
-    case 9: launch_mmqh<C, 4, 2, 2, 4, 1, T>(W, ws, Y, M, N, K, stream); return launch_status();   // 256 x 256, 8 waves
     default: break;
   }
 #endif
