@@ -44,7 +44,7 @@ ROTATE_BYTES = 640 << 20       # distinct weight bytes walked per rotation (> 2x
 # what it reads for a 256 MiB device copy (x2.000 and x1.000); summarised in profiles/bench_mmvq_q4_k_bs1_mmq_q6_k.txt.
 # Counters cannot be read from inside this process, so these are constants of the measured build, not live values.
 TRAFFIC_MMVQ_Q4_K_14336x4096 = 33.37e6 + 0.02e6
-TRAFFIC_MMQ_Q6_K_M512 = {"18944x3584": 159.7e6 + 19.4e6, "3584x18944": 272.5e6 + 29.4e6}  # GEMM kernel of the half engine
+TRAFFIC_MMQ_Q6_K_M512 = {"18944x3584": 159.7e6 + 48.2e6, "3584x18944": 272.9e6 + 29.4e6}  # GEMM kernel of the half engine, read + written
 
 
 def _events_ms(fn, iters):
