@@ -50,13 +50,17 @@ __device__ __forceinline__ void dq8_q8_0(const uint8_t* __restrict__ w, int64_t 
   }
 }
 
-__device__ __forceinline__ void scale_min_k4(const uint8_t* __restrict__ s, int j, int& sc, int& mn) {
+// 6-bit scale and min of sub-block j from the 12 packed bytes, given as the three dwords that hold bytes 0-3, 4-7 and
+// 8-11 (dequantize.cuh:156-163).  Shifts only: indexing the bytes through a pointer would put them in scratch memory.
+__device__ __forceinline__ void scale_min_k4(uint32_t b03, uint32_t b47, uint32_t b8b, int j, int& sc, int& mn) {
+  const int sh = 8 * (j & 3);
+  const uint32_t lo = (b03 >> sh) & 0xFF, mid = (b47 >> sh) & 0xFF, hi = (b8b >> sh) & 0xFF;
   if (j < 4) {
-    sc = s[j] & 63;
-    mn = s[j + 4] & 63;
+    sc = (int)(lo & 63);
+    mn = (int)(mid & 63);
   } else {
-    sc = (s[j + 4] & 0xF) | ((s[j - 4] >> 6) << 4);
-    mn = (s[j + 4] >> 4) | ((s[j] >> 6) << 4);
+    sc = (int)((hi & 0xF) | ((lo >> 6) << 4));
+    mn = (int)((hi >> 4) | ((mid >> 6) << 4));
   }
 }
 
@@ -68,9 +72,8 @@ __device__ __forceinline__ void dq8_q4_k(const uint8_t* __restrict__ w, int64_t 
   const uint4 hdr = *(const uint4*)blk;  // 144-byte blocks keep 16-byte alignment
   const h16 dall = __builtin_bit_cast(h16, (uint16_t)(hdr.x & 0xFFFF));
   const h16 dmin = __builtin_bit_cast(h16, (uint16_t)(hdr.x >> 16));
-  const uint32_t sw[3] = {hdr.y, hdr.z, hdr.w};
   int sc, mn;
-  scale_min_k4((const uint8_t*)sw, j, sc, mn);
+  scale_min_k4(hdr.y, hdr.z, hdr.w, j, sc, mn);
   const h16 d1 = dall * (h16)sc;
   const h16 m1 = dmin * (h16)mn;
   const uint2 q = *(const uint2*)(blk + 16 + 32 * (j >> 1) + pos);
@@ -225,9 +228,8 @@ __device__ __forceinline__ void dq8_q5_k(const uint8_t* __restrict__ w, int64_t 
   const uint4 hdr = *(const uint4*)blk;  // 176-byte blocks keep 16-byte alignment
   const h16 dall = __builtin_bit_cast(h16, (uint16_t)(hdr.x & 0xFFFF));
   const h16 dmin = __builtin_bit_cast(h16, (uint16_t)(hdr.x >> 16));
-  const uint32_t sw[3] = {hdr.y, hdr.z, hdr.w};
   int sc, mn;
-  scale_min_k4((const uint8_t*)sw, j, sc, mn);
+  scale_min_k4(hdr.y, hdr.z, hdr.w, j, sc, mn);
   const h16 d1 = dall * (h16)sc;
   const h16 m1 = dmin * (h16)mn;
   const uint2 q = *(const uint2*)(blk + 48 + 32 * (j >> 1) + pos);

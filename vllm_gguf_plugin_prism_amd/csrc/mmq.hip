@@ -247,9 +247,6 @@ __global__ __launch_bounds__(64 * WM * WN * (MODE == MODE_PINGPONG || MODE == MO
   typename F::Raw r_w[WP];
 
   auto fetch = [&](int k0) {
-#ifdef GGUF_DBG_NOFETCH
-    if (k0 > 0 && K > 0) return;
-#endif
     const int kb0 = k0 >> 5;
 #pragma unroll
     for (int i = 0; i < AQ; ++i) r_aq[i] = *(const uint4*)(aq_src[i] + k0);  // q8 rows are padded to 512, always readable
@@ -265,9 +262,6 @@ __global__ __launch_bounds__(64 * WM * WN * (MODE == MODE_PINGPONG || MODE == MO
     }
   };
   auto stash = [&](int k0) {
-#ifdef GGUF_DBG_NOSTASH
-    if (k0 > 0 && K > 0) return;
-#endif
     const int kb0 = k0 >> 5;
 #pragma unroll
     for (int i = 0; i < AQ; ++i) {

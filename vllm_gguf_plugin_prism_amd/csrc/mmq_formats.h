@@ -61,14 +61,12 @@ struct MQ8_0 {  // vecdotq.cuh:165-177, 869-921
 // Q4_K / Q5_K: for the eight sub-blocks of super-block b8, C * d * sc_j and C * d * sc_j - dmin * m_j from the
 // 16-byte block header (6-bit packing: dequantize.cuh:156-163); C is the centre subtracted from the codes
 __device__ __forceinline__ void k4_offs8(const uint8_t* row, int bs, int b8, int nkb, float c, float (&cs)[8], float (&cm)[8]) {
-  if (8 * b8 >= nkb) {
-#pragma unroll
-    for (int e = 0; e < 8; ++e) cs[e] = cm[e] = 0.0f;
-    return;
-  }
-  const uint4 hdr = ld<uint4>(row + (int64_t)b8 * bs);
-  const float d = (float)__builtin_bit_cast(_Float16, (uint16_t)(hdr.x & 0xFFFF));
-  const float dmin = (float)__builtin_bit_cast(_Float16, (uint16_t)(hdr.x >> 16));
+  // past the row's end: re-read the last super-block and scale it to nothing (no early return: a branch around the
+  // stores to cs / cm would move the two arrays to scratch memory)
+  const bool in = 8 * b8 < nkb;
+  const uint4 hdr = ld<uint4>(row + (int64_t)min(b8, max(nkb / 8 - 1, 0)) * bs);
+  const float d = in ? (float)__builtin_bit_cast(_Float16, (uint16_t)(hdr.x & 0xFFFF)) : 0.0f;
+  const float dmin = in ? (float)__builtin_bit_cast(_Float16, (uint16_t)(hdr.x >> 16)) : 0.0f;
   const uint32_t lo = hdr.y, mid = hdr.z, hi = hdr.w;  // scale bytes 0..3, 4..7, 8..11
 #pragma unroll
   for (int j = 0; j < 4; ++j) {

@@ -136,13 +136,7 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void mmqh_kernel(const uint8_t* 
                                                                   const char* __restrict__ ws, int64_t ws_row_bytes,
                                                                   T* __restrict__ Y, float* __restrict__ partial, int M, int N,
                                                                   int K, int Kp, int tiles_x, int whole_tiles, int shared_tiles, int splits,
-                                                                  int64_t w_pitch, int64_t ldy, const T* __restrict__ bias, int dbg) {
-#ifndef GGUF_MMQ_TUNE
-  (void)dbg;
-#define DBG_SKIP(bit, cond) false
-#else
-#define DBG_SKIP(bit, cond) ((dbg & (bit)) && (cond))
-#endif
+                                                                  int64_t w_pitch, int64_t ldy, const T* __restrict__ bias) {
   using F = typename C::Fmt;
   constexpr int NT = 64 * WM * WN;
   constexpr int KS = 64;                 // elements of K per step
@@ -189,7 +183,6 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void mmqh_kernel(const uint8_t* 
 
   auto fetch_a = [&](auto stage, int t) {
     constexpr int S = decltype(stage)::value;
-    if (DBG_SKIP(2, t > 0)) return;
 #pragma unroll
     for (int i = 0; i < AQ; ++i) r_aq[S][i] = *(const u32x4*)(aq_src[i] + t * KS);  // rows are padded with zeros to a multiple of 512
   };
@@ -204,12 +197,10 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void mmqh_kernel(const uint8_t* 
   };
   auto fetch_w = [&](auto stage, int t) {
     constexpr int S = decltype(stage)::value;
-    if (DBG_SKIP(8, t >= DG)) return;
     r_w[S] = F::fetch(w_row, min(t * KB + kb_dec, nkb_total - 1));  // clamped: a block past K is re-read and decoded to zeros
   };
   auto decode = [&](auto stage, int t, int buf) {
     constexpr int S = decltype(stage)::value;
-    if (DBG_SKIP(4, t >= DG)) return;
     _Float16* wt = tiles + buf * TILE + M_T * LDH;
     const int kb = t * KB + kb_dec;
     uint32_t q[8];
@@ -235,7 +226,6 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void mmqh_kernel(const uint8_t* 
   // keeps the LDS pipe busy for the whole step, and the matrix work of one wave runs under the reads of the other
   // wave on its SIMD.
   auto contract = [&](int buf, int slices) {
-    if (DBG_SKIP(16, true)) return;
     const _Float16* xs = tiles + buf * TILE;
     const _Float16* wt = xs + M_T * LDH;
     v8h af[KS / 16][TM], bf[KS / 16][TN];
@@ -383,15 +373,6 @@ __global__ __launch_bounds__(64 * WM * WN, OCC) void mmqh_kernel(const uint8_t* 
   }
 }
 
-static int tune_dbg() {
-#ifdef GGUF_MMQ_TUNE
-  static const int v = [] { const char* e = getenv("GGUF_MMQH_DBG"); return e ? atoi(e) : 0; }();
-  return v;
-#else
-  return 0;
-#endif
-}
-
 // Y tile = T(sum of its `splits` fp32 partial tiles / 16), gridDim.y workgroups per split tile, fixed order of addition
 template <int M_T, int N_T, typename T>
 __global__ __launch_bounds__(256) void mmqh_reduce_kernel(const float* __restrict__ partial, T* __restrict__ Y, int M, int N,
@@ -447,7 +428,7 @@ static void launch_mmqh(const void* W, const void* ws, void* Y, int M, int N, in
   const _Float16* xh = (const _Float16*)((const char*)ws + (int64_t)M * q8_row_bytes(K));
   hipLaunchKernelGGL(kern, dim3(whole + shared * splits), dim3(64 * WM * WN), lds, stream, (const uint8_t*)W, xh, (const char*)ws,
                      q8_row_bytes(K), (T*)Y, partial, M, N, K, (int)q8_kp(K), tiles_x, whole, shared > 0 ? shared : 1, splits, w_pitch, ldy,
-                     (const T*)la.bias, tune_dbg());
+                     (const T*)la.bias);
   if (shared > 0)
     hipLaunchKernelGGL((mmqh_reduce_kernel<M_T, N_T, T>), dim3(shared, M_T * N_T / 1024), dim3(256), 0, stream, partial, (T*)Y, M, N, tiles_x,
                        whole, splits, ldy, (const T*)la.bias);
