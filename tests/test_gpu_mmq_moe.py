@@ -305,6 +305,31 @@ def test_moe_vec_grouped_and_per_pair_grids(qtype, t, top_k, e):
     assert o.rel_l2(y.cpu().numpy(), o.moe_a8_vec(xv, w, ids, top_k, qtype, n, t)) <= 1e-5
 
 
+@pytest.mark.parametrize("dt", ["f32", "f16"])
+@pytest.mark.parametrize("qtype", MMQ_TYPES)
+def test_moe_vec_shared_experts_keep_gemv_semantics(qtype, dt):
+    """With two or more pairs per expert the per-pair operator runs on the grouped tile kernel (all tile formats but
+    Q5_0).  Its results must stay those of the GEMV: for Q4_K / Q5_K the offset term multiplies the quant sums, not the
+    stored block sums the tile operator ggml_moe_a8 uses (the two differ by about 1e-2 on these weights)."""
+    ops = _ops()
+    rng = np.random.default_rng(970 + qtype)
+    t, top_k, e, n, k = 40, 4, 8, 200, 768
+    w = np.stack([o.make_weights(rng, qtype, n, k) for _ in range(e)])
+    xd, xv = _x(rng, t, k, dt)
+    ids, _ = _routing(rng, t, e, top_k)
+    y = ops.ggml_moe_a8_vec(xd, _dev(w), _dev(ids), top_k, qtype, n, t)
+    assert y.shape == (t * top_k, n) and y.dtype == TORCH_DT[dt]
+    want = o.moe_a8_vec(xv, w, ids, top_k, qtype, n, t)
+    assert o.rel_l2(y.float().cpu().numpy(), want) <= (1e-5 if dt == "f32" else 1e-3)
+    # an expert id outside [0, experts) names no weights: its pairs are left out, the others are unaffected
+    bad = ids.copy()
+    bad[3, 1] = e + 5
+    y2 = ops.ggml_moe_a8_vec(xd, _dev(w), _dev(bad), top_k, qtype, n, t)
+    keep = np.ones(t * top_k, dtype=bool)
+    keep[3 * top_k + 1] = False
+    assert torch.equal(y2[torch.from_numpy(keep).cuda()], y[torch.from_numpy(keep).cuda()])
+
+
 @pytest.mark.parametrize("qtype", ALL)
 def test_moe_vec_matches_oracle(qtype):
     ops = _ops()

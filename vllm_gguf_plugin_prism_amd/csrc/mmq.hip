@@ -143,6 +143,8 @@ struct MoeArgs {
   int64_t expert_stride;  // bytes
   int top_k;
   int num_pairs;          // tokens * top_k
+  int gemv_sums;          // offset term of Q4_K / Q5_K: 0 = times the stored block sum (the reference's tile kernels,
+                          // vecdotq.cuh:369-372), 1 = times d8 * (sum of the quants) (its GEMV, vecdotq.cuh:328-351)
 };
 
 // MODE selects how staging and contraction overlap:
@@ -220,6 +222,7 @@ __global__ __launch_bounds__(64 * WM * WN * (MODE == MODE_PINGPONG || MODE == MO
   }
   const float* as_src[AS];  // activation block scales
   bool as_ok[AS];
+  const int sum_plane = (MOE && moe.gemv_sums ? 2 : 1) * (Kp / 32);  // planes of a workspace row behind d: s8, then d8 * sum(q)
 #pragma unroll
   for (int i = 0; i < AS; ++i) {
     const int p = tid + NT * i, m = min(p / KB, M_T - 1), kb = p % KB;
@@ -253,7 +256,7 @@ __global__ __launch_bounds__(64 * WM * WN * (MODE == MODE_PINGPONG || MODE == MO
 #pragma unroll
     for (int i = 0; i < AS; ++i) {
       r_ad[i] = as_src[i][kb0];
-      if (F::HAS_MIN && !F::MIN16) r_aa[i] = as_src[i][kb0 + Kp / 32];
+      if (F::HAS_MIN && !F::MIN16) r_aa[i] = as_src[i][kb0 + sum_plane];
     }
 #pragma unroll
     for (int i = 0; i < WP; ++i) {
@@ -601,6 +604,52 @@ static bool mmq_type_ok(int type) {
   }
 }
 
+// The per-pair MoE GEMV (ggml_moe_a8_vec, gguf_kernel.cu:395-530) on the grouped tile kernel, for calls in which the
+// experts are shared by enough pairs: the rows are quantized once, the routing sort runs in the workspace behind
+// them, and every expert block is one pass over the expert's weights on the matrix cores instead of one pass per
+// group of pairs on the vector ALUs.  Results keep the GEMV's semantics: Q4_K / Q5_K take their offset term from the
+// quant sums (MoeArgs::gemv_sums); Q5_0 is the one tile format whose tile arithmetic differs from its GEMV
+// (vecdotq.cuh:98-125 against :668-749) and stays on the vector kernel.
+bool moe_vec_tiles_ok(int type, int64_t pairs, int64_t num_experts) {
+  if (!mmq_type_ok(type) || type == T_Q5_0) return false;
+  return num_experts > 0 && num_experts <= 256 && pairs >= 2 * num_experts;  // the tile kernel takes expert ids 0..255 (moe.cuh:33)
+}
+
+int64_t moe_vec_tiles_workspace(int64_t tokens, int64_t top_k, int64_t K, int64_t num_experts) {
+  const int64_t sorted_cap = tokens * top_k + num_experts * 31;
+  return tokens * q8_row_bytes(K) + (sorted_cap + sorted_cap / 32 + 2) * 4;
+}
+
+int moe_vec_tiles(const void* X, int xdtype, void* workspace, const void* W, const int32_t* topk_ids, void* Y, int type, int N,
+                  int K, int top_k, int tokens, int act, int num_experts, hipStream_t s) {
+  const int pairs = tokens * top_k;
+  int rc = quantize_q8_1(X, xdtype, workspace, tokens, K, s, act);
+  if (rc != GGUF_OK) return rc;
+  const int64_t sorted_cap = (int64_t)pairs + (int64_t)num_experts * 31;
+  const int64_t block_cap = sorted_cap / 32 + 1;
+  int32_t* sorted = (int32_t*)((char*)workspace + (int64_t)tokens * q8_row_bytes(K));  // rows are a multiple of 4 bytes long
+  int32_t* experts = sorted + sorted_cap;
+  int32_t* post = experts + block_cap;
+  rc = gguf_moe_align_block_size(topk_ids, pairs, num_experts, 32, sorted, sorted_cap, experts, block_cap, post, (gguf_stream_t)s);
+  if (rc != GGUF_OK) return rc;
+  const int64_t stride = (int64_t)N * (K / block_elems(type)) * block_bytes(type);
+  MoeArgs moe = {sorted, experts, post, stride, top_k, pairs, type == T_Q4_K || type == T_Q5_K ? 1 : 0};
+  const int ns = (int)(sorted_cap / 32 * 32);   // blocks past the padded total see expert -1 and leave
+  switch (type) {
+    case T_Q4_0: return moe_fmt<MQ4_0>(W, workspace, Y, xdtype, N, K, ns, moe, s);
+    case T_Q4_1: return moe_fmt<MQ4_1>(W, workspace, Y, xdtype, N, K, ns, moe, s);
+    case T_Q5_1: return moe_fmt<MQ5_1>(W, workspace, Y, xdtype, N, K, ns, moe, s);
+    case T_Q8_0: return moe_fmt<MQ8_0>(W, workspace, Y, xdtype, N, K, ns, moe, s);
+    case T_Q2_K: return moe_fmt<MQ2_K>(W, workspace, Y, xdtype, N, K, ns, moe, s);
+    case T_Q3_K: return moe_fmt<MQ3_K>(W, workspace, Y, xdtype, N, K, ns, moe, s);
+    case T_Q4_K: return moe_fmt<MQ4_K>(W, workspace, Y, xdtype, N, K, ns, moe, s);
+    case T_Q5_K: return moe_fmt<MQ5_K>(W, workspace, Y, xdtype, N, K, ns, moe, s);
+    case T_Q6_K: return moe_fmt<MQ6_K>(W, workspace, Y, xdtype, N, K, ns, moe, s);
+    case T_IQ4_XS: return moe_fmt<MIQ4_XS>(W, workspace, Y, xdtype, N, K, ns, moe, s);
+    case T_IQ2_XXS: return moe_fmt<MIQ2_XXS>(W, workspace, Y, xdtype, N, K, ns, moe, s);
+  }
+  return GGUF_ERR_TYPE;
+}
 
 // mmq_h.hip
 int mmq_half(const void* W, const void* ws, void* Y, int dtype, int type, int M, int N, int K, float* partial,
@@ -716,7 +765,7 @@ extern "C" int gguf_moe_mmq_act(const void* X, int xdtype, void* q8_workspace, c
   hipLaunchKernelGGL(zero_rows_kernel, dim3((unsigned)((n16 + 255) / 256)), dim3(256), 0, s, (uint4*)Y, n16);
   const int rc = quantize_q8_1(X, xdtype, q8_workspace, tokens, K, s, act);
   if (rc != GGUF_OK) return rc;
-  MoeArgs moe = {sorted_token_ids, expert_ids, num_tokens_post_padded, expert_stride_bytes, (int)top_k, (int)(tokens * top_k)};
+  MoeArgs moe = {sorted_token_ids, expert_ids, num_tokens_post_padded, expert_stride_bytes, (int)top_k, (int)(tokens * top_k), 0};
   const int ns = (int)(num_sorted / 32 * 32);  // a trailing partial block is ignored, like the reference's integer division
   if (ns == 0) return launch_status();
   switch (type) {

@@ -88,10 +88,20 @@ extern "C" int gguf_moe_vec_act(const void* X, int xdtype, void* q8_workspace, c
                                 void* Y, int type, int64_t N, int64_t K, int64_t top_k, int64_t tokens, int act,
                                 int64_t num_experts, int64_t workspace_bytes, gguf_stream_t stream);
 
+namespace gguf {
+// mmq.hip: the same operator on the grouped tile kernel, for calls whose experts are shared by enough pairs
+bool moe_vec_tiles_ok(int type, int64_t pairs, int64_t num_experts);
+int64_t moe_vec_tiles_workspace(int64_t tokens, int64_t top_k, int64_t K, int64_t num_experts);
+int moe_vec_tiles(const void* X, int xdtype, void* workspace, const void* W, const int32_t* topk_ids, void* Y, int type, int N,
+                  int K, int top_k, int tokens, int act, int num_experts, hipStream_t s);
+}  // namespace gguf
+
 extern "C" int64_t gguf_moe_vec_workspace_bytes(int64_t tokens, int64_t top_k, int64_t K, int64_t num_experts) {
   if (tokens < 0 || top_k <= 0 || K <= 0 || num_experts < 0) return 0;
   const int64_t sorted_cap = tokens * top_k + num_experts * 7;  // room for groups of up to eight pairs per expert block
-  return tokens * gguf::q8_row_bytes(K) + (sorted_cap + (sorted_cap + 3) / 4 + 1) * 4;
+  const int64_t vec = tokens * gguf::q8_row_bytes(K) + (sorted_cap + (sorted_cap + 3) / 4 + 1) * 4;
+  const int64_t tiles = gguf::moe_vec_tiles_workspace(tokens, top_k, K, num_experts);   // blocks of 32 pairs per expert
+  return vec > tiles ? vec : tiles;
 }
 
 extern "C" int gguf_moe_vec(const void* X, int xdtype, void* q8_workspace, const void* W, const int32_t* topk_ids, void* Y,
@@ -117,6 +127,9 @@ extern "C" int gguf_moe_vec_act(const void* X, int xdtype, void* q8_workspace, c
   const int ne = num_experts > 0 && num_experts <= 1024 ? (int)num_experts : 0;
   // the workspace holds at least the quantized activations; a caller that provides more says so
   const int64_t scratch_bytes = workspace_bytes > tokens * q8_row_bytes(K) ? workspace_bytes : tokens * q8_row_bytes(K);
+  if (ne > 0 && moe_vec_tiles_ok(type, pairs, ne) &&
+      scratch_bytes >= moe_vec_tiles_workspace(tokens, top_k, K, ne))
+    return moe_vec_tiles(X, xdtype, q8_workspace, W, topk_ids, Y, type, (int)N, (int)K, (int)top_k, (int)tokens, act, ne, s);
   switch (type) {
     case T_Q4_0: return moe_vec_group_std_a(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, ne, q8_workspace, scratch_bytes, s);
     case T_Q4_1: return moe_vec_group_std_a(type, W, X, Y, xdtype, (int)N, (int)K, topk_ids, (int)top_k, pairs, act, ne, q8_workspace, scratch_bytes, s);
