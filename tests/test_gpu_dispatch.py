@@ -82,7 +82,8 @@ def test_embedding_lookup_is_gather_of_exact_dequant(qt):
 
 
 @pytest.mark.parametrize("tokens,top_k,experts,block", [(1, 8, 64, 32), (7, 2, 4, 32), (512, 8, 64, 32), (33, 3, 5, 4),
-                                                        (2000, 2, 300, 32), (5, 1, 3, 8)])
+                                                        (2000, 2, 300, 32), (5, 1, 3, 8), (9000, 8, 1024, 16),
+                                                        (4096, 8, 64, 64), (100, 1, 1, 32)])
 def test_native_moe_align_block_size_matches_checker(tokens, top_k, experts, block):
     from vllm_gguf_plugin_prism_amd import ops
 
@@ -101,6 +102,26 @@ def test_native_moe_align_block_size_matches_checker(tokens, top_k, experts, blo
     # the torch statement of the same sort agrees too
     st, et, nt = D.moe_align_block_size(torch.from_numpy(ids), block, experts)
     assert int(nt[0]) == total and np.array_equal(st.numpy()[:total], s[:total])
+
+
+def test_native_moe_align_skips_experts_out_of_range():
+    from vllm_gguf_plugin_prism_amd import ops
+
+    rng = np.random.default_rng(77)
+    experts, block = 12, 8
+    ids = rng.integers(-2, experts + 3, size=(300, 4)).astype(np.int32)   # some ids name no expert
+    s, e, n = ops.moe_align_block_size(torch.from_numpy(ids).cuda(), block, experts)
+    s, e, total = s.cpu().numpy(), e.cpu().numpy(), int(n.item())
+    flat = ids.reshape(-1)
+    pos = 0
+    for ex in range(experts):
+        mine = np.nonzero(flat == ex)[0]
+        padded = (len(mine) + block - 1) // block * block
+        assert np.array_equal(s[pos:pos + len(mine)], mine)               # ascending pair index inside the run
+        assert (s[pos + len(mine):pos + padded] == flat.size).all()
+        assert (e[pos // block:(pos + padded) // block] == ex).all()
+        pos += padded
+    assert pos == total and (s[total:] == flat.size).all() and (e[total // block:] == -1).all()
 
 
 @pytest.mark.parametrize("dt", [torch.float16, torch.bfloat16, torch.float32])

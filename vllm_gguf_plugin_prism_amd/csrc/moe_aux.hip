@@ -16,79 +16,89 @@ constexpr int ALIGN_MAX_EXPERTS = 1024;
 //   sorted_ids[pos]  flat pair index, or `numel` in padding and unused slots
 //   expert_ids[b]    expert of block b, -1 past the padded total
 //   num_post_padded  padded total
-// Stable order (ascending pair index inside a run) makes the result a pure function of the input.  Pairs are taken
-// 1024 at a time; inside a chunk a pair's rank among equal experts is (same-expert pairs in earlier waves) +
-// (same-expert lanes below it in its wave), the first from a per-wave histogram in LDS, the second from ballots.
+// Stable order (ascending pair index inside a run) makes the result a pure function of the input.
+// Every wave owns a contiguous stretch of the pairs.  Pass 1 counts experts per wave (a private histogram row in LDS);
+// a scan over experts and, per expert, over waves turns the rows into the first slot of each (wave, expert); pass 2
+// walks the stretch again 64 pairs at a time, places every pair at its row's cursor plus the number of lanes below it
+// with the same expert, and moves the cursor on.  The lanes that share an expert are found with one ballot per bit
+// of the expert id.  A wave's LDS operations complete in order, so its row needs no barrier inside a pass.
 __global__ __launch_bounds__(ALIGN_THREADS) void moe_align_kernel(const int32_t* __restrict__ topk_ids, int numel,
                                                                   int num_experts, int block,
                                                                   int32_t* __restrict__ sorted_ids, int sorted_capacity,
                                                                   int32_t* __restrict__ expert_ids, int expert_capacity,
                                                                   int32_t* __restrict__ num_post_padded) {
   extern __shared__ int lds[];
-  int* start = lds;                          // [E] first slot of the expert's run, then its running cursor
-  int* wave_cnt = lds + num_experts;         // [ALIGN_WAVES][E] per-wave histogram of the current chunk
+  int* start = lds;                          // [E] pairs of the expert, then the first slot of its run
+  int* cursor = lds + num_experts;           // [ALIGN_WAVES][E] per-wave counts, then per-wave cursors
   __shared__ int total_padded;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int per_wave = ((numel + ALIGN_WAVES - 1) / ALIGN_WAVES + 63) / 64 * 64;
+  const int w_begin = min(wave * per_wave, numel), w_end = min(w_begin + per_wave, numel);
+  int* mine = cursor + wave * num_experts;
 
   for (int i = tid; i < sorted_capacity; i += ALIGN_THREADS) sorted_ids[i] = numel;
-  for (int e = tid; e < num_experts; e += ALIGN_THREADS) start[e] = 0;
-  __syncthreads();
-  for (int i = tid; i < numel; i += ALIGN_THREADS) {
+  for (int e = lane; e < num_experts; e += 64) mine[e] = 0;
+  for (int i = w_begin + lane; i < w_end; i += 64) {
     const int e = topk_ids[i];
-    if (e >= 0 && e < num_experts) atomicAdd(&start[e], 1);  // counts: the sum does not depend on the order of adds
+    if (e >= 0 && e < num_experts) atomicAdd(&mine[e], 1);  // counts: the sum does not depend on the order of adds
   }
   __syncthreads();
-  if (tid == 0) {
-    int pos = 0;
-    for (int e = 0; e < num_experts; ++e) {
-      const int padded = (start[e] + block - 1) / block * block;
-      start[e] = pos;
-      pos += padded;
-    }
-    total_padded = pos;
-    num_post_padded[0] = pos;
-  }
-  __syncthreads();
-  // expert of every block: expert e owns blocks [start[e], start[e+1]) / block
   for (int e = tid; e < num_experts; e += ALIGN_THREADS) {
+    int sum = 0;
+    for (int w = 0; w < ALIGN_WAVES; ++w) sum += cursor[w * num_experts + e];
+    start[e] = sum;
+  }
+  __syncthreads();
+  if (wave == 0) {  // exclusive scan of the padded counts, 64 experts at a time
+    int running = 0;
+    for (int e0 = 0; e0 < num_experts; e0 += 64) {
+      const int e = e0 + lane;
+      const int padded = e < num_experts ? (start[e] + block - 1) / block * block : 0;
+      int incl = padded;
+#pragma unroll
+      for (int d = 1; d < 64; d <<= 1) {
+        const int below = __shfl_up(incl, d);
+        if (lane >= d) incl += below;
+      }
+      if (e < num_experts) start[e] = running + incl - padded;
+      running += __shfl(incl, 63);
+    }
+    if (lane == 0) {
+      total_padded = running;
+      num_post_padded[0] = running;
+    }
+  }
+  __syncthreads();
+  for (int e = tid; e < num_experts; e += ALIGN_THREADS) {
+    // expert e owns blocks [start[e], start[e+1]) / block; its waves' cursors follow each other inside the run
     const int end = e + 1 < num_experts ? start[e + 1] : total_padded;
     for (int b = start[e] / block; b < end / block && b < expert_capacity; ++b) expert_ids[b] = e;
+    int pos = start[e];
+    for (int w = 0; w < ALIGN_WAVES; ++w) {
+      const int c = cursor[w * num_experts + e];
+      cursor[w * num_experts + e] = pos;
+      pos += c;
+    }
   }
   for (int b = total_padded / block + tid; b < expert_capacity; b += ALIGN_THREADS) expert_ids[b] = -1;
+  __syncthreads();
 
-  for (int c0 = 0; c0 < numel; c0 += ALIGN_THREADS) {
-    for (int i = tid; i < ALIGN_WAVES * num_experts; i += ALIGN_THREADS) wave_cnt[i] = 0;
-    __syncthreads();
-    const int i = c0 + tid;
-    int e = i < numel ? topk_ids[i] : -1;
+  const int bits = 32 - __clz(max(num_experts - 1, 1));
+  for (int i0 = w_begin; i0 < w_end; i0 += 64) {
+    const int i = i0 + lane;
+    int e = i < w_end ? topk_ids[i] : -1;
     if (e >= num_experts) e = -1;
-    // rank among the lanes of this wave with the same expert, and this wave's count of it
-    int rank_in_wave = 0;
-    unsigned long long todo = __ballot(e >= 0);
-    while (todo) {
-      const int leader = __ffsll((long long)todo) - 1;
-      const int e0 = __shfl(e, leader);
-      const unsigned long long same = __ballot(e == e0);
-      if (e == e0) {
-        rank_in_wave = __popcll(same & ((1ull << lane) - 1));
-        if (lane == leader) wave_cnt[wave * num_experts + e0] = __popcll(same);
-      }
-      todo &= ~same;
+    unsigned long long same = __ballot(e >= 0);   // lanes with this lane's expert
+    for (int b = 0; b < bits; ++b) {
+      const unsigned long long set = __ballot((e >> b) & 1);
+      same &= ((e >> b) & 1) ? set : ~set;
     }
-    __syncthreads();
     if (e >= 0) {
-      int before = 0;
-      for (int w = 0; w < wave; ++w) before += wave_cnt[w * num_experts + e];
-      const int pos = start[e] + before + rank_in_wave;
+      const int below = __popcll(same & ((1ull << lane) - 1));
+      const int pos = mine[e] + below;
       if (pos < sorted_capacity) sorted_ids[pos] = i;
+      if (below == 0) mine[e] = pos + __popcll(same);   // one lane per expert moves the cursor; read above, written here
     }
-    __syncthreads();
-    for (int ee = tid; ee < num_experts; ee += ALIGN_THREADS) {
-      int sum = 0;
-      for (int w = 0; w < ALIGN_WAVES; ++w) sum += wave_cnt[w * num_experts + ee];
-      start[ee] += sum;
-    }
-    __syncthreads();
   }
 }
 
@@ -122,6 +132,14 @@ extern "C" int gguf_moe_align_block_size(const int32_t* topk_ids, int64_t numel,
     return GGUF_ERR_SHAPE;
   if (!sorted_token_ids || !expert_ids || !num_tokens_post_padded || (numel > 0 && !topk_ids)) return GGUF_ERR_NULL;
   const size_t lds = (size_t)(1 + ALIGN_WAVES) * num_experts * sizeof(int);
+  if (lds > 65536) {
+    static bool configured = false;  // opt in to > 64 KB of dynamic LDS once
+    if (!configured) {
+      (void)hipFuncSetAttribute((const void*)moe_align_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                (int)((1 + ALIGN_WAVES) * ALIGN_MAX_EXPERTS * sizeof(int)));
+      configured = true;
+    }
+  }
   hipLaunchKernelGGL(moe_align_kernel, dim3(1), dim3(ALIGN_THREADS), lds, (hipStream_t)stream, topk_ids, (int)numel,
                      (int)num_experts, (int)block, sorted_token_ids, (int)sorted_capacity, expert_ids, (int)expert_capacity,
                      num_tokens_post_padded);
