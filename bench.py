@@ -86,6 +86,93 @@ def _graph_ms(fn, calls, replays):
     return start.elapsed_time(stop) / (replays * calls)
 
 
+def _timed_ms(fn, calls):
+    """Graph-timed milliseconds per call where the calls can be captured, event-timed otherwise."""
+    import torch
+
+    try:
+        return _graph_ms(fn, calls, 5)
+    except Exception:  # a call that cannot be captured: time the eager launches
+        torch.cuda.synchronize()
+        for i in range(3):
+            fn(i)
+        return _events_ms(fn, calls * 5)
+
+
+def _other_configs(rng, dev):
+    """The BASELINE configurations the headline does not cover, each as time per call and the rate its roofline names."""
+    import torch
+
+    from vllm_gguf_plugin_prism_amd import dispatch, ops, synth
+
+    Q8_0, Q4_0, IQ2_XXS, IQ4_XS = 8, 2, 16, 23
+    res = {}
+
+    def gemv_bytes(qt, n, k, m):
+        qk, bs = ops.quant_sizes(qt)
+        return n * (k // qk) * bs + 2 * m * k + 2 * m * n
+
+    def xs(m, k):
+        return torch.from_numpy(rng.standard_normal((m, k)).astype(np.float32)).to(torch.float16).to(dev)
+
+    # config 1: Q8_0 [3072,1024] dequantize and batch-1 GEMV (3.3 MB: launch-bound)
+    n, k = 3072, 1024
+    w = torch.from_numpy(synth.make_weights(rng, Q8_0, n, k)).to(dev)
+    x = xs(1, k)
+    ms = _timed_ms(lambda i: ops.ggml_dequantize(w, Q8_0, n, k, torch.float16), 20)
+    res["config1_q8_0_dequant_fp16"] = {"us": ms * 1e3, "GBps": (w.numel() + 2 * n * k) / (ms * 1e-3) / 1e9}
+    ms = _timed_ms(lambda i: ops.ggml_mul_mat_vec_a8(w, x, Q8_0, n), 20)
+    res["config1_q8_0_gemv_bs1"] = {"us": ms * 1e3, "GBps": gemv_bytes(Q8_0, n, k, 1) / (ms * 1e-3) / 1e9}
+
+    # config 2: batch sweep on [14336,4096]; the reference's policy sends batch 4 and 8 at this N to the tile GEMM
+    n, k = 14336, 4096
+    copies = [torch.from_numpy(np.concatenate([synth.make_weights(rng, Q4_K, 2048, k) for _ in range(n // 2048)])).to(dev)]
+    copies += [copies[0].clone() for _ in range(19)]          # 20 x 33 MB, walked in turn
+    for b in (1, 2, 4, 8):
+        x = xs(b, k)
+        path = dispatch.select_mul_mat_path(Q4_K, b, n)
+        ms = _timed_ms(lambda i: dispatch.fused_mul_mat_gguf(x, copies[i % 20], Q4_K), 20)
+        res[f"config2_q4_k_14336x4096_bs{b}"] = {"path": path, "us": ms * 1e3,
+                                                "GBps": gemv_bytes(Q4_K, n, k, b) / (ms * 1e-3) / 1e9}
+        if path != "mmvq":
+            ms = _timed_ms(lambda i: ops.ggml_mul_mat_vec_a8(copies[i % 20], x, Q4_K, n), 20)
+            res[f"config2_q4_k_14336x4096_bs{b}_gemv"] = {"path": "mmvq (forced)", "us": ms * 1e3,
+                                                         "GBps": gemv_bytes(Q4_K, n, k, b) / (ms * 1e-3) / 1e9}
+    del copies
+
+    # config 4: codebook formats, raw valid blocks
+    for qt, name, n, k in ((IQ4_XS, "iq4_xs", 5120, 5120), (IQ2_XXS, "iq2_xxs", 17408, 5120)):
+        nc = 16
+        base = torch.from_numpy(synth.random_blocks(rng, qt, n, k)).to(dev)
+        cp = [base] + [base.clone() for _ in range(nc - 1)]
+        x = xs(1, k)
+        ms = _timed_ms(lambda i: ops.ggml_mul_mat_vec_a8(cp[i % nc], x, qt, n), nc)
+        res[f"config4_{name}_gemv_bs1"] = {"us": ms * 1e3, "GBps": gemv_bytes(qt, n, k, 1) / (ms * 1e-3) / 1e9}
+        x = xs(256, k)
+        ms = _timed_ms(lambda i: dispatch.fused_mul_mat_gguf(x, base, qt), 10)
+        res[f"config4_{name}_m256_dequant_then_gemm"] = {"us": ms * 1e3, "TFLOPS": 2.0 * 256 * n * k / (ms * 1e-3) / 1e12}
+        ms = _timed_ms(lambda i: ops.ggml_mul_mat_a8(base, x, qt, n), 10)
+        res[f"config4_{name}_m256_a8_gemm"] = {"us": ms * 1e3, "TOPS": 2.0 * 256 * n * k / (ms * 1e-3) / 1e12}
+        del cp, base
+
+    # config 5: 64-expert top-8 Q4_0 MoE layer, whole layer (two expert GEMMs, gated activation, weighted sum)
+    E, H, I, top_k = 64, 2048, 1024, 8
+    w13 = torch.from_numpy(np.stack([synth.random_blocks(rng, Q4_0, 2 * I, H) for _ in range(E)])).to(dev)
+    w2 = torch.from_numpy(np.stack([synth.random_blocks(rng, Q4_0, H, I) for _ in range(E)])).to(dev)
+    expert_bytes = (w13.numel() + w2.numel()) // E
+    for t in (1, 64, 512):
+        x = xs(t, H)
+        tw, ids = torch.topk(torch.softmax(torch.randn(t, E, device=dev), 1), top_k)
+        ids = ids.to(torch.int32).contiguous()
+        tw = tw.to(torch.float16)
+        ms = _timed_ms(lambda i: dispatch.fused_moe_gguf(x, w13, w2, tw, ids, Q4_0, Q4_0, "silu"), 5)
+        distinct = int(torch.unique(ids).numel())
+        res[f"config5_moe_q4_0_T{t}"] = {"path": dispatch.select_moe_path(Q4_0, Q4_0, t), "us": ms * 1e3,
+                                         "TOPS": 2.0 * t * top_k * 3 * I * H / (ms * 1e-3) / 1e12,
+                                         "distinct_expert_GBps": distinct * expert_bytes / (ms * 1e-3) / 1e9}
+    return res
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -93,6 +180,9 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-mmq", action="store_true", help="skip the Q6_K MMQ leg")
+    ap.add_argument("--all-configs", action="store_true",
+                    help="also time the other BASELINE configurations (1: Q8_0, 2: batch sweep, 4: i-quants, 5: MoE layer) "
+                         "into an 'other_configs' object; about a minute more")
     ap.add_argument("--profile", action="store_true",
                     help="counter-collection mode: eager launches only (no HIP graph), no CPU leg, M=512 only for "
                          "the MMQ leg, and one 256 MiB device copy at the end to calibrate byte counters")
@@ -234,6 +324,9 @@ def main() -> int:
             "sample": f"Q4_K [{n},{k}] batch 1: numpy fp32 block dequantize ({best[1] * 1e3:.1f} ms) + torch fp32 matmul "
                       f"({best[2] * 1e3:.1f} ms), best of {reps - 1} after 1 warm-up; os.cpu_count()={os.cpu_count()}",
         }
+
+    if args.all_configs:
+        out["other_configs"] = _other_configs(rng, dev)
 
     if args.profile:
         # one plain device-to-device copy of known size: its FETCH_SIZE / WRITE_SIZE readings give the scale of

@@ -46,6 +46,29 @@ def test_mmq_matches_a8_oracle_fp32(qtype, m):
         assert err <= 1e-5, (o.TYPE_NAMES[qtype], m, n, k, err)
 
 
+@pytest.mark.parametrize("dt", ["f32", "f16"])
+@pytest.mark.parametrize("qtype", MMQ_TYPES)
+def test_mmq_handful_of_rows_keeps_tile_semantics(qtype, dt):
+    """Up to eight rows of X run on the streaming GEMV kernel.  The operator is still the tile GEMM: Q4_K / Q5_K take
+    their offset from the stored block sums and Q5_0 from the quant sums, which is where the reference's two operators
+    part (the oracle's "mmq" and "mmvq" results differ by 1e-2 .. 1e-4 on these weights)."""
+    ops = _ops()
+    rng = np.random.default_rng(450 + qtype)
+    n, k = 200, 1536
+    w = o.make_weights(rng, qtype, n, k)
+    wd = _dev(w)
+    for m in (1, 2, 3, 4, 5, 6, 8):
+        xd, xv = _x(rng, m, k, dt)
+        y = ops.ggml_mul_mat_a8(wd, xd, qtype, n)
+        assert y.shape == (m, n) and y.dtype == TORCH_DT[dt]
+        err = o.rel_l2(y.float().cpu().numpy(), o.mul_mat_a8(w, xv, qtype, n, "mmq"))
+        assert err <= (1e-5 if dt == "f32" else 1e-3), (o.TYPE_NAMES[qtype], m, err)
+        # the engines asked for by name are still the tile kernels
+        if dt == "f16":
+            yi = ops.ggml_mul_mat_a8(wd, xd, qtype, n, engine="int8")
+            assert o.rel_l2(yi.float().cpu().numpy(), y.float().cpu().numpy()) <= 1e-3
+
+
 @pytest.mark.parametrize("engine", ["auto", "int8", "half"])
 @pytest.mark.parametrize("dt", ["f16", "bf16"])
 @pytest.mark.parametrize("qtype", MMQ_TYPES)

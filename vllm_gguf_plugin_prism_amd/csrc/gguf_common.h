@@ -150,6 +150,7 @@ struct LinearArgs {
   int64_t w_pitch = 0;         // bytes between rows of W; 0 = rows are dense
   int64_t ldy = 0;             // elements between rows of Y; 0 = N
   const void* bias = nullptr;  // N values of Y's dtype, added to every row of the result after it is rounded; or null
+  bool tile_sums = false;      // GEMV kernels only: form the offset term as the reference's tile kernels do (see TileSums)
 };
 // out = round(round(v) + bias): the reference rounds the product to the output dtype and then adds in that dtype
 template <typename T>
@@ -163,6 +164,7 @@ __device__ __forceinline__ T finish(float v, const T* bias, int64_t n) {
 int quantize_q8_1(const void* x, int xdtype, void* ws, int64_t M, int64_t K, hipStream_t stream, int act = 0,
                   void* half_plane = nullptr);
 
+constexpr int GGUF_NOT_TAKEN = 1;  // internal: a route that declined the call (never returned through the C ABI)
 inline int launch_status() { return hipGetLastError() == hipSuccess ? GGUF_OK : GGUF_ERR_LAUNCH; }
 
 }  // namespace gguf

@@ -651,6 +651,10 @@ int moe_vec_tiles(const void* X, int xdtype, void* workspace, const void* W, con
   return GGUF_ERR_TYPE;
 }
 
+// mmvq.hip
+int mmvq_any(int type, const void* W, const void* x, void* q8_workspace, void* Y, int xdtype, int64_t N, int64_t K, int64_t M,
+             hipStream_t s, const LinearArgs& la);
+
 // mmq_h.hip
 int mmq_half(const void* W, const void* ws, void* Y, int dtype, int type, int M, int N, int K, float* partial,
              int64_t partial_bytes, hipStream_t s, const LinearArgs& la);
@@ -686,6 +690,14 @@ extern "C" int gguf_mmq_linear(const void* W, int64_t w_row_pitch_bytes, const v
   if (N == 0 || M == 0) return GGUF_OK;
   if (!W || !x || !q8_workspace || !Y) return GGUF_ERR_NULL;
   hipStream_t s = (hipStream_t)stream;
+  if (engine == GGUF_MMQ_AUTO && M <= 8) {
+    // a handful of rows: the streaming GEMV kernel with the tile kernels' offset sums reads W once at close to the
+    // GEMV's rate and is exact in int8; it declines shapes it does not cover
+    LinearArgs lt = la;
+    lt.tile_sums = true;
+    const int rc = mmvq_any(type, W, x, q8_workspace, Y, xdtype, N, K, M, s, lt);
+    if (rc != GGUF_NOT_TAKEN) return rc;
+  }
   if (engine == GGUF_MMQ_AUTO) engine = (xdtype != GGUF_DTYPE_F32 && mmq_half_supported(type)) ? GGUF_MMQ_HALF : GGUF_MMQ_INT8;
   if (engine == GGUF_MMQ_HALF) {
     void* half_plane = (char*)q8_workspace + M * q8_row_bytes(K);

@@ -36,22 +36,10 @@ int moe_vec_group_iq_c(int type, const void* W, const void* x, void* Y, int dtyp
 
 }  // namespace gguf
 
-extern "C" int gguf_mmvq_linear(const void* W, int64_t w_row_pitch_bytes, const void* x, int xdtype, void* q8_workspace, void* Y,
-                                int64_t y_row_pitch, const void* bias, int type, int64_t N, int64_t K, int64_t M,
-                                gguf_stream_t stream) {
-  using namespace gguf;
-  const int qk = block_elems(type);
-  if (qk == 0) return GGUF_ERR_TYPE;
-  if (N < 0 || M < 0 || K <= 0 || K % qk != 0 || N > 0x7FFFFFF0LL || K > 0x7FFFFFF0LL) return GGUF_ERR_SHAPE;
-  if (w_row_pitch_bytes < K / qk * block_bytes(type) || y_row_pitch < N) return GGUF_ERR_SHAPE;
-  LinearArgs la;
-  la.w_pitch = w_row_pitch_bytes;
-  la.ldy = y_row_pitch;
-  la.bias = bias;
-  if (xdtype < 0 || xdtype > 2) return GGUF_ERR_DTYPE;
-  if (N == 0 || M == 0) return GGUF_OK;
-  if (!W || !x || !q8_workspace || !Y) return GGUF_ERR_NULL;
-  hipStream_t s = (hipStream_t)stream;
+namespace gguf {
+// one GEMV call after validation; with la.tile_sums the result is GGUF_NOT_TAKEN where the streaming kernel does not apply
+int mmvq_any(int type, const void* W, const void* x, void* q8_workspace, void* Y, int xdtype, int64_t N, int64_t K, int64_t M,
+             hipStream_t s, const LinearArgs& la) {
   switch (type) {
     case T_Q4_0: return mmvq_group_std_a(type, W, x, q8_workspace, Y, xdtype, N, K, M, s, la);
     case T_Q4_1: return mmvq_group_std_a(type, W, x, q8_workspace, Y, xdtype, N, K, M, s, la);
@@ -74,6 +62,25 @@ extern "C" int gguf_mmvq_linear(const void* W, int64_t w_row_pitch_bytes, const 
     case T_IQ1_M: return mmvq_group_iq_c(type, W, x, q8_workspace, Y, xdtype, N, K, M, s, la);
   }
   return GGUF_ERR_TYPE;
+}
+}  // namespace gguf
+
+extern "C" int gguf_mmvq_linear(const void* W, int64_t w_row_pitch_bytes, const void* x, int xdtype, void* q8_workspace, void* Y,
+                                int64_t y_row_pitch, const void* bias, int type, int64_t N, int64_t K, int64_t M,
+                                gguf_stream_t stream) {
+  using namespace gguf;
+  const int qk = block_elems(type);
+  if (qk == 0) return GGUF_ERR_TYPE;
+  if (N < 0 || M < 0 || K <= 0 || K % qk != 0 || N > 0x7FFFFFF0LL || K > 0x7FFFFFF0LL) return GGUF_ERR_SHAPE;
+  if (w_row_pitch_bytes < K / qk * block_bytes(type) || y_row_pitch < N) return GGUF_ERR_SHAPE;
+  LinearArgs la;
+  la.w_pitch = w_row_pitch_bytes;
+  la.ldy = y_row_pitch;
+  la.bias = bias;
+  if (xdtype < 0 || xdtype > 2) return GGUF_ERR_DTYPE;
+  if (N == 0 || M == 0) return GGUF_OK;
+  if (!W || !x || !q8_workspace || !Y) return GGUF_ERR_NULL;
+  return mmvq_any(type, W, x, q8_workspace, Y, xdtype, N, K, M, (hipStream_t)stream, la);
 }
 
 extern "C" int gguf_mmvq(const void* W, const void* x, int xdtype, void* q8_workspace, void* Y, int type, int64_t N,

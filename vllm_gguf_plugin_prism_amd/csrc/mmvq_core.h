@@ -219,10 +219,21 @@ __global__ __launch_bounds__(256) void mmvq_kernel(const uint8_t* __restrict__ W
 #define GGUF_MMVQ_WG_PER_CU 1
 #endif
 
-template <class F, int MT, int NW, int D, typename T>
+// The reference's GEMV and its tile GEMM (ggml_mul_mat_a8) differ in three formats, and only in which per-block sum
+// of the activations meets the offset: Q4_K / Q5_K multiply their mins by d8*sum(q) in the GEMV (vecdotq.cuh:328-351,
+// 384-441) and by the stored sum of the unquantized values in the tiles (:369-372, :1325-1415); Q5_0 subtracts
+// 16 * (stored sum) in the GEMV (:98-125) while its tiles use signed codes, i.e. 16 * d8*sum(q) (:668-749).  With
+// TILE set the streaming kernel keeps the other plane of the quantizer's output for these formats, which turns it
+// into the tile GEMM for a handful of rows of X.
+template <class F> struct TileSums { static constexpr bool swaps = false; };
+template <> struct TileSums<FmtQ5_0> { static constexpr bool swaps = true; };
+template <> struct TileSums<FmtQ4_K> { static constexpr bool swaps = true; };
+template <> struct TileSums<FmtQ5_K> { static constexpr bool swaps = true; };
+
+template <class F, int MT, int NW, int D, typename T, bool TILE = false>
 __global__ __launch_bounds__(64 * NW) void mmvq_stream_kernel(const uint8_t* __restrict__ W, const T* __restrict__ X,
                                                                T* __restrict__ Y, int N, int K, int rows_per_wg, int64_t w_pitch,
-                                                               int64_t ldy, const T* __restrict__ bias) {
+                                                               int64_t ldy, const T* __restrict__ bias, int m_act) {
   extern __shared__ __align__(16) char smem[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: row arithmetic stays on the scalar unit
@@ -269,7 +280,7 @@ __global__ __launch_bounds__(64 * NW) void mmvq_stream_kernel(const uint8_t* __r
   // wait for the weight loads behind them.  Groups past the end are clamped and their stores predicated.
   constexpr int NT = 64 * NW;
   const int g8 = K >> 3;
-  const int qtotal = MT * g8;  // a multiple of 4, so quads stay whole
+  const int qtotal = m_act * g8;  // a multiple of 4, so quads stay whole; rows m_act .. MT-1 of the tile are never stored
   typename F::Regs pre[D];
   auto quantize_group = [&](const raw8<T>& raw, int q) {
     const int qc = min(q, qtotal - 1);
@@ -285,8 +296,9 @@ __global__ __launch_bounds__(64 * NW) void mmvq_stream_kernel(const uint8_t* __r
       *(uint2*)(lq + (size_t)m * K + 8 * j) = qq.q;
       if ((j & 3) == 0) {
         ldv[m * nb + (j >> 2)] = qq.d;
-        if (F::AUX == AUX_S8) lav[m * nb + (j >> 2)] = qq.s;
-        if (F::AUX == AUX_DU) lav[m * nb + (j >> 2)] = qq.du;
+        constexpr bool SWAP = TILE && TileSums<F>::swaps;
+        if (F::AUX == AUX_S8) lav[m * nb + (j >> 2)] = SWAP ? qq.du : qq.s;
+        if (F::AUX == AUX_DU) lav[m * nb + (j >> 2)] = SWAP ? qq.s : qq.du;
       }
     }
   };
@@ -358,7 +370,7 @@ __global__ __launch_bounds__(64 * NW) void mmvq_stream_kernel(const uint8_t* __r
     const int row = i / MT, m = i - row * MT;
     float v = 0.0f;
     for (int st = 0; st < S; ++st) v += part[(row * S + st) * MT + m];
-    Y[(int64_t)m * ldy + r_begin + row] = finish<T>(v, bias, r_begin + row);
+    if (m < m_act) Y[(int64_t)m * ldy + r_begin + row] = finish<T>(v, bias, r_begin + row);
   }
 }
 
@@ -373,24 +385,25 @@ static int num_cus() {
   return n;
 }
 
-template <class F, int MT, int D, typename T>
+template <class F, int MT, int D, typename T, bool TILE>
 static void launch_stream_d(const void* W, const T* X, T* Y, int N, int K, int rows_per_wg, int grid, size_t lds, const LinearArgs& la,
-                            hipStream_t stream) {
+                            hipStream_t stream, int m_act) {
   constexpr int NW = GGUF_MMVQ_NW;
-  auto kern = mmvq_stream_kernel<F, MT, NW, D, T>;
+  auto kern = mmvq_stream_kernel<F, MT, NW, D, T, TILE>;
   static bool big_lds = false;
   if (lds > 64 * 1024 && !big_lds) {
     (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
     big_lds = true;
   }
   hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * NW), lds, stream, (const uint8_t*)W, X, Y, N, K, rows_per_wg,
-                     la.w_pitch ? la.w_pitch : (int64_t)(K / F::QK) * F::BS, la.ldy ? la.ldy : (int64_t)N, (const T*)la.bias);
+                     la.w_pitch ? la.w_pitch : (int64_t)(K / F::QK) * F::BS, la.ldy ? la.ldy : (int64_t)N, (const T*)la.bias, m_act);
 }
 
 // Returns false when the shape does not fit the streaming kernel (a row longer than NW waves, or activations
 // that do not fit in LDS); the caller then takes the workspace path.
-template <class F, int MT, typename T>
-static bool launch_stream(const void* W, const T* X, T* Y, int N, int K, hipStream_t stream, const LinearArgs& la) {
+template <class F, int MT, typename T, bool TILE = false>
+static bool launch_stream(const void* W, const T* X, T* Y, int N, int K, hipStream_t stream, const LinearArgs& la, int m_act = MT) {
+  // m_act <= MT rows of X are there; the kernel computes MT and stores m_act
   constexpr int NW = GGUF_MMVQ_NW;
   const int nb = K / 32, S = (nb + 63) / 64;
   if (S > NW) return false;
@@ -403,9 +416,12 @@ static bool launch_stream(const void* W, const T* X, T* Y, int N, int K, hipStre
                      (size_t)rows_per_wg * S * MT * 4;
   if (lds > 150 * 1024) return false;
   const int per_wave = (rows_per_wg + slots - 1) / slots;  // rows each wave walks; the pipeline depth never exceeds it
-  if (per_wave >= GGUF_MMVQ_DEPTH) launch_stream_d<F, MT, GGUF_MMVQ_DEPTH, T>(W, X, Y, N, K, rows_per_wg, grid, lds, la, stream);
-  else if (per_wave >= 2) launch_stream_d<F, MT, 2, T>(W, X, Y, N, K, rows_per_wg, grid, lds, la, stream);
-  else launch_stream_d<F, MT, 1, T>(W, X, Y, N, K, rows_per_wg, grid, lds, la, stream);
+  if constexpr (MT <= 4) {
+    if (per_wave >= GGUF_MMVQ_DEPTH) { launch_stream_d<F, MT, GGUF_MMVQ_DEPTH, T, TILE>(W, X, Y, N, K, rows_per_wg, grid, lds, la, stream, m_act); return true; }
+    if (per_wave >= 2) { launch_stream_d<F, MT, 2, T, TILE>(W, X, Y, N, K, rows_per_wg, grid, lds, la, stream, m_act); return true; }
+  }
+  // eight activation rows in registers leave room for one weight row in flight per wave
+  launch_stream_d<F, MT, 1, T, TILE>(W, X, Y, N, K, rows_per_wg, grid, lds, la, stream, m_act);
   return true;
 }
 
@@ -413,7 +429,7 @@ static bool launch_stream(const void* W, const T* X, T* Y, int N, int K, hipStre
 #define GGUF_MMVQ_RPW 2
 #endif
 #ifndef GGUF_MMVQ_MAX_FUSED_M
-#define GGUF_MMVQ_MAX_FUSED_M 4
+#define GGUF_MMVQ_MAX_FUSED_M 8
 #endif
 constexpr int MAX_FUSED_M = GGUF_MMVQ_MAX_FUSED_M;  // up to this many vectors are quantized inside the GEMV itself
 
@@ -445,14 +461,29 @@ template <class F, typename T>
 static int mmvq_typed(const void* W, const void* x, void* ws, void* Y, int xdtype, int64_t N, int64_t K, int64_t M,
                       hipStream_t stream, const LinearArgs& la) {
   const int64_t ldy = la.ldy ? la.ldy : N;
+  if (la.tile_sums) {
+    // the tile GEMM's arithmetic for a handful of rows; GGUF_NOT_TAKEN sends the caller back to its tile kernels
+    if (M > MAX_FUSED_M) return GGUF_NOT_TAKEN;
+    const T* xs = (const T*)x;
+    bool ok;
+    if constexpr (TileSums<F>::swaps) {
+      if (M <= 4) ok = launch_stream<F, 4, T, true>(W, xs, (T*)Y, (int)N, (int)K, stream, la, (int)M);
+      else ok = launch_stream<F, 8, T, true>(W, xs, (T*)Y, (int)N, (int)K, stream, la, (int)M);
+    } else {  // the two operators agree on these formats: the GEMV's own kernels serve
+      if (M == 1) ok = launch_stream<F, 1, T>(W, xs, (T*)Y, (int)N, (int)K, stream, la);
+      else if (M == 2) ok = launch_stream<F, 2, T>(W, xs, (T*)Y, (int)N, (int)K, stream, la);
+      else if (M <= 4) ok = launch_stream<F, 4, T>(W, xs, (T*)Y, (int)N, (int)K, stream, la, (int)M);
+      else ok = launch_stream<F, 8, T>(W, xs, (T*)Y, (int)N, (int)K, stream, la, (int)M);
+    }
+    return ok ? launch_status() : GGUF_NOT_TAKEN;
+  }
   if (M <= MAX_FUSED_M) {
     const T* xs = (const T*)x;
     bool ok;
     if (M == 1) ok = launch_stream<F, 1, T>(W, xs, (T*)Y, (int)N, (int)K, stream, la);
     else if (M == 2) ok = launch_stream<F, 2, T>(W, xs, (T*)Y, (int)N, (int)K, stream, la);
-    else if (M == 4) ok = launch_stream<F, 4, T>(W, xs, (T*)Y, (int)N, (int)K, stream, la);
-    else ok = launch_stream<F, 2, T>(W, xs, (T*)Y, (int)N, (int)K, stream, la) &&
-              launch_stream<F, 1, T>(W, xs + 2 * K, (T*)Y + 2 * ldy, (int)N, (int)K, stream, la);
+    else if (M <= 4) ok = launch_stream<F, 4, T>(W, xs, (T*)Y, (int)N, (int)K, stream, la, (int)M);
+    else ok = launch_stream<F, 8, T>(W, xs, (T*)Y, (int)N, (int)K, stream, la, (int)M);
     if (ok) return launch_status();
   }
   const int rc = quantize_q8_1(x, xdtype, ws, M, K, stream);
