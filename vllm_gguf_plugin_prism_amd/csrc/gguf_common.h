@@ -74,6 +74,24 @@ __device__ __forceinline__ T ld(const void* p) {
   __builtin_memcpy(&v, p, sizeof(T));
   return v;
 }
+// A block whose size is 2 modulo 4 (18, 22, 34 bytes) starts at an even address that is a multiple of 4 for every
+// other block only.  A 16-byte load from such an address costs the memory pipeline about twice an aligned one, so
+// the block is fetched as the ND = (size + 2) / 4 whole dwords that cover it from the dword boundary at or below it
+// -- the first and the last of them hold at least one byte of the block, so nothing outside the dwords the block
+// touches is read -- and the fields are cut out with funnel shifts.  Returns the bit offset (0 or 16) of the block
+// inside w[0].
+template <int ND>
+__device__ __forceinline__ uint32_t ld_block_dwords(const uint8_t* p, uint32_t (&w)[ND]) {
+  const uintptr_t a = (uintptr_t)p;
+  const __attribute__((address_space(1))) uint32_t* q = (const __attribute__((address_space(1))) uint32_t*)(a & ~(uintptr_t)3);
+#pragma unroll
+  for (int i = 0; i < ND; ++i) w[i] = q[i];
+  return (uint32_t)(a & 2) * 8;
+}
+// bits [bits, bits + 32) of the 64-bit value hi:lo, bits in 0..32
+__device__ __forceinline__ uint32_t funnel(uint32_t lo, uint32_t hi, uint32_t bits) {
+  return (uint32_t)((((uint64_t)hi << 32) | lo) >> bits);
+}
 __device__ __forceinline__ float ld_f16(const void* p) { return (float)ld<_Float16>(p); }
 __device__ __forceinline__ _Float16 ld_h(const void* p) { return ld<_Float16>(p); }
 

@@ -11,8 +11,12 @@ struct FmtQ4_0 {
   struct Regs { uint16_t d; uint4 q; };
   static __device__ __forceinline__ void init_tables(char*) {}
   static __device__ __forceinline__ Regs load(const uint8_t* row, int u0, int u, const char*) {
-    const uint8_t* b = row + (int64_t)(u0 + u) * BS;
-    Regs r; r.d = ld<uint16_t>(b); r.q = ld<uint4>(b + 2); return r;
+    uint32_t w[5];
+    const uint32_t sh = ld_block_dwords(row + (int64_t)(u0 + u) * BS, w), shq = sh + 16;
+    Regs r;
+    r.d = (uint16_t)(w[0] >> sh);
+    r.q = make_uint4(funnel(w[0], w[1], shq), funnel(w[1], w[2], shq), funnel(w[2], w[3], shq), funnel(w[3], w[4], shq));
+    return r;
   }
   struct ActRegs { int4 lo, hi; float d, a; };
   static __device__ __forceinline__ ActRegs load_act(const Act& x, int u) {
@@ -41,8 +45,13 @@ struct FmtQ8_0 {
   struct Regs { uint16_t d; uint4 q0, q1; };
   static __device__ __forceinline__ void init_tables(char*) {}
   static __device__ __forceinline__ Regs load(const uint8_t* row, int u0, int u, const char*) {
-    const uint8_t* b = row + (int64_t)(u0 + u) * BS;
-    Regs r; r.d = ld<uint16_t>(b); r.q0 = ld<uint4>(b + 2); r.q1 = ld<uint4>(b + 18); return r;
+    uint32_t w[9];
+    const uint32_t sh = ld_block_dwords(row + (int64_t)(u0 + u) * BS, w), shq = sh + 16;
+    Regs r;
+    r.d = (uint16_t)(w[0] >> sh);
+    r.q0 = make_uint4(funnel(w[0], w[1], shq), funnel(w[1], w[2], shq), funnel(w[2], w[3], shq), funnel(w[3], w[4], shq));
+    r.q1 = make_uint4(funnel(w[4], w[5], shq), funnel(w[5], w[6], shq), funnel(w[6], w[7], shq), funnel(w[7], w[8], shq));
+    return r;
   }
   struct ActRegs { int4 a0, a1; float d; };
   static __device__ __forceinline__ ActRegs load_act(const Act& x, int u) {
@@ -366,7 +375,13 @@ struct FmtQ5 {
     const uint8_t* b = row + (int64_t)(u0 + u) * BS;
     Regs r;
     if (HAS_M) { r.dm = ld<uint32_t>(b); r.qh = ld<uint32_t>(b + 4); r.q = ld<uint4>(b + 8); }
-    else { r.dm = ld<uint16_t>(b); r.qh = ld<uint32_t>(b + 2); r.q = ld<uint4>(b + 6); }
+    else {
+      uint32_t w[6];
+      const uint32_t sh = ld_block_dwords(b, w), shq = sh + 16;
+      r.dm = (w[0] >> sh) & 0xFFFFu;
+      r.qh = funnel(w[0], w[1], shq);
+      r.q = make_uint4(funnel(w[1], w[2], shq), funnel(w[2], w[3], shq), funnel(w[3], w[4], shq), funnel(w[4], w[5], shq));
+    }
     return r;
   }
   typedef FmtQ4_0::ActRegs ActRegs;
