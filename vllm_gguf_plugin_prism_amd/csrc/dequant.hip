@@ -55,13 +55,11 @@ __device__ __forceinline__ void dq8_q8_0(const uint8_t* __restrict__ w, int64_t 
 __device__ __forceinline__ void scale_min_k4(uint32_t b03, uint32_t b47, uint32_t b8b, int j, int& sc, int& mn) {
   const int sh = 8 * (j & 3);
   const uint32_t lo = (b03 >> sh) & 0xFF, mid = (b47 >> sh) & 0xFF, hi = (b8b >> sh) & 0xFF;
-  if (j < 4) {
-    sc = (int)(lo & 63);
-    mn = (int)(mid & 63);
-  } else {
-    sc = (int)((hi & 0xF) | ((lo >> 6) << 4));
-    mn = (int)((hi >> 4) | ((mid >> 6) << 4));
-  }
+  // both forms are computed and one is selected: a branch here would make the compiler hold back the loads behind it
+  const int sc_lo = (int)(lo & 63), mn_lo = (int)(mid & 63);
+  const int sc_hi = (int)((hi & 0xF) | ((lo >> 6) << 4)), mn_hi = (int)((hi >> 4) | ((mid >> 6) << 4));
+  sc = j < 4 ? sc_lo : sc_hi;
+  mn = j < 4 ? mn_lo : mn_hi;
 }
 
 // Q4_K: dequantize.cuh:165-196.  d1 = d*sc, m1 = dmin*m (each rounded), y = fma(d1, q, -m1).
@@ -70,13 +68,13 @@ __device__ __forceinline__ void dq8_q4_k(const uint8_t* __restrict__ w, int64_t 
   const int r = (int)(e0 & 255);
   const int j = r >> 5, pos = r & 31;
   const uint4 hdr = *(const uint4*)blk;  // 144-byte blocks keep 16-byte alignment
+  const uint2 q = *(const uint2*)(blk + 16 + 32 * (j >> 1) + pos);   // both loads are in flight before either is used
   const h16 dall = __builtin_bit_cast(h16, (uint16_t)(hdr.x & 0xFFFF));
   const h16 dmin = __builtin_bit_cast(h16, (uint16_t)(hdr.x >> 16));
   int sc, mn;
   scale_min_k4(hdr.y, hdr.z, hdr.w, j, sc, mn);
   const h16 d1 = dall * (h16)sc;
   const h16 m1 = dmin * (h16)mn;
-  const uint2 q = *(const uint2*)(blk + 16 + 32 * (j >> 1) + pos);
   const int sh = (j & 1) ? 4 : 0;
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
@@ -106,6 +104,17 @@ __device__ __forceinline__ void dq8_q6_k(const uint8_t* __restrict__ w, int64_t 
   }
 }
 
+// kvalues_iq4nl (ggml-common.h:1060) of four 4-bit codes held one per byte, as four signed bytes: the table sits
+// in four registers and v_perm picks from it, instead of eight byte loads from memory per thread.
+__device__ __forceinline__ int kvalues_iq4nl4(uint32_t idx) {
+  constexpr uint32_t T0 = 0xBFAD9881u, T1 = 0xF6EADDCFu, T2 = 0x26190D01u, T3 = 0x71594535u;  // -127 -104 -83 -65 | ... | 53 69 89 113
+  const uint32_t sel = idx & 0x07070707u;
+  const uint32_t lo = __builtin_amdgcn_perm(T1, T0, sel);
+  const uint32_t hi = __builtin_amdgcn_perm(T3, T2, sel);
+  const uint32_t m = ((idx >> 3) & 0x01010101u) * 0xFFu;
+  return (int)((hi & m) | (lo & ~m));
+}
+
 // IQ4_XS: dequantize.cuh:420-435 (fp32).
 __device__ __forceinline__ void dq8_iq4_xs(const uint8_t* __restrict__ w, int64_t e0, float (&o)[8]) {
   const uint8_t* blk = w + (e0 >> 8) * 136;
@@ -116,11 +125,9 @@ __device__ __forceinline__ void dq8_iq4_xs(const uint8_t* __restrict__ w, int64_
   const float d = ld_f16(blk) * (float)(ls - 32);
   const uint2 q = ld<uint2>(blk + 8 + 16 * ib + (pos & 15));
   const int shq = pos >> 4 ? 4 : 0;
+  const int v0 = kvalues_iq4nl4((q.x >> shq) & 0x0F0F0F0Fu), v1 = kvalues_iq4nl4((q.y >> shq) & 0x0F0F0F0Fu);
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const uint32_t word = i < 4 ? q.x : q.y;
-    o[i] = d * (float)k_kvalues_iq4nl[(word >> (8 * (i & 3) + shq)) & 0xF];
-  }
+  for (int i = 0; i < 8; ++i) o[i] = d * (float)(int8_t)((i < 4 ? v0 : v1) >> (8 * (i & 3)));
 }
 
 // IQ2_XXS: dequantize.cuh:258-275 (fp32).  Grid magnitudes are decoded from the 16-bit code word.
@@ -198,8 +205,12 @@ __device__ __forceinline__ void dq8_q2_k(const uint8_t* __restrict__ w, int64_t 
 
 // 6-bit scale `is` of a Q3_K block, minus nothing (dequantize.cuh:137-140); s points at the 12 scale bytes.
 __device__ __forceinline__ int q3k_scale(const uint8_t* __restrict__ s, int is) {
-  const int lo = is < 8 ? (s[is] & 0xF) : (s[is - 8] >> 4);
-  const int hi = (s[8 + (is & 3)] >> (2 * (is >> 2))) & 3;
+  // the twelve bytes as three dwords, fields by shifts: byte loads at computed offsets behind a branch would be
+  // issued one after the other
+  const uint32_t s0 = ld<uint32_t>(s), s1 = ld<uint32_t>(s + 4), s2 = ld<uint32_t>(s + 8);
+  const uint32_t lo8 = ((is & 4) ? s1 : s0) >> (8 * (is & 3));        // byte is % 8
+  const int lo = (int)((lo8 >> (is < 8 ? 0 : 4)) & 0xF);
+  const int hi = (int)((s2 >> (8 * (is & 3) + 2 * (is >> 2))) & 3);
   return lo | (hi << 4);
 }
 
@@ -208,9 +219,9 @@ __device__ __forceinline__ void dq8_q3_k(const uint8_t* __restrict__ w, int64_t 
   const uint8_t* blk = w + (e0 >> 8) * 110;
   const int r = (int)(e0 & 255);
   const int n = r >> 7, j = (r >> 5) & 3, l0 = r & 31;
-  const h16 dl = ld_h(blk + 108) * (h16)(q3k_scale(blk + 96, r >> 4) - 32);
   const uint2 q = ld<uint2>(blk + 32 + 32 * n + l0);
   const uint2 hm = ld<uint2>(blk + l0);
+  const h16 dl = ld_h(blk + 108) * (h16)(q3k_scale(blk + 96, r >> 4) - 32);
   const int hb = 4 * n + j;
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
@@ -226,14 +237,14 @@ __device__ __forceinline__ void dq8_q5_k(const uint8_t* __restrict__ w, int64_t 
   const int r = (int)(e0 & 255);
   const int j = r >> 5, pos = r & 31;
   const uint4 hdr = *(const uint4*)blk;  // 176-byte blocks keep 16-byte alignment
+  const uint2 q = *(const uint2*)(blk + 48 + 32 * (j >> 1) + pos);
+  const uint2 qh = *(const uint2*)(blk + 16 + pos);
   const h16 dall = __builtin_bit_cast(h16, (uint16_t)(hdr.x & 0xFFFF));
   const h16 dmin = __builtin_bit_cast(h16, (uint16_t)(hdr.x >> 16));
   int sc, mn;
   scale_min_k4(hdr.y, hdr.z, hdr.w, j, sc, mn);
   const h16 d1 = dall * (h16)sc;
   const h16 m1 = dmin * (h16)mn;
-  const uint2 q = *(const uint2*)(blk + 48 + 32 * (j >> 1) + pos);
-  const uint2 qh = *(const uint2*)(blk + 16 + pos);
   const int sh = (j & 1) ? 4 : 0;
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
@@ -365,11 +376,9 @@ __device__ __forceinline__ void dq8_iq4_nl(const uint8_t* __restrict__ w, int64_
   const float d = ld_f16(blk);
   const uint2 q = ld<uint2>(blk + 2 + (pos & 15));
   const int sh = pos >> 4 ? 4 : 0;
+  const int v0 = kvalues_iq4nl4((q.x >> sh) & 0x0F0F0F0Fu), v1 = kvalues_iq4nl4((q.y >> sh) & 0x0F0F0F0Fu);
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const uint32_t word = i < 4 ? q.x : q.y;
-    o[i] = d * (float)k_kvalues_iq4nl[(word >> (8 * (i & 3) + sh)) & 0xF];
-  }
+  for (int i = 0; i < 8; ++i) o[i] = d * (float)(int8_t)((i < 4 ? v0 : v1) >> (8 * (i & 3)));
 }
 
 template <typename OutT>
