@@ -93,7 +93,9 @@ int gguf_mmq(const void* W, const void* x, int xdtype, void* q8_workspace, void*
  *   GGUF_MMQ_HALF  half-precision MFMA on operands that carry their scales (activation d8*q and weight d*q, each
  *                  rounded to half): two to three times faster, relative deviation about 2e-4 in the l2 norm, below
  *                  the rounding of a half or bfloat16 result.  Not for fp32 results; not for Q4_1 / Q5_1.
- *   GGUF_MMQ_AUTO  HALF where it applies, INT8 otherwise.
+ *   GGUF_MMQ_AUTO  HALF where it applies, INT8 otherwise; with M <= 8 the streaming GEMV kernel instead, switched to
+ *                  this operator's offset sums (Q4_K, Q5_K, Q5_0 are the formats where the reference's GEMV and its
+ *                  tile GEMM form them differently), which is exact in int8 and reads W once at the GEMV's rate.
  * workspace_bytes is the size of q8_workspace; 0 stands for the minimum, M * gguf_q8_1_row_bytes(K).  Given
  * gguf_mmq_workspace_bytes(M, N, K) bytes, the half engine splits K over several workgroups per output tile when the
  * output alone has too few tiles to occupy the chip (few tokens or a narrow N with a long K), keeping fp32 partial
@@ -151,8 +153,11 @@ int gguf_moe_vec(const void* X, int xdtype, void* q8_workspace, const void* W, c
  * gguf_moe_vec_act also takes the number of experts in W (0 = unknown) and the size of the workspace (0 = the
  * minimum, tokens * gguf_q8_1_row_bytes(K)).  When tokens*top_k >= 2*num_experts and the workspace has room for the
  * routing sort as well -- gguf_moe_vec_workspace_bytes() -- the pairs are sorted by expert, the activations quantized
- * once, and four pairs of an expert share each pass over its weights, so a shared expert is read about once per call
- * rather than once per pair (the reference's grid re-reads it per pair, moe_vec.cuh:3-53).  Same results either way. */
+ * once, and the pairs of an expert share each pass over its weights, so a shared expert is read about once per call
+ * rather than once per pair (the reference's grid re-reads it per pair, moe_vec.cuh:3-53): 32 pairs per pass on the
+ * grouped int8-MFMA kernel for the formats that have tiles (up to 256 experts; Q5_0 excepted), four per pass on the
+ * vector kernel for the others.  The operator's arithmetic is the GEMV's on every route (Q4_K / Q5_K offsets from the
+ * quant sums); results agree to fp32 summation order. */
 int64_t gguf_moe_vec_workspace_bytes(int64_t tokens, int64_t top_k, int64_t K, int64_t num_experts);
 int gguf_moe_mmq_act(const void* X, int xdtype, void* q8_workspace, const void* W, int64_t expert_stride_bytes,
                      const int32_t* sorted_token_ids, const int32_t* expert_ids, const int32_t* num_tokens_post_padded,
