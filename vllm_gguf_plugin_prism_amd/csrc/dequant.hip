@@ -391,10 +391,9 @@ __device__ __forceinline__ void store8(OutT* __restrict__ y, const OutT (&v)[8])
   }
 }
 
-// eight dense values of packed elements [e0, e0 + 8) of `w`, stored at `dst`
+// eight dense values of packed elements [e0, e0 + 8) of `w`
 template <int TYPE, typename OutT>
-__device__ __forceinline__ void dequant8(const uint8_t* __restrict__ w, int64_t e0, OutT* __restrict__ dst) {
-  alignas(16) OutT out[8];
+__device__ __forceinline__ void dequant8_values(const uint8_t* __restrict__ w, int64_t e0, OutT (&out)[8]) {
   constexpr bool F32_MATH = TYPE == T_IQ4_XS || TYPE == T_IQ2_XXS || TYPE == T_IQ2_XS || TYPE == T_IQ2_S || TYPE == T_IQ3_XXS ||
                             TYPE == T_IQ3_S || TYPE == T_IQ1_S || TYPE == T_IQ1_M || TYPE == T_IQ4_NL;
   if constexpr (F32_MATH) {
@@ -425,14 +424,28 @@ __device__ __forceinline__ void dequant8(const uint8_t* __restrict__ w, int64_t 
 #pragma unroll
     for (int i = 0; i < 8; ++i) out[i] = from_half<OutT>(h[i]);
   }
+}
+
+// the same, stored at `dst`
+template <int TYPE, typename OutT>
+__device__ __forceinline__ void dequant8(const uint8_t* __restrict__ w, int64_t e0, OutT* __restrict__ dst) {
+  alignas(16) OutT out[8];
+  dequant8_values<TYPE, OutT>(w, e0, out);
   store8<OutT>(dst, out);
 }
 
+// A workgroup covers 4096 consecutive elements; every thread produces two groups of eight, 2048 elements apart, and
+// decodes both before it stores either, so that the loads of the two groups (and, for the codebook formats, their
+// dependent table lookups) are in flight together.  Groups past the end are computed on the last group and not stored.
 template <int TYPE, typename OutT>
 __global__ __launch_bounds__(256) void dequant_kernel(const uint8_t* __restrict__ w, OutT* __restrict__ y, int64_t nelem) {
-  const int64_t e0 = ((int64_t)blockIdx.x * 256 + threadIdx.x) * 8;
-  if (e0 >= nelem) return;
-  dequant8<TYPE, OutT>(w, e0, y + e0);
+  const int64_t e0 = (int64_t)blockIdx.x * 4096 + threadIdx.x * 8, e1 = e0 + 2048;
+  const int64_t last = nelem - 8;
+  alignas(16) OutT a[8], b[8];
+  dequant8_values<TYPE, OutT>(w, e0 < last ? e0 : last, a);
+  dequant8_values<TYPE, OutT>(w, e1 < last ? e1 : last, b);
+  if (e0 < nelem) store8<OutT>(y + e0, a);
+  if (e1 < nelem) store8<OutT>(y + e1, b);
 }
 
 // Row gather fused with dequantisation: Y[i, :] = dense(W[ids[i], :]).  A row whose id is outside [0, n_rows) is
@@ -456,8 +469,7 @@ __global__ __launch_bounds__(256) void dequant_rows_kernel(const uint8_t* __rest
 
 template <int TYPE>
 static int launch_dequant(const void* w, void* y, int ydtype, int64_t nelem, hipStream_t stream) {
-  const int64_t threads = nelem / 8;
-  const unsigned grid = (unsigned)((threads + 255) / 256);
+  const unsigned grid = (unsigned)((nelem + 4095) / 4096);
   GGUF_DISPATCH_DTYPE(ydtype, hipLaunchKernelGGL((dequant_kernel<TYPE, scalar_t>), dim3(grid), dim3(256), 0, stream,
                                                  (const uint8_t*)w, (scalar_t*)y, nelem));
   return launch_status();
