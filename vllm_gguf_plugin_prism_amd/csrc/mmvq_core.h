@@ -230,7 +230,7 @@ template <> struct TileSums<FmtQ5_0> { static constexpr bool swaps = true; };
 template <> struct TileSums<FmtQ4_K> { static constexpr bool swaps = true; };
 template <> struct TileSums<FmtQ5_K> { static constexpr bool swaps = true; };
 
-template <class F, int MT, int NW, int D, typename T, bool TILE = false>
+template <class F, int MT, int NW, int D, typename T, bool TILE = false, bool FULL = true>
 __global__ __launch_bounds__(64 * NW) void mmvq_stream_kernel(const uint8_t* __restrict__ W, const T* __restrict__ X,
                                                                T* __restrict__ Y, int N, int K, int rows_per_wg, int64_t w_pitch,
                                                                int64_t ldy, const T* __restrict__ bias, int m_act) {
@@ -280,7 +280,10 @@ __global__ __launch_bounds__(64 * NW) void mmvq_stream_kernel(const uint8_t* __r
   // wait for the weight loads behind them.  Groups past the end are clamped and their stores predicated.
   constexpr int NT = 64 * NW;
   const int g8 = K >> 3;
-  const int qtotal = m_act * g8;  // a multiple of 4, so quads stay whole; rows m_act .. MT-1 of the tile are never stored
+  // FULL: all MT rows of the tile exist (m_act == MT), known at compile time.  Otherwise rows m_act .. MT-1 are
+  // computed on whatever the LDS holds and never stored.
+  const int rows_x = FULL ? MT : m_act;
+  const int qtotal = rows_x * g8;  // a multiple of 4, so quads stay whole
   typename F::Regs pre[D];
   auto quantize_group = [&](const raw8<T>& raw, int q) {
     const int qc = min(q, qtotal - 1);
@@ -370,7 +373,7 @@ __global__ __launch_bounds__(64 * NW) void mmvq_stream_kernel(const uint8_t* __r
     const int row = i / MT, m = i - row * MT;
     float v = 0.0f;
     for (int st = 0; st < S; ++st) v += part[(row * S + st) * MT + m];
-    if (m < m_act) Y[(int64_t)m * ldy + r_begin + row] = finish<T>(v, bias, r_begin + row);
+    if (FULL || m < m_act) Y[(int64_t)m * ldy + r_begin + row] = finish<T>(v, bias, r_begin + row);
   }
 }
 
@@ -385,11 +388,11 @@ static int num_cus() {
   return n;
 }
 
-template <class F, int MT, int D, typename T, bool TILE>
+template <class F, int MT, int D, typename T, bool TILE, bool FULL>
 static void launch_stream_d(const void* W, const T* X, T* Y, int N, int K, int rows_per_wg, int grid, size_t lds, const LinearArgs& la,
                             hipStream_t stream, int m_act) {
   constexpr int NW = GGUF_MMVQ_NW;
-  auto kern = mmvq_stream_kernel<F, MT, NW, D, T, TILE>;
+  auto kern = mmvq_stream_kernel<F, MT, NW, D, T, TILE, FULL>;
   static bool big_lds = false;
   if (lds > 64 * 1024 && !big_lds) {
     (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
@@ -416,12 +419,18 @@ static bool launch_stream(const void* W, const T* X, T* Y, int N, int K, hipStre
                      (size_t)rows_per_wg * S * MT * 4;
   if (lds > 150 * 1024) return false;
   const int per_wave = (rows_per_wg + slots - 1) / slots;  // rows each wave walks; the pipeline depth never exceeds it
-  if constexpr (MT <= 4) {
-    if (per_wave >= GGUF_MMVQ_DEPTH) { launch_stream_d<F, MT, GGUF_MMVQ_DEPTH, T, TILE>(W, X, Y, N, K, rows_per_wg, grid, lds, la, stream, m_act); return true; }
-    if (per_wave >= 2) { launch_stream_d<F, MT, 2, T, TILE>(W, X, Y, N, K, rows_per_wg, grid, lds, la, stream, m_act); return true; }
-  }
-  // eight activation rows in registers leave room for one weight row in flight per wave
-  launch_stream_d<F, MT, 1, T, TILE>(W, X, Y, N, K, rows_per_wg, grid, lds, la, stream, m_act);
+  const auto go = [&](auto full) {
+    constexpr bool FULL = decltype(full)::value;
+    if constexpr (MT <= 4) {
+      if (per_wave >= GGUF_MMVQ_DEPTH) { launch_stream_d<F, MT, GGUF_MMVQ_DEPTH, T, TILE, FULL>(W, X, Y, N, K, rows_per_wg, grid, lds, la, stream, m_act); return; }
+      if (per_wave >= 2) { launch_stream_d<F, MT, 2, T, TILE, FULL>(W, X, Y, N, K, rows_per_wg, grid, lds, la, stream, m_act); return; }
+    }
+    // eight activation rows in registers leave room for one weight row in flight per wave
+    launch_stream_d<F, MT, 1, T, TILE, FULL>(W, X, Y, N, K, rows_per_wg, grid, lds, la, stream, m_act);
+  };
+  if constexpr (MT <= 2) go(std::true_type{});   // the callers of the 1- and 2-row tiles always fill them
+  else if (m_act == MT) go(std::true_type{});
+  else go(std::false_type{});
   return true;
 }
 
