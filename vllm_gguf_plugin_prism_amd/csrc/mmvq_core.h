@@ -290,11 +290,7 @@ __global__ __launch_bounds__(64 * NW) void mmvq_stream_kernel(const uint8_t* __r
     const int m = qc / g8, j = qc - m * g8;
     float xv[8];
     raw.cvt(xv);
-#ifdef GGUF_DBG_NOQUANT
-    Q8Quad qq; qq.q = make_uint2(__builtin_bit_cast(uint32_t, xv[0]), __builtin_bit_cast(uint32_t, xv[7])); qq.d = xv[1]; qq.s = xv[2]; qq.du = xv[3];
-#else
     const Q8Quad qq = q8_1_quantize8(xv);
-#endif
     if (q < qtotal) {
       *(uint2*)(lq + (size_t)m * K + 8 * j) = qq.q;
       if ((j & 3) == 0) {
@@ -353,11 +349,7 @@ __global__ __launch_bounds__(64 * NW) void mmvq_stream_kernel(const uint8_t* __r
       float acc[MT];
 #pragma unroll
       for (int m = 0; m < MT; ++m) {
-#ifdef GGUF_DBG_NODOT
-        const float v = (float)(((const uint32_t*)&pre[d])[0] ^ ((const uint32_t*)&pre[d])[sizeof(typename F::Regs) / 4 - 1]);
-#else
         const float v = F::dot(pre[d], act[m], u);
-#endif
         acc[m] = lane_on ? v : 0.0f;
       }
       pre[d] = load_row(i + D);  // refill the slot: D - 1 other slots are still in flight
