@@ -277,3 +277,12 @@ def test_shard_operators_reject_bad_views():
         ops.ggml_mul_mat_a8(w, x, o.Q4_K, 64, bias=torch.zeros(64, dtype=torch.float32, device="cuda"))
     with pytest.raises(ValueError):
         ops.ggml_mul_mat_a8(w.t(), x, o.Q4_K, 64)
+    # packed blocks at an odd address or rows an odd number of bytes apart cannot be GGUF data
+    buf = torch.zeros(64 * 289 + 1, dtype=torch.uint8, device="cuda")
+    odd_base = buf[1:1 + 64 * 288].view(64, 288)
+    odd_pitch = buf[:64 * 289].view(64, 289)[:, :288]
+    for bad in (odd_base, odd_pitch):
+        with pytest.raises(ValueError):
+            ops.ggml_mul_mat_vec_a8(bad, x, o.Q4_K, 64)
+        with pytest.raises(ValueError):
+            ops.ggml_mul_mat_a8(bad, x, o.Q4_K, 64)

@@ -689,6 +689,7 @@ extern "C" int gguf_mmq_linear(const void* W, int64_t w_row_pitch_bytes, const v
   if (engine == GGUF_MMQ_HALF && xdtype == GGUF_DTYPE_F32) return GGUF_ERR_DTYPE;
   if (N == 0 || M == 0) return GGUF_OK;
   if (!W || !x || !q8_workspace || !Y) return GGUF_ERR_NULL;
+  if (((uintptr_t)W & 1) || (w_row_pitch_bytes & 1)) return GGUF_ERR_SHAPE;  // packed blocks sit at even addresses
   hipStream_t s = (hipStream_t)stream;
   if (engine == GGUF_MMQ_AUTO && M <= 8) {
     // a handful of rows: the streaming GEMV kernel with the tile kernels' offset sums reads W once at close to the

@@ -80,6 +80,8 @@ extern "C" int gguf_mmvq_linear(const void* W, int64_t w_row_pitch_bytes, const 
   if (xdtype < 0 || xdtype > 2) return GGUF_ERR_DTYPE;
   if (N == 0 || M == 0) return GGUF_OK;
   if (!W || !x || !q8_workspace || !Y) return GGUF_ERR_NULL;
+  // packed blocks sit at even addresses (every block size is even): the GEMV's block loads rely on it
+  if (((uintptr_t)W & 1) || (w_row_pitch_bytes & 1)) return GGUF_ERR_SHAPE;
   return mmvq_any(type, W, x, q8_workspace, Y, xdtype, N, K, M, (hipStream_t)stream, la);
 }
 
@@ -129,6 +131,7 @@ extern "C" int gguf_moe_vec_act(const void* X, int xdtype, void* q8_workspace, c
   if (xdtype < 0 || xdtype > 2) return GGUF_ERR_DTYPE;
   if (N == 0 || tokens == 0) return GGUF_OK;
   if (!X || !q8_workspace || !W || !topk_ids || !Y) return GGUF_ERR_NULL;
+  if ((uintptr_t)W & 1) return GGUF_ERR_SHAPE;  // packed blocks sit at even addresses
   hipStream_t s = (hipStream_t)stream;
   const int pairs = (int)(tokens * top_k);
   const int ne = num_experts > 0 && num_experts <= 1024 ? (int)num_experts : 0;
