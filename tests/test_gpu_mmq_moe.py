@@ -46,6 +46,26 @@ def test_mmq_matches_a8_oracle_fp32(qtype, m):
         assert err <= 1e-5, (o.TYPE_NAMES[qtype], m, n, k, err)
 
 
+@pytest.mark.parametrize("qtype", [o.Q4_0, o.Q5_0, o.Q5_1, o.Q8_0, o.Q2_K, o.Q3_K, o.Q4_K, o.Q5_K, o.Q6_K])
+def test_mmq_2048_tokens_as_the_reference_tests_them(qtype):
+    """The largest batch of the reference's test_mmq (tests/test_kernels.py:150-196: 7, 83, 128, 2048 tokens on
+    hidden sizes 256 and 1024), here against the a8 oracle instead of gguf-py: fp32 through the integer engine,
+    fp16 through the library's choice."""
+    ops = _ops()
+    rng = np.random.default_rng(480 + qtype)
+    m = 2048
+    for n, k in [(256, 1024), (1024, 256)]:
+        w = o.make_weights(rng, qtype, n, k)
+        wd = _dev(w)
+        xd, xv = _x(rng, m, k, "f32")
+        exp = o.mul_mat_a8(w, xv, qtype, n, "mmq")
+        assert o.rel_l2(ops.ggml_mul_mat_a8(wd, xd, qtype, n).cpu().numpy(), exp) <= 1e-5
+        xh, xhv = _x(rng, m, k, "f16")
+        y = ops.ggml_mul_mat_a8(wd, xh, qtype, n)
+        assert y.shape == (m, n) and y.dtype == torch.float16
+        assert o.rel_l2(y.float().cpu().numpy(), o.mul_mat_a8(w, xhv, qtype, n, "mmq")) <= 1e-3
+
+
 @pytest.mark.parametrize("dt", ["f32", "f16"])
 @pytest.mark.parametrize("qtype", MMQ_TYPES)
 def test_mmq_handful_of_rows_keeps_tile_semantics(qtype, dt):
