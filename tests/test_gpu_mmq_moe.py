@@ -315,6 +315,26 @@ def test_moe_grouped_matches_oracle(qtype, t, top_k, e):
     assert o.rel_l2(y2.cpu().numpy(), exp2) <= 1e-5
 
 
+@pytest.mark.parametrize("qtype", [o.Q4_0, o.Q4_K])
+@pytest.mark.parametrize("t,top_k", [(2048, 8), (83, 4)])
+def test_moe_256_experts_as_the_reference_tests_them(qtype, t, top_k):
+    """Expert count and token counts of the reference's test_moe (tests/test_kernels.py:313-361: 256 experts, top-4 and
+    top-8, up to 2048 tokens), both operators, on a narrower layer so that the fp64 oracle stays in seconds."""
+    ops = _ops()
+    rng = np.random.default_rng(760 + qtype + t)
+    e, n, k = 256, 128, 512
+    w = np.stack([o.make_weights(rng, qtype, n, k) for _ in range(e)])
+    wd = _dev(w)
+    xd, xv = _x(rng, t, k, "f32")
+    ids, _ = _routing(rng, t, e, top_k)
+    blk = ops.ggml_moe_get_block_size(qtype)
+    s, eids, npost = o.moe_align_block_size(ids, blk, e)
+    y = ops.ggml_moe_a8(xd, wd, _dev(s), _dev(eids), _dev(npost), qtype, n, top_k, t)
+    assert o.rel_l2(y.cpu().numpy(), o.moe_a8(xv, w, s, eids, npost, qtype, n, top_k, t, blk)) <= 1e-5
+    yv = ops.ggml_moe_a8_vec(xd, wd, _dev(ids), top_k, qtype, n, t)
+    assert o.rel_l2(yv.cpu().numpy(), o.moe_a8_vec(xv, w, ids, top_k, qtype, n, t)) <= 1e-5
+
+
 def test_moe_grouped_padding_and_bad_experts_write_nothing():
     ops = _ops()
     rng = np.random.default_rng(800)
