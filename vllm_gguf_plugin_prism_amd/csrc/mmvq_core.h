@@ -195,10 +195,10 @@ __global__ __launch_bounds__(256) void mmvq_kernel(const uint8_t* __restrict__ W
   }
 }
 
-// ------------------------------------------------------------------ streaming kernel (M <= 4)
+// ------------------------------------------------------------------ streaming kernel (M <= 8)
 // The decode case is one pass over a few tens of MB, i.e. a handful of HBM latencies long, so the
-// whole game is to have every weight byte requested in the first microsecond and nothing else on
-// the critical path.
+// whole game is to keep a steady, bounded stream of weight requests going from the first microsecond
+// and to have nothing else on the critical path.
 //   * One fat workgroup (NW waves) per CU owns a contiguous band of rows.  A row of K/32 units needs
 //     S = ceil(K/2048) waves; the workgroup runs NW/S rows side by side ("slots"), and a lane keeps
 //     the same unit column for its whole life.
@@ -212,8 +212,10 @@ __global__ __launch_bounds__(256) void mmvq_kernel(const uint8_t* __restrict__ W
 #ifndef GGUF_MMVQ_NW
 #define GGUF_MMVQ_NW 16
 #endif
+// D = 2: measured against 1, 3, 4, 5 and "every row at once" on 33 MB matrices, two row-loads in flight per wave
+// (32 per CU and lane column) give the highest rate; deeper pipelines lose bandwidth, they do not gain latency cover.
 #ifndef GGUF_MMVQ_DEPTH
-#define GGUF_MMVQ_DEPTH 4
+#define GGUF_MMVQ_DEPTH 2
 #endif
 #ifndef GGUF_MMVQ_WG_PER_CU
 #define GGUF_MMVQ_WG_PER_CU 1
@@ -415,7 +417,6 @@ static bool launch_stream(const void* W, const T* X, T* Y, int N, int K, hipStre
     constexpr bool FULL = decltype(full)::value;
     if constexpr (MT <= 4) {
       if (per_wave >= GGUF_MMVQ_DEPTH) { launch_stream_d<F, MT, GGUF_MMVQ_DEPTH, T, TILE, FULL>(W, X, Y, N, K, rows_per_wg, grid, lds, la, stream, m_act); return; }
-      if (per_wave >= 2) { launch_stream_d<F, MT, 2, T, TILE, FULL>(W, X, Y, N, K, rows_per_wg, grid, lds, la, stream, m_act); return; }
     }
     // eight activation rows in registers leave room for one weight row in flight per wave
     launch_stream_d<F, MT, 1, T, TILE, FULL>(W, X, Y, N, K, rows_per_wg, grid, lds, la, stream, m_act);
