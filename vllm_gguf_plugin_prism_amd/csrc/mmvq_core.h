@@ -382,10 +382,9 @@ static int num_cus() {
   return n;
 }
 
-template <class F, int MT, int D, typename T, bool TILE, bool FULL>
+template <class F, int MT, int D, typename T, bool TILE, bool FULL, int NW>
 static void launch_stream_d(const void* W, const T* X, T* Y, int N, int K, int rows_per_wg, int grid, size_t lds, const LinearArgs& la,
                             hipStream_t stream, int m_act) {
-  constexpr int NW = GGUF_MMVQ_NW;
   auto kern = mmvq_stream_kernel<F, MT, NW, D, T, TILE, FULL>;
   static bool big_lds = false;
   if (lds > 64 * 1024 && !big_lds) {
@@ -398,10 +397,9 @@ static void launch_stream_d(const void* W, const T* X, T* Y, int N, int K, int r
 
 // Returns false when the shape does not fit the streaming kernel (a row longer than NW waves, or activations
 // that do not fit in LDS); the caller then takes the workspace path.
-template <class F, int MT, typename T, bool TILE = false>
+template <class F, int MT, typename T, bool TILE = false, int NW = GGUF_MMVQ_NW>
 static bool launch_stream(const void* W, const T* X, T* Y, int N, int K, hipStream_t stream, const LinearArgs& la, int m_act = MT) {
   // m_act <= MT rows of X are there; the kernel computes MT and stores m_act
-  constexpr int NW = GGUF_MMVQ_NW;
   const int nb = K / 32, S = (nb + 63) / 64;
   if (S > NW) return false;
   const int slots = NW / S;
@@ -416,10 +414,10 @@ static bool launch_stream(const void* W, const T* X, T* Y, int N, int K, hipStre
   const auto go = [&](auto full) {
     constexpr bool FULL = decltype(full)::value;
     if constexpr (MT <= 4) {
-      if (per_wave >= GGUF_MMVQ_DEPTH) { launch_stream_d<F, MT, GGUF_MMVQ_DEPTH, T, TILE, FULL>(W, X, Y, N, K, rows_per_wg, grid, lds, la, stream, m_act); return; }
+      if (per_wave >= GGUF_MMVQ_DEPTH) { launch_stream_d<F, MT, GGUF_MMVQ_DEPTH, T, TILE, FULL, NW>(W, X, Y, N, K, rows_per_wg, grid, lds, la, stream, m_act); return; }
     }
     // eight activation rows in registers leave room for one weight row in flight per wave
-    launch_stream_d<F, MT, 1, T, TILE, FULL>(W, X, Y, N, K, rows_per_wg, grid, lds, la, stream, m_act);
+    launch_stream_d<F, MT, 1, T, TILE, FULL, NW>(W, X, Y, N, K, rows_per_wg, grid, lds, la, stream, m_act);
   };
   if constexpr (MT <= 2) go(std::true_type{});   // the callers of the 1- and 2-row tiles always fill them
   else if (m_act == MT) go(std::true_type{});
@@ -482,7 +480,10 @@ static int mmvq_typed(const void* W, const void* x, void* ws, void* Y, int xdtyp
   if (M <= MAX_FUSED_M) {
     const T* xs = (const T*)x;
     bool ok;
-    if (M == 1) ok = launch_stream<F, 1, T>(W, xs, (T*)Y, (int)N, (int)K, stream, la);
+    // A small matrix (a row fits two waves, at most 16 rows per CU) is over in a few microseconds, much of it the
+    // dispatch of the workgroups: half as many waves, each walking twice the rows, start and finish sooner.
+    if (M == 1 && K <= 4096 && N <= 16 * num_cus()) ok = launch_stream<F, 1, T, false, 8>(W, xs, (T*)Y, (int)N, (int)K, stream, la);
+    else if (M == 1) ok = launch_stream<F, 1, T>(W, xs, (T*)Y, (int)N, (int)K, stream, la);
     else if (M == 2) ok = launch_stream<F, 2, T>(W, xs, (T*)Y, (int)N, (int)K, stream, la);
     else if (M <= 4) ok = launch_stream<F, 4, T>(W, xs, (T*)Y, (int)N, (int)K, stream, la, (int)M);
     else ok = launch_stream<F, 8, T>(W, xs, (T*)Y, (int)N, (int)K, stream, la, (int)M);
