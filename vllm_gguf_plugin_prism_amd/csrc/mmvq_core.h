@@ -221,6 +221,57 @@ __global__ __launch_bounds__(256) void mmvq_kernel(const uint8_t* __restrict__ W
 #define GGUF_MMVQ_WG_PER_CU 1
 #endif
 
+// MT per-lane values -> the sum over this lane's row of 16 lanes of value number (lane mod MT), in every lane.
+// Exchange step k pairs lanes 2^k apart: a lane keeps the half of its values whose class bit k equals its own lane
+// bit and adds the partner's copy of the same values.  The order of additions is fixed by the lane numbers.
+template <int CTRL>
+__device__ __forceinline__ float dpp_f(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
+}
+template <int MT>
+__device__ __forceinline__ float rows16_sums(const float (&a)[MT], int lane) {
+  constexpr int XOR1 = 0xB1, XOR2 = 0x4E, ROR4 = 0x124, ROR8 = 0x128, ROR12 = 0x12C;
+  float v;
+  if constexpr (MT == 1) {
+    v = a[0];
+    v += dpp_f<XOR1>(v);
+    v += dpp_f<XOR2>(v);
+    v += dpp_f<ROR4>(v);
+  } else {
+    const bool b0 = lane & 1;
+    float k[MT / 2];
+#pragma unroll
+    for (int p = 0; p < MT / 2; ++p) {          // classes 2p and 2p+1
+      const float keep = b0 ? a[2 * p + 1] : a[2 * p], give = b0 ? a[2 * p] : a[2 * p + 1];
+      k[p] = keep + dpp_f<XOR1>(give);
+    }
+    if constexpr (MT == 2) {
+      v = k[0] + dpp_f<XOR2>(k[0]);
+      v += dpp_f<ROR4>(v);
+    } else {
+      const bool b1 = lane & 2;
+      float q[MT / 4];
+#pragma unroll
+      for (int p = 0; p < MT / 4; ++p) {        // classes 4p + (lane & 1) and 4p + 2 + (lane & 1)
+        const float keep = b1 ? k[2 * p + 1] : k[2 * p], give = b1 ? k[2 * p] : k[2 * p + 1];
+        q[p] = keep + dpp_f<XOR2>(give);
+      }
+      if constexpr (MT == 4) {
+        v = q[0] + dpp_f<ROR4>(q[0]);
+      } else {
+        static_assert(MT == 8, "tiles of 1, 2, 4 or 8 rows");
+        const bool b2 = lane & 4;
+        const float keep = b2 ? q[1] : q[0], give = b2 ? q[0] : q[1];
+        // the partner four lanes away: below for lanes with bit 2 set, above for the others
+        const float down = dpp_f<ROR4>(give), up = dpp_f<ROR12>(give);
+        v = keep + (b2 ? down : up);
+      }
+    }
+  }
+  v += dpp_f<ROR8>(v);
+  return v;
+}
+
 // The reference's GEMV and its tile GEMM (ggml_mul_mat_a8) differ in three formats, and only in which per-block sum
 // of the activations meets the offset: Q4_K / Q5_K multiply their mins by d8*sum(q) in the GEMV (vecdotq.cuh:328-351,
 // 384-441) and by the stored sum of the unquantized values in the tiles (:369-372, :1325-1415); Q5_0 subtracts
@@ -246,7 +297,7 @@ __global__ __launch_bounds__(64 * NW) void mmvq_stream_kernel(const uint8_t* __r
   float* ldv = (float*)(smem + (size_t)MT * K);  // [MT][nb]
   float* lav = ldv + MT * nb;                  // [MT][nb]
   char* tab = (char*)(lav + (F::AUX != AUX_NONE ? MT * nb : 0));
-  float* part = (float*)(tab + F::TABLE_BYTES);  // [rows_per_wg][S][MT]
+  float* part = (float*)(tab + F::TABLE_BYTES);  // [rows_per_wg][S][4 rows of 16 lanes][MT]
 
   const int r_begin = blockIdx.x * rows_per_wg;
   const int r_end = min(N, r_begin + rows_per_wg);
@@ -355,18 +406,19 @@ __global__ __launch_bounds__(64 * NW) void mmvq_stream_kernel(const uint8_t* __r
         acc[m] = lane_on ? v : 0.0f;
       }
       pre[d] = load_row(i + D);  // refill the slot: D - 1 other slots are still in flight
-#pragma unroll
-      for (int m = 0; m < MT; ++m) {
-        const float v = wave_sum(acc[m]);
-        if (lane == 0 && row_ok) part[((slot + slots * i) * S + step) * MT + m] = v;
-      }
+      // The MT sums over the wave are formed together: after log2(MT) exchange steps in which a lane keeps the value
+      // of the class (lane mod MT) it belongs to and hands the other to its partner, one value per lane is left to
+      // add up over lanes of equal class, instead of MT values over all lanes.  Rotations by 4 and 8 inside a row of 16
+      // lanes finish that; the four rows of the wave leave their totals in LDS for the adder below.
+      const float v = rows16_sums<MT>(acc, lane);
+      if ((lane & 15) < MT && row_ok) part[(((slot + slots * i) * S + step) * 4 + (lane >> 4)) * MT + (lane & 15)] = v;
     }
   }
   __syncthreads();
   for (int i = tid; i < nrows * MT; i += 64 * NW) {
     const int row = i / MT, m = i - row * MT;
     float v = 0.0f;
-    for (int st = 0; st < S; ++st) v += part[(row * S + st) * MT + m];
+    for (int st = 0; st < 4 * S; ++st) v += part[(row * 4 * S + st) * MT + m];
     if (FULL || m < m_act) Y[(int64_t)m * ldy + r_begin + row] = finish<T>(v, bias, r_begin + row);
   }
 }
@@ -388,7 +440,7 @@ static void launch_stream_d(const void* W, const T* X, T* Y, int N, int K, int r
   auto kern = mmvq_stream_kernel<F, MT, NW, D, T, TILE, FULL>;
   static bool big_lds = false;
   if (lds > 64 * 1024 && !big_lds) {
-    (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 150 * 1024);
+    (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
     big_lds = true;
   }
   hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * NW), lds, stream, (const uint8_t*)W, X, Y, N, K, rows_per_wg,
@@ -408,8 +460,8 @@ static bool launch_stream(const void* W, const T* X, T* Y, int N, int K, hipStre
   if (rows_per_wg < slots) rows_per_wg = slots;  // at least one row per slot
   const int grid = (N + rows_per_wg - 1) / rows_per_wg;
   const size_t lds = (size_t)MT * K + (size_t)MT * nb * 4 * (F::AUX != AUX_NONE ? 2 : 1) + F::TABLE_BYTES +
-                     (size_t)rows_per_wg * S * MT * 4;
-  if (lds > 150 * 1024) return false;
+                     (size_t)rows_per_wg * S * 4 * MT * 4;
+  if (lds > 160 * 1024) return false;
   const int per_wave = (rows_per_wg + slots - 1) / slots;  // rows each wave walks; the pipeline depth never exceeds it
   const auto go = [&](auto full) {
     constexpr bool FULL = decltype(full)::value;
