@@ -225,8 +225,8 @@ def test_mmq_half_engine_splits_the_last_round():
     assert float(err.max()) <= 1.5e-3 and float((y.double() - ref).norm() / ref.norm()) <= 6e-4
     ws = torch.empty(m * _lib.lib().gguf_q8_1_row_bytes(k), dtype=torch.uint8, device="cuda")
     y_plain = torch.empty_like(y, dtype=torch.float16)
-    rc = _lib.lib().gguf_mmq(w.data_ptr(), xd.data_ptr(), 1, ws.data_ptr(), y_plain.data_ptr(), o.Q6_K, n, k, m,
-                             torch.cuda.current_stream().cuda_stream)
+    rc = _lib.lib().gguf_mmq_engine(w.data_ptr(), xd.data_ptr(), 1, ws.data_ptr(), y_plain.data_ptr(), o.Q6_K, n, k, m,
+                                    ops.MMQ_ENGINES["half"], ws.numel(), torch.cuda.current_stream().cuda_stream)
     assert rc == 0
     assert float((y_plain.double() - y.double()).norm() / ref.norm()) <= 4e-4
 

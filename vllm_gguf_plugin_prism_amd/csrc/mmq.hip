@@ -661,6 +661,11 @@ int mmq_half(const void* W, const void* ws, void* Y, int dtype, int type, int M,
 bool mmq_half_supported(int type);
 int64_t mmq_half_partial_bytes(int M, int N, int K);
 
+// mmq_i.hip
+int mmq_int(const void* W, const void* ws, void* Y, int dtype, int type, int M, int N, int K, float* partial,
+            int64_t partial_bytes, hipStream_t s, const LinearArgs& la);
+int64_t mmq_int_partial_bytes(int M, int N, int K);
+
 }  // namespace gguf
 
 // bytes of the quantized rows and their half-precision copy, rounded up so that what follows is aligned
@@ -668,7 +673,8 @@ static int64_t mmq_rows_bytes(int64_t M, int64_t K) { return (M * (gguf::q8_row_
 
 extern "C" int64_t gguf_mmq_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   if (M <= 0 || N <= 0 || K <= 0 || M > 0x7FFFFFF0LL || N > 0x7FFFFFF0LL || K > 0x7FFFFFF0LL) return 0;
-  return mmq_rows_bytes(M, K) + gguf::mmq_half_partial_bytes((int)M, (int)N, (int)K);
+  const int64_t ph = gguf::mmq_half_partial_bytes((int)M, (int)N, (int)K), pi = gguf::mmq_int_partial_bytes((int)M, (int)N, (int)K);
+  return mmq_rows_bytes(M, K) + (ph > pi ? ph : pi);
 }
 
 extern "C" int gguf_mmq_linear(const void* W, int64_t w_row_pitch_bytes, const void* x, int xdtype, void* q8_workspace, void* Y,
@@ -699,17 +705,19 @@ extern "C" int gguf_mmq_linear(const void* W, int64_t w_row_pitch_bytes, const v
     const int rc = mmvq_any(type, W, x, q8_workspace, Y, xdtype, N, K, M, s, lt);
     if (rc != GGUF_NOT_TAKEN) return rc;
   }
-  if (engine == GGUF_MMQ_AUTO) engine = (xdtype != GGUF_DTYPE_F32 && mmq_half_supported(type)) ? GGUF_MMQ_HALF : GGUF_MMQ_INT8;
+  if (engine == GGUF_MMQ_AUTO) engine = GGUF_MMQ_INT8;   // the reference's arithmetic; the half engine is for callers that ask
+  float* partial = (float*)((char*)q8_workspace + mmq_rows_bytes(M, K));
+  const int64_t partial_bytes = workspace_bytes > mmq_rows_bytes(M, K) ? workspace_bytes - mmq_rows_bytes(M, K) : 0;
   if (engine == GGUF_MMQ_HALF) {
     void* half_plane = (char*)q8_workspace + M * q8_row_bytes(K);
     const int rc = quantize_q8_1(x, xdtype, q8_workspace, M, K, s, 0, half_plane);
     if (rc != GGUF_OK) return rc;
-    float* partial = (float*)((char*)q8_workspace + mmq_rows_bytes(M, K));
-    const int64_t partial_bytes = workspace_bytes > mmq_rows_bytes(M, K) ? workspace_bytes - mmq_rows_bytes(M, K) : 0;
     return mmq_half(W, q8_workspace, Y, xdtype, type, (int)M, (int)N, (int)K, partial, partial_bytes, s, la);
   }
-  const int rc = quantize_q8_1(x, xdtype, q8_workspace, M, K, s);
+  int rc = quantize_q8_1(x, xdtype, q8_workspace, M, K, s);
   if (rc != GGUF_OK) return rc;
+  rc = mmq_int(W, q8_workspace, Y, xdtype, type, (int)M, (int)N, (int)K, partial, partial_bytes, s, la);
+  if (rc != GGUF_NOT_TAKEN) return rc;
   switch (type) {
     case T_Q4_0: return mmq_fmt<MQ4_0>(W, q8_workspace, Y, xdtype, (int)M, (int)N, (int)K, s, la);
     case T_Q4_1: return mmq_fmt<MQ4_1>(W, q8_workspace, Y, xdtype, (int)M, (int)N, (int)K, s, la);
