@@ -39,6 +39,7 @@ extern "C" {
 #define GGUF_ERR_SHAPE (-3)  /* K not a multiple of the block size, negative size, ... */
 #define GGUF_ERR_NULL (-4)   /* required pointer is null */
 #define GGUF_ERR_LAUNCH (-5) /* hipLaunchKernel reported an error */
+#define GGUF_ERR_WORKSPACE (-6) /* the call needs more workspace than the entry point has */
 
 typedef void* gguf_stream_t; /* a hipStream_t */
 
@@ -106,6 +107,22 @@ int gguf_mmq(const void* W, const void* x, int xdtype, void* q8_workspace, void*
 int64_t gguf_mmq_workspace_bytes(int64_t M, int64_t N, int64_t K);
 int gguf_mmq_engine(const void* W, const void* x, int xdtype, void* q8_workspace, void* Y, int type, int64_t N, int64_t K,
                     int64_t M, int engine, int64_t workspace_bytes, gguf_stream_t stream);
+
+/* gguf_mmq without a workspace argument, for callers that cannot allocate device memory: code running under HIP graph
+ * capture, tight serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference (whose
+ * operator allocates its result and workspace through torch on every call, gguf_kernel.cu:228-231).  The quantized rows and, for
+ * shapes whose K is split, the fp32 partial tiles live in a fixed 32 MiB array of device memory that the library
+ * holds on every GPU it runs on until the process ends; the call allocates and frees nothing.  Arithmetic, engine
+ * choice and results are those of gguf_mmq_engine(..., GGUF_MMQ_AUTO, workspace_bytes) given the same room for
+ * partial tiles.  GGUF_ERR_WORKSPACE if the quantized rows alone, M * roundup(K, 512) / 32 * 44 bytes rounded up to
+ * 256, exceed the array.  Every call on a GPU uses that GPU's one array: calls that overlap on one GPU (two
+ * streams, two threads) race; calls on one stream are ordered and need no clearing between them.
+ * gguf_mmq_static_capacity returns the array's size (0 if the current device cannot be queried) and, as its side
+ * effect, looks up the array's address for the current device; callers that are about to capture call it once
+ * before they begin, so that the first gguf_mmq_static inside the capture does no set-up. */
+int64_t gguf_mmq_static_capacity(void);
+int gguf_mmq_static(const void* W, const void* x, int xdtype, void* Y, int type, int64_t N, int64_t K, int64_t M,
+                    gguf_stream_t stream);
 
 /* The two a8 operators for one shard of a merged linear layer.  quantization/linear.py:229-262 keeps the shards of a
  * fused layer (q/k/v, gate/up) in one uint8 tensor padded to the widest row; when their ggml types differ it copies

@@ -35,7 +35,7 @@ def handle():
 
 def test_header_declares_the_bound_entry_points():
     assert declared_symbols() == sorted(_lib.EXPORTS)
-    assert len(declared_symbols()) == 23
+    assert len(declared_symbols()) == 25
 
 
 def test_every_declared_symbol_is_exported(handle):

@@ -14,6 +14,7 @@ ERRORS = {
     -3: "bad shape (K must be a positive multiple of the block size; sizes must be non-negative)",
     -4: "null pointer",
     -5: "kernel launch failed",
+    -6: "the call needs more workspace than this entry point has",
 }
 
 _lib = None
@@ -38,6 +39,9 @@ _SIGNATURES = {
     "gguf_mmq_linear": (_c.c_int, [_c.c_void_p, _c.c_int64, _c.c_void_p, _c.c_int, _c.c_void_p, _c.c_void_p, _c.c_int64,
                                    _c.c_void_p, _c.c_int, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int, _c.c_int64, _c.c_void_p]),
     "gguf_mmq_workspace_bytes": (_c.c_int64, [_c.c_int64, _c.c_int64, _c.c_int64]),
+    "gguf_mmq_static_capacity": (_c.c_int64, []),
+    "gguf_mmq_static": (_c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_int, _c.c_void_p, _c.c_int, _c.c_int64, _c.c_int64, _c.c_int64,
+                                   _c.c_void_p]),
     "gguf_mmq_engine": (_c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_int, _c.c_void_p, _c.c_void_p, _c.c_int, _c.c_int64,
                                    _c.c_int64, _c.c_int64, _c.c_int, _c.c_int64, _c.c_void_p]),
     "gguf_dequant_gemm": (_c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_int, _c.c_void_p, _c.c_void_p, _c.c_int, _c.c_int64,

@@ -677,9 +677,25 @@ extern "C" int64_t gguf_mmq_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   return mmq_rows_bytes(M, K) + (ph > pi ? ph : pi);
 }
 
+// gguf_mmq_linear with the size of the workspace's row region given by the caller: rows_bytes < 0 stands for the public
+// layout (quantized rows, then room for their half-precision copy); the entry point that brings its own workspace
+// keeps the quantized rows only and never runs the half engine.
+namespace gguf {
+int mmq_linear_impl(const void* W, int64_t w_row_pitch_bytes, const void* x, int xdtype, void* q8_workspace, void* Y,
+                    int64_t y_row_pitch, const void* bias, int type, int64_t N, int64_t K, int64_t M, int engine,
+                    int64_t workspace_bytes, int64_t rows_bytes, gguf_stream_t stream);
+}
+
 extern "C" int gguf_mmq_linear(const void* W, int64_t w_row_pitch_bytes, const void* x, int xdtype, void* q8_workspace, void* Y,
                                int64_t y_row_pitch, const void* bias, int type, int64_t N, int64_t K, int64_t M, int engine,
                                int64_t workspace_bytes, gguf_stream_t stream) {
+  return gguf::mmq_linear_impl(W, w_row_pitch_bytes, x, xdtype, q8_workspace, Y, y_row_pitch, bias, type, N, K, M, engine,
+                               workspace_bytes, -1, stream);
+}
+
+int gguf::mmq_linear_impl(const void* W, int64_t w_row_pitch_bytes, const void* x, int xdtype, void* q8_workspace, void* Y,
+                          int64_t y_row_pitch, const void* bias, int type, int64_t N, int64_t K, int64_t M, int engine,
+                          int64_t workspace_bytes, int64_t rows_bytes, gguf_stream_t stream) {
   using namespace gguf;
   const int qk = block_elems(type);
   if (qk == 0 || !mmq_type_ok(type)) return GGUF_ERR_TYPE;
@@ -706,8 +722,10 @@ extern "C" int gguf_mmq_linear(const void* W, int64_t w_row_pitch_bytes, const v
     if (rc != GGUF_NOT_TAKEN) return rc;
   }
   if (engine == GGUF_MMQ_AUTO) engine = GGUF_MMQ_INT8;   // the reference's arithmetic; the half engine is for callers that ask
-  float* partial = (float*)((char*)q8_workspace + mmq_rows_bytes(M, K));
-  const int64_t partial_bytes = workspace_bytes > mmq_rows_bytes(M, K) ? workspace_bytes - mmq_rows_bytes(M, K) : 0;
+  if (rows_bytes < 0) rows_bytes = mmq_rows_bytes(M, K);
+  else if (engine == GGUF_MMQ_HALF) return GGUF_ERR_SHAPE;   // no room for the half-precision rows in this layout
+  float* partial = (float*)((char*)q8_workspace + rows_bytes);
+  const int64_t partial_bytes = workspace_bytes > rows_bytes ? workspace_bytes - rows_bytes : 0;
   if (engine == GGUF_MMQ_HALF) {
     void* half_plane = (char*)q8_workspace + M * q8_row_bytes(K);
     const int rc = quantize_q8_1(x, xdtype, q8_workspace, M, K, s, 0, half_plane);
