@@ -173,6 +173,75 @@ def _other_configs(rng, dev):
     return res
 
 
+def _probes(rng, dev):
+    """What one launch can reach on this machine before any arithmetic, and where the GEMV kernel's time goes.
+
+    Prints a text report (the profiles/ summaries are made from it).  Uses libgguf_probes.so: plain streaming reads by
+    launch geometry over rotating matrix-sized buffers in one HIP graph, and the library's streaming GEMV kernel built
+    with its phase trace on."""
+    import ctypes
+
+    import torch
+
+    from vllm_gguf_plugin_prism_amd import build as _build, synth
+
+    if not _build.PROBES_LIB.exists():
+        raise RuntimeError(f"{_build.PROBES_LIB} is missing: python -m vllm_gguf_plugin_prism_amd.build")
+    h = ctypes.CDLL(str(_build.PROBES_LIB))
+    vp, i64, ci = ctypes.c_void_p, ctypes.c_int64, ctypes.c_int
+    h.gguf_probe_read.argtypes = [vp, i64, ci, ci, ci, ci, vp, vp]
+    h.gguf_probe_mmvq_q4_k.argtypes = [vp, vp, vp, i64, i64, vp]
+    h.gguf_probe_mmvq_trace.argtypes = [vp, ci]
+    stream = lambda: torch.cuda.current_stream().cuda_stream  # noqa: E731
+    sink = torch.zeros(4, dtype=torch.int32, device=dev)
+
+    print("== plain streaming read of one matrix-sized buffer per launch, 20 distinct buffers per HIP graph (660 MB walked)")
+    print("   (a launch reads the buffer once, 16 bytes per lane and load; best of 3 graph replays)")
+    for nbytes in (33030144, 9437184):
+        bufs = [torch.full((nbytes,), i + 1, dtype=torch.uint8, device=dev) for i in range(20)]
+        rows = []
+        for threads, per_cu in ((256, 1), (256, 2), (256, 4), (256, 8), (256, 32), (512, 1), (512, 2), (512, 4), (1024, 1), (1024, 2)):
+            for unroll in (2, 4, 8):
+                for nt in (0, 1):
+                    def call(i, threads=threads, per_cu=per_cu, unroll=unroll, nt=nt):
+                        rc = h.gguf_probe_read(bufs[i % 20].data_ptr(), nbytes, threads, 256 * per_cu, unroll, nt, sink.data_ptr(), stream())
+                        assert rc == 0
+                    ms = min(_graph_ms(call, 20, 1) for _ in range(3))
+                    rows.append((ms * 1e3, threads, per_cu, unroll, nt))
+        rows.sort()
+        print(f"-- {nbytes / 1e6:.1f} MB per launch: fastest and slowest geometries of {len(rows)}")
+        for us, threads, per_cu, unroll, nt in rows[:6] + rows[-2:]:
+            print(f"   {us:6.2f} us  {nbytes / us / 1e6:5.2f} TB/s  ({100 * nbytes / us / 1e6 / 8.0:4.1f} % of 8 TB/s)  {threads:4d} threads x {per_cu:2d} workgroups per CU, "
+                  f"{unroll} loads in flight per lane, {'non-temporal' if nt else 'plain'} loads")
+        del bufs
+
+    print("== streaming GEMV kernel, Q4_K batch 1 fp16: wall-clock times of five points, microseconds after the first wave")
+    print("   of the launch entered (median over workgroups; first wave / last wave of a workgroup); 10 ns clock")
+    for n, k in CFG2_SHAPES:
+        ws = [torch.from_numpy(np.concatenate([synth.make_weights(rng, Q4_K, min(2048, n - r), k) for r in range(0, n, 2048)], axis=0)).to(dev)]
+        ws += [ws[0].clone() for _ in range(int(700e6 // ws[0].numel()))]
+        x = torch.from_numpy(rng.standard_normal((1, k)).astype(np.float32)).to(torch.float16).to(dev)
+        y = torch.empty((1, n), dtype=torch.float16, device=dev)
+        acc = []
+        for rep in range(len(ws) * 2):
+            rc = h.gguf_probe_mmvq_q4_k(ws[rep % len(ws)].data_ptr(), x.data_ptr(), y.data_ptr(), n, k, stream())
+            assert rc == 0
+            torch.cuda.synchronize()
+            nwg = 256
+            buf = (ctypes.c_ulonglong * (nwg * 16))()
+            assert h.gguf_probe_mmvq_trace(buf, nwg) == 0
+            t = np.frombuffer(buf, dtype=np.uint64).reshape(nwg, 2, 8)[:, :, :5].astype(np.int64)
+            if rep >= len(ws):          # the first pass over the copies warms code and page tables up
+                acc.append((t - t[:, :, 0].min()) * 0.01)
+        t = np.median(np.stack(acc), axis=0)          # [workgroup][first/last wave][point], median over launches
+        names = ("entered", "own activations quantized", "all activations in LDS", "own rows walked", "results stored")
+        print(f"-- [{n},{k}], {n * (k // 256) * 144 / 1e6:.1f} MB")
+        for p, name in enumerate(names):
+            a, b = np.median(t[:, 0, p]), np.median(t[:, 1, p])
+            print(f"   {name:28s} {a:6.2f} / {b:6.2f}   (latest workgroup {t[:, :, p].max():6.2f})")
+        del ws
+
+
 def main() -> int:
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -186,6 +255,9 @@ def main() -> int:
     ap.add_argument("--profile", action="store_true",
                     help="counter-collection mode: eager launches only (no HIP graph), no CPU leg, M=512 only for "
                          "the MMQ leg, and one 256 MiB device copy at the end to calibrate byte counters")
+    ap.add_argument("--probes", action="store_true",
+                    help="print the measurement probes instead of the benchmark line: the plain-read ceiling of one launch "
+                         "by geometry, and the phase timeline of the streaming GEMV kernel")
     args = ap.parse_args()
     if args.profile:
         args.no_cpu = True
@@ -203,6 +275,9 @@ def main() -> int:
         return 3
     dev = torch.device("cuda:0")
     rng = np.random.default_rng(0)
+    if args.probes:
+        _probes(rng, dev)
+        return 0
 
     # ---------------------------------------------------------------- config 2: Q4_K batch-1 GEMV
     mats = []

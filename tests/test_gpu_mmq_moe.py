@@ -284,6 +284,36 @@ def test_config3_q6_k_qwen_mlp_slices(m):
         assert o.rel_l2(y, o.mul_mat_a8(w, xv, o.Q6_K, n, "mmq")) <= 1e-3
 
 
+@pytest.mark.parametrize("engine", ["auto", "half"])
+@pytest.mark.parametrize("m", [128, 512, 2048])
+@pytest.mark.parametrize("n,k", [(18944, 3584), (3584, 18944)])
+def test_config3_q6_k_full_size(n, k, m, engine):
+    """Config 3 at its real shapes, with the tile plans the benchmark times: whole tiles, the tiles of a sparse last
+    round split along K ([18944,3584] at M = 512: rows from 16384 on; at M = 2048: rows from 18432 on) and outputs
+    with too few tiles for the chip, every tile split ([3584,18944]).  The fp64 oracle checks a sample of weight rows
+    over all token rows, chosen to fall into each of those groups; doubling the activations must double every result
+    exactly, which looks at the whole output."""
+    from vllm_gguf_plugin_prism_amd import synth
+    ops = _ops()
+    rng = np.random.default_rng(31 + m + n)
+    w = synth.random_blocks(rng, o.Q6_K, n, k)       # raw valid blocks, d ~ U(1e-4, 1e-2): a numpy quantizer at this size takes a minute
+    x = rng.standard_normal((m, k)).astype(np.float16)
+    wd, xd = _dev(w), torch.from_numpy(x).cuda()
+    y = ops.ggml_mul_mat_a8(wd, xd, o.Q6_K, n, engine=engine)
+    assert y.shape == (m, n) and y.dtype == torch.float16
+    marks = [0, 64, 16384 - 32, 16384, 18432 - 32, 18432]
+    rows = np.unique(np.concatenate([np.arange(a, a + 40) for a in marks if a + 40 <= n] + [np.arange(n - 70, n), rng.integers(0, n, 24)]))
+    want = o.mul_mat_a8(w[rows], x.astype(np.float32), o.Q6_K, len(rows), "mmq")
+    assert o.rel_l2(y[:, torch.from_numpy(rows).cuda()].float().cpu().numpy(), want) <= 1e-3
+    y2 = ops.ggml_mul_mat_a8(wd, xd * 2, o.Q6_K, n, engine=engine)
+    if engine == "auto":
+        normal = y.abs() >= 2.0 ** -13          # a result in the half subnormals has fewer bits than its double
+        assert torch.equal(y2[normal], (y * 2)[normal])
+        assert o.rel_l2(y2.float().cpu().numpy(), 2 * y.float().cpu().numpy()) <= 1e-6
+    else:   # the half engine rounds d8 * q to half: doubling keeps that exact too, short of overflow
+        assert o.rel_l2(y2.float().cpu().numpy(), 2 * y.float().cpu().numpy()) <= 1e-3
+
+
 def _routing(rng, t, e, top_k):
     logits = rng.standard_normal((t, e)).astype(np.float32)
     ids = np.argsort(-logits, axis=1)[:, :top_k].astype(np.int32)

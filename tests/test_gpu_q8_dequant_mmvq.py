@@ -82,7 +82,7 @@ def test_dequantize_default_dtype_and_shape_label():
 
 
 @pytest.mark.parametrize("qtype", ALL)
-@pytest.mark.parametrize("m", [1, 2, 3, 5, 8, 11])
+@pytest.mark.parametrize("m", [1, 2, 3, 5, 8, 9, 10, 11, 16])   # past eight rows: passes of eight, then 1, 2, 3 rows or none
 def test_mmvq_matches_a8_oracle(qtype, m):
     ops = _ops()
     rng = np.random.default_rng(200 + qtype * 16 + m)
@@ -148,6 +148,24 @@ def test_config2_q4_k_full_size(shape):
     y1 = ops.ggml_mul_mat_vec_a8(wd, xa, o.Q4_K, n).float()
     y2 = ops.ggml_mul_mat_vec_a8(wd, (xa * 2).to(torch.float16), o.Q4_K, n).float()
     assert o.rel_l2(y2.cpu().numpy(), 2 * y1.cpu().numpy()) <= 2e-3
+
+
+@pytest.mark.parametrize("shape", [(4096, 4096), (14336, 4096), (4096, 14336)])
+@pytest.mark.parametrize("m", [4, 8])
+def test_config2_q4_k_full_size_batch_4_and_8(shape, m):
+    """The batch sweep of config 2 at its real shapes through the reference's dispatch policy (linear.py:38-49): batch 4
+    on the 4096-row matrices is a GEMV, everything else here goes to ggml_mul_mat_a8, whose offset term uses the stored
+    block sums.  The oracle follows the path the policy names."""
+    from vllm_gguf_plugin_prism_amd import dispatch as D
+    n, k = shape
+    rng = np.random.default_rng(21 + m)
+    w = o.make_weights(rng, o.Q4_K, n, k)
+    xd, xv = _x(rng, m, k, "f16")
+    path = D.select_mul_mat_path(o.Q4_K, m, n)
+    assert path == ("mmvq" if (n <= 5120 and m <= 6) else "mmq")
+    y = D.fused_mul_mat_gguf(xd, _to_dev(w), o.Q4_K)
+    assert y.shape == (m, n) and y.dtype == torch.float16
+    assert o.rel_l2(y.float().cpu().numpy(), o.mul_mat_a8(w, xv, o.Q4_K, n, path)) <= 1e-3
 
 
 def test_empty_and_errors():

@@ -15,6 +15,8 @@ from pathlib import Path
 PKG = Path(__file__).resolve().parent
 CSRC = PKG / "csrc"
 LIB = PKG / "libgguf_hip.so"
+PROBES_SRC = CSRC / "probes" / "probes.hip"      # measurement probes for bench.py, a library of their own
+PROBES_LIB = PKG / "libgguf_probes.so"
 HIPCC = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
 FLAGS = [
     "--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC",
@@ -51,6 +53,14 @@ def build(verbose: bool = True) -> Path:
     if res.returncode != 0:
         raise RuntimeError("link failed:\n" + res.stderr)
     os.replace(tmp, LIB)
+    probes_obj = objdir / "probes.o"
+    _compile(PROBES_SRC, probes_obj)
+    tmp = PROBES_LIB.with_suffix(".so.tmp")
+    cmd = [HIPCC, "--offload-arch=gfx950", "-shared", "-fPIC", str(probes_obj), "-o", str(tmp)]
+    res = subprocess.run(cmd, capture_output=True, text=True)
+    if res.returncode != 0:
+        raise RuntimeError("link of the probe library failed:\n" + res.stderr)
+    os.replace(tmp, PROBES_LIB)
     if verbose:
         print(f"built {LIB} from {len(srcs)} sources", file=sys.stderr)
     return LIB

@@ -283,6 +283,19 @@ template <> struct TileSums<FmtQ5_0> { static constexpr bool swaps = true; };
 template <> struct TileSums<FmtQ4_K> { static constexpr bool swaps = true; };
 template <> struct TileSums<FmtQ5_K> { static constexpr bool swaps = true; };
 
+// Profiling builds (the probe library only) record when the first and the last wave of every workgroup pass five
+// points of the kernel, on the 100 MHz wall clock that all CUs share.
+#ifdef GGUF_TRACE_PHASES
+__device__ unsigned long long g_mmvq_phases[1024 * 2 * 8];
+#define GGUF_PHASE(i)                                                                                 \
+  do {                                                                                                \
+    if ((tid & 63) == 0 && (wave == 0 || wave == NW - 1) && blockIdx.x < 1024)                        \
+      g_mmvq_phases[(blockIdx.x * 2 + (wave ? 1 : 0)) * 8 + (i)] = __builtin_amdgcn_s_memrealtime(); \
+  } while (0)
+#else
+#define GGUF_PHASE(i) do {} while (0)
+#endif
+
 template <class F, int MT, int NW, int D, typename T, bool TILE = false, bool FULL = true>
 __global__ __launch_bounds__(64 * NW) void mmvq_stream_kernel(const uint8_t* __restrict__ W, const T* __restrict__ X,
                                                                T* __restrict__ Y, int N, int K, int rows_per_wg, int64_t w_pitch,
@@ -290,6 +303,7 @@ __global__ __launch_bounds__(64 * NW) void mmvq_stream_kernel(const uint8_t* __r
   extern __shared__ __align__(16) char smem[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: row arithmetic stays on the scalar unit
+  GGUF_PHASE(0);                               // entry
   const int nb = K >> 5;                       // 32-weight units per row
   const int S = (nb + 63) >> 6;                // waves per row
   const int slots = NW / S;                    // rows in flight side by side (>= 1, checked by the host)
@@ -356,7 +370,13 @@ __global__ __launch_bounds__(64 * NW) void mmvq_stream_kernel(const uint8_t* __r
   };
   auto prologue = [&](auto qg_tag) {
     constexpr int QG = decltype(qg_tag)::value;
-    raw8<T> xraw[QG];
+    if constexpr (QG == 0) {   // a wave with no activation values to quantize: its weights only
+      if (qtotal <= NT) __builtin_amdgcn_s_barrier();   // (see below: the others' activation requests go first)
+#pragma unroll
+      for (int d = 0; d < D; ++d) pre[d] = load_row(d);
+      return;
+    }
+    raw8<T> xraw[QG > 0 ? QG : 1];
 #pragma unroll
     for (int g = 0; g < QG; ++g) {
       const int qc = min(tid + g * NT, qtotal - 1);
@@ -364,13 +384,23 @@ __global__ __launch_bounds__(64 * NW) void mmvq_stream_kernel(const uint8_t* __r
       xraw[g].load(X + (int64_t)m * K + 8 * j);
     }
     __builtin_amdgcn_sched_barrier(0);
+    if constexpr (QG == 1) {
+      // One request per thread covers the activations: hold every wave's weight requests back until all of those
+      // are out.  The memory pipeline serves a CU's requests in order, and a late wave's activation request would
+      // otherwise wait behind the weight requests of the waves that started before it, and the barrier below with it.
+      __builtin_amdgcn_s_barrier();
+      __builtin_amdgcn_sched_barrier(0);
+    }
 #pragma unroll
     for (int d = 0; d < D; ++d) pre[d] = load_row(d);
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int g = 0; g < QG; ++g) quantize_group(xraw[g], tid + g * NT);
   };
-  if (qtotal <= NT) prologue(std::integral_constant<int, 1>{});
+  // (wave-uniform: a wave whose first lane is past the last group takes no part in the quantisation and reaches the
+  // barrier as soon as its weight requests are out, instead of after a load and a quantisation nobody uses)
+  if (wave * 64 >= qtotal) prologue(std::integral_constant<int, 0>{});
+  else if (qtotal <= NT) prologue(std::integral_constant<int, 1>{});
   else if (qtotal <= 2 * NT) prologue(std::integral_constant<int, 2>{});
   else prologue(std::integral_constant<int, 4>{});
   for (int q = tid + 4 * NT; q - tid < qtotal; q += NT) {  // uniform trip count; only for K * MT > 32 * NT
@@ -380,7 +410,9 @@ __global__ __launch_bounds__(64 * NW) void mmvq_stream_kernel(const uint8_t* __r
     r.load(X + (int64_t)m2 * K + 8 * j2);
     quantize_group(r, q);
   }
+  GGUF_PHASE(1);                               // own share of the activations quantized
   __syncthreads();
+  GGUF_PHASE(2);                               // every wave's share is in LDS
 
   // this lane's column of every activation vector, held in registers for the whole row loop
   typename F::ActRegs act[MT];
@@ -414,6 +446,7 @@ __global__ __launch_bounds__(64 * NW) void mmvq_stream_kernel(const uint8_t* __r
       if ((lane & 15) < MT && row_ok) part[(((slot + slots * i) * S + step) * 4 + (lane >> 4)) * MT + (lane & 15)] = v;
     }
   }
+  GGUF_PHASE(3);                               // own rows walked
   __syncthreads();
   for (int i = tid; i < nrows * MT; i += 64 * NW) {
     const int row = i / MT, m = i - row * MT;
@@ -421,6 +454,7 @@ __global__ __launch_bounds__(64 * NW) void mmvq_stream_kernel(const uint8_t* __r
     for (int st = 0; st < 4 * S; ++st) v += part[(row * 4 * S + st) * MT + m];
     if (FULL || m < m_act) Y[(int64_t)m * ldy + r_begin + row] = finish<T>(v, bias, r_begin + row);
   }
+  GGUF_PHASE(4);                               // results stored
 }
 
 static int num_cus() {
