@@ -11,19 +11,21 @@ included), rotating over distinct weight copies that together exceed the 256 MB
 Infinity Cache, with every input resident in HBM before the clock starts.
 
 Beside it:
-  roofline      the GEMV kernel against the 8 TB/s HBM peak, timed per launch with HIP events
-  mmq           the second half of the metric: Q6_K prefill GEMM at M=512 (BASELINE config 3) in TOPS
-                against the 5.03 POPS dense int8 MFMA peak the metric names, with its own roofline.
-                gguf_mmq's default engine for half results multiplies on half-precision MFMA
-                (2.5 PFLOP/s peak, also reported); the int8-MFMA engine is timed beside it
+  roofline      the GEMV kernel against the 8 TB/s HBM peak, timed per launch with HIP events over at least 100 launches
+  mmq           the second half of the metric: Q6_K prefill GEMM at M=512 (BASELINE config 3) in TOPS against the
+                5.03 POPS dense int8 MFMA peak, on the operator's default engine: exact int8 dot products on
+                v_mfma_i32_32x32x32_i8 with fp32 block scales, the reference's arithmetic.  The opt-in engine that
+                multiplies dequantized operands on half-precision MFMA is timed beside it as ``half_engine``
+  other_configs the remaining BASELINE configurations (1: Q8_0 small, 2: batch sweep, 4: codebook formats, 5: MoE layer)
   cpu_baseline  the reference's CPU path (block dequantize + fp32 matmul) restated in numpy/torch,
-                timed on this host's cores on a bounded sample of the same workload
+                timed on one host core on a bounded sample of the same workload
 """
 from __future__ import annotations
 
 import argparse
 import json
 import os
+import re
 import sys
 import time
 
@@ -34,17 +36,25 @@ sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
 INT8_PEAK_TOPS = 5033.0        # dense int8 MFMA, K=32/64 shapes (256 CU x 8192 op/clk x 2.4 GHz)
-INT8_LEGACY_PEAK_TOPS = 2516.0  # legacy K=16 shapes run at half that rate
 F16_PEAK_TFLOPS = 2516.0       # dense half-precision MFMA
 Q4_K, Q6_K = 12, 14
 CFG2_SHAPES = [(4096, 4096), (14336, 4096), (4096, 14336)]
 CFG3_SHAPES = [(18944, 3584), (3584, 18944)]
 ROTATE_BYTES = 640 << 20       # distinct weight bytes walked per rotation (> 2x the 256 MB cache)
-# HBM bytes per launch from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE runs of `bench.py --profile`, each counter scaled by
-# what it reads for a 256 MiB device copy (x2.000 and x1.000); summarised in profiles/bench_mmvq_q4_k_bs1_mmq_q6_k.txt.
-# Counters cannot be read from inside this process, so these are constants of the measured build, not live values.
-TRAFFIC_MMVQ_Q4_K_14336x4096 = 33.37e6 + 0.02e6
-TRAFFIC_MMQ_Q6_K_M512 = {"18944x3584": 159.7e6 + 48.2e6, "3584x18944": 272.9e6 + 29.4e6}  # GEMM kernel of the half engine, read + written
+MIN_LAUNCHES = 100             # every reported per-launch time is an average over at least this many launches
+# HBM bytes per launch cannot be read from inside this process: they come from rocprofv3 --pmc FETCH_SIZE and WRITE_SIZE
+# runs of `bench.py --profile`, each counter scaled by what it reads for a 256 MiB device copy.  The summary of those runs
+# carries one `traffic_bytes_per_launch <key> = <bytes>` line per kernel; without the file the figure is null.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "pmc_hbm_traffic_mmvq_q4_k_mmq_q6_k.txt")
+
+
+def _traffic(key):
+    try:
+        text = open(TRAFFIC_FILE).read()
+    except OSError:
+        return None
+    m = re.search(rf"^traffic_bytes_per_launch\s+{re.escape(key)}\s*=\s*([0-9.eE+]+)", text, re.M)
+    return float(m.group(1)) if m else None
 
 
 def _events_ms(fn, iters):
@@ -86,20 +96,23 @@ def _graph_ms(fn, calls, replays):
     return start.elapsed_time(stop) / (replays * calls)
 
 
-def _timed_ms(fn, calls):
-    """Graph-timed milliseconds per call where the calls can be captured, event-timed otherwise."""
+def _timed_ms(fn, calls, eager=False):
+    """Milliseconds per call over at least MIN_LAUNCHES calls: graph-timed where the calls can be captured (and
+    ``eager`` is not asked for), event-timed otherwise."""
     import torch
 
-    try:
-        return _graph_ms(fn, calls, 5)
-    except Exception:  # a call that cannot be captured: time the eager launches
-        torch.cuda.synchronize()
-        for i in range(3):
-            fn(i)
-        return _events_ms(fn, calls * 5)
+    replays = -(-MIN_LAUNCHES // calls)
+    if not eager:
+        try:
+            return _graph_ms(fn, calls, replays)
+        except Exception:  # a call that cannot be captured: time the eager launches
+            torch.cuda.synchronize()
+    for i in range(3):
+        fn(i)
+    return _events_ms(fn, calls * replays)
 
 
-def _other_configs(rng, dev):
+def _other_configs(rng, dev, w_14336x4096):
     """The BASELINE configurations the headline does not cover, each as time per call and the rate its roofline names."""
     import torch
 
@@ -126,7 +139,7 @@ def _other_configs(rng, dev):
 
     # config 2: batch sweep on [14336,4096]; the reference's policy sends batch 4 and 8 at this N to the tile GEMM
     n, k = 14336, 4096
-    copies = [torch.from_numpy(np.concatenate([synth.make_weights(rng, Q4_K, 2048, k) for _ in range(n // 2048)])).to(dev)]
+    copies = [torch.from_numpy(w_14336x4096).to(dev)]
     copies += [copies[0].clone() for _ in range(19)]          # 20 x 33 MB, walked in turn
     for b in (1, 2, 4, 8):
         x = xs(b, k)
@@ -249,21 +262,21 @@ def main() -> int:
     ap.add_argument("--warmup", type=int, default=20)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-mmq", action="store_true", help="skip the Q6_K MMQ leg")
-    ap.add_argument("--all-configs", action="store_true",
-                    help="also time the other BASELINE configurations (1: Q8_0, 2: batch sweep, 4: i-quants, 5: MoE layer) "
-                         "into an 'other_configs' object; about a minute more")
+    ap.add_argument("--no-other", action="store_true",
+                    help="skip the other BASELINE configurations (1: Q8_0, 2: batch sweep, 4: i-quants, 5: MoE layer), "
+                         "which otherwise go into an 'other_configs' object (about half a minute)")
     ap.add_argument("--profile", action="store_true",
-                    help="counter-collection mode: eager launches only (no HIP graph), no CPU leg, M=512 only for "
-                         "the MMQ leg, and one 256 MiB device copy at the end to calibrate byte counters")
+                    help="counter-collection mode: eager launches only (no HIP graph), no CPU leg, no other configurations, "
+                         "M=512 only for the MMQ leg, and one 256 MiB device copy at the end to calibrate byte counters")
     ap.add_argument("--probes", action="store_true",
                     help="print the measurement probes instead of the benchmark line: the plain-read ceiling of one launch "
                          "by geometry, and the phase timeline of the streaming GEMV kernel")
     args = ap.parse_args()
     if args.profile:
-        args.no_cpu = True
+        args.no_cpu = args.no_other = True
     if args.gpus != 1:
         print("bench.py measures one GPU: this build has no multi-GPU path (the operators shard by "
-              "rows/columns of W with no communication; see DESIGN.md). Run with --gpus 1.", file=sys.stderr)
+              "rows/columns of W with no communication). Run with --gpus 1.", file=sys.stderr)
         return 2
 
     import torch
@@ -305,8 +318,10 @@ def main() -> int:
         step(i)
     torch.cuda.synchronize()
     eager_ms = (time.perf_counter() - t0) * 1e3 / args.steps
-    # the same K steps as one HIP graph: host launch cost out of the timed region
-    graph_ms = eager_ms if args.profile else _graph_ms(step, ncopies, max(1, args.steps // ncopies))
+    # the same steps as one HIP graph of a full rotation over the weight copies, replayed: host launch cost out of the
+    # timed region.  At least K steps and at least MIN_LAUNCHES kernel launches are timed whatever K is.
+    replays = max(-(-args.steps // ncopies), -(-MIN_LAUNCHES // (len(CFG2_SHAPES) * ncopies)))
+    graph_ms = eager_ms if args.profile else _graph_ms(step, ncopies, replays)
     ms_per_step = min(eager_ms, graph_ms)
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
 
@@ -314,64 +329,66 @@ def main() -> int:
     per_shape = {}
     for n, k, copies, x in mats:
         one = lambda i, n=n, copies=copies, x=x: ops.ggml_mul_mat_vec_a8(copies[i % ncopies], x, Q4_K, n)  # noqa: E731
-        ms = _events_ms(one, ncopies * 4) if args.profile else _graph_ms(one, ncopies * 4, 10)
+        ms = _timed_ms(one, ncopies * 4, eager=args.profile)
         b = n * (k // 256) * 144 + 2 * k + 2 * n
-        per_shape[f"{n}x{k}"] = {"us_per_call": ms * 1e3, "GBps": b / (ms * 1e-3) / 1e9, "bytes": b}
+        per_shape[f"{n}x{k}"] = {"us_per_call": ms * 1e3, "GBps": b / (ms * 1e-3) / 1e9, "bytes": b,
+                                 "launches_timed": ncopies * 4 * -(-MIN_LAUNCHES // (ncopies * 4))}
     big = per_shape["14336x4096"]
     roofline = {"bound": "hbm", "achieved": big["GBps"], "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                "frac": big["GBps"] / HBM_PEAK_GBS, "traffic": TRAFFIC_MMVQ_Q4_K_14336x4096,
+                "frac": big["GBps"] / HBM_PEAK_GBS, "traffic": _traffic("mmvq_q4_k_14336x4096_bs1"),
                 "algorithmic_bytes": big["bytes"],
-                "kernel": "mmvq Q4_K [14336,4096] bs1 (activation quantisation + GEMV per call)",
+                "kernel": "mmvq Q4_K [14336,4096] bs1 (one kernel per call: activation quantisation fused into the GEMV)",
                 "per_shape": per_shape}
 
     out = {
         "metric": "Q4_K GEMV HBM GB/s (% peak) @bs1; Q6_K MMQ int8 TOPS (% peak) @M=512",
         "value": value, "unit": "GB/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms_per_step, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "int8 dot products, fp32 accumulate, fp16 in/out", "data": "synthetic (seeded N(0,0.02) weights quantized to Q4_K, N(0,1) fp16 activations)",
+        "dtype": "int8 dot products, fp32 accumulate, fp16 in/out",
+        "data": "synthetic (seeded N(0,0.02) weights quantized to Q4_K, N(0,1) fp16 activations)",
         "config": {"workload": "BASELINE config 2: Q4_K batch-1 MMVQ over [4096,4096],[14336,4096],[4096,14336]",
                    "weight_copies_rotated": ncopies, "rotated_bytes": ncopies * total_copy_bytes,
                    "eager_ms_per_step": eager_ms, "graph_ms_per_step": graph_ms,
+                   "graph_steps_timed": 0 if args.profile else replays * ncopies,
                    "pct_of_hbm_peak": 100.0 * value / HBM_PEAK_GBS},
         "roofline": roofline,
     }
 
     # ---------------------------------------------------------------- config 3: Q6_K MMQ at M=512
     if not args.no_mmq:
-        mmq, mmq_int8 = {}, {}
+        tables = {"auto": {}, "half": {}}
         for n, k in CFG3_SHAPES:
             w = np.concatenate([synth.make_weights(rng, Q6_K, min(2048, n - r), k) for r in range(0, n, 2048)], axis=0)
             wd = torch.from_numpy(w).to(dev)
             for m in ((512,) if args.profile else (128, 512, 2048)):
                 x = torch.from_numpy(rng.standard_normal((m, k)).astype(np.float32)).to(torch.float16).to(dev)
-                for engine in (("auto",) if args.profile else ("auto", "int8")):
-                    for _ in range(3):
-                        ops.ggml_mul_mat_a8(wd, x, Q6_K, n, engine=engine)
-                    ms = _events_ms(lambda i: ops.ggml_mul_mat_a8(wd, x, Q6_K, n, engine=engine), 20)
+                for engine, table in tables.items():
+                    call = lambda i, engine=engine: ops.ggml_mul_mat_a8(wd, x, Q6_K, n, engine=engine)  # noqa: E731
+                    ms = _timed_ms(call, 20, eager=args.profile)
                     tops = 2.0 * m * n * k / (ms * 1e-3) / 1e12
-                    (mmq if engine == "auto" else mmq_int8)[f"{n}x{k}@M{m}"] = {
-                        "ms": ms, "TOPS": tops, "frac_int8_peak": tops / INT8_PEAK_TOPS}
+                    table[f"{n}x{k}@M{m}"] = {"ms": ms, "TOPS": tops, "frac_int8_peak": tops / INT8_PEAK_TOPS}
             del wd
         ops_total = sum(2.0 * 512 * n * k for n, k in CFG3_SHAPES)
 
         def at_m512(table):
             t_total = sum(v["ms"] for key, v in table.items() if key.endswith("@M512")) * 1e-3
-            return ops_total / t_total / 1e12 if t_total else None
+            return ops_total / t_total / 1e12
 
-        tops512 = at_m512(mmq)
+        tops512, half512 = at_m512(tables["auto"]), at_m512(tables["half"])
         out["mmq"] = {
             "metric": "Q6_K MMQ int8 TOPS @M=512", "value": tops512, "unit": "TOPS",
-            "engine": "half-precision MFMA on dequantized operands (gguf_mmq's choice for fp16 results)",
-            "dtype": "f16 products, f32 accumulation",
+            "engine": "gguf_mmq's default: exact int8 dot products on v_mfma_i32_32x32x32_i8, fp32 block scales",
+            "dtype": "int8 products, int32 sums per block, fp32 accumulation",
             "roofline": {"bound": "mfma", "achieved": tops512, "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
-                         "frac": tops512 / INT8_PEAK_TOPS, "traffic": TRAFFIC_MMQ_Q6_K_M512,
-                         "denominator": "5.03 POPS dense int8, the peak the metric names; the engine that runs issues "
-                                        f"v_mfma_f32_32x32x16_f16, whose own peak is {F16_PEAK_TFLOPS} TFLOP/s",
-                         "frac_of_f16_mfma_peak": tops512 / F16_PEAK_TFLOPS},
-            "per_shape": mmq,
-            "int8_engine": {"value": at_m512(mmq_int8), "unit": "TOPS", "per_shape": mmq_int8,
-                            "note": "engine='int8': the reference's integer arithmetic on v_mfma_i32_32x32x16_i8"},
-            "note": "time per call = activation quantisation kernel + GEMM kernel (+ the partial-sum kernel where K is split)",
+                         "frac": tops512 / INT8_PEAK_TOPS,
+                         "traffic": {f"{n}x{k}": _traffic(f"mmqi_q6_k_{n}x{k}_m512") for n, k in CFG3_SHAPES}},
+            "per_shape": tables["auto"],
+            "half_engine": {"value": half512, "unit": "TOPS", "frac_of_f16_mfma_peak": half512 / F16_PEAK_TFLOPS,
+                            "per_shape": tables["half"],
+                            "note": "engine='half', opt-in: dequantized operands on v_mfma_f32_32x32x16_f16; not the "
+                                    "reference's arithmetic (operands rounded to half), so not the headline"},
+            "note": "time per call = activation quantisation kernel + GEMM kernel (+ the partial-sum kernel where K is split), "
+                    "averaged over 100 calls",
         }
 
     # ---------------------------------------------------------------- CPU baseline (bounded sample)
@@ -381,6 +398,8 @@ def main() -> int:
         n, k = CFG2_SHAPES[0]
         w = host_w[(n, k)]
         x32 = torch.from_numpy(rng.standard_normal((1, k)).astype(np.float32))
+        threads_before = torch.get_num_threads()
+        torch.set_num_threads(1)           # numpy's block decode is one thread; the matmul leg is held to the same
         best = None
         t_end = time.perf_counter() + 20.0
         reps = 0
@@ -393,15 +412,16 @@ def main() -> int:
             if reps > 0 and (best is None or t2 - t0 < best[0]):
                 best = (t2 - t0, t1 - t0, t2 - t1)
             reps += 1
+        torch.set_num_threads(threads_before)
         qbytes = n * (k // 256) * 144
         out["cpu_baseline"] = {
-            "value": qbytes / best[0] / 1e9, "unit": "GB/s", "cores": torch.get_num_threads(), "kind": "port",
-            "sample": f"Q4_K [{n},{k}] batch 1: numpy fp32 block dequantize ({best[1] * 1e3:.1f} ms) + torch fp32 matmul "
-                      f"({best[2] * 1e3:.1f} ms), best of {reps - 1} after 1 warm-up; os.cpu_count()={os.cpu_count()}",
+            "value": qbytes / best[0] / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
+            "sample": f"Q4_K [{n},{k}] batch 1 on one thread: numpy fp32 block dequantize ({best[1] * 1e3:.1f} ms) + torch fp32 "
+                      f"matmul ({best[2] * 1e3:.1f} ms), best of {reps - 1} after 1 warm-up",
         }
 
-    if args.all_configs:
-        out["other_configs"] = _other_configs(rng, dev)
+    if not args.no_other:
+        out["other_configs"] = _other_configs(rng, dev, host_w[(14336, 4096)])
 
     if args.profile:
         # one plain device-to-device copy of known size: its FETCH_SIZE / WRITE_SIZE readings give the scale of

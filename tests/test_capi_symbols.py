@@ -79,3 +79,37 @@ def test_argument_validation_needs_no_gpu(handle):
     assert handle.gguf_mmvq(None, None, 1, None, None, 99, 16, 256, 1, None) == -1
     assert handle.gguf_mmvq(None, None, 1, None, None, 12, 16, 100, 1, None) == -3
     assert handle.gguf_mmq(None, None, 1, None, None, 23, 16, 256, 1, None) in (-1, -4)
+
+
+def _ctype_of(decl: str):
+    """ctypes class of one C parameter or return type as include/gguf_hip.h spells it."""
+    d = re.sub(r"\bconst\b", "", decl).strip()
+    if d.startswith("char") and "*" in d:
+        return ctypes.c_char_p
+    if "*" in d or d.startswith("gguf_stream_t"):
+        return ctypes.c_void_p            # every pointer, and the stream handle, crosses as an address
+    base = d.split()[0]
+    return {"int": ctypes.c_int, "int64_t": ctypes.c_int64, "void": None}[base]
+
+
+def declared_prototypes():
+    text = re.sub(r"/\*.*?\*/", "", HEADER.read_text(), flags=re.S)
+    text = re.sub(r"^\s*#.*$", "", text, flags=re.M)
+    protos = {}
+    for m in re.finditer(r"([A-Za-z_][A-Za-z0-9_ \*]*?)\b(gguf_[a-z0-9_]+)\s*\(([^)]*)\)\s*;", text):
+        ret, name, params = m.group(1).strip(), m.group(2), m.group(3).strip()
+        args = [] if params in ("", "void") else [_ctype_of(p) for p in params.split(",")]
+        protos[name] = (_ctype_of(ret), args)
+    return protos
+
+
+def test_ctypes_signatures_match_the_header_type_for_type():
+    """Argument count, order and width of every binding against the prototype it calls: an int passed where the
+    header says int64_t, or two arguments swapped between a pointer and a size, would corrupt the call frame the way
+    a surplus argument once did."""
+    protos = declared_prototypes()
+    assert sorted(protos) == sorted(_lib.EXPORTS)
+    for name, (res, args) in _lib._SIGNATURES.items():
+        want_res, want_args = protos[name]
+        assert res is want_res, (name, res, want_res)
+        assert list(args) == want_args, (name, [a.__name__ for a in args], [a.__name__ for a in want_args])

@@ -365,6 +365,35 @@ def test_moe_256_experts_as_the_reference_tests_them(qtype, t, top_k):
     assert o.rel_l2(yv.cpu().numpy(), o.moe_a8_vec(xv, w, ids, top_k, qtype, n, t)) <= 1e-5
 
 
+def test_more_than_256_experts_take_the_per_pair_operator():
+    """The grouped kernel keeps the reference's guard on expert ids (moe.cuh:33), so the wrapper refuses a tensor of
+    more than 256 experts and the layer-level dispatch sends such a layer to the per-pair operator, which has no
+    limit; the result must match the per-token definition of the layer."""
+    from vllm_gguf_plugin_prism_amd import dispatch as D
+    ops = _ops()
+    rng = np.random.default_rng(777)
+    e, n, k, t, top_k, qtype = 300, 64, 256, 70, 2, o.Q8_0
+    w = np.stack([o.make_weights(rng, qtype, n, k) for _ in range(e)])
+    xd, xv = _x(rng, t, k, "f32")
+    ids, wts = _routing(rng, t, e, top_k)
+    ids[0, 0] = 299                                    # an expert the grouped kernel would have dropped
+    ids[0, 1] = 3
+    blk = ops.ggml_moe_get_block_size(qtype)
+    s, eids, npost = o.moe_align_block_size(ids, blk, e)
+    with pytest.raises(NotImplementedError):
+        ops.ggml_moe_a8(xd, _dev(w), _dev(s), _dev(eids), _dev(npost), qtype, n, top_k, t)
+    yv = ops.ggml_moe_a8_vec(xd, _dev(w), _dev(ids), top_k, qtype, n, t)
+    assert o.rel_l2(yv.cpu().numpy(), o.moe_a8_vec(xv, w, ids, top_k, qtype, n, t)) <= 1e-5
+    assert D.select_moe_path(qtype, qtype, t) == "grouped"        # what the reference's policy says for 70 tokens
+    w2 = np.stack([o.make_weights(rng, qtype, k, n // 2) for _ in range(e)])
+    got = D.fused_moe_gguf(xd, _dev(w), _dev(w2), torch.from_numpy(wts).cuda(), _dev(ids), qtype, qtype, "silu")
+    h = o.moe_a8_vec(xv, w, ids, top_k, qtype, n, t)
+    a = o.silu_and_mul(h.astype(np.float64)).astype(np.float32)
+    y = o.moe_a8_vec(a, w2, ids.reshape(-1), 1, qtype, k, t * top_k).reshape(t, top_k, k)
+    want = (y * wts[:, :, None]).sum(1)
+    assert o.rel_l2(got.cpu().numpy(), want) <= 1e-4
+
+
 def test_moe_grouped_padding_and_bad_experts_write_nothing():
     ops = _ops()
     rng = np.random.default_rng(800)

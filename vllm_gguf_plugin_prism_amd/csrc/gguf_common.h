@@ -5,6 +5,8 @@
 #include <hip/hip_fp16.h>
 #include <stdint.h>
 
+#include <atomic>
+
 #include "../../include/gguf_hip.h"
 
 namespace gguf {
@@ -181,6 +183,33 @@ __device__ __forceinline__ T finish(float v, const T* bias, int64_t n) {
 // q8_1_device.h).  half_plane: if not null, also the dequantized rows in half precision, [M][q8_kp(K)].
 int quantize_q8_1(const void* x, int xdtype, void* ws, int64_t M, int64_t K, hipStream_t stream, int act = 0,
                   void* half_plane = nullptr);
+
+// Opt a kernel in to more than 64 KB of dynamic LDS, once per device: `done` is the caller's bit set of the devices
+// already served (one static per kernel instantiation).  The attribute belongs to the device the kernel's code object
+// is loaded on, so a second GPU in the same process needs its own call.
+template <typename K>
+static inline void allow_large_lds(K kern, size_t lds, std::atomic<uint64_t>& done) {
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev > 63) dev = 0;
+  const uint64_t bit = 1ull << dev;
+  if (done.load(std::memory_order_relaxed) & bit) return;
+  (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+  done.fetch_or(bit, std::memory_order_relaxed);
+}
+
+// compute units of the current device (asked once per device)
+static inline int num_cus() {
+  static std::atomic<int> cached[64];
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev > 63) dev = 0;
+  int n = cached[dev].load(std::memory_order_relaxed);
+  if (n == 0) {
+    hipDeviceProp_t prop;
+    n = hipGetDeviceProperties(&prop, dev) == hipSuccess && prop.multiProcessorCount > 0 ? prop.multiProcessorCount : 256;
+    cached[dev].store(n, std::memory_order_relaxed);
+  }
+  return n;
+}
 
 constexpr int GGUF_NOT_TAKEN = 1;  // internal: a route that declined the call (never returned through the C ABI)
 inline int launch_status() { return hipGetLastError() == hipSuccess ? GGUF_OK : GGUF_ERR_LAUNCH; }

@@ -150,22 +150,18 @@ struct MoeArgs {
 // MODE selects how staging and contraction overlap:
 //   MODE_PREFETCH  the next step's global loads are issued before this step's MFMA phase and held in registers;
 //   MODE_PLAIN     load, stage, contract in turn; latency is covered only by other workgroups on the CU;
-//   MODE_PINGPONG  the workgroup is two groups of WM*WN waves with private LDS tiles, side by side in N.  The
-//                  groups run half a period apart, separated by workgroup barriers: while one waits for its
-//                  global loads and unpacks them, the other runs its MFMA + rescale phase, so the vector ALU
-//                  (the bound of this kernel) always has a group to work for.
 //   MODE_KSPLIT    MODE_PLAIN with twice the waves: all of them stage the step together, then each half of the
 //                  workgroup contracts half of the step's 32-blocks for the same outputs, and the two partial tiles
 //                  are added through LDS at the end.  For shapes with too few output tiles to fill the chip.
-enum { MODE_PREFETCH = 0, MODE_PLAIN = 1, MODE_PINGPONG = 2, MODE_KSPLIT = 3 };
+enum { MODE_PREFETCH = 0, MODE_PLAIN = 1, MODE_KSPLIT = 3 };
 
 template <class F, int WM, int WN, int TM, int TN, int KS, int OCC, int MODE, typename T, bool MOE>
-__global__ __launch_bounds__(64 * WM * WN * (MODE == MODE_PINGPONG || MODE == MODE_KSPLIT ? 2 : 1), OCC) void mmq_kernel(const uint8_t* __restrict__ W, const char* __restrict__ ws,
+__global__ __launch_bounds__(64 * WM * WN * (MODE == MODE_KSPLIT ? 2 : 1), OCC) void mmq_kernel(const uint8_t* __restrict__ W, const char* __restrict__ ws,
                                                          T* __restrict__ Y, int M, int N, int K, int64_t ws_row_bytes,
                                                          MoeArgs moe, int64_t w_pitch, int64_t ldy, const T* __restrict__ bias) {
   constexpr int GW = WM * WN;            // waves that share one set of accumulators' tile
   constexpr int KW = MODE == MODE_KSPLIT ? 2 : 1;  // wave sets splitting the 32-blocks of a step
-  constexpr int NT = 64 * GW * KW;       // threads that stage one tile (the whole workgroup unless MODE_PINGPONG)
+  constexpr int NT = 64 * GW * KW;       // threads that stage one tile: the whole workgroup
   constexpr int KB = KS / 32;            // q8_1 blocks per step
   constexpr int GR = KS / 16;            // 16-byte granules per activation row and step
   constexpr int LDK = Pitch<F::G, KS>::value;
@@ -174,22 +170,20 @@ __global__ __launch_bounds__(64 * WM * WN * (MODE == MODE_PINGPONG || MODE == MO
   constexpr int AQ = (M_T * GR + NT - 1) / NT;  // activation granules per thread and step
   constexpr int AS = (M_T * KB + NT - 1) / NT;  // activation block scales per thread and step
   constexpr int WP = (N_T * KB + NT - 1) / NT;  // (weight row, 32-block) pairs per thread and step
-  static_assert(!(MOE && MODE == MODE_PINGPONG), "the grouped variant has no ping-pong form");
   extern __shared__ __align__(16) char smem[];
-  const int group = MODE == MODE_PINGPONG ? (int)threadIdx.x / NT : 0;  // wave-uniform
-  int8_t* xq = (int8_t*)smem + (size_t)group * mmq_group_lds_bytes<F, WM, WN, TM, TN, KS>();  // [M_T][LDK]
+  int8_t* xq = (int8_t*)smem;                       // [M_T][LDK]
   int8_t* wq = xq + M_T * LDK;                      // [N_T][LDK]
   float* xd = (float*)(wq + N_T * LDK);             // [KB][M_T]  q8_1 block scales
   float* xa = xd + KB * M_T;                        // [KB][M_T] q8_1 block sums (HAS_MIN), or [2*KB][M_T] quant sums (MIN16)
   float* wsc = xa + (!F::HAS_MIN ? 0 : F::MIN16 ? 2 * KB * M_T : KB * M_T);  // [NG][N_T]
   float* wmn = wsc + NG * N_T;                      // [KB][N_T]  (HAS_MIN)
 
-  const int tid = (int)threadIdx.x - group * NT, lane = tid & 63;  // indices inside the group
+  const int tid = (int)threadIdx.x, lane = tid & 63;
   const int kgrp = (tid >> 6) / GW, wave = (tid >> 6) % GW;         // wave-uniform
   const int wm = wave / WN, wn = wave % WN;
   constexpr int KB_MINE = (KS / 32) / KW;                            // 32-blocks of a step this wave contracts
   const int m_base = blockIdx.y * M_T;
-  const int n_base = MODE == MODE_PINGPONG ? (blockIdx.x * 2 + group) * N_T : blockIdx.x * N_T;
+  const int n_base = blockIdx.x * N_T;
   const int Kp = (int)q8_kp(K);
   const int64_t rowbytes = w_pitch;   // bytes between rows of W: the dense row size unless the caller's tensor is padded
   const int nkb_total = K >> 5;
@@ -198,7 +192,7 @@ __global__ __launch_bounds__(64 * WM * WN * (MODE == MODE_PINGPONG || MODE == MO
     static_assert(!MOE || M_T == 32, "one expert per 32 sorted slots");
     if (m_base >= moe.num_tokens_post_padded[0]) return;
     const int e = moe.expert_ids[blockIdx.y];
-    if (e < 0 || e > 255) return;
+    if (e < 0 || e > 255) return;   // the reference's guard (moe.cuh:33); callers with more experts are turned away in ops.py
     W += (int64_t)e * moe.expert_stride;
   }
 
@@ -456,24 +450,6 @@ __global__ __launch_bounds__(64 * WM * WN * (MODE == MODE_PINGPONG || MODE == MO
 #pragma unroll
           for (int r = 0; r < 16; ++r) acc[j][i][r] += red[(((wave * TM + j) * TN + i) * 16 + r) * 64 + lane];
     }
-  } else {
-    // phase p: group g stages step (p-g)/2 when p-g is even and contracts step (p-g-1)/2 when it is odd.  A group's
-    // tile is written and read only by that group, in alternating phases, so one barrier per phase orders both.
-    const int nsteps = (K + KS - 1) / KS;
-#pragma unroll 1
-    for (int p = 0; p <= 2 * nsteps; ++p) {
-      const int q = p - group;
-      if (q >= 0 && q < 2 * nsteps) {
-        if ((q & 1) == 0) {
-          fetch((q >> 1) * KS);
-          stash((q >> 1) * KS);
-        } else {
-#pragma unroll 1
-          for (int kb = 0; kb < KB; ++kb) contract(kb);
-        }
-      }
-      __syncthreads();
-    }
   }
 
   // ---- store: lane = one output feature, 16 token rows per tile
@@ -505,32 +481,21 @@ __global__ __launch_bounds__(64 * WM * WN * (MODE == MODE_PINGPONG || MODE == MO
 template <class F, int WM, int WN, int TM, int TN, int KS, int OCC, int MODE, typename T, bool MOE>
 static void launch_mmq(const void* W, const void* ws, void* Y, int M, int N, int K, int m_tiles, const MoeArgs& moe,
                        hipStream_t stream, const LinearArgs& la = LinearArgs()) {
-  constexpr int G = MODE == MODE_PINGPONG ? 2 : 1;
   constexpr int KW = MODE == MODE_KSPLIT ? 2 : 1;
-  constexpr int N_T = 32 * WN * TN * G;
-  constexpr size_t lds = mmq_group_lds_bytes<F, WM, WN, TM, TN, KS>() * G;
+  constexpr int N_T = 32 * WN * TN;
+  constexpr size_t lds = mmq_group_lds_bytes<F, WM, WN, TM, TN, KS>();
   static_assert(mmq_group_lds_bytes<F, WM, WN, TM, TN, KS>() % 16 == 0, "group tiles keep 16-byte alignment");
   auto kern = mmq_kernel<F, WM, WN, TM, TN, KS, OCC, MODE, T, MOE>;
   if constexpr (lds > 65536) {
-    static bool configured = false;  // opt in to > 64 KB of dynamic LDS once per instantiation
-    if (!configured) {
-      (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-      configured = true;
-    }
+    static std::atomic<uint64_t> done{0};
+    allow_large_lds(kern, lds, done);
   }
-  hipLaunchKernelGGL(kern, dim3((N + N_T - 1) / N_T, m_tiles), dim3(64 * WM * WN * G * KW), lds, stream, (const uint8_t*)W, (const char*)ws,
+  hipLaunchKernelGGL(kern, dim3((N + N_T - 1) / N_T, m_tiles), dim3(64 * WM * WN * KW), lds, stream, (const uint8_t*)W, (const char*)ws,
                      (T*)Y, M, N, K, q8_row_bytes(K), moe, la.w_pitch ? la.w_pitch : (int64_t)(K / F::QK) * F::BS,
                      la.ldy ? la.ldy : (int64_t)N, (const T*)la.bias);
 }
 
 
-#ifdef GGUF_MMQ_TUNE
-// tuning builds only: GGUF_MMQ_CFG in the environment forces one tile configuration (fp16 activations only)
-static int tune_cfg() {
-  static const int v = [] { const char* e = getenv("GGUF_MMQ_CFG"); return e ? atoi(e) : 0; }();
-  return v;
-}
-#endif
 
 // Tile choice.  The kernel is bound by vector-ALU issue, not by operand traffic, so small tiles cost little and what
 // matters is that every CU has several workgroups to overlap one group's load latency with another's arithmetic:
@@ -543,17 +508,6 @@ template <class F, typename T>
 static int mmq_typed(const void* W, const void* ws, void* Y, int M, int N, int K, hipStream_t stream, const LinearArgs& la) {
   MoeArgs none = {};
   const int64_t large_tiles = (int64_t)((M + 127) / 128) * ((N + 127) / 128);
-#ifdef GGUF_MMQ_TUNE
-  switch (tune_cfg()) {
-    case 1: launch_mmq<F, 4, 1, 1, 2, 128, 4, MODE_PINGPONG, T, false>(W, ws, Y, M, N, K, (M + 127) / 128, none, stream, la); return launch_status();
-    case 3: launch_mmq<F, 2, 1, 1, 1, 128, 4, MODE_PINGPONG, T, false>(W, ws, Y, M, N, K, (M + 63) / 64, none, stream, la); return launch_status();
-    case 5: launch_mmq<F, 4, 2, 1, 2, 128, 4, MODE_PLAIN, T, false>(W, ws, Y, M, N, K, (M + 127) / 128, none, stream, la); return launch_status();
-    case 6: launch_mmq<F, 2, 2, 1, 1, 128, 4, MODE_PLAIN, T, false>(W, ws, Y, M, N, K, (M + 63) / 64, none, stream, la); return launch_status();
-    case 9: launch_mmq<F, 2, 2, 1, 1, 128, 4, MODE_KSPLIT, T, false>(W, ws, Y, M, N, K, (M + 63) / 64, none, stream, la); return launch_status();
-    case 8: launch_mmq<F, 4, 2, 1, 2, 128, 4, MODE_PREFETCH, T, false>(W, ws, Y, M, N, K, (M + 127) / 128, none, stream, la); return launch_status();
-    default: break;
-  }
-#endif
   const int64_t small_tiles = (int64_t)((M + 63) / 64) * ((N + 63) / 64);
   if (large_tiles >= 400) {
     constexpr int MODE = F::LIGHT ? MODE_PREFETCH : MODE_PLAIN;
@@ -568,13 +522,8 @@ static int mmq_typed(const void* W, const void* ws, void* Y, int M, int N, int K
 
 template <class F>
 static int mmq_fmt(const void* W, const void* ws, void* Y, int dtype, int M, int N, int K, hipStream_t s, const LinearArgs& la) {
-#ifdef GGUF_MMQ_TUNE
-  if (dtype != GGUF_DTYPE_F16) return GGUF_ERR_DTYPE;
-  return mmq_typed<F, _Float16>(W, ws, Y, M, N, K, s, la);
-#else
   GGUF_DISPATCH_DTYPE(dtype, return (mmq_typed<F, scalar_t>(W, ws, Y, M, N, K, s, la)));
   return GGUF_ERR_DTYPE;
-#endif
 }
 
 template <class F, typename T>
@@ -591,9 +540,11 @@ static int moe_fmt(const void* W, const void* ws, void* Y, int dtype, int N, int
   return GGUF_ERR_DTYPE;
 }
 
-__global__ void zero_rows_kernel(uint4* __restrict__ p, int64_t n16) {
-  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x;
+// nbytes of zeros from p (16-byte aligned): whole 16-byte words, then the last thread past them clears the odd bytes
+__global__ void zero_rows_kernel(uint4* __restrict__ p, int64_t nbytes) {
+  const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x, n16 = nbytes >> 4;
   if (i < n16) p[i] = make_uint4(0, 0, 0, 0);
+  else if (i == n16) for (int64_t b = n16 << 4; b < nbytes; ++b) ((uint8_t*)p)[b] = 0;
 }
 
 static bool mmq_type_ok(int type) {
@@ -799,9 +750,8 @@ extern "C" int gguf_moe_mmq_act(const void* X, int xdtype, void* q8_workspace, c
   hipStream_t s = (hipStream_t)stream;
   // rows that no slot names stay zero, as with the reference's zero-filled output (gguf_kernel.cu:301-302)
   const int64_t ybytes = tokens * top_k * N * (xdtype == GGUF_DTYPE_F32 ? 4 : 2);
-  const int64_t n16 = ybytes / 16;
-  if (ybytes % 16 != 0) return GGUF_ERR_SHAPE;
-  hipLaunchKernelGGL(zero_rows_kernel, dim3((unsigned)((n16 + 255) / 256)), dim3(256), 0, s, (uint4*)Y, n16);
+  if ((uintptr_t)Y & 15) return GGUF_ERR_SHAPE;
+  hipLaunchKernelGGL(zero_rows_kernel, dim3((unsigned)((ybytes / 16 + 256) / 256)), dim3(256), 0, s, (uint4*)Y, ybytes);
   const int rc = quantize_q8_1(X, xdtype, q8_workspace, tokens, K, s, act);
   if (rc != GGUF_OK) return rc;
   MoeArgs moe = {sorted_token_ids, expert_ids, num_tokens_post_padded, expert_stride_bytes, (int)top_k, (int)(tokens * top_k), 0};

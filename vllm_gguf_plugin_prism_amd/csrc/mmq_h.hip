@@ -61,9 +61,7 @@ template <class F>
 static int mmqh_fmt(const void* W, const void* ws, void* Y, int dtype, int M, int N, int K, float* partial, int64_t partial_bytes,
                     hipStream_t s, const LinearArgs& la) {
   if (dtype == GGUF_DTYPE_F16) return mmqh_typed<A8Codes<F>, _Float16>(W, ws, Y, M, N, K, partial, partial_bytes, s, la);
-#ifndef GGUF_MMQ_TUNE
   if (dtype == GGUF_DTYPE_BF16) return mmqh_typed<A8Codes<F>, bf16_t>(W, ws, Y, M, N, K, partial, partial_bytes, s, la);
-#endif
   return GGUF_ERR_DTYPE;
 }
 
@@ -71,7 +69,6 @@ static int mmqh_fmt(const void* W, const void* ws, void* Y, int dtype, int M, in
 int mmq_half(const void* W, const void* ws, void* Y, int dtype, int type, int M, int N, int K, float* partial,
              int64_t partial_bytes, hipStream_t s, const LinearArgs& la) {
   switch (type) {
-#ifndef GGUF_MMQ_TUNE
     case T_Q4_0: return mmqh_fmt<MQ4_0>(W, ws, Y, dtype, M, N, K, partial, partial_bytes, s, la);
     case T_Q5_0: return mmqh_fmt<MQ5_0>(W, ws, Y, dtype, M, N, K, partial, partial_bytes, s, la);
     case T_Q8_0: return mmqh_fmt<MQ8_0>(W, ws, Y, dtype, M, N, K, partial, partial_bytes, s, la);
@@ -81,7 +78,6 @@ int mmq_half(const void* W, const void* ws, void* Y, int dtype, int type, int M,
     case T_Q5_K: return mmqh_fmt<MQ5_K>(W, ws, Y, dtype, M, N, K, partial, partial_bytes, s, la);
     case T_IQ4_XS: return mmqh_fmt<MIQ4_XS>(W, ws, Y, dtype, M, N, K, partial, partial_bytes, s, la);
     case T_IQ2_XXS: return mmqh_fmt<MIQ2_XXS>(W, ws, Y, dtype, M, N, K, partial, partial_bytes, s, la);
-#endif
     case T_Q6_K: return mmqh_fmt<MQ6_K>(W, ws, Y, dtype, M, N, K, partial, partial_bytes, s, la);
   }
   return GGUF_ERR_TYPE;

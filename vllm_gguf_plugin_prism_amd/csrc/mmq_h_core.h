@@ -417,11 +417,8 @@ static void launch_mmqh(const void* W, const void* ws, void* Y, int M, int N, in
   constexpr size_t lds = (size_t)(M_T + N_T) * (64 + 8) * 2 * 2;
   auto kern = mmqh_kernel<C, WM, WN, TM, TN, OCC, T>;
   if constexpr (lds > 65536) {
-    static bool configured = false;  // opt in to > 64 KB of dynamic LDS once per instantiation
-    if (!configured) {
-      (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-      configured = true;
-    }
+    static std::atomic<uint64_t> done{0};
+    allow_large_lds(kern, lds, done);
   }
   const int tiles_x = (N + N_T - 1) / N_T, tiles = tiles_x * ((M + M_T - 1) / M_T);
   if (whole < 0) { whole = tiles; shared = 0; splits = 1; }
@@ -434,26 +431,10 @@ static void launch_mmqh(const void* W, const void* ws, void* Y, int M, int N, in
                        whole, splits, ldy, (const T*)la.bias);
 }
 
-#ifdef GGUF_MMQ_TUNE
-static int tune_cfg_h() {
-  static const int v = [] { const char* e = getenv("GGUF_MMQH_CFG"); return e ? atoi(e) : 0; }();
-  return v;
-}
-#endif
 
 template <class C, typename T>
 static int mmqh_typed(const void* W, const void* ws, void* Y, int M, int N, int K, float* partial, int64_t partial_bytes,
                       hipStream_t stream, const LinearArgs& la = LinearArgs()) {
-#ifdef GGUF_MMQ_TUNE
-  switch (tune_cfg_h()) {
-    case 1: launch_mmqh<C, 4, 2, 2, 2, 1, T>(W, ws, Y, M, N, K, stream); return launch_status();   // 256 x 128, 8 waves
-    case 5: launch_mmqh<C, 2, 2, 2, 1, 2, T>(W, ws, Y, M, N, K, stream); return launch_status();   // 128 x 64, 4 waves
-    case 6: launch_mmqh<C, 2, 4, 2, 1, 2, T>(W, ws, Y, M, N, K, stream); return launch_status();   // 128 x 128, 8 waves (64 x 32 each)
-    case 7: launch_mmqh<C, 2, 2, 1, 1, 4, T>(W, ws, Y, M, N, K, stream); return launch_status();   // 64 x 64, 4 waves
-    case 8: launch_mmqh<C, 4, 2, 1, 2, 2, T>(W, ws, Y, M, N, K, stream); return launch_status();   // 128 x 128, 8 waves (32 x 64 each)
-    default: break;
-  }
-#endif
   const MmqhPlan p = mmq_half_plan(M, N, K, partial_bytes);
   switch (p.cfg) {
     case 0: launch_mmqh<C, 4, 2, 2, 2, 1, T>(W, ws, Y, M, N, K, stream, p.whole, p.shared, p.splits, partial, la); break;  // 256 x 128, 8 waves

@@ -30,8 +30,6 @@
 // or the output has too few tiles for the chip, the affected tiles are split along K into fp32 partial tiles that a
 // second kernel adds in fixed order (the result depends on the shape only, not on the run).
 #pragma once
-#include <atomic>
-
 #include "mmq_formats.h"
 
 namespace gguf {
@@ -54,17 +52,6 @@ __device__ __forceinline__ float seeded_times(int bits, float dw, float neg_seed
 // LDS row pitch in bytes.  K=32 operands are read 16 bytes per lane: a 16-byte skew (KS + 16) spreads 8 consecutive
 // rows over all banks.  K=16 operands are read 8 bytes per lane: an 8-byte skew (KS + 8) spreads 16 consecutive rows.
 template <int G, int KS> struct Pitch { static constexpr int value = G == 32 ? KS + 16 : KS + 8; };
-
-// opt in to more than 64 KB of dynamic LDS, once per kernel and device
-template <typename K>
-static void allow_large_lds(K kern, size_t lds, std::atomic<uint64_t>& done) {
-  int dev = 0;
-  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev > 63) dev = 0;
-  const uint64_t bit = 1ull << dev;
-  if (done.load(std::memory_order_relaxed) & bit) return;
-  (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
-  done.fetch_or(bit, std::memory_order_relaxed);
-}
 
 constexpr int MMQI_KS = 128;  // values of K per step
 

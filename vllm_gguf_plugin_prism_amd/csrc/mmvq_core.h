@@ -209,17 +209,10 @@ __global__ __launch_bounds__(256) void mmvq_kernel(const uint8_t* __restrict__ W
 //     row loop touches no LDS except for one partial sum per (row, wave), and refills the load slot it
 //     has just consumed: D row-loads stay in flight per wave.
 //   * Row totals are summed from the per-wave partials in a fixed order.
-#ifndef GGUF_MMVQ_NW
-#define GGUF_MMVQ_NW 16
-#endif
+constexpr int MMVQ_NW = 16;            // waves per workgroup of the streaming kernel
 // D = 2: measured against 1, 3, 4, 5 and "every row at once" on 33 MB matrices, two row-loads in flight per wave
 // (32 per CU and lane column) give the highest rate; deeper pipelines lose bandwidth, they do not gain latency cover.
-#ifndef GGUF_MMVQ_DEPTH
-#define GGUF_MMVQ_DEPTH 2
-#endif
-#ifndef GGUF_MMVQ_WG_PER_CU
-#define GGUF_MMVQ_WG_PER_CU 1
-#endif
+constexpr int MMVQ_DEPTH = 2;
 
 // MT per-lane values -> the sum over this lane's row of 16 lanes of value number (lane mod MT), in every lane.
 // Exchange step k pairs lanes 2^k apart: a lane keeps the half of its values whose class bit k equals its own lane
@@ -457,25 +450,13 @@ __global__ __launch_bounds__(64 * NW) void mmvq_stream_kernel(const uint8_t* __r
   GGUF_PHASE(4);                               // results stored
 }
 
-static int num_cus() {
-  static int n = 0;
-  if (n == 0) {
-    int dev = 0;
-    hipDeviceProp_t prop;
-    if (hipGetDevice(&dev) == hipSuccess && hipGetDeviceProperties(&prop, dev) == hipSuccess) n = prop.multiProcessorCount;
-    if (n <= 0) n = 256;
-  }
-  return n;
-}
-
 template <class F, int MT, int D, typename T, bool TILE, bool FULL, int NW>
 static void launch_stream_d(const void* W, const T* X, T* Y, int N, int K, int rows_per_wg, int grid, size_t lds, const LinearArgs& la,
                             hipStream_t stream, int m_act) {
   auto kern = mmvq_stream_kernel<F, MT, NW, D, T, TILE, FULL>;
-  static bool big_lds = false;
-  if (lds > 64 * 1024 && !big_lds) {
-    (void)hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-    big_lds = true;
+  if (lds > 64 * 1024) {
+    static std::atomic<uint64_t> done{0};
+    allow_large_lds(kern, 160 * 1024, done);
   }
   hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * NW), lds, stream, (const uint8_t*)W, X, Y, N, K, rows_per_wg,
                      la.w_pitch ? la.w_pitch : (int64_t)(K / F::QK) * F::BS, la.ldy ? la.ldy : (int64_t)N, (const T*)la.bias, m_act);
@@ -483,13 +464,13 @@ static void launch_stream_d(const void* W, const T* X, T* Y, int N, int K, int r
 
 // Returns false when the shape does not fit the streaming kernel (a row longer than NW waves, or activations
 // that do not fit in LDS); the caller then takes the workspace path.
-template <class F, int MT, typename T, bool TILE = false, int NW = GGUF_MMVQ_NW>
+template <class F, int MT, typename T, bool TILE = false, int NW = MMVQ_NW>
 static bool launch_stream(const void* W, const T* X, T* Y, int N, int K, hipStream_t stream, const LinearArgs& la, int m_act = MT) {
   // m_act <= MT rows of X are there; the kernel computes MT and stores m_act
   const int nb = K / 32, S = (nb + 63) / 64;
   if (S > NW) return false;
   const int slots = NW / S;
-  const int target = num_cus() * GGUF_MMVQ_WG_PER_CU;
+  const int target = num_cus();
   int rows_per_wg = (N + target - 1) / target;
   if (rows_per_wg < slots) rows_per_wg = slots;  // at least one row per slot
   const int grid = (N + rows_per_wg - 1) / rows_per_wg;
@@ -500,7 +481,7 @@ static bool launch_stream(const void* W, const T* X, T* Y, int N, int K, hipStre
   const auto go = [&](auto full) {
     constexpr bool FULL = decltype(full)::value;
     if constexpr (MT <= 4) {
-      if (per_wave >= GGUF_MMVQ_DEPTH) { launch_stream_d<F, MT, GGUF_MMVQ_DEPTH, T, TILE, FULL, NW>(W, X, Y, N, K, rows_per_wg, grid, lds, la, stream, m_act); return; }
+      if (per_wave >= MMVQ_DEPTH) { launch_stream_d<F, MT, MMVQ_DEPTH, T, TILE, FULL, NW>(W, X, Y, N, K, rows_per_wg, grid, lds, la, stream, m_act); return; }
     }
     // eight activation rows in registers leave room for one weight row in flight per wave
     launch_stream_d<F, MT, 1, T, TILE, FULL, NW>(W, X, Y, N, K, rows_per_wg, grid, lds, la, stream, m_act);
@@ -511,13 +492,8 @@ static bool launch_stream(const void* W, const T* X, T* Y, int N, int K, hipStre
   return true;
 }
 
-#ifndef GGUF_MMVQ_RPW
-#define GGUF_MMVQ_RPW 2
-#endif
-#ifndef GGUF_MMVQ_MAX_FUSED_M
-#define GGUF_MMVQ_MAX_FUSED_M 8
-#endif
-constexpr int MAX_FUSED_M = GGUF_MMVQ_MAX_FUSED_M;  // up to this many vectors are quantized inside the GEMV itself
+constexpr int MMVQ_RPW = 2;     // rows per wave of the workspace kernel
+constexpr int MAX_FUSED_M = 8;  // up to this many vectors are quantized inside the GEMV itself
 
 static inline int kchunk_for(int mt, int K) {
   int kchunk = mt == 1 ? 32768 : mt == 2 ? 16384 : mt == 4 ? 8192 : 4096;
@@ -531,7 +507,7 @@ static inline size_t mmvq_lds(int kchunk) {
 
 template <class F, int MT, typename T, bool FUSEQ>
 static void launch_mt(const void* W, const char* xsrc, T* Y, int N, int K, hipStream_t stream, const LinearArgs& la) {
-  constexpr int RPW = GGUF_MMVQ_RPW;
+  constexpr int RPW = MMVQ_RPW;
   const int kchunk = kchunk_for(MT, K);
   const int grid = (N + 4 * RPW - 1) / (4 * RPW);
   const int64_t xrb = FUSEQ ? (int64_t)K * (int64_t)sizeof(T) : q8_row_bytes(K);
@@ -612,13 +588,8 @@ extern "C" int gguf_moe_align_block_size(const int32_t* topk_ids, int64_t numel,
                                          int32_t* sorted_token_ids, int64_t sorted_capacity, int32_t* expert_ids,
                                          int64_t expert_capacity, int32_t* num_tokens_post_padded, gguf_stream_t stream);
 
-#ifndef GGUF_MOE_VEC_GROUP_RPW
-#define GGUF_MOE_VEC_GROUP_RPW 2
-#endif
-#ifndef GGUF_MOE_VEC_GROUP
-#define GGUF_MOE_VEC_GROUP 4
-#endif
-constexpr int MOE_VEC_GROUP = GGUF_MOE_VEC_GROUP;  // pairs of one expert that share a pass over its weights
+constexpr int MOE_VEC_GROUP_RPW = 2;
+constexpr int MOE_VEC_GROUP = 4;  // pairs of one expert that share a pass over its weights
 
 // With the expert count known and a workspace large enough for the quantized activations plus the routing sort
 // (q8 rows first, then the three sort arrays), pairs are grouped by expert: the activations are quantized once by the
@@ -627,7 +598,7 @@ constexpr int MOE_VEC_GROUP = GGUF_MOE_VEC_GROUP;  // pairs of one expert that s
 template <class F, typename T>
 static int moe_vec_typed(const void* W, const char* x, void* Y, int xdtype, int N, int K, const int32_t* topk_ids, int top_k,
                          int pairs, int act, int num_experts, void* scratch, int64_t scratch_bytes, hipStream_t stream) {
-  constexpr int RPW = GGUF_MMVQ_RPW;
+  constexpr int RPW = MMVQ_RPW;
   const int grid = (N + 4 * RPW - 1) / (4 * RPW);
   const int64_t xrb = (int64_t)K * (int64_t)sizeof(T) * (act == ACT_NONE ? 1 : 2);
   const int tokens = pairs / top_k;
@@ -647,7 +618,7 @@ static int moe_vec_typed(const void* W, const char* x, void* Y, int xdtype, int 
     if (rc != GGUF_OK) return rc;
     const int kchunk = kchunk_for(MOE_VEC_GROUP, K);
     const size_t lds = mmvq_lds<F, MOE_VEC_GROUP>(kchunk);
-    constexpr int GRPW = GGUF_MOE_VEC_GROUP_RPW;  // rows per wave: more rows amortise the staging of the group's activations
+    constexpr int GRPW = MOE_VEC_GROUP_RPW;  // rows per wave: more rows amortise the staging of the group's activations
     const int ggrid = (N + 4 * GRPW - 1) / (4 * GRPW);
     hipLaunchKernelGGL((mmvq_kernel<F, MOE_VEC_GROUP, GRPW, T, true, false>), dim3(ggrid, (unsigned)block_cap), dim3(256), lds, stream,
                        (const uint8_t*)W, (const char*)scratch, (T*)Y, N, K, kchunk, q8_row_bytes(K), (int64_t)N,

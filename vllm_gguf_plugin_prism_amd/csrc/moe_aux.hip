@@ -133,12 +133,8 @@ extern "C" int gguf_moe_align_block_size(const int32_t* topk_ids, int64_t numel,
   if (!sorted_token_ids || !expert_ids || !num_tokens_post_padded || (numel > 0 && !topk_ids)) return GGUF_ERR_NULL;
   const size_t lds = (size_t)(1 + ALIGN_WAVES) * num_experts * sizeof(int);
   if (lds > 65536) {
-    static bool configured = false;  // opt in to > 64 KB of dynamic LDS once
-    if (!configured) {
-      (void)hipFuncSetAttribute((const void*)moe_align_kernel, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                (int)((1 + ALIGN_WAVES) * ALIGN_MAX_EXPERTS * sizeof(int)));
-      configured = true;
-    }
+    static std::atomic<uint64_t> done{0};
+    gguf::allow_large_lds(moe_align_kernel, (1 + ALIGN_WAVES) * ALIGN_MAX_EXPERTS * sizeof(int), done);
   }
   hipLaunchKernelGGL(moe_align_kernel, dim3(1), dim3(ALIGN_THREADS), lds, (hipStream_t)stream, topk_ids, (int)numel,
                      (int)num_experts, (int)block, sorted_token_ids, (int)sorted_capacity, expert_ids, (int)expert_capacity,

@@ -183,6 +183,10 @@ def fused_moe_gguf(x, w1, w2, topk_weights, topk_ids, weight_type: int, weight_t
     top_k = topk_ids.shape[1]
     out_hidden = torch.empty_like(x)
     path = select_moe_path(int(weight_type), int(weight_type2), tokens)
+    if path == "grouped" and w1.shape[0] > ops.MOE_GROUPED_MAX_EXPERTS:
+        # The reference's grouped kernel drops expert ids above 255 without a word (moe.cuh:33) and the one here keeps
+        # that guard; the per-pair operator computes every expert, so a layer with more experts takes it at any batch.
+        path = "vec"
     topk_ids = topk_ids.to(torch.int32).contiguous()
     if path == "grouped":
         experts, rows, _ = w1.shape

@@ -141,10 +141,10 @@ def ggml_mul_mat_a8(W: torch.Tensor, X: torch.Tensor, quant_type: int, row: int,
                     out: torch.Tensor | None = None, bias: torch.Tensor | None = None) -> torch.Tensor:
     """Prefill GEMM ``q8_1(X) @ W^T`` on MFMA (reference: gguf_kernel.cu:220-290).
 
-    ``engine``: ``"int8"`` keeps the reference's integer arithmetic (int8 MFMA, block scales in fp32); ``"half"``
-    multiplies the dequantized operands on half-precision MFMA (faster, about 2e-4 relative deviation, half and
-    bfloat16 results only); ``"auto"`` takes ``"half"`` where it applies.  ``out`` / ``bias`` / sliced ``W``: as for
-    :func:`ggml_mul_mat_vec_a8`."""
+    ``engine``: ``"int8"`` keeps the reference's integer arithmetic (exact int8 dot products per block on int8 MFMA,
+    block scales in fp32) and is what ``"auto"`` means; ``"half"`` is opt-in and multiplies the dequantized operands
+    on half-precision MFMA (faster, about 2e-4 relative deviation from the integer result, half and bfloat16 results
+    only).  ``out`` / ``bias`` / sliced ``W``: as for :func:`ggml_mul_mat_vec_a8`."""
     out, w_pitch, ldy = _shard_args(W, X, quant_type, row, out, bias)
     vecs, col = X.shape
     with torch.cuda.device(X.device):
@@ -176,6 +176,9 @@ def ggml_dequant_gemm(W: torch.Tensor, X: torch.Tensor, quant_type: int, row: in
     return out
 
 
+MOE_GROUPED_MAX_EXPERTS = 256
+
+
 def ggml_moe_a8(
     X: torch.Tensor,
     W: torch.Tensor,
@@ -197,6 +200,10 @@ def ggml_moe_a8(
     for t in (sorted_token_ids, expert_ids, num_tokens_post_padded):
         if t.dtype != torch.int32:
             raise ValueError("MoE index tensors must be int32")
+    if W.dim() == 3 and W.shape[0] > MOE_GROUPED_MAX_EXPERTS:
+        # the kernel keeps the reference's guard and leaves the rows of experts past 255 zero (moe.cuh:33): refuse rather
+        # than return a result with holes; ggml_moe_a8_vec has no such limit
+        raise NotImplementedError(f"ggml_moe_a8 takes at most {MOE_GROUPED_MAX_EXPERTS} experts, got {W.shape[0]}")
     act = _act_code(activation)
     col = X.shape[1] // 2 if act else X.shape[1]
     with torch.cuda.device(X.device):
