@@ -228,26 +228,40 @@ def _probes(rng, dev):
                   f"{unroll} loads in flight per lane, {'non-temporal' if nt else 'plain'} loads")
         del bufs
 
-    print("== streaming GEMV kernel, Q4_K batch 1 fp16: wall-clock times of five points, microseconds after the first wave")
-    print("   of the launch entered (median over workgroups; first wave / last wave of a workgroup); 10 ns clock")
+    print("== streaming GEMV kernel, Q4_K batch 1 fp16: wall-clock times of eight points, microseconds after the first wave")
+    print("   of the launch entered (median over workgroups; first wave / last wave of a workgroup); 10 ns clock;")
+    print("   the launch traced is the last of a HIP graph of back-to-back launches over rotating weight copies")
     for n, k in CFG2_SHAPES:
         ws = [torch.from_numpy(np.concatenate([synth.make_weights(rng, Q4_K, min(2048, n - r), k) for r in range(0, n, 2048)], axis=0)).to(dev)]
         ws += [ws[0].clone() for _ in range(int(700e6 // ws[0].numel()))]
         x = torch.from_numpy(rng.standard_normal((1, k)).astype(np.float32)).to(torch.float16).to(dev)
         y = torch.empty((1, n), dtype=torch.float16, device=dev)
-        acc = []
-        for rep in range(len(ws) * 2):
-            rc = h.gguf_probe_mmvq_q4_k(ws[rep % len(ws)].data_ptr(), x.data_ptr(), y.data_ptr(), n, k, stream())
+
+        def launch(i):
+            rc = h.gguf_probe_mmvq_q4_k(ws[i % len(ws)].data_ptr(), x.data_ptr(), y.data_ptr(), n, k, stream())
             assert rc == 0
+
+        # back-to-back launches over all copies in one HIP graph; the trace buffer holds the last launch of a replay
+        for i in range(3):
+            launch(i)
+        torch.cuda.synchronize()
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            for i in range(len(ws)):
+                launch(i)
+        acc = []
+        nwg = 256
+        for rep in range(12):
+            g.replay()
             torch.cuda.synchronize()
-            nwg = 256
             buf = (ctypes.c_ulonglong * (nwg * 16))()
             assert h.gguf_probe_mmvq_trace(buf, nwg) == 0
-            t = np.frombuffer(buf, dtype=np.uint64).reshape(nwg, 2, 8)[:, :, :5].astype(np.int64)
-            if rep >= len(ws):          # the first pass over the copies warms code and page tables up
+            t = np.frombuffer(buf, dtype=np.uint64).reshape(nwg, 2, 8)[:, :, [0, 5, 6, 7, 1, 2, 3, 4]].astype(np.int64)
+            if rep >= 2:
                 acc.append((t - t[:, :, 0].min()) * 0.01)
         t = np.median(np.stack(acc), axis=0)          # [workgroup][first/last wave][point], median over launches
-        names = ("entered", "own activations quantized", "all activations in LDS", "own rows walked", "results stored")
+        names = ("entered", "kernel arguments read", "activation requests out", "first weight requests out",
+                 "own activations quantized", "all activations in LDS", "own rows walked", "results stored")
         print(f"-- [{n},{k}], {n * (k // 256) * 144 / 1e6:.1f} MB")
         for p, name in enumerate(names):
             a, b = np.median(t[:, 0, p]), np.median(t[:, 1, p])

@@ -276,7 +276,7 @@ template <> struct TileSums<FmtQ5_0> { static constexpr bool swaps = true; };
 template <> struct TileSums<FmtQ4_K> { static constexpr bool swaps = true; };
 template <> struct TileSums<FmtQ5_K> { static constexpr bool swaps = true; };
 
-// Profiling builds (the probe library only) record when the first and the last wave of every workgroup pass five
+// Profiling builds (the probe library only) record when the first and the last wave of every workgroup pass eight
 // points of the kernel, on the 100 MHz wall clock that all CUs share.
 #ifdef GGUF_TRACE_PHASES
 __device__ unsigned long long g_mmvq_phases[1024 * 2 * 8];
@@ -289,37 +289,62 @@ __device__ unsigned long long g_mmvq_phases[1024 * 2 * 8];
 #define GGUF_PHASE(i) do {} while (0)
 #endif
 
+// What the streaming kernel needs before its first memory requests, worked out on the host so that the kernel starts
+// without a division, and packed so that all of its arguments fit the first 64 bytes of the argument block (one
+// fetch).  The quotients by S and by K/8 are taken by multiplication with a rounded-up reciprocal, exact for the small
+// numerators here: wave < 16 with S <= 16, and group index * K/8 < 2^32 because K <= 32768 for this kernel.
+struct StreamGeom {
+  uint32_t w_pitch;       // bytes between rows of W
+  int N, K, rows_per_wg;
+  uint32_t packed;        // m_act | S << 4 | slots << 9 | (4096 / S + 1) << 14
+  uint32_t g8_inv;        // 2^32 / (K / 8) + 1
+  __device__ __forceinline__ int m_act() const { return packed & 15; }
+  __device__ __forceinline__ int S() const { return (packed >> 4) & 31; }          // waves per row: ceil(K / 32 / 64)
+  __device__ __forceinline__ int slots() const { return (packed >> 9) & 31; }      // rows side by side: NW / S (>= 1)
+  __device__ __forceinline__ int slot_of(int wave) const { return (int)(((unsigned)wave * (packed >> 14)) >> 12); }  // wave / S
+};
+static inline StreamGeom stream_geom(int N, int K, int rows_per_wg, int64_t w_pitch, int m_act, int nw) {
+  StreamGeom g;
+  const int S = (K / 32 + 63) / 64;
+  g.w_pitch = (uint32_t)w_pitch;
+  g.N = N;
+  g.K = K;
+  g.rows_per_wg = rows_per_wg;
+  g.packed = (uint32_t)m_act | (uint32_t)S << 4 | (uint32_t)(nw / S) << 9 | (4096u / (uint32_t)S + 1u) << 14;
+  g.g8_inv = (uint32_t)((1ull << 32) / (uint32_t)(K / 8)) + 1u;
+  return g;
+}
+
 template <class F, int MT, int NW, int D, typename T, bool TILE = false, bool FULL = true>
 __global__ __launch_bounds__(64 * NW) void mmvq_stream_kernel(const uint8_t* __restrict__ W, const T* __restrict__ X,
-                                                               T* __restrict__ Y, int N, int K, int rows_per_wg, int64_t w_pitch,
-                                                               int64_t ldy, const T* __restrict__ bias, int m_act) {
+                                                               T* __restrict__ Y, const T* __restrict__ bias, int64_t ldy,
+                                                               StreamGeom geom) {
   extern __shared__ __align__(16) char smem[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: row arithmetic stays on the scalar unit
+  const int N = geom.N, K = geom.K, rows_per_wg = geom.rows_per_wg, m_act = geom.m_act();
   GGUF_PHASE(0);                               // entry
   const int nb = K >> 5;                       // 32-weight units per row
-  const int S = (nb + 63) >> 6;                // waves per row
-  const int slots = NW / S;                    // rows in flight side by side (>= 1, checked by the host)
+  const int S = geom.S();                      // waves per row
+  const int slots = geom.slots();              // rows in flight side by side (>= 1, checked by the host)
   int8_t* lq = (int8_t*)smem;                  // [MT][K]
   float* ldv = (float*)(smem + (size_t)MT * K);  // [MT][nb]
   float* lav = ldv + MT * nb;                  // [MT][nb]
   char* tab = (char*)(lav + (F::AUX != AUX_NONE ? MT * nb : 0));
   float* part = (float*)(tab + F::TABLE_BYTES);  // [rows_per_wg][S][4 rows of 16 lanes][MT]
 
-  const int r_begin = blockIdx.x * rows_per_wg;
+  const int r_begin = blockIdx.x * rows_per_wg;   // (the host launches ceil(N / rows_per_wg) workgroups: r_begin < N)
   const int r_end = min(N, r_begin + rows_per_wg);
-  if (r_begin >= r_end) return;
   const int nrows = r_end - r_begin;
-  const int64_t rowbytes = w_pitch;   // bytes between rows: the dense row size unless the caller's tensor is padded
+  if (nrows > 0) GGUF_PHASE(5);                // kernel arguments have arrived
+  const int64_t rowbytes = geom.w_pitch;   // bytes between rows: the dense row size unless the caller's tensor is padded
 
   // this wave: slot (which of the side-by-side rows) and step (which 64-unit stretch of the row)
-  const int slot = wave / S, step = wave - slot * S;
+  const int slot = geom.slot_of(wave), step = wave - slot * S;   // wave / S, wave % S
   const bool wave_on = slot < slots;           // NW - slots*S waves have no weights to fetch; they still quantize
   const int u_raw = step * 64 + lane;
   const bool lane_on = wave_on && u_raw < nb;
   const int u = min(u_raw, nb - 1);
-  const int my_rows = wave_on && nrows > slot ? (nrows - slot + slots - 1) / slots : 0;  // rows slot, slot+slots, ...
-  const int max_rows = (nrows + slots - 1) / slots;  // trip count of the row loop, same for every wave
 
   if (F::TABLE_BYTES > 0) {
     F::init_tables(tab);
@@ -345,9 +370,10 @@ __global__ __launch_bounds__(64 * NW) void mmvq_stream_kernel(const uint8_t* __r
   const int rows_x = FULL ? MT : m_act;
   const int qtotal = rows_x * g8;  // a multiple of 4, so quads stay whole
   typename F::Regs pre[D];
+  const auto row_of_group = [&](int qc) { return MT == 1 ? 0 : (int)__umulhi((unsigned)qc, geom.g8_inv); };  // qc / g8
   auto quantize_group = [&](const raw8<T>& raw, int q) {
     const int qc = min(q, qtotal - 1);
-    const int m = qc / g8, j = qc - m * g8;
+    const int m = row_of_group(qc), j = qc - m * g8;
     float xv[8];
     raw.cvt(xv);
     const Q8Quad qq = q8_1_quantize8(xv);
@@ -365,15 +391,18 @@ __global__ __launch_bounds__(64 * NW) void mmvq_stream_kernel(const uint8_t* __r
     constexpr int QG = decltype(qg_tag)::value;
     if constexpr (QG == 0) {   // a wave with no activation values to quantize: its weights only
       if (qtotal <= NT) __builtin_amdgcn_s_barrier();   // (see below: the others' activation requests go first)
+      GGUF_PHASE(6);
 #pragma unroll
       for (int d = 0; d < D; ++d) pre[d] = load_row(d);
+      __builtin_amdgcn_sched_barrier(0);
+      GGUF_PHASE(7);
       return;
     }
     raw8<T> xraw[QG > 0 ? QG : 1];
 #pragma unroll
     for (int g = 0; g < QG; ++g) {
       const int qc = min(tid + g * NT, qtotal - 1);
-      const int m = qc / g8, j = qc - m * g8;
+      const int m = row_of_group(qc), j = qc - m * g8;
       xraw[g].load(X + (int64_t)m * K + 8 * j);
     }
     __builtin_amdgcn_sched_barrier(0);
@@ -384,9 +413,13 @@ __global__ __launch_bounds__(64 * NW) void mmvq_stream_kernel(const uint8_t* __r
       __builtin_amdgcn_s_barrier();
       __builtin_amdgcn_sched_barrier(0);
     }
+    GGUF_PHASE(6);                             // activation requests are out (every wave's, where one request covers them)
 #pragma unroll
     for (int d = 0; d < D; ++d) pre[d] = load_row(d);
     __builtin_amdgcn_sched_barrier(0);
+    GGUF_PHASE(7);                             // weight requests of the first rows are out
+#pragma unroll
+    for (int g = 0; g < QG; ++g) xraw[g].hold();   // (keeps the conversions below from moving above the weight requests)
 #pragma unroll
     for (int g = 0; g < QG; ++g) quantize_group(xraw[g], tid + g * NT);
   };
@@ -398,7 +431,7 @@ __global__ __launch_bounds__(64 * NW) void mmvq_stream_kernel(const uint8_t* __r
   else prologue(std::integral_constant<int, 4>{});
   for (int q = tid + 4 * NT; q - tid < qtotal; q += NT) {  // uniform trip count; only for K * MT > 32 * NT
     const int qc = min(q, qtotal - 1);
-    const int m2 = qc / g8, j2 = qc - m2 * g8;
+    const int m2 = row_of_group(qc), j2 = qc - m2 * g8;
     raw8<T> r;
     r.load(X + (int64_t)m2 * K + 8 * j2);
     quantize_group(r, q);
@@ -406,6 +439,9 @@ __global__ __launch_bounds__(64 * NW) void mmvq_stream_kernel(const uint8_t* __r
   GGUF_PHASE(1);                               // own share of the activations quantized
   __syncthreads();
   GGUF_PHASE(2);                               // every wave's share is in LDS
+  // (the two quotients below are the kernel's only divisions; here they run while the first weights are still on their way)
+  const int my_rows = wave_on && nrows > slot ? (nrows - slot + slots - 1) / slots : 0;  // rows slot, slot+slots, ...
+  const int max_rows = (nrows + slots - 1) / slots;  // trip count of the row loop, same for every wave
 
   // this lane's column of every activation vector, held in registers for the whole row loop
   typename F::ActRegs act[MT];
@@ -458,8 +494,9 @@ static void launch_stream_d(const void* W, const T* X, T* Y, int N, int K, int r
     static std::atomic<uint64_t> done{0};
     allow_large_lds(kern, 160 * 1024, done);
   }
-  hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * NW), lds, stream, (const uint8_t*)W, X, Y, N, K, rows_per_wg,
-                     la.w_pitch ? la.w_pitch : (int64_t)(K / F::QK) * F::BS, la.ldy ? la.ldy : (int64_t)N, (const T*)la.bias, m_act);
+  const int64_t w_pitch = la.w_pitch ? la.w_pitch : (int64_t)(K / F::QK) * F::BS;
+  hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * NW), lds, stream, (const uint8_t*)W, X, Y, (const T*)la.bias,
+                     la.ldy ? la.ldy : (int64_t)N, stream_geom(N, K, rows_per_wg, w_pitch, m_act, NW));
 }
 
 // Returns false when the shape does not fit the streaming kernel (a row longer than NW waves, or activations
@@ -469,6 +506,7 @@ static bool launch_stream(const void* W, const T* X, T* Y, int N, int K, hipStre
   // m_act <= MT rows of X are there; the kernel computes MT and stores m_act
   const int nb = K / 32, S = (nb + 63) / 64;
   if (S > NW) return false;
+  if ((la.w_pitch ? la.w_pitch : (int64_t)(K / F::QK) * F::BS) > (int64_t)UINT32_MAX) return false;   // (the kernel holds it in 32 bits)
   const int slots = NW / S;
   const int target = num_cus();
   int rows_per_wg = (N + target - 1) / target;

@@ -18,6 +18,10 @@ template <typename T> struct raw8;
 template <> struct raw8<float> {
   float4 a, b;
   __device__ __forceinline__ void load(const float* p) { a = *(const float4*)p; b = *(const float4*)(p + 4); }
+  // Nothing that uses the loaded values may be scheduled before this point (and the wait for them comes here).
+  __device__ __forceinline__ void hold() {
+    asm volatile("" : "+v"(a.x), "+v"(a.y), "+v"(a.z), "+v"(a.w), "+v"(b.x), "+v"(b.y), "+v"(b.z), "+v"(b.w));
+  }
   __device__ __forceinline__ void cvt(float (&v)[8]) const {
     v[0] = a.x; v[1] = a.y; v[2] = a.z; v[3] = a.w; v[4] = b.x; v[5] = b.y; v[6] = b.z; v[7] = b.w;
   }
@@ -25,6 +29,7 @@ template <> struct raw8<float> {
 template <> struct raw8<_Float16> {
   uint4 a;
   __device__ __forceinline__ void load(const _Float16* p) { a = *(const uint4*)p; }
+  __device__ __forceinline__ void hold() { asm volatile("" : "+v"(a.x), "+v"(a.y), "+v"(a.z), "+v"(a.w)); }
   __device__ __forceinline__ void cvt(float (&v)[8]) const {
     const uint32_t w[4] = {a.x, a.y, a.z, a.w};
 #pragma unroll
@@ -37,6 +42,7 @@ template <> struct raw8<_Float16> {
 template <> struct raw8<bf16_t> {
   uint4 a;
   __device__ __forceinline__ void load(const bf16_t* p) { a = *(const uint4*)p; }
+  __device__ __forceinline__ void hold() { asm volatile("" : "+v"(a.x), "+v"(a.y), "+v"(a.z), "+v"(a.w)); }
   __device__ __forceinline__ void cvt(float (&v)[8]) const {
     const uint32_t w[4] = {a.x, a.y, a.z, a.w};
 #pragma unroll
