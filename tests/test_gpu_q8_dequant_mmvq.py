@@ -55,6 +55,45 @@ def test_q8_1_ties_round_away_from_zero():
     assert q[0, :7].cpu().tolist() == [127, 1, -1, 3, -3, 1, 0]
 
 
+def test_q8_1_near_ties_and_extreme_scales_bit_exact():
+    # Blocks built to sit on the rounding boundary: the block maximum is 127 * d for an arbitrary d, so the scale is d
+    # (or its neighbour), and the other values are (k + 1/2) * d and their neighbours one and two units in the last
+    # place away.  Scales run from the smallest subnormal quotient to near overflow.
+    ops = _ops()
+    rng = np.random.default_rng(4242)
+    rows = []
+    for d in np.concatenate([rng.uniform(0.001, 10.0, 200), 2.0 ** rng.integers(-140, 100, 60), [1.0, 2.0 ** -133, 1e-39, 3e-41, 2.5e36]]).astype(np.float32):
+        blk = np.zeros(32, dtype=np.float32)
+        k = rng.integers(-126, 126, 31).astype(np.float32)
+        base = (k + np.float32(0.5)) * np.float32(d)
+        step = rng.integers(-2, 3, 31)
+        vals = base.copy()
+        for s in (1, 2):
+            up = np.nextafter(vals, np.float32(np.inf), dtype=np.float32)
+            dn = np.nextafter(vals, np.float32(-np.inf), dtype=np.float32)
+            vals = np.where(step >= s, up, np.where(step <= -s, dn, vals))
+        blk[:31] = vals
+        blk[31] = np.float32(127.0) * np.float32(d)
+        rows.append(rng.permutation(blk))
+    x = np.stack(rows).astype(np.float32)
+    x = x[np.isfinite(x).all(axis=1)]
+    x = np.concatenate([x, x[:, ::-1]], axis=1)          # two blocks per row
+    q, ds = ops.quantize_q8_1(torch.from_numpy(x).cuda())
+    qo, do, so = o.quantize_q8_1(x)
+    assert np.array_equal(q.cpu().numpy(), qo)
+    assert np.array_equal(ds[:, :, 0].cpu().numpy(), do.astype(np.float32))
+    # the same values through the GEMV's own quantizer: Q8_0 weights that pick out one element each
+    n, kk = 64, 64
+    w = o.make_weights(rng, o.Q8_0, n, kk)
+    for r in (0, 17, x.shape[0] - 1):
+        xr = torch.from_numpy(x[r : r + 1].copy()).cuda()
+        if not np.isfinite(x[r]).all() or np.abs(x[r]).max() > 1e30 or np.abs(x[r]).max() < 1e-30:
+            continue
+        y = ops.ggml_mul_mat_vec_a8(_to_dev(w), xr, o.Q8_0, n).cpu().numpy()
+        exp = o.mul_mat_a8(w, x[r : r + 1], o.Q8_0, n, "mmvq")
+        assert o.rel_l2(y, exp) <= 1e-5
+
+
 @pytest.mark.parametrize("dt", ["f16", "bf16", "f32"])
 @pytest.mark.parametrize("qtype", ALL)
 def test_dequantize_bit_exact(qtype, dt):

@@ -80,6 +80,13 @@ struct FmtQ4_K {
     const uint8_t* b = row + (int64_t)sb * BS;
     Regs r; r.hdr = ld<uint4>(b); r.q = ld<uint4>(b + 16 + 16 * c); return r;
   }
+  // The 64 units a wave covers are 8 whole blocks, 1152 contiguous bytes; from a copy of them in LDS lane l takes the
+  // header of block l / 8 and its own 16 bytes of qs.
+  static constexpr int SPAN = 8 * BS;
+  static __device__ __forceinline__ Regs from_span(const char* span, int lane) {
+    const char* b = span + (lane >> 3) * BS;
+    Regs r; r.hdr = *(const uint4*)b; r.q = *(const uint4*)(b + 16 + 16 * (lane & 7)); return r;
+  }
   struct ActRegs { int4 lo, hi; float2 d8, du; };
   static __device__ __forceinline__ ActRegs load_act(const Act& x, int u) {
     const int sb = u >> 3, c = u & 7, g = c >> 1, h = c & 1;
@@ -111,7 +118,9 @@ struct FmtQ4_K {
       s0 = dot4((int)(q[i] & 0x0F0F0F0Fu), al[i], s0);
       s1 = dot4((int)((q[i] >> 4) & 0x0F0F0F0Fu), ah[i], s1);
     }
-    const float pos = x.d8.x * (float)(s0 * (int)(a0 & 0xFF)) + x.d8.y * (float)(s1 * (int)(a0 >> 8));
+    // (|s| * scale < 2^21: the product of the two converted factors is the converted integer product, bit for bit, and
+    //  a float multiply issues at four times the rate of a 32-bit integer one)
+    const float pos = x.d8.x * ((float)s0 * (float)(a0 & 0xFF)) + x.d8.y * ((float)s1 * (float)(a0 >> 8));
     const float neg = x.du.x * (float)(a1 & 0xFF) + x.du.y * (float)(a1 >> 8);
     return h2f(r.hdr.x & 0xFFFF) * pos - h2f(r.hdr.x >> 16) * neg;
   }

@@ -106,31 +106,39 @@ __device__ __forceinline__ Q8Quad q8_1_quantize8(const float (&v)[8]) {
 
   const float d = amax / 127.0f;
   const float dd = amax == 0.0f ? 1.0f : d;  // an all-zero block divides 0 by 1: q = 0 without a branch
-  // q = roundf(x / dd), ties away from zero, bit-for-bit what the IEEE quotient gives.  One reciprocal per
-  // lane replaces eight divisions: x * (1/dd) is within 127 * 2^-23 of the true quotient, so it rounds the
-  // same way unless the fraction lies within 2^-14 of a tie; only then is the exact quotient formed.
-  const float rd = 1.0f / dd;
-  int q[8];
-  int isum = 0;
+  // q = roundf(x / dd), ties away from zero, bit-for-bit what the IEEE quotient gives.  The hardware reciprocal
+  // (one ulp) replaces eight divisions: x * rcp(dd) is within 127 * 2^-22 of the true quotient, so it rounds the same
+  // way unless its fraction lies within 2^-14 of a tie, and away from a tie adding half a unit and truncating is the
+  // rounding.  A lane that meets a near-tie among its eight values, or a scale so small that its reciprocal
+  // overflows, forms the exact quotients for all eight instead.
+  const float rd = __builtin_amdgcn_rcpf(dd);
+  float t[8];
+  bool exact = !(rd < 3.0e38f);
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
-    float t = v[i] * rd;
-    float tr = truncf(t);
-    float fr = fabsf(t - tr);
-    if (fabsf(fr - 0.5f) < 6.1035156e-5f) {
-      t = v[i] / dd;
-      tr = truncf(t);
-      fr = fabsf(t - tr);
-    }
-    q[i] = (int)tr + (fr >= 0.5f ? (t < 0.0f ? -1 : 1) : 0);
-    isum += q[i];
+    t[i] = v[i] * rd;
+    const float fr = __builtin_amdgcn_fractf(fabsf(t[i]));
+    exact = exact || fabsf(fr - 0.5f) < 6.1035156e-5f;
   }
+  if (exact) {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const float e = v[i] / dd;
+      const float tr = truncf(e);
+      // the quotient rounded half away from zero, as a value that the add-half-and-truncate below maps to itself
+      t[i] = tr + (fabsf(e - tr) >= 0.5f ? copysignf(1.0f, e) : 0.0f);
+    }
+  }
+  int q[8];
+#pragma unroll
+  for (int i = 0; i < 8; ++i) q[i] = (int)(t[i] + copysignf(0.5f, t[i]));   // (the conversion truncates)
+  Q8Quad r;
+  r.q.x = __builtin_amdgcn_perm(__builtin_amdgcn_perm(q[3], q[2], 0x0c0c0400), __builtin_amdgcn_perm(q[1], q[0], 0x0c0c0400), 0x05040100);
+  r.q.y = __builtin_amdgcn_perm(__builtin_amdgcn_perm(q[7], q[6], 0x0c0c0400), __builtin_amdgcn_perm(q[5], q[4], 0x0c0c0400), 0x05040100);
+  int isum = __builtin_amdgcn_sdot4((int)r.q.x, 0x01010101, 0, false);
+  isum = __builtin_amdgcn_sdot4((int)r.q.y, 0x01010101, isum, false);
   isum += dpp_mov_i<0x4E>(isum);
   isum += dpp_mov_i<0xB1>(isum);
-
-  Q8Quad r;
-  r.q.x = (q[0] & 0xFF) | ((q[1] & 0xFF) << 8) | ((q[2] & 0xFF) << 16) | ((uint32_t)(q[3] & 0xFF) << 24);
-  r.q.y = (q[4] & 0xFF) | ((q[5] & 0xFF) << 8) | ((q[6] & 0xFF) << 16) | ((uint32_t)(q[7] & 0xFF) << 24);
   r.d = (float)(_Float16)d;
   r.s = (float)(_Float16)sum;
   r.du = r.d * (float)isum;
