@@ -88,19 +88,21 @@ int gguf_mmq(const void* W, const void* x, int xdtype, void* q8_workspace, void*
              int64_t M, gguf_stream_t stream);
 
 /* gguf_mmq with the arithmetic engine chosen by the caller.  The reference has one engine (dp4a, mmq.cuh:2-104);
- * this library has two and gguf_mmq picks between them:
+ * this library has two:
  *   GGUF_MMQ_INT8  int8 MFMA on the block codes, block scales applied in fp32: the reference's arithmetic, differing
- *                  only in the order of the fp32 additions;
+ *                  only in the order of the fp32 additions.  This is what gguf_mmq runs.
  *   GGUF_MMQ_HALF  half-precision MFMA on operands that carry their scales (activation d8*q and weight d*q, each
- *                  rounded to half): two to three times faster, relative deviation about 2e-4 in the l2 norm, below
- *                  the rounding of a half or bfloat16 result.  Not for fp32 results; not for Q4_1 / Q5_1.
- *   GGUF_MMQ_AUTO  HALF where it applies, INT8 otherwise; with M <= 8 the streaming GEMV kernel instead, switched to
- *                  this operator's offset sums (Q4_K, Q5_K, Q5_0 are the formats where the reference's GEMV and its
- *                  tile GEMM form them differently), which is exact in int8 and reads W once at the GEMV's rate.
+ *                  rounded to half): about 1.8 times faster, relative deviation about 2e-4 in the l2 norm, below
+ *                  the rounding of a half or bfloat16 result -- but not the reference's arithmetic, so only for
+ *                  callers that ask.  Not for fp32 results; not for Q4_1 / Q5_1.
+ *   GGUF_MMQ_AUTO  INT8; with M <= 8 the streaming GEMV kernel instead, switched to this operator's offset sums
+ *                  (Q4_K, Q5_K, Q5_0 are the formats where the reference's GEMV and its tile GEMM form them
+ *                  differently), which is exact in int8 and reads W once at the GEMV's rate.
  * workspace_bytes is the size of q8_workspace; 0 stands for the minimum, M * gguf_q8_1_row_bytes(K).  Given
- * gguf_mmq_workspace_bytes(M, N, K) bytes, the half engine splits K over several workgroups per output tile when the
- * output alone has too few tiles to occupy the chip (few tokens or a narrow N with a long K), keeping fp32 partial
- * tiles behind the rows and adding them in a second launch.  The result does not depend on the run, only on the shape. */
+ * gguf_mmq_workspace_bytes(M, N, K) bytes, either engine splits K over several workgroups per output tile where the
+ * output tiles alone would leave much of the chip idle (few tokens, a narrow N with a long K, a sparse last round of
+ * tiles), keeping fp32 partial tiles behind the rows and adding them in a second launch in fixed order.  The result
+ * does not depend on the run, only on the shape and on whether the room was given. */
 #define GGUF_MMQ_AUTO 0
 #define GGUF_MMQ_INT8 1
 #define GGUF_MMQ_HALF 2

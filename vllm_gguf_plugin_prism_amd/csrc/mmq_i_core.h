@@ -90,8 +90,11 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void mmqi_kernel(const uint8_t* __
   int wg = blockIdx.x;
   const int whole8 = whole_tiles & ~7;
   if (wg < whole8) wg = (wg & 7) * (whole8 >> 3) + (wg >> 3);
-  const int tile = wg < whole_tiles ? wg : whole_tiles + (wg - whole_tiles) % shared_tiles;
-  const int split = wg < whole_tiles ? 0 : (wg - whole_tiles) / shared_tiles;
+  int sw = wg - whole_tiles;                       // (>= 0: a workgroup on a shared tile; numbered the same way)
+  const int shared8 = (shared_tiles * splits) & ~7;
+  if (sw >= 0 && sw < shared8 && (whole_tiles & 7) == 0) sw = (sw & 7) * (shared8 >> 3) + (sw >> 3);
+  const int tile = wg < whole_tiles ? wg : whole_tiles + sw % shared_tiles;
+  const int split = wg < whole_tiles ? 0 : sw / shared_tiles;
   const int nsplit = wg < whole_tiles ? 1 : splits;
   const int m_base = (tile % tiles_m) * M_T, n_base = (tile / tiles_m) * N_T;
   const int nkb_total = K >> 5;
