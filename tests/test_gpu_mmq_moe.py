@@ -452,6 +452,34 @@ def test_moe_vec_shared_experts_keep_gemv_semantics(qtype, dt):
     assert torch.equal(y2[torch.from_numpy(keep).cuda()], y[torch.from_numpy(keep).cuda()])
 
 
+@pytest.mark.parametrize("dt", ["f32", "f16"])
+@pytest.mark.parametrize("qtype", [o.Q4_0, o.Q8_0, o.Q4_K, o.Q5_K, o.IQ4_XS, o.IQ2_XXS])
+def test_moe_vec_blocks_of_16_slots(qtype, dt):
+    """Up to 16 pairs per expert on average the tile route sorts into blocks of 16 slots and runs the 16-row MFMA kernel:
+    experts with more than 16 pairs (two blocks), with none, a ragged last step of K (for the 32-value formats), an
+    output narrower and one wider than the kernel's 128 features, and an expert id outside the table."""
+    ops = _ops()
+    rng = np.random.default_rng(1200 + qtype)
+    qk = o.QUANT_SIZES[qtype][0]
+    for t, top_k, e, n, k in [(24, 4, 8, 200, 736 if qk == 32 else 768), (64, 8, 64, 72, 512)]:
+        w = np.stack([o.make_weights(rng, qtype, n, k) for _ in range(e)])
+        xd, xv = _x(rng, t, k, dt)
+        ids, _ = _routing(rng, t, e, top_k)
+        if e == 8:
+            ids[:20, 0] = 5          # expert 5 gets at least 20 pairs: two blocks
+            ids[ids == 2] = 3        # expert 2 gets none (pairs are independent: a token may name an expert twice)
+        assert 2 * e <= t * top_k <= 16 * e
+        y = ops.ggml_moe_a8_vec(xd, _dev(w), _dev(ids), top_k, qtype, n, t)
+        want = o.moe_a8_vec(xv, w, ids, top_k, qtype, n, t)
+        assert o.rel_l2(y.float().cpu().numpy(), want) <= (1e-5 if dt == "f32" else 1e-3), (o.TYPE_NAMES[qtype], t, e)
+        bad = ids.copy()
+        bad[1, 0] = e + 3
+        y2 = ops.ggml_moe_a8_vec(xd, _dev(w), _dev(bad), top_k, qtype, n, t)
+        keep = np.ones(t * top_k, dtype=bool)
+        keep[top_k] = False
+        assert torch.equal(y2[torch.from_numpy(keep).cuda()], y[torch.from_numpy(keep).cuda()])
+
+
 @pytest.mark.parametrize("qtype", ALL)
 def test_moe_vec_matches_oracle(qtype):
     ops = _ops()

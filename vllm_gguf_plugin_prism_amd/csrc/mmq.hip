@@ -136,17 +136,6 @@ __host__ __device__ constexpr size_t mmq_group_lds_bytes() {
   return (size_t)(M_T + N_T) * Pitch<F::G, KS>::value + (size_t)(KB + XA) * M_T * 4 + (size_t)(KS / F::G + WMN) * N_T * 4;
 }
 
-struct MoeArgs {
-  const int32_t* sorted_token_ids;
-  const int32_t* expert_ids;
-  const int32_t* num_tokens_post_padded;
-  int64_t expert_stride;  // bytes
-  int top_k;
-  int num_pairs;          // tokens * top_k
-  int gemv_sums;          // offset term of Q4_K / Q5_K: 0 = times the stored block sum (the reference's tile kernels,
-                          // vecdotq.cuh:369-372), 1 = times d8 * (sum of the quants) (its GEMV, vecdotq.cuh:328-351)
-};
-
 // MODE selects how staging and contraction overlap:
 //   MODE_PREFETCH  the next step's global loads are issued before this step's MFMA phase and held in registers;
 //   MODE_PLAIN     load, stage, contract in turn; latency is covered only by other workgroups on the CU;
@@ -571,20 +560,29 @@ int64_t moe_vec_tiles_workspace(int64_t tokens, int64_t top_k, int64_t K, int64_
   return tokens * q8_row_bytes(K) + (sorted_cap + sorted_cap / 32 + 2) * 4;
 }
 
+// moe_tiles16.hip: the same contraction over blocks of 16 slots, for experts with few pairs
+bool moe_tiles16_ok(int type);
+int moe_tiles16(const void* W, const void* ws, void* Y, int dtype, int type, int N, int K, int num_sorted, const MoeArgs& moe,
+                hipStream_t s);
+
 int moe_vec_tiles(const void* X, int xdtype, void* workspace, const void* W, const int32_t* topk_ids, void* Y, int type, int N,
                   int K, int top_k, int tokens, int act, int num_experts, hipStream_t s) {
   const int pairs = tokens * top_k;
   int rc = quantize_q8_1(X, xdtype, workspace, tokens, K, s, act);
   if (rc != GGUF_OK) return rc;
-  const int64_t sorted_cap = (int64_t)pairs + (int64_t)num_experts * 31;
-  const int64_t block_cap = sorted_cap / 32 + 1;
+  // Blocks of 16 slots while an expert has 16 pairs or fewer on average (most of a 32-slot block would be padding),
+  // blocks of 32 above.  The routing arrays of either fit the room moe_vec_tiles_workspace reports.
+  const int blk = pairs <= 16 * num_experts && moe_tiles16_ok(type) ? 16 : 32;
+  const int64_t sorted_cap = (int64_t)pairs + (int64_t)num_experts * (blk - 1);
+  const int64_t block_cap = sorted_cap / blk + 1;
   int32_t* sorted = (int32_t*)((char*)workspace + (int64_t)tokens * q8_row_bytes(K));  // rows are a multiple of 4 bytes long
   int32_t* experts = sorted + sorted_cap;
   int32_t* post = experts + block_cap;
-  rc = gguf_moe_align_block_size(topk_ids, pairs, num_experts, 32, sorted, sorted_cap, experts, block_cap, post, (gguf_stream_t)s);
+  rc = gguf_moe_align_block_size(topk_ids, pairs, num_experts, blk, sorted, sorted_cap, experts, block_cap, post, (gguf_stream_t)s);
   if (rc != GGUF_OK) return rc;
   const int64_t stride = (int64_t)N * (K / block_elems(type)) * block_bytes(type);
   MoeArgs moe = {sorted, experts, post, stride, top_k, pairs, type == T_Q4_K || type == T_Q5_K ? 1 : 0};
+  if (blk == 16) return moe_tiles16(W, workspace, Y, xdtype, type, N, K, (int)(sorted_cap / 16 * 16), moe, s);
   const int ns = (int)(sorted_cap / 32 * 32);   // blocks past the padded total see expert -1 and leave
   switch (type) {
     case T_Q4_0: return moe_fmt<MQ4_0>(W, workspace, Y, xdtype, N, K, ns, moe, s);

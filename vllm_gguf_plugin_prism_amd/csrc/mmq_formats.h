@@ -6,6 +6,18 @@
 
 namespace gguf {
 
+// The routing of the grouped MoE contraction (reference: csrc/gguf/moe.cuh:5-129), as moe_align_block_size leaves it.
+struct MoeArgs {
+  const int32_t* sorted_token_ids;
+  const int32_t* expert_ids;
+  const int32_t* num_tokens_post_padded;
+  int64_t expert_stride;  // bytes
+  int top_k;
+  int num_pairs;          // tokens * top_k
+  int gemv_sums;          // offset term of Q4_K / Q5_K: 0 = times the stored block sum (the reference's tile kernels,
+                          // vecdotq.cuh:369-372), 1 = times d8 * (sum of the quants) (its GEMV, vecdotq.cuh:328-351)
+};
+
 // --------------------------------------------------------------------------------------------
 // Format policies: unpack one 32-element block of one weight row to int8 (8 dwords, element order)
 // plus fp32 scale(s) and, where the format has one, the fp32 offset factor multiplied by the
