@@ -141,13 +141,13 @@ def _other_configs(rng, dev, w_14336x4096):
     n, k = 14336, 4096
     copies = [torch.from_numpy(w_14336x4096).to(dev)]
     copies += [copies[0].clone() for _ in range(19)]          # 20 x 33 MB, walked in turn
-    for b in (1, 2, 4, 8):
+    for b in (1, 2, 4, 8, 16, 32):      # (the baseline names 1, 2, 4, 8; 16 and 32 show the few-row tile route)
         x = xs(b, k)
         path = dispatch.select_mul_mat_path(Q4_K, b, n)
         ms = _timed_ms(lambda i: dispatch.fused_mul_mat_gguf(x, copies[i % 20], Q4_K), 20)
         res[f"config2_q4_k_14336x4096_bs{b}"] = {"path": path, "us": ms * 1e3,
                                                 "GBps": gemv_bytes(Q4_K, n, k, b) / (ms * 1e-3) / 1e9}
-        if path != "mmvq":
+        if path != "mmvq" and b <= 8:
             ms = _timed_ms(lambda i: ops.ggml_mul_mat_vec_a8(copies[i % 20], x, Q4_K, n), 20)
             res[f"config2_q4_k_14336x4096_bs{b}_gemv"] = {"path": "mmvq (forced)", "us": ms * 1e3,
                                                          "GBps": gemv_bytes(Q4_K, n, k, b) / (ms * 1e-3) / 1e9}

@@ -453,6 +453,33 @@ def test_moe_vec_shared_experts_keep_gemv_semantics(qtype, dt):
 
 
 @pytest.mark.parametrize("dt", ["f32", "f16"])
+@pytest.mark.parametrize("qtype", [o.Q4_0, o.Q8_0, o.Q4_K, o.Q5_K, o.IQ4_XS, o.IQ2_XXS, o.Q6_K])
+def test_mmq_nine_to_32_rows(qtype, dt):
+    """9 to 32 rows of X run on 16-row tiles with K split over the chip (Q6_K up to 16 rows, the large tiles above): both
+    sides of the 16- and 32-row edges, an output narrower than a tile and one that is not a multiple of it, a short K
+    that cannot be split and a long one that is, and the same call without room for partial tiles."""
+    ops = _ops()
+    rng = np.random.default_rng(1300 + qtype)
+    from vllm_gguf_plugin_prism_amd import _lib
+    lib = _lib.lib()
+    for m, n, k in [(9, 72, 512), (16, 200, 1024), (17, 384, 2048), (32, 130, 4096), (33, 130, 1024)]:
+        w = o.make_weights(rng, qtype, n, k)
+        xd, xv = _x(rng, m, k, dt)
+        y = ops.ggml_mul_mat_a8(_dev(w), xd, qtype, n)
+        want = o.mul_mat_a8(w, xv, qtype, n, "mmq")
+        tol = 1e-5 if dt == "f32" else 1e-3
+        assert o.rel_l2(y.float().cpu().numpy(), want) <= tol, (o.TYPE_NAMES[qtype], m, n, k)
+        # the minimum workspace: no room for partial tiles, so K is not split; same arithmetic, other summation order
+        nbytes = m * lib.gguf_q8_1_row_bytes(k)
+        ws = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+        y2 = torch.empty_like(y)
+        rc = lib.gguf_mmq_engine(_dev(w).data_ptr(), xd.data_ptr(), {"f32": 0, "f16": 1, "bf16": 2}[dt], ws.data_ptr(), y2.data_ptr(),
+                                 int(qtype), n, k, m, 1, nbytes, torch.cuda.current_stream().cuda_stream)
+        assert rc == 0
+        assert o.rel_l2(y2.float().cpu().numpy(), want) <= tol
+
+
+@pytest.mark.parametrize("dt", ["f32", "f16"])
 @pytest.mark.parametrize("qtype", [o.Q4_0, o.Q8_0, o.Q4_K, o.Q5_K, o.IQ4_XS, o.IQ2_XXS])
 def test_moe_vec_blocks_of_16_slots(qtype, dt):
     """Up to 16 pairs per expert on average the tile route sorts into blocks of 16 slots and runs the 16-row MFMA kernel:

@@ -604,11 +604,18 @@ int moe_vec_tiles(const void* X, int xdtype, void* workspace, const void* W, con
 int mmvq_any(int type, const void* W, const void* x, void* q8_workspace, void* Y, int xdtype, int64_t N, int64_t K, int64_t M,
              hipStream_t s, const LinearArgs& la);
 
+constexpr int MMQ_ROWS16_MAX = 32;   // up to this many rows of X the integer path runs the 16-row tile kernel
+
 // mmq_h.hip
 int mmq_half(const void* W, const void* ws, void* Y, int dtype, int type, int M, int N, int K, float* partial,
              int64_t partial_bytes, hipStream_t s, const LinearArgs& la);
 bool mmq_half_supported(int type);
 int64_t mmq_half_partial_bytes(int M, int N, int K);
+
+// moe_tiles16.hip: the 16-row tile kernel for 9 .. 32 rows of X (GGUF_NOT_TAKEN for formats it does not cover)
+int mmq_rows16(const void* W, const void* ws, void* Y, int dtype, int type, int M, int N, int K, float* partial, int64_t partial_bytes,
+               hipStream_t s, const LinearArgs& la);
+int64_t mmq_rows16_partial_bytes(int M, int N, int K);
 
 // mmq_i.hip
 int mmq_int(const void* W, const void* ws, void* Y, int dtype, int type, int M, int N, int K, float* partial,
@@ -623,7 +630,9 @@ static int64_t mmq_rows_bytes(int64_t M, int64_t K) { return (M * (gguf::q8_row_
 extern "C" int64_t gguf_mmq_workspace_bytes(int64_t M, int64_t N, int64_t K) {
   if (M <= 0 || N <= 0 || K <= 0 || M > 0x7FFFFFF0LL || N > 0x7FFFFFF0LL || K > 0x7FFFFFF0LL) return 0;
   const int64_t ph = gguf::mmq_half_partial_bytes((int)M, (int)N, (int)K), pi = gguf::mmq_int_partial_bytes((int)M, (int)N, (int)K);
-  return mmq_rows_bytes(M, K) + (ph > pi ? ph : pi);
+  const int64_t p16 = M <= gguf::MMQ_ROWS16_MAX ? gguf::mmq_rows16_partial_bytes((int)M, (int)N, (int)K) : 0;
+  const int64_t p = ph > pi ? ph : pi;
+  return mmq_rows_bytes(M, K) + (p > p16 ? p : p16);
 }
 
 // gguf_mmq_linear with the size of the workspace's row region given by the caller: rows_bytes < 0 stands for the public
@@ -683,6 +692,10 @@ int gguf::mmq_linear_impl(const void* W, int64_t w_row_pitch_bytes, const void* 
   }
   int rc = quantize_q8_1(x, xdtype, q8_workspace, M, K, s);
   if (rc != GGUF_OK) return rc;
+  if (M <= MMQ_ROWS16_MAX) {   // a few rows: 16-row tiles, K split over the chip
+    rc = mmq_rows16(W, q8_workspace, Y, xdtype, type, (int)M, (int)N, (int)K, partial, partial_bytes, s, la);
+    if (rc != GGUF_NOT_TAKEN) return rc;
+  }
   rc = mmq_int(W, q8_workspace, Y, xdtype, type, (int)M, (int)N, (int)K, partial, partial_bytes, s, la);
   if (rc != GGUF_NOT_TAKEN) return rc;
   switch (type) {

@@ -16,14 +16,25 @@ namespace gguf {
 
 typedef int v4i_t __attribute__((ext_vector_type(4)));
 
-template <class F, typename T, int NW, int OCC>
+// Dense mode (MOE = false): the same tile for a plain product with 9 to 32 rows of X, where the 64 x 128 tiles of the
+// integer engine would multiply mostly padding and leave most of the chip idle.  `tiles` output tiles of 16 rows x
+// 16 CT NW features, each split `splits` ways along K when the output alone has too few tiles to fill the chip; split
+// tiles leave fp32 partial tiles that mmqi_reduce_kernel adds in fixed order.
+struct Dense16 {
+  int M, splits;
+  int64_t w_pitch, ldy;
+  float* partial;
+};
+
+template <class F, typename T, int NW, int OCC, bool MOE = true>
 __global__ __launch_bounds__(64 * NW, OCC) void moe16_kernel(const uint8_t* __restrict__ W, const char* __restrict__ ws, int64_t ws_row_bytes,
-                                                        T* __restrict__ Y, int N, int K, int Kp, int tiles_m, int tiles, MoeArgs moe) {
-  static_assert(F::G == 32, "formats whose weight scale holds for a whole 32-value block");
+                                                        T* __restrict__ Y, int N, int K, int Kp, int tiles_m, int tiles, MoeArgs moe,
+                                                        Dense16 dn, const T* __restrict__ bias) {
+  static_assert(!(F::G == 16 && F::HAS_MIN), "16-deep formats with per-group offsets keep the 32-row kernel");
   constexpr int NT = 64 * NW, KS = MMQI_KS, KB = KS / 32, GR = KS / 16, LDK = Pitch<32, KS>::value;
   constexpr int M_T = 16, CT = 2, N_T = 16 * CT * NW;   // two 16-feature tiles per wave
   constexpr int PAIRS = N_T * KB, WP = PAIRS / NT;  // (weight row, 32-block) pairs per step, per thread
-  constexpr int DEPTH = 2;
+  constexpr int DEPTH = F::G == 16 ? 1 : 2;          // (two stages of the large Q6_K / Q3_K blocks do not fit the registers)
   constexpr size_t BUF = (size_t)(M_T + N_T) * LDK + (size_t)KB * M_T * 4 * (F::HAS_MIN ? 2 : 1) + (size_t)KB * N_T * 8;
   static_assert(BUF % 16 == 0 && PAIRS % NT == 0 && M_T * GR <= NT, "buffers keep 16-byte alignment; shares divide evenly");
   extern __shared__ __align__(16) char smem[];
@@ -32,24 +43,36 @@ __global__ __launch_bounds__(64 * NW, OCC) void moe16_kernel(const uint8_t* __re
   const int lcol = lane & 15, lgrp = lane >> 4;     // MFMA operand: row / column lcol, k values [8 lgrp, +8); result rows 4 lgrp + r
 
   int wg = blockIdx.x;
-  const int tiles8 = tiles & ~7;                    // workgroups go to the 8 XCDs in turn: give each a contiguous run
-  if (wg < tiles8) wg = (wg & 7) * (tiles8 >> 3) + (wg >> 3);
-  const int block = wg % tiles_m, m_base = block * M_T, n_base = (wg / tiles_m) * N_T;
-  if (m_base >= moe.num_tokens_post_padded[0]) return;
-  const int e = moe.expert_ids[block];
-  if (e < 0 || e > 255) return;                     // the reference's guard (moe.cuh:33)
-  W += (int64_t)e * moe.expert_stride;
-  const int64_t w_pitch = (int64_t)(K / F::QK) * F::BS;
-  const int nkb_total = K >> 5, nsteps = (K + KS - 1) / KS;
-  const auto src_row = [&](int m) {                 // the token row behind slot m of the block; row 0 stands in for padding
-    const int pair = moe.sorted_token_ids[m_base + m];
-    return pair < moe.num_pairs ? pair / moe.top_k : 0;
+  const int nsplit = MOE ? 1 : dn.splits;
+  const int total = tiles * nsplit, total8 = total & ~7;   // workgroups go to the 8 XCDs in turn: give each a contiguous run
+  if (wg < total8) wg = (wg & 7) * (total8 >> 3) + (wg >> 3);
+  const int tile = wg % tiles, split = wg / tiles;
+  const int block = tile % tiles_m, m_base = block * M_T, n_base = (tile / tiles_m) * N_T;
+  int64_t w_pitch = (int64_t)(K / F::QK) * F::BS;
+  if constexpr (MOE) {
+    if (m_base >= moe.num_tokens_post_padded[0]) return;
+    const int e = moe.expert_ids[block];
+    if (e < 0 || e > 255) return;                   // the reference's guard (moe.cuh:33)
+    W += (int64_t)e * moe.expert_stride;
+  } else {
+    w_pitch = dn.w_pitch;
+  }
+  const int nkb_total = K >> 5, nsteps_all = (K + KS - 1) / KS;
+  const int per_split = (nsteps_all + nsplit - 1) / nsplit;
+  const int t0 = split * per_split, nsteps = max(0, min(nsteps_all, t0 + per_split) - t0);
+  const auto src_row = [&](int m) {                 // the row of the quantized activations behind tile row m
+    if constexpr (MOE) {
+      const int pair = moe.sorted_token_ids[m_base + m];
+      return pair < moe.num_pairs ? pair / moe.top_k : 0;    // row 0 stands in for padding
+    } else {
+      return min(m_base + m, dn.M - 1);             // rows past M repeat the last row; never stored
+    }
   };
 
   // ---- per-thread staging plan, fixed over K
   const char* const aq_src = ws + (int64_t)src_row(min(tid / GR, M_T - 1)) * ws_row_bytes + 16 * (tid % GR);   // threads < 128
   const float* const as_src = (const float*)(ws + (int64_t)src_row(min(tid, M_T - 1)) * ws_row_bytes + Kp);     // threads < 16
-  const int sum_plane = (moe.gemv_sums ? 2 : 1) * (Kp / 32);
+  const int sum_plane = (MOE && moe.gemv_sums ? 2 : 1) * (Kp / 32);
   const uint8_t* w_src[WP];
 #pragma unroll
   for (int i = 0; i < WP; ++i) w_src[i] = W + (int64_t)min(n_base + (tid + NT * i) / KB, N - 1) * w_pitch;
@@ -92,10 +115,10 @@ __global__ __launch_bounds__(64 * NW, OCC) void moe16_kernel(const uint8_t* __re
       uint32_t q[8];
       float s0, s1, mn = 0.0f, mn1 = 0.0f;
       F::unpack(r.w[i], kb0 + kb, q, s0, s1, mn, mn1);
-      if (kb0 + kb >= nkb_total) s0 = mn = 0.0f;      // a block past K was re-read: scaled to nothing
+      if (kb0 + kb >= nkb_total) s0 = s1 = mn = 0.0f;   // a block past K was re-read: scaled to nothing
       *(uint4*)(wq + n * LDK + 32 * kb) = make_uint4(q[0], q[1], q[2], q[3]);
       *(uint4*)(wq + n * LDK + 32 * kb + 16) = make_uint4(q[4], q[5], q[6], q[7]);
-      wsc[kb * N_T + n] = (f32x2){s0, -mn};
+      wsc[kb * N_T + n] = F::G == 32 ? (f32x2){s0, -mn} : (f32x2){s0, s1};   // 16-deep formats: one scale per half
     }
   };
 
@@ -114,22 +137,43 @@ __global__ __launch_bounds__(64 * NW, OCC) void moe16_kernel(const uint8_t* __re
     const f32x2* wsc = (const f32x2*)(xd + KB * M_T * (F::HAS_MIN ? 2 : 1));
 #pragma unroll
     for (int kb = 0; kb < KB; ++kb) {
-      const long a = *(const long*)(xq + lcol * LDK + 32 * kb + 8 * lgrp);
       const f32x4 d8 = *(const f32x4*)(xd + kb * M_T + 4 * lgrp);
       f32x4 s8 = {0.0f, 0.0f, 0.0f, 0.0f};
       if constexpr (F::HAS_MIN) s8 = *(const f32x4*)(xs + kb * M_T + 4 * lgrp);
+      if constexpr (F::G == 32) {
+        const long a = *(const long*)(xq + lcol * LDK + 32 * kb + 8 * lgrp);
 #pragma unroll
-      for (int c = 0; c < CT; ++c) {
-        const int col = 32 * wave + 16 * c + lcol;
-        const long b = *(const long*)(wq + col * LDK + 32 * kb + 8 * lgrp);
-        const f32x2 sc = wsc[kb * N_T + col];
-        const v4i_t s = __builtin_amdgcn_mfma_i32_16x16x32_i8(a, b, seed, 0, 0, 0);
-        const float nsd = -kSeed * sc[0];
+        for (int c = 0; c < CT; ++c) {
+          const int col = 32 * wave + 16 * c + lcol;
+          const long b = *(const long*)(wq + col * LDK + 32 * kb + 8 * lgrp);
+          const f32x2 sc = wsc[kb * N_T + col];
+          const v4i_t s = __builtin_amdgcn_mfma_i32_16x16x32_i8(a, b, seed, 0, 0, 0);
+          const float nsd = -kSeed * sc[0];
 #pragma unroll
-        for (int r = 0; r < 4; ++r) {
-          const float t = seeded_times(s[r], sc[0], nsd);   // = RN(S * dw)
-          acc[c][r] = __builtin_fmaf(t, d8[r], acc[c][r]);
-          if constexpr (F::HAS_MIN) acc[c][r] = __builtin_fmaf(s8[r], sc[1], acc[c][r]);
+          for (int r = 0; r < 4; ++r) {
+            const float t = seeded_times(s[r], sc[0], nsd);   // = RN(S * dw)
+            acc[c][r] = __builtin_fmaf(t, d8[r], acc[c][r]);
+            if constexpr (F::HAS_MIN) acc[c][r] = __builtin_fmaf(s8[r], sc[1], acc[c][r]);
+          }
+        }
+      } else {
+        // the weight scale changes every 16 values: one MFMA per half block, the same K=32 instruction with the
+        // activations of the other half zeroed (k groups 0, 1 are the first half, 2, 3 the second)
+        const long a = *(const long*)(xq + lcol * LDK + 32 * kb + 8 * lgrp);
+        const long a0 = lgrp < 2 ? a : 0L, a1 = lgrp < 2 ? 0L : a;
+#pragma unroll
+        for (int c = 0; c < CT; ++c) {
+          const int col = 32 * wave + 16 * c + lcol;
+          const long b = *(const long*)(wq + col * LDK + 32 * kb + 8 * lgrp);
+          const f32x2 sc = wsc[kb * N_T + col];
+          const v4i_t sa = __builtin_amdgcn_mfma_i32_16x16x32_i8(a0, b, seed, 0, 0, 0);
+          const v4i_t sb = __builtin_amdgcn_mfma_i32_16x16x32_i8(a1, b, seed, 0, 0, 0);
+          const float nsa = -kSeed * sc[0], nsb = -kSeed * sc[1];
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            acc[c][r] = __builtin_fmaf(seeded_times(sa[r], sc[0], nsa), d8[r], acc[c][r]);
+            acc[c][r] = __builtin_fmaf(seeded_times(sb[r], sc[1], nsb), d8[r], acc[c][r]);
+          }
         }
       }
     }
@@ -141,36 +185,55 @@ __global__ __launch_bounds__(64 * NW, OCC) void moe16_kernel(const uint8_t* __re
   // them before a stage is decoded, which leaves the second stage about one turn of lead.  Making every thread issue
   // every load gives exact counts and was measured slower, 63 against 53 us for the first expert GEMM of the 64-token
   // layer: the redundant activation loads cost more than the lead gains.)
-  fetch(0, stage[0]);
-  stash(0, 0, stage[0]);
+  if (nsteps > 0) {
+    fetch(t0, stage[0]);
+    stash(t0, 0, stage[0]);
 #pragma unroll
-  for (int d = 0; d < DEPTH; ++d)
-    if (1 + d < nsteps) fetch(1 + d, stage[d]);
-  __syncthreads();
-  for (int j0 = 0; j0 < nsteps; j0 += DEPTH) {
+    for (int d = 0; d < DEPTH; ++d)
+      if (1 + d < nsteps) fetch(t0 + 1 + d, stage[d]);
+    __syncthreads();
+    for (int j0 = 0; j0 < nsteps; j0 += DEPTH) {
 #pragma unroll
-    for (int d = 0; d < DEPTH; ++d) {   // (stage indices are compile-time: the stages live in registers)
-      const int j = j0 + d;
-      if (j < nsteps) {
-        if (j + 1 < nsteps) {
-          stash(j + 1, (j + 1) & 1, stage[d]);
-          if (j + 1 + DEPTH < nsteps) fetch(j + 1 + DEPTH, stage[d]);
+      for (int d = 0; d < DEPTH; ++d) {   // (stage indices are compile-time: the stages live in registers)
+        const int j = j0 + d;
+        if (j < nsteps) {
+          if (j + 1 < nsteps) {
+            stash(t0 + j + 1, (j + 1) & 1, stage[d]);
+            if (j + 1 + DEPTH < nsteps) fetch(t0 + j + 1 + DEPTH, stage[d]);
+          }
+          contract(j & 1);
+          __syncthreads();
         }
-        contract(j & 1);
-        __syncthreads();
       }
     }
   }
 
-  // ---- store: lane = one output feature of each of its tiles, four slots
+  // ---- store: lane = one output feature of each of its tiles, four rows
+  if constexpr (!MOE) {
+    if (nsplit > 1) {   // the whole partial tile, edges included: the adder masks them
+      float* const mine = dn.partial + ((int64_t)tile * nsplit + split) * (M_T * N_T);
+#pragma unroll
+      for (int r = 0; r < 4; ++r)
+#pragma unroll
+        for (int c = 0; c < CT; ++c) mine[(4 * lgrp + r) * N_T + 32 * wave + 16 * c + lcol] = acc[c][r];
+      return;
+    }
+  }
 #pragma unroll
   for (int r = 0; r < 4; ++r) {
-    const int pair = moe.sorted_token_ids[m_base + 4 * lgrp + r];
-    if (pair >= moe.num_pairs) continue;
+    int64_t row;
+    if constexpr (MOE) {
+      const int pair = moe.sorted_token_ids[m_base + 4 * lgrp + r];
+      if (pair >= moe.num_pairs) continue;
+      row = (int64_t)pair * N;
+    } else {
+      if (m_base + 4 * lgrp + r >= dn.M) continue;
+      row = (int64_t)(m_base + 4 * lgrp + r) * dn.ldy;
+    }
 #pragma unroll
     for (int c = 0; c < CT; ++c) {
       const int nn = n_base + 32 * wave + 16 * c + lcol;
-      if (nn < N) Y[(int64_t)pair * N + nn] = finish<T>(acc[c][r], (const T*)nullptr, nn);
+      if (nn < N) Y[row + nn] = finish<T>(acc[c][r], MOE ? (const T*)nullptr : bias, nn);
     }
   }
 }
@@ -190,8 +253,75 @@ static int moe16_typed(const void* W, const void* ws, void* Y, int N, int K, int
   const int tiles_m = num_sorted / 16, tiles = tiles_m * ((N + N_T - 1) / N_T);
   if (tiles == 0) return GGUF_OK;
   hipLaunchKernelGGL(kern, dim3(tiles), dim3(64 * NW), lds, stream, (const uint8_t*)W, (const char*)ws, q8_row_bytes(K), (T*)Y, N, K,
-                     (int)q8_kp(K), tiles_m, tiles, moe);
+                     (int)q8_kp(K), tiles_m, tiles, moe, Dense16{}, (const T*)nullptr);
   return launch_status();
+}
+
+// The plain product for 9 .. 32 rows of X on the same tile.  The chip holds 3 x 256 workgroups of this kernel: an output
+// with fewer tiles is split along K (at least four steps of 128 values per stretch, at most 16 ways) when the workspace
+// has room for the partial tiles.  Measured on Q4_K [14336,4096] at 16 rows: aiming at 384 workgroups 26.3 us, 768
+// 24.4 us, 1536 28.7 us, no split 46.5 us.
+static inline int dense16_splits(int M, int N, int K, int64_t partial_bytes_available) {
+  const int64_t tiles = (int64_t)((M + 15) / 16) * ((N + 127) / 128);
+  const int nsteps = (K + MMQI_KS - 1) / MMQI_KS;
+  int s = tiles > 0 ? (int)(768 / tiles) : 1;
+  if (s > nsteps / 4) s = nsteps / 4;   // a stretch shorter than four steps is mostly prologue
+  if (s > 16) s = 16;
+  if (s < 2) return 1;
+  return tiles * s * (16 * 128 * 4) <= partial_bytes_available ? s : 1;
+}
+int64_t mmq_rows16_partial_bytes(int M, int N, int K) {
+  const int s = dense16_splits(M, N, K, INT64_MAX);
+  return s > 1 ? (int64_t)((M + 15) / 16) * ((N + 127) / 128) * s * (16 * 128 * 4) : 0;
+}
+
+template <class F, typename T>
+static int dense16_typed(const void* W, const void* ws, void* Y, int M, int N, int K, float* partial, int64_t partial_bytes,
+                         hipStream_t stream, const LinearArgs& la) {
+  constexpr int NW = 4, N_T = 32 * NW, OCC = sizeof(typename F::Raw) > 64 ? 2 : 3;
+  constexpr size_t BUF = (size_t)(16 + N_T) * Pitch<32, MMQI_KS>::value + (size_t)4 * 16 * 4 * (F::HAS_MIN ? 2 : 1) + (size_t)4 * N_T * 8;
+  constexpr size_t lds = 2 * BUF;
+  auto kern = moe16_kernel<F, T, NW, OCC, false>;
+  if constexpr (lds > 65536) {
+    static std::atomic<uint64_t> done{0};
+    allow_large_lds(kern, lds, done);
+  }
+  const int tiles_m = (M + 15) / 16, tiles = tiles_m * ((N + N_T - 1) / N_T);
+  const int splits = dense16_splits(M, N, K, partial_bytes);
+  const int64_t w_pitch = la.w_pitch ? la.w_pitch : (int64_t)(K / F::QK) * F::BS, ldy = la.ldy ? la.ldy : (int64_t)N;
+  hipLaunchKernelGGL(kern, dim3(tiles * splits), dim3(64 * NW), lds, stream, (const uint8_t*)W, (const char*)ws, q8_row_bytes(K), (T*)Y, N, K,
+                     (int)q8_kp(K), tiles_m, tiles, MoeArgs{}, Dense16{M, splits, w_pitch, ldy, partial}, (const T*)la.bias);
+  if (splits > 1)
+    hipLaunchKernelGGL((mmqi_reduce_kernel<16, N_T, T>), dim3(tiles, 2), dim3(256), 0, stream, partial, (T*)Y, M, N, tiles_m, 0, splits,
+                       ldy, (const T*)la.bias);
+  return launch_status();
+}
+
+template <class F>
+static int dense16_fmt(const void* W, const void* ws, void* Y, int dtype, int M, int N, int K, float* partial, int64_t partial_bytes,
+                       hipStream_t s, const LinearArgs& la) {
+  GGUF_DISPATCH_DTYPE(dtype, return (dense16_typed<F, scalar_t>(W, ws, Y, M, N, K, partial, partial_bytes, s, la)));
+  return GGUF_ERR_DTYPE;
+}
+
+// q8_1(X) . W^T for a few rows of X (the quantized rows are in the workspace); GGUF_NOT_TAKEN for other formats.
+int mmq_rows16(const void* W, const void* ws, void* Y, int dtype, int type, int M, int N, int K, float* partial, int64_t partial_bytes,
+               hipStream_t s, const LinearArgs& la) {
+  // the 16-deep formats pay two MFMAs and four vector instructions per result and block here as in the large tiles, and
+  // with two 16-row tiles (17 .. 32 rows) the large tiles are as fast: Q6_K [14336,4096] 44 us either way
+  if ((type == T_Q6_K || type == T_Q3_K) && M > 16) return GGUF_NOT_TAKEN;
+  switch (type) {
+    case T_Q4_0: return dense16_fmt<MQ4_0>(W, ws, Y, dtype, M, N, K, partial, partial_bytes, s, la);
+    case T_Q8_0: return dense16_fmt<MQ8_0>(W, ws, Y, dtype, M, N, K, partial, partial_bytes, s, la);
+    case T_Q5_0: return dense16_fmt<MQ5_0>(W, ws, Y, dtype, M, N, K, partial, partial_bytes, s, la);
+    case T_Q3_K: return dense16_fmt<MQ3_K>(W, ws, Y, dtype, M, N, K, partial, partial_bytes, s, la);
+    case T_Q6_K: return dense16_fmt<MQ6_K>(W, ws, Y, dtype, M, N, K, partial, partial_bytes, s, la);
+    case T_Q4_K: return dense16_fmt<MQ4_K>(W, ws, Y, dtype, M, N, K, partial, partial_bytes, s, la);
+    case T_Q5_K: return dense16_fmt<MQ5_K>(W, ws, Y, dtype, M, N, K, partial, partial_bytes, s, la);
+    case T_IQ4_XS: return dense16_fmt<MIQ4_XS>(W, ws, Y, dtype, M, N, K, partial, partial_bytes, s, la);
+    case T_IQ2_XXS: return dense16_fmt<MIQ2_XXS>(W, ws, Y, dtype, M, N, K, partial, partial_bytes, s, la);
+  }
+  return GGUF_NOT_TAKEN;
 }
 
 template <class F>
@@ -202,8 +332,8 @@ static int moe16_fmt(const void* W, const void* ws, void* Y, int dtype, int N, i
 
 bool moe_tiles16_ok(int type) {
   switch (type) {
-    case T_Q4_0: case T_Q8_0: case T_Q4_K: case T_Q5_K: case T_IQ4_XS: case T_IQ2_XXS: return true;
-    default: return false;   // 16-deep formats and those with other scale rules keep the 32-slot kernel
+    case T_Q4_0: case T_Q8_0: case T_Q3_K: case T_Q4_K: case T_Q5_K: case T_Q6_K: case T_IQ4_XS: case T_IQ2_XXS: return true;
+    default: return false;   // formats with other scale rules (Q4_1, Q5_1, Q2_K; Q5_0 in the per-pair operator) keep the 32-slot kernel
   }
 }
 
@@ -213,6 +343,8 @@ int moe_tiles16(const void* W, const void* ws, void* Y, int dtype, int type, int
   switch (type) {
     case T_Q4_0: return moe16_fmt<MQ4_0>(W, ws, Y, dtype, N, K, num_sorted, moe, s);
     case T_Q8_0: return moe16_fmt<MQ8_0>(W, ws, Y, dtype, N, K, num_sorted, moe, s);
+    case T_Q3_K: return moe16_fmt<MQ3_K>(W, ws, Y, dtype, N, K, num_sorted, moe, s);
+    case T_Q6_K: return moe16_fmt<MQ6_K>(W, ws, Y, dtype, N, K, num_sorted, moe, s);
     case T_Q4_K: return moe16_fmt<MQ4_K>(W, ws, Y, dtype, N, K, num_sorted, moe, s);
     case T_Q5_K: return moe16_fmt<MQ5_K>(W, ws, Y, dtype, N, K, num_sorted, moe, s);
     case T_IQ4_XS: return moe16_fmt<MIQ4_XS>(W, ws, Y, dtype, N, K, num_sorted, moe, s);
