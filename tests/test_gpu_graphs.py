@@ -28,12 +28,13 @@ def _capture(fn):
     return graph, out
 
 
-@pytest.mark.parametrize("case", ["mmvq", "mmq_half", "mmq_half_split", "mmq_int8", "dequant_gemm", "moe_vec_grouped"])
+@pytest.mark.parametrize("case", ["mmvq", "mmq_half", "mmq_half_split", "mmq_int8", "mmq_int8_split", "mmq_16_rows", "dequant_gemm",
+                                  "moe_vec_grouped", "moe_vec_blocks_of_16"])
 def test_replays_match_eager(case):
     from vllm_gguf_plugin_prism_amd import ops
     rng = np.random.default_rng(abs(hash(case)) % 1000)
-    if case == "moe_vec_grouped":
-        e, t, top_k, n, k = 8, 16, 4, 256, 512
+    if case in ("moe_vec_grouped", "moe_vec_blocks_of_16"):
+        e, t, top_k, n, k = (8, 40, 4, 256, 512) if case == "moe_vec_grouped" else (16, 24, 4, 200, 1024)   # 20 / 6 pairs per expert
         w = _dev(np.stack([o.make_weights(rng, o.Q4_0, n, k) for _ in range(e)]))
         ids = _dev(np.stack([rng.choice(e, size=top_k, replace=False) for _ in range(t)]).astype(np.int32))
         xs = [torch.randn(t, k, dtype=torch.float16, device="cuda") for _ in range(3)]
@@ -42,6 +43,7 @@ def test_replays_match_eager(case):
     else:
         qtype, m, n, k = {"mmvq": (o.Q4_K, 1, 512, 1024), "mmq_half": (o.Q6_K, 96, 384, 1024),
                           "mmq_half_split": (o.Q4_K, 200, 250, 4096), "mmq_int8": (o.Q6_K, 96, 384, 1024),
+                          "mmq_int8_split": (o.Q4_K, 200, 250, 4096), "mmq_16_rows": (o.Q4_K, 12, 300, 4096),
                           "dequant_gemm": (o.IQ4_XS, 64, 256, 1024)}[case]
         w = _dev(o.make_weights(rng, qtype, n, k))
         xs = [torch.randn(m, k, dtype=torch.float16, device="cuda") for _ in range(3)]
@@ -51,7 +53,7 @@ def test_replays_match_eager(case):
         elif case == "dequant_gemm":
             fn = lambda: ops.ggml_dequant_gemm(w, x, qtype, n)
         else:
-            engine = "int8" if case == "mmq_int8" else "half"
+            engine = "half" if case.startswith("mmq_half") else "int8"
             fn = lambda: ops.ggml_mul_mat_a8(w, x, qtype, n, engine=engine)
     graph, out = _capture(fn)
     for xi in xs:
