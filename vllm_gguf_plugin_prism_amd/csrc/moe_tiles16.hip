@@ -1,15 +1,18 @@
-// The grouped MoE contraction for experts with few pairs: 16 sorted slots per block instead of 32.
+// 16-row tiles of the integer engine on v_mfma_i32_16x16x32_i8, for the two places where a 32-row tile is mostly
+// padding: the grouped MoE contraction for experts with few pairs (blocks of 16 sorted slots instead of 32), and the
+// plain tile GEMM with 9 to 32 rows of X.
 //
 // With about eight pairs per expert (64 tokens, top-8 of 64 experts) three quarters of a 32-row tile are padding,
 // and what the integer engine pays per tile -- the rescale of every MFMA result by its two block scales on the vector
-// ALU -- does not shrink with the padding.  This kernel contracts a block of 16 slots with v_mfma_i32_16x16x32_i8:
-// four results per lane and 16 x 16 tile instead of sixteen per 32 x 32, so the vector work per weight block halves
-// and the kernel's time is set by how fast the experts' weights stream in.  Arithmetic and semantics are those of
-// the 32-slot kernels (reference: csrc/gguf/moe.cuh:5-129; block dot products exact in int32, scales in fp32).
+// ALU -- does not shrink with the padding.  A 16 x 16 tile holds four results per lane instead of the sixteen of a
+// 32 x 32 one, so the vector work per weight block halves.  Arithmetic and semantics are those of the 32-row kernels
+// (reference: csrc/gguf/moe.cuh:5-129 and mmq.cuh:2-104; block dot products exact in int32, scales in fp32).  The
+// formats whose weight scale changes every 16 values (Q6_K, Q3_K) issue the K=32 instruction twice per block, each
+// time with the activations of the other half zeroed: gfx950 has no 16 x 16 x 16 int8 MFMA.
 //
-// Work split: a workgroup of NW waves owns (one block of 16 slots) x (32 NW output features) and walks K in steps of
-// 128 values; a wave owns 32 features = two 16 x 16 tiles.  The packed blocks of the weight rows are decoded once per
-// step into LDS (two buffers, one barrier per step); global loads run two steps ahead in registers.
+// Work split: a workgroup of NW waves owns 16 rows x (32 NW) output features and walks K in steps of 128 values; a
+// wave owns 32 features = two 16 x 16 tiles.  The packed blocks of the weight rows are decoded once per step into LDS
+// (two buffers, one barrier per step); global loads run two steps ahead in registers (one for Q6_K / Q3_K).
 #include "mmq_i_core.h"
 
 namespace gguf {
