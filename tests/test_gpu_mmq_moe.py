@@ -480,24 +480,25 @@ def test_mmq_nine_to_32_rows(qtype, dt):
 
 
 @pytest.mark.parametrize("dt", ["f32", "f16", "bf16"])
-def test_mmq_q4_k_up_to_16_rows_from_packed_blocks(dt):
-    """Q4_K with at most 16 rows of X builds its MFMA operands straight from the packed blocks, K split over the waves
+@pytest.mark.parametrize("qtype", [o.Q4_K, o.Q5_K])
+def test_mmq_q4_k_q5_k_up_to_16_rows_from_packed_blocks(qtype, dt):
+    """Q4_K and Q5_K with at most 16 rows of X build their MFMA operands straight from the packed blocks, K split over the waves
     of a workgroup: one super-block of K, a stretch that fills LDS (K = 4096), K beyond it (split over workgroups as
     well, and the same call without room for partial tiles), few columns (split down to a super-block per wave), the
     two-column-tile variant of wide outputs with a ragged last tile, a row slice of a wider weight tensor with bias
     into a column slice of a wider result, and a slice whose rows are not 16-byte aligned (which takes the staged
     kernel)."""
     ops = _ops()
-    rng = np.random.default_rng(1400)
+    rng = np.random.default_rng(1400 + qtype)
     from vllm_gguf_plugin_prism_amd import _lib
     lib = _lib.lib()
     tol = 1e-5 if dt == "f32" else (1e-3 if dt == "f16" else 8e-3)
     for m, n, k in [(9, 72, 256), (16, 200, 4096), (16, 40, 8192), (13, 96, 4096), (12, 10250, 512), (1, 33, 768)]:
-        w = o.make_weights(rng, o.Q4_K, n, k)
+        w = o.make_weights(rng, qtype, n, k)
         xd, xv = _x(rng, m, k, dt)
-        want = o.mul_mat_a8(w, xv, o.Q4_K, n, "mmq")
+        want = o.mul_mat_a8(w, xv, qtype, n, "mmq")
         if m > 8:
-            y = ops.ggml_mul_mat_a8(_dev(w), xd, o.Q4_K, n)
+            y = ops.ggml_mul_mat_a8(_dev(w), xd, qtype, n)
             assert o.rel_l2(y.float().cpu().numpy(), want) <= tol, (m, n, k)
         # through the engine entry point with the integer engine named (no GEMV route for few rows) and the minimum
         # workspace
@@ -505,22 +506,22 @@ def test_mmq_q4_k_up_to_16_rows_from_packed_blocks(dt):
         ws = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
         y2 = torch.empty((m, n), dtype=TORCH_DT[dt], device="cuda")
         rc = lib.gguf_mmq_engine(_dev(w).data_ptr(), xd.data_ptr(), {"f32": 0, "f16": 1, "bf16": 2}[dt], ws.data_ptr(), y2.data_ptr(),
-                                 int(o.Q4_K), n, k, m, 1, nbytes, torch.cuda.current_stream().cuda_stream)
+                                 int(qtype), n, k, m, 1, nbytes, torch.cuda.current_stream().cuda_stream)
         assert rc == 0
         assert o.rel_l2(y2.float().cpu().numpy(), want) <= tol, (m, n, k, "minimum workspace")
     # shard of a merged layer: rows 8 .. 8 + n of a taller tensor whose rows are 32 bytes longer than the blocks,
     # bias, result columns 5 .. 5 + n of a wider tensor
     m, n, k = 14, 150, 1024
-    row_bytes = k // 256 * 144
+    row_bytes = k // 256 * o.QUANT_SIZES[qtype][1]
     for pad, where in ((32, "aligned"), (2, "unaligned")):
         tall = rng.integers(0, 256, (n + 20, row_bytes + pad), dtype=np.uint8)
-        w = o.make_weights(rng, o.Q4_K, n, k)
+        w = o.make_weights(rng, qtype, n, k)
         tall[8:8 + n, :row_bytes] = w
         xd, xv = _x(rng, m, k, dt)
         bias = torch.from_numpy(rng.standard_normal(n).astype(np.float32)).to(TORCH_DT[dt]).cuda()
         wide = torch.full((m, n + 11), 7.0, dtype=TORCH_DT[dt], device="cuda")
-        ops.ggml_mul_mat_a8(_dev(tall)[8:8 + n, :row_bytes], xd, o.Q4_K, n, out=wide[:, 5:5 + n], bias=bias)
-        want = o.mul_mat_a8(w, xv, o.Q4_K, n, "mmq") + bias.float().cpu().numpy()
+        ops.ggml_mul_mat_a8(_dev(tall)[8:8 + n, :row_bytes], xd, qtype, n, out=wide[:, 5:5 + n], bias=bias)
+        want = o.mul_mat_a8(w, xv, qtype, n, "mmq") + bias.float().cpu().numpy()
         assert o.rel_l2(wide[:, 5:5 + n].float().cpu().numpy(), want) <= tol, where
         assert torch.all(wide[:, :5] == 7.0) and torch.all(wide[:, 5 + n:] == 7.0)
 

@@ -35,10 +35,10 @@ struct Direct16Args {
   float* partial;
 };
 
-template <typename T, int KSPL, int CT>
+template <typename T, int KSPL, int CT, bool Q5>
 __global__ __launch_bounds__(64 * KSPL, 4) void rows16_q4k_kernel(const uint8_t* __restrict__ W, const char* __restrict__ ws,
                                                                     T* __restrict__ Y, const T* __restrict__ bias, Direct16Args a) {
-  constexpr int NT = 64 * KSPL, N_T = 16 * CT, BS = 144;
+  constexpr int NT = 64 * KSPL, N_T = 16 * CT, BS = Q5 ? 176 : 144, QS = Q5 ? 48 : 16;   // block bytes, offset of qs
   constexpr int MAX_SB = kDirectMaxSb;
   extern __shared__ __align__(16) char smem[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -63,14 +63,17 @@ __global__ __launch_bounds__(64 * KSPL, 4) void rows16_q4k_kernel(const uint8_t*
 #pragma unroll
   for (int c = 0; c < CT; ++c)
     wrow[c] = W + (int64_t)min(n_base + 16 * c + lcol, a.N - 1) * a.w_pitch + (int64_t)sb0 * BS;
-  struct Blk { uint4 hdr; u4_d q[2]; };
+  // Q5_K: the fifth bits of values l and 32 + l .. 224 + l of the super-block are the bits of qh[l]; a piece covers
+  // l = 16 (g % 2) .. + 15 of its blocks, so the lane takes that half of qh (bit number = block number)
+  struct Blk { uint4 hdr; u4_d q[2]; u4_d qh; };
   auto fetch = [&](int sb, Blk (&b)[CT]) {
 #pragma unroll
     for (int c = 0; c < CT; ++c) {
       const uint8_t* p = wrow[c] + sb * BS;
       b[c].hdr = *(const uint4*)p;
+      if constexpr (Q5) b[c].qh = *(const u4_d*)(p + 16 + 16 * (lgrp & 1));
 #pragma unroll
-      for (int i = 0; i < 2; ++i) b[c].q[i] = *(const u4_d*)(p + 16 + 64 * i + 16 * lgrp);
+      for (int i = 0; i < 2; ++i) b[c].q[i] = *(const u4_d*)(p + QS + 64 * i + 16 * lgrp);
     }
   };
   // ---- activations of super-blocks [sb0, sb0 + nmine) -> LDS: xq[16][pitch] int8, xsc[nmine * 8][16] half2 (d8, s8).
@@ -144,7 +147,11 @@ __global__ __launch_bounds__(64 * KSPL, 4) void rows16_q4k_kernel(const uint8_t*
           const v4i_d zero = {0, 0, 0, 0};
           v4i_d bv;
 #pragma unroll
-          for (int e = 0; e < 4; ++e) bv[e] = (int)((h ? b[c].q[i][e] >> 4 : b[c].q[i][e]) & 0x0F0F0F0Fu);
+          for (int e = 0; e < 4; ++e) {
+            uint32_t v = (h ? b[c].q[i][e] >> 4 : b[c].q[i][e]) & 0x0F0F0F0Fu;
+            if constexpr (Q5) v |= ((b[c].qh[e] >> (4 * i + h + 2 * (lgrp >> 1))) & 0x01010101u) << 4;
+            bv[e] = (int)v;
+          }
 #pragma unroll
           for (int sel = 0; sel < 2; ++sel) {
             const int blkno = 4 * i + 2 * sel + h;
@@ -195,9 +202,9 @@ struct Direct16Plan {
   int ct, tiles, gsplits, per_wg;
   int64_t partial_bytes() const { return gsplits > 1 ? (int64_t)tiles * gsplits * (16 * 16 * ct * 4) : 0; }
 };
-static Direct16Plan direct16_plan(int N, int K, int64_t partial_bytes_available) {
+static Direct16Plan direct16_plan(int type, int N, int K, int64_t partial_bytes_available) {
   Direct16Plan p;
-  p.ct = (N + 31) / 32 >= 320 ? 2 : 1;
+  p.ct = type == T_Q4_K && (N + 31) / 32 >= 320 ? 2 : 1;   // (with Q5_K's fifth bits two column tiles do not fit the registers)
   p.tiles = (N + 16 * p.ct - 1) / (16 * p.ct);
   const int nsb = K / 256;
   p.gsplits = (nsb + kDirectMaxSb - 1) / kDirectMaxSb;
@@ -211,20 +218,23 @@ static Direct16Plan direct16_plan(int N, int K, int64_t partial_bytes_available)
   }
   return p;
 }
-int64_t rows16_direct_partial_bytes(int N, int K) { return K % 256 ? 0 : direct16_plan(N, K, INT64_MAX).partial_bytes(); }
+int64_t rows16_direct_partial_bytes(int N, int K) {   // (the format is not known where the workspace is sized)
+  if (K % 256) return 0;
+  return std::max(direct16_plan(T_Q4_K, N, K, INT64_MAX).partial_bytes(), direct16_plan(T_Q5_K, N, K, INT64_MAX).partial_bytes());
+}
 
-template <typename T, int CT>
+template <typename T, int CT, bool Q5>
 static int rows16_q4k_launch(const void* W, const void* ws, void* Y, int M, int N, int K, float* partial, const Direct16Plan& p,
                              hipStream_t stream, const LinearArgs& la) {
   constexpr int KSPL = kDirectKspl, N_T = 16 * CT;
   const size_t act = (size_t)16 * (p.per_wg * 256 + 16) + (size_t)p.per_wg * 8 * 16 * 4, red = (size_t)KSPL * 16 * N_T * 4;
   const size_t lds = act > red ? act : red;
-  auto kern = rows16_q4k_kernel<T, KSPL, CT>;
+  auto kern = rows16_q4k_kernel<T, KSPL, CT, Q5>;
   if (lds > 65536) {
     static std::atomic<uint64_t> done{0};
     allow_large_lds(kern, 80 * 1024, done);
   }
-  Direct16Args a = {M, N, K, (int)q8_kp(K), p.gsplits, p.per_wg, q8_row_bytes(K), la.w_pitch ? la.w_pitch : (int64_t)(K / 256) * 144,
+  Direct16Args a = {M, N, K, (int)q8_kp(K), p.gsplits, p.per_wg, q8_row_bytes(K), la.w_pitch ? la.w_pitch : (int64_t)(K / 256) * (Q5 ? 176 : 144),
                     la.ldy ? la.ldy : (int64_t)N, partial};
   hipLaunchKernelGGL(kern, dim3(p.tiles * p.gsplits), dim3(64 * KSPL), lds, stream, (const uint8_t*)W, (const char*)ws, (T*)Y,
                      (const T*)la.bias, a);
@@ -234,22 +244,32 @@ static int rows16_q4k_launch(const void* W, const void* ws, void* Y, int M, int 
   return launch_status();
 }
 
-template <typename T>
+template <typename T, bool Q5>
 static int rows16_q4k_typed(const void* W, const void* ws, void* Y, int M, int N, int K, float* partial, const Direct16Plan& p,
                             hipStream_t stream, const LinearArgs& la) {
-  if (p.ct == 2) return rows16_q4k_launch<T, 2>(W, ws, Y, M, N, K, partial, p, stream, la);
-  return rows16_q4k_launch<T, 1>(W, ws, Y, M, N, K, partial, p, stream, la);
+  if constexpr (!Q5)
+    if (p.ct == 2) return rows16_q4k_launch<T, 2, Q5>(W, ws, Y, M, N, K, partial, p, stream, la);
+  return rows16_q4k_launch<T, 1, Q5>(W, ws, Y, M, N, K, partial, p, stream, la);
 }
 
-// Q4_K, at most 16 rows of X, W and its row pitch 16-byte aligned; GGUF_NOT_TAKEN otherwise.
+// Whether rows16_direct() would run this call.
+bool rows16_direct_takes(const void* W, int64_t w_pitch, int type, int M, int N, int K, int64_t partial_bytes) {
+  if ((type != T_Q4_K && type != T_Q5_K) || M > 16 || K % 256) return false;
+  const int64_t pitch = w_pitch ? w_pitch : (int64_t)(K / 256) * (type == T_Q5_K ? 176 : 144);
+  if (((uintptr_t)W & 15) || (pitch & 15)) return false;
+  return direct16_plan(type, N, K, partial_bytes).gsplits != 0;
+}
+
+// Q4_K or Q5_K, at most 16 rows of X, W and its row pitch 16-byte aligned; GGUF_NOT_TAKEN otherwise.
 int rows16_direct(const void* W, const void* ws, void* Y, int dtype, int type, int M, int N, int K, float* partial, int64_t partial_bytes,
                   hipStream_t s, const LinearArgs& la) {
-  if (type != T_Q4_K || M > 16 || K % 256) return GGUF_NOT_TAKEN;
-  const int64_t pitch = la.w_pitch ? la.w_pitch : (int64_t)(K / 256) * 144;
-  if (((uintptr_t)W & 15) || (pitch & 15)) return GGUF_NOT_TAKEN;
-  const Direct16Plan p = direct16_plan(N, K, partial_bytes);
-  if (p.gsplits == 0) return GGUF_NOT_TAKEN;
-  GGUF_DISPATCH_DTYPE(dtype, return (rows16_q4k_typed<scalar_t>(W, ws, Y, M, N, K, partial, p, s, la)));
+  if (!rows16_direct_takes(W, la.w_pitch, type, M, N, K, partial_bytes)) return GGUF_NOT_TAKEN;
+  const Direct16Plan p = direct16_plan(type, N, K, partial_bytes);
+  if (type == T_Q5_K) {
+    GGUF_DISPATCH_DTYPE(dtype, return (rows16_q4k_typed<scalar_t, true>(W, ws, Y, M, N, K, partial, p, s, la)));
+    return GGUF_ERR_DTYPE;
+  }
+  GGUF_DISPATCH_DTYPE(dtype, return (rows16_q4k_typed<scalar_t, false>(W, ws, Y, M, N, K, partial, p, s, la)));
   return GGUF_ERR_DTYPE;
 }
 
