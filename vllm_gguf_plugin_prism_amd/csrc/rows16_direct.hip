@@ -17,6 +17,10 @@
 // nothing overlaps that traffic: the kernel that did so spent 13 of its 17 us outside the weight stream (Q4_K
 // [14336,4096], 16 rows).  Workgroups split K between them only when the stretch does not fit LDS (K > 4096) or the
 // output has too few column groups to fill the chip.
+// More than 16 rows as further passes of 16 over the weights a wave holds were measured and lose to the staged tiles:
+// every pass repeats the rescaling, which is what the kernel spends its arithmetic on ([14336,4096] at 32 rows 37
+// against 32 us, at 64 rows 60 against 37 us).  One workgroup per CU instead of two, so that the rounds of workgroups
+// overlap each other's phases, is slower too (19.5 against 16.8 us).
 // Arithmetic as in the other integer tile kernels (mmq.cuh:2-104, vecdotq.cuh:353-379: exact int32 block sums,
 // `d*sc*d8*S - dmin*m*s8` with the stored block sums s8).
 #include "mmq_i_core.h"
