@@ -29,12 +29,14 @@ def _capture(fn):
 
 
 @pytest.mark.parametrize("case", ["mmvq", "mmq_half", "mmq_half_split", "mmq_int8", "mmq_int8_split", "mmq_16_rows", "dequant_gemm",
-                                  "moe_vec_grouped", "moe_vec_blocks_of_16"])
+                                  "moe_vec_grouped", "moe_vec_blocks_of_16", "moe_vec_few_pairs"])
 def test_replays_match_eager(case):
     from vllm_gguf_plugin_prism_amd import ops
     rng = np.random.default_rng(abs(hash(case)) % 1000)
-    if case in ("moe_vec_grouped", "moe_vec_blocks_of_16"):
-        e, t, top_k, n, k = (8, 40, 4, 256, 512) if case == "moe_vec_grouped" else (16, 24, 4, 200, 1024)   # 20 / 6 pairs per expert
+    if case.startswith("moe_vec"):
+        # 20 / 6 / 0.25 pairs per expert: blocks of 32 slots, of 16, every pair on its own
+        e, t, top_k, n, k = {"moe_vec_grouped": (8, 40, 4, 256, 512), "moe_vec_blocks_of_16": (16, 24, 4, 200, 1024),
+                             "moe_vec_few_pairs": (32, 2, 4, 200, 1024)}[case]
         w = _dev(np.stack([o.make_weights(rng, o.Q4_0, n, k) for _ in range(e)]))
         ids = _dev(np.stack([rng.choice(e, size=top_k, replace=False) for _ in range(t)]).astype(np.int32))
         xs = [torch.randn(t, k, dtype=torch.float16, device="cuda") for _ in range(3)]

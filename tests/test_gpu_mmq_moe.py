@@ -427,6 +427,39 @@ def test_moe_vec_grouped_and_per_pair_grids(qtype, t, top_k, e):
     assert o.rel_l2(y.cpu().numpy(), o.moe_a8_vec(xv, w, ids, top_k, qtype, n, t)) <= 1e-5
 
 
+@pytest.mark.parametrize("dt", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("qtype", [o.Q4_0, o.Q8_0, o.Q4_K, o.Q6_K, o.IQ4_XS, o.IQ2_XXS])
+def test_moe_vec_few_pairs_stream_each_expert(qtype, dt):
+    """With fewer than two pairs per expert every pair walks its expert's matrix on the streaming GEMV kernel, which
+    quantizes the pair's token itself: rows that are whole 2048-value spans (the staged loads of Q4_K) and shorter
+    ones, an output that does not divide into the workgroups' bands, the gated activation of the layer's second GEMM
+    folded into the quantisation, and an expert id outside the table (left out, the others unaffected)."""
+    ops = _ops()
+    rng = np.random.default_rng(1500 + qtype)
+    tol = {"f32": 1e-5, "f16": 1e-3, "bf16": 8e-3}[dt]
+    for t, top_k, e, n, k in [(1, 8, 64, 200, 2048), (3, 2, 8, 77, 512), (5, 1, 16, 300, 1024)]:
+        w = np.stack([o.make_weights(rng, qtype, n, k) for _ in range(e)])
+        xd, xv = _x(rng, t, k, dt)
+        ids, _ = _routing(rng, t, e, top_k)
+        assert t * top_k < 2 * e
+        y = ops.ggml_moe_a8_vec(xd, _dev(w), _dev(ids), top_k, qtype, n, t)
+        want = o.moe_a8_vec(xv, w, ids, top_k, qtype, n, t)
+        assert o.rel_l2(y.float().cpu().numpy(), want) <= tol, (o.TYPE_NAMES[qtype], t, e, k)
+        bad = ids.copy()
+        bad[0, 0] = e + 2
+        y2 = ops.ggml_moe_a8_vec(xd, _dev(w), _dev(bad), top_k, qtype, n, t)
+        assert torch.equal(y2[1:], y[1:])
+        # second GEMM of a layer: rows [gate | up] per pair, act(gate) * up quantized inside the kernel
+        pairs = t * top_k
+        h = (torch.randn(pairs, 2 * k, device="cuda") * 2).to(TORCH_DT[dt])
+        sep = (torch.nn.functional.silu(h[:, :k]) * h[:, k:]).contiguous()
+        flat = _dev(ids.reshape(pairs, 1))
+        got = ops.ggml_moe_a8_vec(h, _dev(w), flat, 1, qtype, n, pairs, activation="silu")
+        ref = o.moe_a8_vec(sep.float().cpu().numpy(), w, ids.reshape(pairs, 1), 1, qtype, n, pairs)
+        # (torch's and the kernel's exp may differ in the last bit of a few activations: a quant moves by one step at most)
+        assert o.rel_l2(got.float().cpu().numpy(), ref) <= max(tol, 5e-4), (o.TYPE_NAMES[qtype], "gated", t, e, k)
+
+
 @pytest.mark.parametrize("dt", ["f32", "f16"])
 @pytest.mark.parametrize("qtype", MMQ_TYPES)
 def test_moe_vec_shared_experts_keep_gemv_semantics(qtype, dt):

@@ -336,10 +336,12 @@ static inline StreamGeom stream_geom(int N, int K, int rows_per_wg, int64_t w_pi
   return g;
 }
 
-template <class F, int MT, int NW, int D, typename T, bool TILE = false, bool FULL = true, bool STAGED = false>
-__global__ __launch_bounds__(64 * NW) void mmvq_stream_kernel(const uint8_t* __restrict__ W, const T* __restrict__ X,
-                                                               T* __restrict__ Y, const T* __restrict__ bias, int64_t ldy,
-                                                               StreamGeom geom) {
+// GATED (one activation row only): the row of X is [gate | up], K values each, and what is quantized is
+// T(T(act(gate)) * up), the values a separate act-and-multiply kernel would have stored (fused_moe.py:44-51,80).
+template <class F, int MT, int NW, int D, typename T, bool TILE, bool FULL, bool STAGED, bool GATED>
+__device__ __forceinline__ void mmvq_stream_body(const uint8_t* __restrict__ W, const T* __restrict__ X, T* __restrict__ Y,
+                                                 const T* __restrict__ bias, int64_t ldy, const StreamGeom& geom, int act_fn) {
+  static_assert(!GATED || MT == 1, "the gated variant quantizes one row");
   extern __shared__ __align__(16) char smem[];
   const int tid = threadIdx.x, lane = tid & 63;
   const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);  // wave-uniform: row arithmetic stays on the scalar unit
@@ -401,11 +403,16 @@ __global__ __launch_bounds__(64 * NW) void mmvq_stream_kernel(const uint8_t* __r
   const int qtotal = rows_x * g8;  // a multiple of 4, so quads stay whole
   std::conditional_t<STAGED, SpanRegs<STAGED ? SPAN : 1040>, typename F::Regs> pre[D];
   const auto row_of_group = [&](int qc) { return MT == 1 ? 0 : (int)__umulhi((unsigned)qc, geom.g8_inv); };  // qc / g8
-  auto quantize_group = [&](const raw8<T>& raw, int q) {
+  auto quantize_group = [&](const raw8<T>& raw, const raw8<T>& up, int q) {
     const int qc = min(q, qtotal - 1);
     const int m = row_of_group(qc), j = qc - m * g8;
     float xv[8];
     raw.cvt(xv);
+    if constexpr (GATED) {
+      float uv[8];
+      up.cvt(uv);
+      gate8<T>(xv, uv, act_fn);
+    }
     const Q8Quad qq = q8_1_quantize8(xv);
     if (q < qtotal) {
       *(uint2*)(lq + (size_t)m * K + 8 * j) = qq.q;
@@ -428,12 +435,13 @@ __global__ __launch_bounds__(64 * NW) void mmvq_stream_kernel(const uint8_t* __r
       GGUF_PHASE(7);
       return;
     }
-    raw8<T> xraw[QG > 0 ? QG : 1];
+    raw8<T> xraw[QG > 0 ? QG : 1], xup[GATED && QG > 0 ? QG : 1];
 #pragma unroll
     for (int g = 0; g < QG; ++g) {
       const int qc = min(tid + g * NT, qtotal - 1);
       const int m = row_of_group(qc), j = qc - m * g8;
       xraw[g].load(X + (int64_t)m * K + 8 * j);
+      if constexpr (GATED) xup[g].load(X + K + 8 * j);
     }
     __builtin_amdgcn_sched_barrier(0);
     if constexpr (QG == 1) {
@@ -449,9 +457,12 @@ __global__ __launch_bounds__(64 * NW) void mmvq_stream_kernel(const uint8_t* __r
     __builtin_amdgcn_sched_barrier(0);
     GGUF_PHASE(7);                             // weight requests of the first rows are out
 #pragma unroll
-    for (int g = 0; g < QG; ++g) xraw[g].hold();   // (keeps the conversions below from moving above the weight requests)
+    for (int g = 0; g < QG; ++g) {   // (keeps the conversions below from moving above the weight requests)
+      xraw[g].hold();
+      if constexpr (GATED) xup[g].hold();
+    }
 #pragma unroll
-    for (int g = 0; g < QG; ++g) quantize_group(xraw[g], tid + g * NT);
+    for (int g = 0; g < QG; ++g) quantize_group(xraw[g], xup[GATED ? g : 0], tid + g * NT);
   };
   // (wave-uniform: a wave whose first lane is past the last group takes no part in the quantisation and reaches the
   // barrier as soon as its weight requests are out, instead of after a load and a quantisation nobody uses)
@@ -462,9 +473,10 @@ __global__ __launch_bounds__(64 * NW) void mmvq_stream_kernel(const uint8_t* __r
   for (int q = tid + 4 * NT; q - tid < qtotal; q += NT) {  // uniform trip count; only for K * MT > 32 * NT
     const int qc = min(q, qtotal - 1);
     const int m2 = row_of_group(qc), j2 = qc - m2 * g8;
-    raw8<T> r;
+    raw8<T> r, ru;
     r.load(X + (int64_t)m2 * K + 8 * j2);
-    quantize_group(r, q);
+    if constexpr (GATED) ru.load(X + K + 8 * j2);
+    quantize_group(r, GATED ? ru : r, q);
   }
   GGUF_PHASE(1);                               // own share of the activations quantized
   __syncthreads();
@@ -526,6 +538,33 @@ __global__ __launch_bounds__(64 * NW) void mmvq_stream_kernel(const uint8_t* __r
   GGUF_PHASE(4);                               // results stored
 }
 
+template <class F, int MT, int NW, int D, typename T, bool TILE = false, bool FULL = true, bool STAGED = false>
+__global__ __launch_bounds__(64 * NW) void mmvq_stream_kernel(const uint8_t* __restrict__ W, const T* __restrict__ X,
+                                                               T* __restrict__ Y, const T* __restrict__ bias, int64_t ldy,
+                                                               StreamGeom geom) {
+  mmvq_stream_body<F, MT, NW, D, T, TILE, FULL, STAGED, false>(W, X, Y, bias, ldy, geom, ACT_NONE);
+}
+
+// The per-pair MoE operator on the same kernel (reference: csrc/gguf/moe_vec.cuh:3-53): blockIdx.y is the flat
+// (token, k) pair z; its expert topk_ids[z] picks the weight matrix (experts densely packed), its token z / top_k the
+// activation row, and the result is row z of Y.  A pair whose expert id is outside [0, num_experts) (when the caller
+// says how many there are) names no weights and is left out.
+struct MoeStreamArgs {
+  const int32_t* topk_ids;
+  int64_t expert_bytes;   // between the matrices of two experts
+  int64_t x_pitch;        // elements between activation rows: K, or 2 K for [gate | up] rows
+  int top_k, num_experts, act;
+};
+template <class F, int NW, int D, typename T, bool STAGED, bool GATED>
+__global__ __launch_bounds__(64 * NW) void mmvq_stream_moe_kernel(const uint8_t* __restrict__ W, const T* __restrict__ X,
+                                                                   T* __restrict__ Y, MoeStreamArgs moe, StreamGeom geom) {
+  const int z = blockIdx.y;
+  const int e = moe.topk_ids[z];
+  if (moe.num_experts > 0 && (e < 0 || e >= moe.num_experts)) return;
+  mmvq_stream_body<F, 1, NW, D, T, false, true, STAGED, GATED>(W + (int64_t)e * moe.expert_bytes, X + (int64_t)(z / moe.top_k) * moe.x_pitch,
+                                                               Y + (int64_t)z * geom.N, nullptr, (int64_t)geom.N, geom, moe.act);
+}
+
 template <class F, int MT, int D, typename T, bool TILE, bool FULL, int NW, bool STAGED = false>
 static void launch_stream_d(const void* W, const T* X, T* Y, int N, int K, int rows_per_wg, int grid, size_t lds, const LinearArgs& la,
                             hipStream_t stream, int m_act) {
@@ -576,6 +615,46 @@ static bool launch_stream(const void* W, const T* X, T* Y, int N, int K, hipStre
   if constexpr (MT <= 2) go(std::true_type{});   // the callers of the 1- and 2-row tiles always fill them
   else if (m_act == MT) go(std::true_type{});
   else go(std::false_type{});
+  return true;
+}
+
+// The per-pair MoE operator on the streaming kernel: about one workgroup per CU in all, each walking a band of one
+// pair's expert matrix.  Returns false for shapes the streaming kernel does not take.
+template <class F, typename T, bool GATED>
+static bool launch_stream_moe(const void* W, const T* X, T* Y, int N, int K, const int32_t* topk_ids, int top_k, int pairs, int act,
+                              int num_experts, hipStream_t stream) {
+  constexpr int NW = MMVQ_NW;
+  const int nb = K / 32, S = (nb + 63) / 64;
+  if (S > NW || pairs > 65535) return false;
+  const int64_t pitch = (int64_t)(K / F::QK) * F::BS;
+  if (pitch > (int64_t)UINT32_MAX) return false;
+  const int slots = NW / S;
+  const int64_t target = num_cus();
+  int rows_per_wg = (int)(((int64_t)N * pairs + target - 1) / target);
+  if (rows_per_wg < slots) rows_per_wg = slots;
+  if (rows_per_wg > N) rows_per_wg = N;
+  const int grid = (N + rows_per_wg - 1) / rows_per_wg;
+  const size_t lds = (size_t)K + (size_t)nb * 4 * (F::AUX != AUX_NONE ? 2 : 1) + F::TABLE_BYTES + (size_t)rows_per_wg * S * 4 * 4;
+  if (lds > 160 * 1024) return false;
+  const int per_wave = (rows_per_wg + slots - 1) / slots;
+  const MoeStreamArgs moe = {topk_ids, (int64_t)N * pitch, (int64_t)K * (GATED ? 2 : 1), top_k, num_experts, act};
+  const StreamGeom geom = stream_geom(N, K, rows_per_wg, pitch, 1, NW);
+  const auto go = [&](auto kern, size_t bytes) {
+    if (bytes > 64 * 1024) {
+      static std::atomic<uint64_t> done{0};   // (one per kernel: the lambda's body is instantiated per argument type)
+      allow_large_lds(kern, 160 * 1024, done);
+    }
+    hipLaunchKernelGGL(kern, dim3(grid, pairs), dim3(64 * NW), bytes, stream, (const uint8_t*)W, X, Y, moe, geom);
+  };
+  if constexpr (SpanOf<F>::value > 0) {
+    const size_t lds_staged = lds + (size_t)NW * SpanOf<F>::value;
+    if (per_wave >= MMVQ_DEPTH && nb % 64 == 0 && pitch % 16 == 0 && (uintptr_t)W % 16 == 0 && lds_staged <= 160 * 1024) {
+      go(mmvq_stream_moe_kernel<F, NW, MMVQ_DEPTH, T, true, GATED>, lds_staged);
+      return true;
+    }
+  }
+  if (per_wave >= MMVQ_DEPTH) go(mmvq_stream_moe_kernel<F, NW, MMVQ_DEPTH, T, false, GATED>, lds);
+  else go(mmvq_stream_moe_kernel<F, NW, 1, T, false, GATED>, lds);
   return true;
 }
 
@@ -712,6 +791,10 @@ static int moe_vec_typed(const void* W, const char* x, void* Y, int xdtype, int 
                        MoeVecArgs{topk_ids, sorted, experts, top_k, pairs, (int)ACT_NONE}, (int64_t)(K / F::QK) * F::BS, (const T*)nullptr);
     return launch_status();
   }
+  // one workgroup row per pair: the streaming kernel where the shape fits it
+  if (act == ACT_NONE ? launch_stream_moe<F, T, false>(W, (const T*)x, (T*)Y, N, K, topk_ids, top_k, pairs, act, num_experts, stream)
+                      : launch_stream_moe<F, T, true>(W, (const T*)x, (T*)Y, N, K, topk_ids, top_k, pairs, act, num_experts, stream))
+    return launch_status();
   const int kchunk = kchunk_for(1, K);
   const size_t lds = mmvq_lds<F, 1>(kchunk);
   for (int z0 = 0; z0 < pairs; z0 += 65535) {

@@ -63,16 +63,21 @@ __device__ __forceinline__ void load8(const T* p, float (&v)[8]) {
 // separate act-and-multiply kernel would have stored in dtype T (the MoE layer applies it between its two GEMMs,
 // quantization/fused_moe.py:44-51,80).  act: 1 = SiLU, 2 = GELU (erf form).
 enum { ACT_NONE = 0, ACT_SILU = 1, ACT_GELU = 2 };
+// g <- T(T(act(g)) * u) for eight values already widened to fp32
 template <typename T>
-__device__ __forceinline__ void load8_gated(const T* gate, const T* up, int act, float (&v)[8]) {
-  float g[8], u[8];
-  load8<T>(gate, g);
-  load8<T>(up, u);
+__device__ __forceinline__ void gate8(float (&g)[8], const float (&u)[8], int act) {
 #pragma unroll
   for (int i = 0; i < 8; ++i) {
     const float a = act == ACT_SILU ? g[i] / (1.0f + expf(-g[i])) : g[i] * 0.5f * (1.0f + erff(g[i] * 0.70710678118654752440f));
-    v[i] = to_f32<T>(from_f32<T>(to_f32<T>(from_f32<T>(a)) * u[i]));  // T x T products are exact in fp32, so one rounding each
+    g[i] = to_f32<T>(from_f32<T>(to_f32<T>(from_f32<T>(a)) * u[i]));  // T x T products are exact in fp32, so one rounding each
   }
+}
+template <typename T>
+__device__ __forceinline__ void load8_gated(const T* gate, const T* up, int act, float (&v)[8]) {
+  float u[8];
+  load8<T>(gate, v);
+  load8<T>(up, u);
+  gate8<T>(v, u, act);
 }
 
 template <int CTRL>
