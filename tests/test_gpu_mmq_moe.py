@@ -513,14 +513,14 @@ def test_mmq_nine_to_32_rows(qtype, dt):
 
 
 @pytest.mark.parametrize("dt", ["f32", "f16", "bf16"])
-@pytest.mark.parametrize("qtype", [o.Q4_K, o.Q5_K])
-def test_mmq_q4_k_q5_k_up_to_16_rows_from_packed_blocks(qtype, dt):
-    """Q4_K and Q5_K with at most 16 rows of X build their MFMA operands straight from the packed blocks, K split over the waves
+@pytest.mark.parametrize("qtype", [o.Q4_K, o.Q5_K, o.Q6_K])
+def test_mmq_k_quants_up_to_16_rows_from_packed_blocks(qtype, dt):
+    """Q4_K, Q5_K and Q6_K with at most 16 rows of X build their MFMA operands straight from the packed blocks, K split over the waves
     of a workgroup: one super-block of K, a stretch that fills LDS (K = 4096), K beyond it (split over workgroups as
     well, and the same call without room for partial tiles), few columns (split down to a super-block per wave), the
     two-column-tile variant of wide outputs with a ragged last tile, a row slice of a wider weight tensor with bias
-    into a column slice of a wider result, and a slice whose rows are not 16-byte aligned (which takes the staged
-    kernel)."""
+    into a column slice of a wider result, and a slice whose rows are not 16-byte aligned (Q4_K / Q5_K take the staged
+    kernel there, Q6_K blocks are at even addresses anyway)."""
     ops = _ops()
     rng = np.random.default_rng(1400 + qtype)
     from vllm_gguf_plugin_prism_amd import _lib

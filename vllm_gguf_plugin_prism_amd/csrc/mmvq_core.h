@@ -659,7 +659,6 @@ static bool launch_stream_moe(const void* W, const T* X, T* Y, int N, int K, con
 }
 
 constexpr int MMVQ_RPW = 2;     // rows per wave of the workspace kernel
-constexpr int MAX_FUSED_M = 8;  // up to this many vectors are quantized inside the GEMV itself
 
 static inline int kchunk_for(int mt, int K) {
   int kchunk = mt == 1 ? 32768 : mt == 2 ? 16384 : mt == 4 ? 8192 : 4096;
@@ -685,51 +684,53 @@ static void launch_mt(const void* W, const char* xsrc, T* Y, int N, int K, hipSt
 }
 
 
+// Rows of X the streaming kernel takes in one launch.  Eight rows of activation registers spill for the formats whose
+// units carry the most scale data (measured on [14336,4096]: Q6_K 83 us at eight rows against 19 us at four, Q2_K 82
+// against 20, Q3_K 73 against 20): those take four rows per pass.
+template <class F> struct StreamRows { static constexpr int max = 8; };
+template <> struct StreamRows<FmtQ2_K> { static constexpr int max = 4; };
+template <> struct StreamRows<FmtQ3_K> { static constexpr int max = 4; };
+template <> struct StreamRows<FmtQ6_K> { static constexpr int max = 4; };
+
 template <class F, typename T>
 static int mmvq_typed(const void* W, const void* x, void* ws, void* Y, int xdtype, int64_t N, int64_t K, int64_t M,
                       hipStream_t stream, const LinearArgs& la) {
   const int64_t ldy = la.ldy ? la.ldy : N;
+  constexpr int MAXR = StreamRows<F>::max;
   if (la.tile_sums) {
     // the tile GEMM's arithmetic for a handful of rows; GGUF_NOT_TAKEN sends the caller back to its tile kernels
-    if (M > MAX_FUSED_M) return GGUF_NOT_TAKEN;
+    if (M > MAXR) return GGUF_NOT_TAKEN;
     const T* xs = (const T*)x;
-    bool ok;
+    bool ok = false;
     if constexpr (TileSums<F>::swaps) {
       if (M <= 4) ok = launch_stream<F, 4, T, true>(W, xs, (T*)Y, (int)N, (int)K, stream, la, (int)M);
-      else ok = launch_stream<F, 8, T, true>(W, xs, (T*)Y, (int)N, (int)K, stream, la, (int)M);
+      else if constexpr (MAXR == 8) ok = launch_stream<F, 8, T, true>(W, xs, (T*)Y, (int)N, (int)K, stream, la, (int)M);
     } else {  // the two operators agree on these formats: the GEMV's own kernels serve
       if (M == 1) ok = launch_stream<F, 1, T>(W, xs, (T*)Y, (int)N, (int)K, stream, la);
       else if (M == 2) ok = launch_stream<F, 2, T>(W, xs, (T*)Y, (int)N, (int)K, stream, la);
       else if (M <= 4) ok = launch_stream<F, 4, T>(W, xs, (T*)Y, (int)N, (int)K, stream, la, (int)M);
-      else ok = launch_stream<F, 8, T>(W, xs, (T*)Y, (int)N, (int)K, stream, la, (int)M);
+      else if constexpr (MAXR == 8) ok = launch_stream<F, 8, T>(W, xs, (T*)Y, (int)N, (int)K, stream, la, (int)M);
     }
     return ok ? launch_status() : GGUF_NOT_TAKEN;
   }
-  if (M <= MAX_FUSED_M) {
-    const T* xs = (const T*)x;
-    bool ok;
-    // A small matrix (a row fits two waves, at most 16 rows per CU) is over in a few microseconds, much of it the
-    // dispatch of the workgroups: half as many waves, each walking twice the rows, start and finish sooner.
-    if (M == 1 && K <= 4096 && N <= 16 * num_cus()) ok = launch_stream<F, 1, T, false, 8>(W, xs, (T*)Y, (int)N, (int)K, stream, la);
-    else if (M == 1) ok = launch_stream<F, 1, T>(W, xs, (T*)Y, (int)N, (int)K, stream, la);
-    else if (M == 2) ok = launch_stream<F, 2, T>(W, xs, (T*)Y, (int)N, (int)K, stream, la);
-    else if (M <= 4) ok = launch_stream<F, 4, T>(W, xs, (T*)Y, (int)N, (int)K, stream, la, (int)M);
-    else ok = launch_stream<F, 8, T>(W, xs, (T*)Y, (int)N, (int)K, stream, la, (int)M);
-    if (ok) return launch_status();
-  } else {
-    // More rows than a tile holds: eight at a time through the same kernel.  Each pass reads W again, as the workspace
-    // kernel below also does per eight rows, but at the streaming kernel's rate (Q4_K [14336,4096] at 16 rows: 42 us
-    // against 76 us).  If the first pass does not fit the kernel none has been launched and the workspace path runs.
+  {
+    // Up to MAXR rows are one launch.  More rows than a tile holds go MAXR at a time through the same kernel: each pass
+    // reads W again, as the workspace kernel below also does per eight rows, but at the streaming kernel's rate (Q4_K
+    // [14336,4096] at 16 rows: 42 us against 76 us).  If the first pass does not fit the kernel none has been launched
+    // and the workspace path runs.
     const T* xs = (const T*)x;
     bool ok = true;
-    for (int64_t m0 = 0; m0 < M && ok; m0 += 8) {
-      const int rows = (int)(M - m0 < 8 ? M - m0 : 8);
+    for (int64_t m0 = 0; m0 < M && ok; m0 += MAXR) {
+      const int rows = (int)(M - m0 < MAXR ? M - m0 : MAXR);
       const T* xm = xs + m0 * K;
       T* ym = (T*)Y + m0 * ldy;
-      if (rows > 4) ok = launch_stream<F, 8, T>(W, xm, ym, (int)N, (int)K, stream, la, rows);
-      else if (rows > 2) ok = launch_stream<F, 4, T>(W, xm, ym, (int)N, (int)K, stream, la, rows);
+      // A small matrix (a row fits two waves, at most 16 rows per CU) is over in a few microseconds, much of it the
+      // dispatch of the workgroups: half as many waves, each walking twice the rows, start and finish sooner.
+      if (M == 1 && K <= 4096 && N <= 16 * num_cus()) ok = launch_stream<F, 1, T, false, 8>(W, xm, ym, (int)N, (int)K, stream, la);
+      else if (rows == 1) ok = launch_stream<F, 1, T>(W, xm, ym, (int)N, (int)K, stream, la);
       else if (rows == 2) ok = launch_stream<F, 2, T>(W, xm, ym, (int)N, (int)K, stream, la);
-      else ok = launch_stream<F, 1, T>(W, xm, ym, (int)N, (int)K, stream, la);
+      else if (rows <= 4) ok = launch_stream<F, 4, T>(W, xm, ym, (int)N, (int)K, stream, la, rows);
+      else if constexpr (MAXR == 8) ok = launch_stream<F, 8, T>(W, xm, ym, (int)N, (int)K, stream, la, rows);
       if (!ok && m0 > 0) return GGUF_ERR_LAUNCH;   // cannot happen: a later pass needs no more than the first
     }
     if (ok) return launch_status();

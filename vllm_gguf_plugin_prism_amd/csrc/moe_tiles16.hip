@@ -318,7 +318,7 @@ int mmq_rows16(const void* W, const void* ws, void* Y, int dtype, int type, int 
   // the 16-deep formats pay two MFMAs and four vector instructions per result and block here as in the large tiles, and
   // with two 16-row tiles (17 .. 32 rows) the large tiles are as fast: Q6_K [14336,4096] 44 us either way
   if ((type == T_Q6_K || type == T_Q3_K) && M > 16) return GGUF_NOT_TAKEN;
-  {   // Q4_K with at most 16 rows: straight from the packed blocks
+  {   // Q4_K, Q5_K, Q6_K with at most 16 rows: straight from the packed blocks
     const int rc = rows16_direct(W, ws, Y, dtype, type, M, N, K, partial, partial_bytes, s, la);
     if (rc != GGUF_NOT_TAKEN) return rc;
   }

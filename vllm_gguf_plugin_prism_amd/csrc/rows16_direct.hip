@@ -1,15 +1,22 @@
-// The tile GEMM for up to 16 rows of X without LDS staging of the weights (Q4_K).
+// The tile GEMM for up to 16 rows of X without LDS staging of the weights (Q4_K, Q5_K, Q6_K).
 //
 // With at most 16 rows every weight is used by exactly one MFMA, so staging the decoded weights in LDS buys no reuse:
-// it only reshapes them into the MFMA operand layout, at the price of a barrier per step of K.  For Q4_K that layout
-// can be read straight from the packed block.  The 32 values of block kb of a super-block are the low (kb even) or
-// high (kb odd) nibbles of the 32 bytes qs[32 (kb / 2) ..], and the operand lane (column c, k group g) of a 64-deep
-// int8 MFMA supplies 16 values.  A lane fetches, per super-block and column, the 16-byte header and the two 16-byte
-// pieces qs[64 i + 16 g ..], i = 0, 1: the four lanes of a column read 64 contiguous bytes per load (8-byte pieces,
-// the layout of the 32-deep MFMA, stream at 60 % of that rate: 16 rows x 32 bytes per load instruction).  A piece
-// holds half a block in its low nibbles and half of the next block in its high nibbles; k groups 0, 1 of a column hold
-// one pair of blocks and groups 2, 3 the pair after it, so each MFMA runs with the activations of the other two groups
-// zeroed: eight MFMAs per super-block and column tile, one per block.  Only the activations go through LDS.
+// it only reshapes them into the MFMA operand layout, at the price of a barrier per step of K.  For these formats that
+// layout can be read straight from the packed block.  The operand lane (column c, k group g) of a 64-deep int8 MFMA
+// supplies 16 values.
+//   Q4_K: the 32 values of block kb of a super-block are the low (kb even) or high (kb odd) nibbles of the 32 bytes
+//   qs[32 (kb / 2) ..].  A lane fetches, per super-block and column, the 16-byte header and the two 16-byte pieces
+//   qs[64 i + 16 g ..], i = 0, 1: the four lanes of a column read 64 contiguous bytes per load (8-byte pieces, the
+//   layout of the 32-deep MFMA, stream at 60 % of that rate: 16 rows x 32 bytes per load instruction).  A piece holds
+//   half a block in its low nibbles and half of the next block in its high nibbles; k groups 0, 1 of a column hold one
+//   pair of blocks and groups 2, 3 the pair after it, so each MFMA runs with the activations of the other two groups
+//   zeroed: eight MFMAs per super-block and column tile, one per block.
+//   Q5_K: the same, with the 16 bytes of qh that hold the pieces' fifth bits.
+//   Q6_K: a scale covers 16 values, which is what one lane holds: four MFMAs per piece and nibble, each with the
+//   activations of one k group and zeros for the other three.  The 210-byte blocks sit at even addresses, so most of
+//   the 16-byte loads are unaligned, which costs about 30 % (measured with the blocks moved to 208-byte spacing);
+//   fetching whole dwords from the boundary below and funnel-shifting recovers 4 % of that and was not kept.
+// Only the activations go through LDS.
 //
 // K is split over the eight waves of a workgroup, not over workgroups: a workgroup owns 16 or 32 columns, each wave
 // takes up to two super-blocks, and the eight partial tiles are added through LDS in the order of K.  A split over
@@ -17,12 +24,16 @@
 // nothing overlaps that traffic: the kernel that did so spent 13 of its 17 us outside the weight stream (Q4_K
 // [14336,4096], 16 rows).  Workgroups split K between them only when the stretch does not fit LDS (K > 4096) or the
 // output has too few column groups to fill the chip.
+// With 32 columns a wave takes its two 16-column tiles in turn, the second requested as the registers of the first
+// become free: the staged activations serve both, the second tile's loads overlap the first's arithmetic, and the
+// kernel keeps the registers of one tile (both tiles held at once: Q4_K [14336,4096] 16.8 against 15.3 us; four tiles
+// in turn gain nothing over two).
 // More than 16 rows as further passes of 16 over the weights a wave holds were measured and lose to the staged tiles:
 // every pass repeats the rescaling, which is what the kernel spends its arithmetic on ([14336,4096] at 32 rows 37
 // against 32 us, at 64 rows 60 against 37 us).  One workgroup per CU instead of two, so that the rounds of workgroups
 // overlap each other's phases, is slower too (19.5 against 16.8 us).
-// Arithmetic as in the other integer tile kernels (mmq.cuh:2-104, vecdotq.cuh:353-379: exact int32 block sums,
-// `d*sc*d8*S - dmin*m*s8` with the stored block sums s8).
+// Arithmetic as in the other integer tile kernels (mmq.cuh:2-104, vecdotq.cuh:353-379, 467-491: exact int32 block
+// sums, `d*sc*d8*S - dmin*m*s8` with the stored block sums s8; Q6_K `d*sc*d8*S` per 16 values).
 #include "mmq_i_core.h"
 
 namespace gguf {
@@ -39,10 +50,16 @@ struct Direct16Args {
   float* partial;
 };
 
-template <typename T, int KSPL, int CT, bool Q5>
-__global__ __launch_bounds__(64 * KSPL, 4) void rows16_q4k_kernel(const uint8_t* __restrict__ W, const char* __restrict__ ws,
-                                                                    T* __restrict__ Y, const T* __restrict__ bias, Direct16Args a) {
-  constexpr int NT = 64 * KSPL, N_T = 16 * CT, BS = Q5 ? 176 : 144, QS = Q5 ? 48 : 16;   // block bytes, offset of qs
+enum { DIRECT_Q4_K = 0, DIRECT_Q5_K = 1, DIRECT_Q6_K = 2 };
+
+// NP: 16-column tiles a wave takes in turn (the workgroup owns 16 NP columns)
+template <typename T, int KSPL, int NP, int FMT>
+__global__ __launch_bounds__(64 * KSPL, 4) void rows16_direct_kernel(const uint8_t* __restrict__ W, const char* __restrict__ ws,
+                                                                      T* __restrict__ Y, const T* __restrict__ bias, Direct16Args a) {
+  constexpr bool Q5 = FMT == DIRECT_Q5_K, Q6 = FMT == DIRECT_Q6_K;
+  constexpr int NT = 64 * KSPL, N_T = 16 * NP;
+  constexpr int BS = Q6 ? 210 : Q5 ? 176 : 144, QS = Q5 ? 48 : 16;   // block bytes, offset of qs (Q4_K, Q5_K)
+  constexpr int XROWS = Q6 ? 17 : 16;                    // Q6_K: a row of zeros behind the 16 rows of X
   constexpr int MAX_SB = kDirectMaxSb;
   extern __shared__ __align__(16) char smem[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -52,34 +69,45 @@ __global__ __launch_bounds__(64 * KSPL, 4) void rows16_q4k_kernel(const uint8_t*
   const int tiles = (a.N + N_T - 1) / N_T;
   int wg = blockIdx.x;
   const int total8 = (tiles * a.gsplits) & ~7;
-  if (wg < total8) wg = (wg & 7) * (total8 >> 3) + (wg >> 3);
+  if (wg < total8) wg = (wg & 7) * (total8 >> 3) + (wg >> 3);   // each of the 8 XCDs gets a contiguous run of tiles
   const int tile = wg % tiles, gs = wg / tiles, n_base = tile * N_T;
   const int nsb = a.K >> 8;                               // super-blocks per row
   const int sb0 = gs * a.per_wg, nmine = min(nsb, sb0 + a.per_wg) - sb0;   // >= 1 (host)
   const int pw = (nmine + KSPL - 1) / KSPL;
   const int my0 = ks * pw, my1 = min(nmine, my0 + pw);    // this wave's super-blocks, relative to sb0
 
-  // ---- this wave's columns; its first two super-blocks are requested before anything else.  Per super-block and
-  // column a lane (column c, k group g) holds the header and two 16-byte pieces of qs, [64 i + 16 g, + 16) for i = 0, 1:
-  // the four lanes of a column read 64 contiguous bytes per load.  Piece i of lane g is half g % 2 of the byte pair
-  // row 2 i + g / 2, i.e. 16 values of block 4 i + 2 (g / 2) in the low nibbles and of the block after it in the high.
-  const uint8_t* wrow[CT];
+  // ---- this wave's columns, and what a lane holds of one super-block of one column
+  const uint8_t* wrow[NP];
 #pragma unroll
-  for (int c = 0; c < CT; ++c)
-    wrow[c] = W + (int64_t)min(n_base + 16 * c + lcol, a.N - 1) * a.w_pitch + (int64_t)sb0 * BS;
+  for (int q = 0; q < NP; ++q) wrow[q] = W + (int64_t)min(n_base + 16 * q + lcol, a.N - 1) * a.w_pitch + (int64_t)sb0 * BS;
+  // Q4_K: the header and the pieces qs[64 i + 16 g ..]: piece i of lane g is half g % 2 of the byte pair row
+  // 2 i + g / 2, i.e. 16 values of block 4 i + 2 (g / 2) in the low nibbles and of the block after it in the high.
   // Q5_K: the fifth bits of values l and 32 + l .. 224 + l of the super-block are the bits of qh[l]; a piece covers
-  // l = 16 (g % 2) .. + 15 of its blocks, so the lane takes that half of qh (bit number = block number)
-  struct Blk { uint4 hdr; u4_d q[2]; u4_d qh; };
-  auto fetch = [&](int sb, Blk (&b)[CT]) {
+  // l = 16 (g % 2) .. + 15 of its blocks, so the lane takes that half of qh (bit number = block number).
+  // Q6_K (loads of any alignment): per half n of the super-block a lane takes ql[64 n + 16 g ..] -- its low nibbles
+  // are the 16-value scale group 8 n + g, its high nibbles group 8 n + 4 + g -- the 16 bytes of qh that hold their
+  // upper two bits, and with all lanes of its column the 16 scales and d.
+  struct Blk4 { uint4 hdr; u4_d q[2]; u4_d qh; };
+  struct Blk6 { u4_d ql[2], qh[2], sc; uint32_t d; };
+  using Blk = std::conditional_t<Q6, Blk6, Blk4>;
+  auto fetch = [&](int q, int sb, Blk& b) {
+    const uint8_t* p = wrow[q] + sb * BS;
+    if constexpr (Q6) {
 #pragma unroll
-    for (int c = 0; c < CT; ++c) {
-      const uint8_t* p = wrow[c] + sb * BS;
-      b[c].hdr = *(const uint4*)p;
-      if constexpr (Q5) b[c].qh = *(const u4_d*)(p + 16 + 16 * (lgrp & 1));
+      for (int n = 0; n < 2; ++n) {
+        b.ql[n] = ld<u4_d>(p + 64 * n + 16 * lgrp);
+        b.qh[n] = ld<u4_d>(p + 128 + 32 * n + 16 * (lgrp & 1));
+      }
+      b.sc = ld<u4_d>(p + 192);
+      b.d = ld<uint16_t>(p + 208);
+    } else {
+      b.hdr = *(const uint4*)p;
+      if constexpr (Q5) b.qh = *(const u4_d*)(p + 16 + 16 * (lgrp & 1));
 #pragma unroll
-      for (int i = 0; i < 2; ++i) b[c].q[i] = *(const u4_d*)(p + QS + 64 * i + 16 * lgrp);
+      for (int i = 0; i < 2; ++i) b.q[i] = *(const u4_d*)(p + QS + 64 * i + 16 * lgrp);
     }
   };
+
   // ---- activations of super-blocks [sb0, sb0 + nmine) -> LDS: xq[16][pitch] int8, xsc[nmine * 8][16] half2 (d8, s8).
   // Requested before the weights: loads return in order, so the wait for the activations must not include the
   // weights.  Every thread issues every load (clamped to the last granule) so that the loads in flight can be counted.
@@ -87,7 +115,7 @@ __global__ __launch_bounds__(64 * KSPL, 4) void rows16_q4k_kernel(const uint8_t*
   constexpr int TPR = NT / 16, AI = 16 * MAX_SB / TPR, SI = 8 * MAX_SB / TPR;
   const int pitch = nmine * 256 + 16;
   int8_t* xq = (int8_t*)smem;
-  h2_d* xsc = (h2_d*)(smem + 16 * pitch);
+  h2_d* xsc = (h2_d*)(smem + XROWS * pitch);
   const int gpr = nmine * 16, spr = nmine * 8;             // 16-byte granules, blocks per row
   const int am = tid / TPR, at = tid % TPR;
   const char* const arow = ws + (int64_t)min(am, a.M - 1) * a.ws_row_bytes;
@@ -102,39 +130,72 @@ __global__ __launch_bounds__(64 * KSPL, 4) void rows16_q4k_kernel(const uint8_t*
     dreg[i] = asc[kb];
     sreg[i] = asc[a.Kp / 32 + kb];
   }
-  Blk cur[CT], nxt[CT];
-  fetch(min(my0, nmine - 1), cur);
-  fetch(min(my0 + 1, nmine - 1), nxt);
+  Blk cur, nxt;
+  fetch(0, min(my0, nmine - 1), cur);
+  fetch(0, min(my0 + 1, nmine - 1), nxt);
   // (threads past the end store the last piece once more: a guarded store would draw its load into the guard)
 #pragma unroll
   for (int i = 0; i < AI; ++i) *(u4_d*)(xq + am * pitch + 16 * min(at + TPR * i, gpr - 1)) = areg[i];
 #pragma unroll
   for (int i = 0; i < SI; ++i)   // both are half-precision values widened to fp32 by the quantizer: the narrowing is exact
     xsc[min(at + TPR * i, spr - 1) * 16 + am] = (h2_d){(_Float16)dreg[i], (_Float16)sreg[i]};
+  if constexpr (Q6)
+    for (int i = tid; i < gpr; i += NT) *(u4_d*)(xq + 16 * pitch + 16 * i) = (u4_d){0u, 0u, 0u, 0u};
 
-  float acc[CT][4];
+  float acc[NP][4];
 #pragma unroll
-  for (int c = 0; c < CT; ++c)
+  for (int q = 0; q < NP; ++q)
 #pragma unroll
-    for (int r = 0; r < 4; ++r) acc[c][r] = 0.0f;
+    for (int r = 0; r < 4; ++r) acc[q][r] = 0.0f;
   const v4i_d seed = {kSeedBits, kSeedBits, kSeedBits, kSeedBits};
   __syncthreads();
 
-  // One super-block of this wave's two column tiles.  An MFMA of 64 values takes 16 per lane: k groups 0, 1 of a
-  // piece hold one block and groups 2, 3 the block two further on, so each is contracted with the activations of the
-  // other pair of groups zeroed.
-  auto consume = [&](int s, const Blk (&b)[CT], bool valid) {
-    const int8_t* xrow = xq + lcol * pitch + s * 256 + 64 * (lgrp >> 1) + 16 * (lgrp & 1);
+  // One super-block of column tile q.  (A super-block past the wave's stretch was re-read: it is scaled to nothing.)
+  auto consume = [&](int q, int s, const Blk& b, bool valid) {
+    if constexpr (Q6) {
+      // the activations of k group t for the lanes of that group, the row of zeros for the others
+      const int8_t* xsel[4];
 #pragma unroll
-    for (int c = 0; c < CT; ++c) {   // (one column tile at a time: both tiles' scales at once do not fit the registers)
+      for (int t = 0; t < 4; ++t) xsel[t] = xq + (lgrp == t ? lcol : 16) * pitch + s * 256 + 16 * lgrp;
+      const float d = valid ? (float)__builtin_bit_cast(_Float16, (uint16_t)b.d) : 0.0f;
+#pragma unroll
+      for (int n = 0; n < 2; ++n)
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+          v4i_d bv;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            const uint32_t lo = (h ? b.ql[n][e] >> 4 : b.ql[n][e]) & 0x0F0F0F0Fu;
+            const uint32_t hi = (b.qh[n][e] >> (4 * h + 2 * (lgrp >> 1))) & 0x03030303u;
+            bv[e] = (int)sub_bytes(lo | (hi << 4), 0x20202020u);
+          }
+          const uint4 sc4 = *(const uint4*)(xsc + (s * 8 + 4 * n + 2 * h) * 16 + 4 * lgrp);       // block 4 n + 2 h
+          const uint4 sc5 = *(const uint4*)(xsc + (s * 8 + 4 * n + 2 * h + 1) * 16 + 4 * lgrp);   // and the next
+          const uint32_t d8w[2][4] = {{sc4.x, sc4.y, sc4.z, sc4.w}, {sc5.x, sc5.y, sc5.z, sc5.w}};
+#pragma unroll
+          for (int t = 0; t < 4; ++t) {
+            const int grp = 8 * n + 4 * h + t;             // 16 values 128 n + 64 h + 16 t .. of the super-block
+            const v4i_d av = *(const v4i_d*)(xsel[t] + 128 * n + 64 * h);
+            const v4i_d S = __builtin_amdgcn_mfma_i32_16x16x64_i8(av, bv, seed, 0, 0, 0);
+            const int sc = (int)(int8_t)((b.sc[grp >> 2] >> (8 * (grp & 3))) & 0xFF);
+            const float w = d * (float)sc, nsw = -kSeed * w;
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const h2_d hh = __builtin_bit_cast(h2_d, d8w[t >> 1][r]);
+              acc[q][r] = __builtin_fmaf(seeded_times(S[r], w, nsw), (float)hh[0], acc[q][r]);
+            }
+          }
+        }
+    } else {
+      const int8_t* xrow = xq + lcol * pitch + s * 256 + 64 * (lgrp >> 1) + 16 * (lgrp & 1);
       // 6-bit scales and mins of the 8 sub-blocks (dequantize.cuh:156-163), times d and dmin
       float dw[8], mw[8];
-      const uint32_t dm = valid ? b[c].hdr.x : 0u;       // a super-block past the stretch was re-read: scaled to nothing
+      const uint32_t dm = valid ? b.hdr.x : 0u;
       const float d = (float)__builtin_bit_cast(_Float16, (uint16_t)(dm & 0xFFFF));
       const float dmin = (float)__builtin_bit_cast(_Float16, (uint16_t)(dm >> 16));
       // the twelve scale bytes: sc, m of blocks 0..3 in the low six bits of bytes 0..3, 4..7; of blocks 4..7 the
       // low four bits in the nibbles of bytes 8..11 and the high two in the top bits of bytes 0..3, 4..7
-      const uint32_t s_lo = b[c].hdr.y, s_mid = b[c].hdr.z, s_hi = b[c].hdr.w;
+      const uint32_t s_lo = b.hdr.y, s_mid = b.hdr.z, s_hi = b.hdr.w;
       const uint32_t sc4[2] = {s_lo & 0x3F3F3F3Fu, (s_hi & 0x0F0F0F0Fu) | ((s_lo >> 2) & 0x30303030u)};
       const uint32_t mn4[2] = {s_mid & 0x3F3F3F3Fu, ((s_hi >> 4) & 0x0F0F0F0Fu) | ((s_mid >> 2) & 0x30303030u)};
 #pragma unroll
@@ -152,8 +213,8 @@ __global__ __launch_bounds__(64 * KSPL, 4) void rows16_q4k_kernel(const uint8_t*
           v4i_d bv;
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
-            uint32_t v = (h ? b[c].q[i][e] >> 4 : b[c].q[i][e]) & 0x0F0F0F0Fu;
-            if constexpr (Q5) v |= ((b[c].qh[e] >> (4 * i + h + 2 * (lgrp >> 1))) & 0x01010101u) << 4;
+            uint32_t v = (h ? b.q[i][e] >> 4 : b.q[i][e]) & 0x0F0F0F0Fu;
+            if constexpr (Q5) v |= ((b.qh[e] >> (4 * i + h + 2 * (lgrp >> 1))) & 0x01010101u) << 4;
             bv[e] = (int)v;
           }
 #pragma unroll
@@ -161,23 +222,38 @@ __global__ __launch_bounds__(64 * KSPL, 4) void rows16_q4k_kernel(const uint8_t*
             const int blkno = 4 * i + 2 * sel + h;
             const v4i_d asel = (lgrp >> 1) == sel ? av : zero;
             const v4i_d S = __builtin_amdgcn_mfma_i32_16x16x64_i8(asel, bv, seed, 0, 0, 0);
-            const uint4 sc4 = *(const uint4*)(xsc + (s * 8 + blkno) * 16 + 4 * lgrp);
-            const uint32_t scw[4] = {sc4.x, sc4.y, sc4.z, sc4.w};
+            const uint4 x4 = *(const uint4*)(xsc + (s * 8 + blkno) * 16 + 4 * lgrp);
+            const uint32_t scw[4] = {x4.x, x4.y, x4.z, x4.w};
             const float w = dw[blkno], nsw = -kSeed * w, nm = -mw[blkno];
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
               const h2_d hh = __builtin_bit_cast(h2_d, scw[r]);
-              acc[c][r] = __builtin_fmaf(seeded_times(S[r], w, nsw), (float)hh[0], acc[c][r]);
-              acc[c][r] = __builtin_fmaf((float)hh[1], nm, acc[c][r]);
+              acc[q][r] = __builtin_fmaf(seeded_times(S[r], w, nsw), (float)hh[0], acc[q][r]);
+              acc[q][r] = __builtin_fmaf((float)hh[1], nm, acc[q][r]);
             }
           }
         }
     }
   };
   static_assert(MAX_SB <= 2 * KSPL, "a wave holds at most two super-blocks");
-  // (both unconditionally: a load whose only use is guarded is moved into the guard, behind the barrier)
-  consume(min(my0, nmine - 1), cur, my0 < my1);
-  consume(min(my0 + 1, nmine - 1), nxt, my0 + 1 < my1);
+  // (both super-blocks unconditionally: a load whose only use is guarded is moved into the guard, behind the barrier)
+#pragma unroll
+  for (int q = 0; q < NP; ++q) {
+    // the next tile is requested as soon as a super-block's registers are free (the fences keep the compiler from
+    // starting those loads before that, which would need the registers of both tiles)
+    consume(q, min(my0, nmine - 1), cur, my0 < my1);
+    if (q + 1 < NP) {
+      __builtin_amdgcn_sched_barrier(0);
+      fetch(q + 1, min(my0, nmine - 1), cur);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+    consume(q, min(my0 + 1, nmine - 1), nxt, my0 + 1 < my1);
+    if (q + 1 < NP) {
+      __builtin_amdgcn_sched_barrier(0);
+      fetch(q + 1, min(my0 + 1, nmine - 1), nxt);
+      __builtin_amdgcn_sched_barrier(0);
+    }
+  }
 
   // ---- the KSPL partial tiles are added in the order of K
   __syncthreads();                                        // every wave is done with the activations
@@ -185,7 +261,7 @@ __global__ __launch_bounds__(64 * KSPL, 4) void rows16_q4k_kernel(const uint8_t*
 #pragma unroll
   for (int r = 0; r < 4; ++r)
 #pragma unroll
-    for (int c = 0; c < CT; ++c) red[(ks * 16 + 4 * lgrp + r) * N_T + 16 * c + lcol] = acc[c][r];
+    for (int q = 0; q < NP; ++q) red[(ks * 16 + 4 * lgrp + r) * N_T + 16 * q + lcol] = acc[q][r];
   __syncthreads();
   float* const mine = a.gsplits > 1 ? a.partial + ((int64_t)tile * a.gsplits + gs) * (16 * N_T) : nullptr;
   for (int e = tid; e < 16 * N_T; e += NT) {
@@ -198,18 +274,18 @@ __global__ __launch_bounds__(64 * KSPL, 4) void rows16_q4k_kernel(const uint8_t*
   }
 }
 
-// How a call is laid out.  One column tile per wave (16 columns per workgroup) until that gives 640 workgroups, two
-// above (measured on K = 4096 at 16 rows: N = 4096 8.9 against 13.5 us, N = 8192 11.3, N = 14336 16.8 against 17.5 us).
-// Workgroups split K between them when a stretch would not fit LDS (K > 4096), or down to one super-block per wave
-// when the output has fewer than 192 column groups.
+// How a call is laid out.  16 columns per workgroup until that gives 640 workgroups, 32 above (measured on Q4_K,
+// K = 4096 at 16 rows: N = 4096 8.9 against 13.5 us, N = 8192 11.3, N = 14336 15.3 against 17.5 us).  Workgroups split K
+// between them when a stretch would not fit LDS (K > 4096), or down to one super-block per wave when the output has
+// fewer than 192 column groups.
 struct Direct16Plan {
-  int ct, tiles, gsplits, per_wg;
-  int64_t partial_bytes() const { return gsplits > 1 ? (int64_t)tiles * gsplits * (16 * 16 * ct * 4) : 0; }
+  int np, tiles, gsplits, per_wg;   // np: 16-column tiles per workgroup
+  int64_t partial_bytes() const { return gsplits > 1 ? (int64_t)tiles * gsplits * (16 * 16 * np * 4) : 0; }
 };
-static Direct16Plan direct16_plan(int type, int N, int K, int64_t partial_bytes_available) {
+static Direct16Plan direct16_plan(int N, int K, int64_t partial_bytes_available) {
   Direct16Plan p;
-  p.ct = type == T_Q4_K && (N + 31) / 32 >= 320 ? 2 : 1;   // (with Q5_K's fifth bits two column tiles do not fit the registers)
-  p.tiles = (N + 16 * p.ct - 1) / (16 * p.ct);
+  p.np = (N + 31) / 32 >= 320 ? 2 : 1;
+  p.tiles = (N + 16 * p.np - 1) / (16 * p.np);
   const int nsb = K / 256;
   p.gsplits = (nsb + kDirectMaxSb - 1) / kDirectMaxSb;
   if (p.tiles * p.gsplits < 192) p.gsplits = std::max(p.gsplits, std::min(384 / p.tiles, nsb / kDirectKspl));
@@ -222,23 +298,23 @@ static Direct16Plan direct16_plan(int type, int N, int K, int64_t partial_bytes_
   }
   return p;
 }
-int64_t rows16_direct_partial_bytes(int N, int K) {   // (the format is not known where the workspace is sized)
-  if (K % 256) return 0;
-  return std::max(direct16_plan(T_Q4_K, N, K, INT64_MAX).partial_bytes(), direct16_plan(T_Q5_K, N, K, INT64_MAX).partial_bytes());
-}
+int64_t rows16_direct_partial_bytes(int N, int K) { return K % 256 ? 0 : direct16_plan(N, K, INT64_MAX).partial_bytes(); }
 
-template <typename T, int CT, bool Q5>
-static int rows16_q4k_launch(const void* W, const void* ws, void* Y, int M, int N, int K, float* partial, const Direct16Plan& p,
-                             hipStream_t stream, const LinearArgs& la) {
-  constexpr int KSPL = kDirectKspl, N_T = 16 * CT;
-  const size_t act = (size_t)16 * (p.per_wg * 256 + 16) + (size_t)p.per_wg * 8 * 16 * 4, red = (size_t)KSPL * 16 * N_T * 4;
+static inline int direct_block_bytes(int type) { return type == T_Q6_K ? 210 : type == T_Q5_K ? 176 : 144; }
+
+template <typename T, int NP, int FMT>
+static int rows16_direct_launch(const void* W, const void* ws, void* Y, int M, int N, int K, float* partial, const Direct16Plan& p,
+                                hipStream_t stream, const LinearArgs& la) {
+  constexpr int KSPL = kDirectKspl, N_T = 16 * NP, XROWS = FMT == DIRECT_Q6_K ? 17 : 16;
+  constexpr int BS = FMT == DIRECT_Q6_K ? 210 : FMT == DIRECT_Q5_K ? 176 : 144;
+  const size_t act = (size_t)XROWS * (p.per_wg * 256 + 16) + (size_t)p.per_wg * 8 * 16 * 4, red = (size_t)KSPL * 16 * N_T * 4;
   const size_t lds = act > red ? act : red;
-  auto kern = rows16_q4k_kernel<T, KSPL, CT, Q5>;
+  auto kern = rows16_direct_kernel<T, KSPL, NP, FMT>;
   if (lds > 65536) {
     static std::atomic<uint64_t> done{0};
     allow_large_lds(kern, 80 * 1024, done);
   }
-  Direct16Args a = {M, N, K, (int)q8_kp(K), p.gsplits, p.per_wg, q8_row_bytes(K), la.w_pitch ? la.w_pitch : (int64_t)(K / 256) * (Q5 ? 176 : 144),
+  Direct16Args a = {M, N, K, (int)q8_kp(K), p.gsplits, p.per_wg, q8_row_bytes(K), la.w_pitch ? la.w_pitch : (int64_t)(K / 256) * BS,
                     la.ldy ? la.ldy : (int64_t)N, partial};
   hipLaunchKernelGGL(kern, dim3(p.tiles * p.gsplits), dim3(64 * KSPL), lds, stream, (const uint8_t*)W, (const char*)ws, (T*)Y,
                      (const T*)la.bias, a);
@@ -248,32 +324,35 @@ static int rows16_q4k_launch(const void* W, const void* ws, void* Y, int M, int 
   return launch_status();
 }
 
-template <typename T, bool Q5>
-static int rows16_q4k_typed(const void* W, const void* ws, void* Y, int M, int N, int K, float* partial, const Direct16Plan& p,
-                            hipStream_t stream, const LinearArgs& la) {
-  if constexpr (!Q5)
-    if (p.ct == 2) return rows16_q4k_launch<T, 2, Q5>(W, ws, Y, M, N, K, partial, p, stream, la);
-  return rows16_q4k_launch<T, 1, Q5>(W, ws, Y, M, N, K, partial, p, stream, la);
+template <typename T, int FMT>
+static int rows16_direct_typed(const void* W, const void* ws, void* Y, int M, int N, int K, float* partial, const Direct16Plan& p,
+                               hipStream_t stream, const LinearArgs& la) {
+  if (p.np == 2) return rows16_direct_launch<T, 2, FMT>(W, ws, Y, M, N, K, partial, p, stream, la);
+  return rows16_direct_launch<T, 1, FMT>(W, ws, Y, M, N, K, partial, p, stream, la);
 }
 
 // Whether rows16_direct() would run this call.
 bool rows16_direct_takes(const void* W, int64_t w_pitch, int type, int M, int N, int K, int64_t partial_bytes) {
-  if ((type != T_Q4_K && type != T_Q5_K) || M > 16 || K % 256) return false;
-  const int64_t pitch = w_pitch ? w_pitch : (int64_t)(K / 256) * (type == T_Q5_K ? 176 : 144);
-  if (((uintptr_t)W & 15) || (pitch & 15)) return false;
-  return direct16_plan(type, N, K, partial_bytes).gsplits != 0;
+  if ((type != T_Q4_K && type != T_Q5_K && type != T_Q6_K) || M > 16 || K % 256) return false;
+  const int64_t pitch = w_pitch ? w_pitch : (int64_t)(K / 256) * direct_block_bytes(type);
+  if (type != T_Q6_K && (((uintptr_t)W & 15) || (pitch & 15))) return false;   // (Q6_K blocks are at even addresses anyway)
+  return direct16_plan(N, K, partial_bytes).gsplits != 0;
 }
 
-// Q4_K or Q5_K, at most 16 rows of X, W and its row pitch 16-byte aligned; GGUF_NOT_TAKEN otherwise.
+// Q4_K, Q5_K (W and its row pitch 16-byte aligned) or Q6_K, at most 16 rows of X; GGUF_NOT_TAKEN otherwise.
 int rows16_direct(const void* W, const void* ws, void* Y, int dtype, int type, int M, int N, int K, float* partial, int64_t partial_bytes,
                   hipStream_t s, const LinearArgs& la) {
   if (!rows16_direct_takes(W, la.w_pitch, type, M, N, K, partial_bytes)) return GGUF_NOT_TAKEN;
-  const Direct16Plan p = direct16_plan(type, N, K, partial_bytes);
-  if (type == T_Q5_K) {
-    GGUF_DISPATCH_DTYPE(dtype, return (rows16_q4k_typed<scalar_t, true>(W, ws, Y, M, N, K, partial, p, s, la)));
+  const Direct16Plan p = direct16_plan(N, K, partial_bytes);
+  if (type == T_Q6_K) {
+    GGUF_DISPATCH_DTYPE(dtype, return (rows16_direct_typed<scalar_t, DIRECT_Q6_K>(W, ws, Y, M, N, K, partial, p, s, la)));
     return GGUF_ERR_DTYPE;
   }
-  GGUF_DISPATCH_DTYPE(dtype, return (rows16_q4k_typed<scalar_t, false>(W, ws, Y, M, N, K, partial, p, s, la)));
+  if (type == T_Q5_K) {
+    GGUF_DISPATCH_DTYPE(dtype, return (rows16_direct_typed<scalar_t, DIRECT_Q5_K>(W, ws, Y, M, N, K, partial, p, s, la)));
+    return GGUF_ERR_DTYPE;
+  }
+  GGUF_DISPATCH_DTYPE(dtype, return (rows16_direct_typed<scalar_t, DIRECT_Q4_K>(W, ws, Y, M, N, K, partial, p, s, la)));
   return GGUF_ERR_DTYPE;
 }
 
