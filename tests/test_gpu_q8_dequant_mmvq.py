@@ -207,6 +207,37 @@ def test_config2_q4_k_full_size_batch_4_and_8(shape, m):
     assert o.rel_l2(y.float().cpu().numpy(), o.mul_mat_a8(w, xv, o.Q4_K, n, path)) <= 1e-3
 
 
+@pytest.mark.parametrize("dt", ["f32", "f16"])
+@pytest.mark.parametrize("qtype", [o.Q4_K, o.Q5_K, o.Q6_K])
+def test_mmvq_five_rows_or_more_of_a_large_matrix(qtype, dt):
+    """From five rows on, a K-quant matrix of at least 8M weights runs the GEMV operator on 16-row MFMA tiles read from
+    the packed blocks (16 rows per launch), with the GEMV's arithmetic: for Q4_K / Q5_K the offset term multiplies
+    d8 * sum(q8), not the stored block sum of the tile operator (the two differ by about 1e-2 on these weights).  A
+    matrix below that size and K beyond 4096 (no room for partial tiles in this operator's workspace) stay on the
+    streaming kernel; all must agree with the GEMV oracle."""
+    ops = _ops()
+    rng = np.random.default_rng(1600 + qtype)
+    tol = 1e-5 if dt == "f32" else 1e-3
+    for n, k, ms in [(2048, 4096, (5, 16, 21)), (1100, 8192, (6,)), (300, 1024, (7,))]:
+        w = o.make_weights(rng, qtype, n, k)
+        wd = _to_dev(w)
+        for m in ms:
+            xd, xv = _x(rng, m, k, dt)
+            y = ops.ggml_mul_mat_vec_a8(wd, xd, qtype, n)
+            want = o.mul_mat_a8(w, xv, qtype, n, "mmvq")
+            assert o.rel_l2(y.float().cpu().numpy(), want) <= tol, (o.TYPE_NAMES[qtype], n, k, m)
+    # with bias, into a column slice of a wider result
+    n, k, m = 2048, 4096, 9
+    w = o.make_weights(rng, qtype, n, k)
+    xd, xv = _x(rng, m, k, dt)
+    bias = torch.from_numpy(rng.standard_normal(n).astype(np.float32)).to(TORCH_DT[dt]).cuda()
+    wide = torch.full((m, n + 8), 3.0, dtype=TORCH_DT[dt], device="cuda")
+    ops.ggml_mul_mat_vec_a8(_to_dev(w), xd, qtype, n, out=wide[:, 8:], bias=bias)
+    want = o.mul_mat_a8(w, xv, qtype, n, "mmvq") + bias.float().cpu().numpy()
+    assert o.rel_l2(wide[:, 8:].float().cpu().numpy(), want) <= tol
+    assert torch.all(wide[:, :8] == 3.0)
+
+
 def test_empty_and_errors():
     ops = _ops()
     rng = np.random.default_rng(3)

@@ -310,7 +310,7 @@ static int dense16_fmt(const void* W, const void* ws, void* Y, int dtype, int M,
 }
 
 int rows16_direct(const void* W, const void* ws, void* Y, int dtype, int type, int M, int N, int K, float* partial, int64_t partial_bytes,
-                  hipStream_t s, const LinearArgs& la);   // rows16_direct.hip
+                  hipStream_t s, const LinearArgs& la, bool gemv_sums);   // rows16_direct.hip
 
 // q8_1(X) . W^T for a few rows of X (the quantized rows are in the workspace); GGUF_NOT_TAKEN for other formats.
 int mmq_rows16(const void* W, const void* ws, void* Y, int dtype, int type, int M, int N, int K, float* partial, int64_t partial_bytes,
@@ -319,7 +319,7 @@ int mmq_rows16(const void* W, const void* ws, void* Y, int dtype, int type, int 
   // with two 16-row tiles (17 .. 32 rows) the large tiles are as fast: Q6_K [14336,4096] 44 us either way
   if ((type == T_Q6_K || type == T_Q3_K) && M > 16) return GGUF_NOT_TAKEN;
   {   // Q4_K, Q5_K, Q6_K with at most 16 rows: straight from the packed blocks
-    const int rc = rows16_direct(W, ws, Y, dtype, type, M, N, K, partial, partial_bytes, s, la);
+    const int rc = rows16_direct(W, ws, Y, dtype, type, M, N, K, partial, partial_bytes, s, la, false);
     if (rc != GGUF_NOT_TAKEN) return rc;
   }
   switch (type) {

@@ -52,8 +52,9 @@ struct Direct16Args {
 
 enum { DIRECT_Q4_K = 0, DIRECT_Q5_K = 1, DIRECT_Q6_K = 2 };
 
-// NP: 16-column tiles a wave takes in turn (the workgroup owns 16 NP columns)
-template <typename T, int KSPL, int NP, int FMT>
+// NP: 16-column tiles a wave takes in turn (the workgroup owns 16 NP columns).  GSUM (Q4_K, Q5_K): the offset term
+// multiplies d8 * sum(q8), the GEMV operator's arithmetic (vecdotq.cuh:328-351), instead of the stored block sum.
+template <typename T, int KSPL, int NP, int FMT, bool GSUM>
 __global__ __launch_bounds__(64 * KSPL, 4) void rows16_direct_kernel(const uint8_t* __restrict__ W, const char* __restrict__ ws,
                                                                       T* __restrict__ Y, const T* __restrict__ bias, Direct16Args a) {
   constexpr bool Q5 = FMT == DIRECT_Q5_K, Q6 = FMT == DIRECT_Q6_K;
@@ -128,7 +129,7 @@ __global__ __launch_bounds__(64 * KSPL, 4) void rows16_direct_kernel(const uint8
   for (int i = 0; i < SI; ++i) {
     const int kb = min(at + TPR * i, spr - 1);
     dreg[i] = asc[kb];
-    sreg[i] = asc[a.Kp / 32 + kb];
+    sreg[i] = asc[(GSUM ? 2 : 1) * (a.Kp / 32) + kb];   // the stored sum s8, or du = d8 * sum(q8)
   }
   Blk cur, nxt;
   fetch(0, min(my0, nmine - 1), cur);
@@ -137,8 +138,13 @@ __global__ __launch_bounds__(64 * KSPL, 4) void rows16_direct_kernel(const uint8
 #pragma unroll
   for (int i = 0; i < AI; ++i) *(u4_d*)(xq + am * pitch + 16 * min(at + TPR * i, gpr - 1)) = areg[i];
 #pragma unroll
-  for (int i = 0; i < SI; ++i)   // both are half-precision values widened to fp32 by the quantizer: the narrowing is exact
-    xsc[min(at + TPR * i, spr - 1) * 16 + am] = (h2_d){(_Float16)dreg[i], (_Float16)sreg[i]};
+  for (int i = 0; i < SI; ++i) {
+    // d8 and s8 are half-precision values widened to fp32 by the quantizer: the narrowing is exact.  du is not one, but
+    // du / d8 = sum(q8) is an integer of at most 13 bits, exact as a quotient and as a half; the product is formed again
+    // where it is used.
+    const float second = GSUM ? (dreg[i] != 0.0f ? sreg[i] / dreg[i] : 0.0f) : sreg[i];
+    xsc[min(at + TPR * i, spr - 1) * 16 + am] = (h2_d){(_Float16)dreg[i], (_Float16)second};
+  }
   if constexpr (Q6)
     for (int i = tid; i < gpr; i += NT) *(u4_d*)(xq + 16 * pitch + 16 * i) = (u4_d){0u, 0u, 0u, 0u};
 
@@ -229,7 +235,8 @@ __global__ __launch_bounds__(64 * KSPL, 4) void rows16_direct_kernel(const uint8
             for (int r = 0; r < 4; ++r) {
               const h2_d hh = __builtin_bit_cast(h2_d, scw[r]);
               acc[q][r] = __builtin_fmaf(seeded_times(S[r], w, nsw), (float)hh[0], acc[q][r]);
-              acc[q][r] = __builtin_fmaf((float)hh[1], nm, acc[q][r]);
+              const float sx = GSUM ? (float)hh[0] * (float)hh[1] : (float)hh[1];
+              acc[q][r] = __builtin_fmaf(sx, nm, acc[q][r]);
             }
           }
         }
@@ -302,14 +309,14 @@ int64_t rows16_direct_partial_bytes(int N, int K) { return K % 256 ? 0 : direct1
 
 static inline int direct_block_bytes(int type) { return type == T_Q6_K ? 210 : type == T_Q5_K ? 176 : 144; }
 
-template <typename T, int NP, int FMT>
+template <typename T, int NP, int FMT, bool GSUM>
 static int rows16_direct_launch(const void* W, const void* ws, void* Y, int M, int N, int K, float* partial, const Direct16Plan& p,
                                 hipStream_t stream, const LinearArgs& la) {
   constexpr int KSPL = kDirectKspl, N_T = 16 * NP, XROWS = FMT == DIRECT_Q6_K ? 17 : 16;
   constexpr int BS = FMT == DIRECT_Q6_K ? 210 : FMT == DIRECT_Q5_K ? 176 : 144;
   const size_t act = (size_t)XROWS * (p.per_wg * 256 + 16) + (size_t)p.per_wg * 8 * 16 * 4, red = (size_t)KSPL * 16 * N_T * 4;
   const size_t lds = act > red ? act : red;
-  auto kern = rows16_direct_kernel<T, KSPL, NP, FMT>;
+  auto kern = rows16_direct_kernel<T, KSPL, NP, FMT, GSUM>;
   if (lds > 65536) {
     static std::atomic<uint64_t> done{0};
     allow_large_lds(kern, 80 * 1024, done);
@@ -326,9 +333,15 @@ static int rows16_direct_launch(const void* W, const void* ws, void* Y, int M, i
 
 template <typename T, int FMT>
 static int rows16_direct_typed(const void* W, const void* ws, void* Y, int M, int N, int K, float* partial, const Direct16Plan& p,
-                               hipStream_t stream, const LinearArgs& la) {
-  if (p.np == 2) return rows16_direct_launch<T, 2, FMT>(W, ws, Y, M, N, K, partial, p, stream, la);
-  return rows16_direct_launch<T, 1, FMT>(W, ws, Y, M, N, K, partial, p, stream, la);
+                               hipStream_t stream, const LinearArgs& la, bool gemv_sums) {
+  if constexpr (FMT != DIRECT_Q6_K) {   // (Q6_K has no offset term: the two operators agree)
+    if (gemv_sums) {
+      if (p.np == 2) return rows16_direct_launch<T, 2, FMT, true>(W, ws, Y, M, N, K, partial, p, stream, la);
+      return rows16_direct_launch<T, 1, FMT, true>(W, ws, Y, M, N, K, partial, p, stream, la);
+    }
+  }
+  if (p.np == 2) return rows16_direct_launch<T, 2, FMT, false>(W, ws, Y, M, N, K, partial, p, stream, la);
+  return rows16_direct_launch<T, 1, FMT, false>(W, ws, Y, M, N, K, partial, p, stream, la);
 }
 
 // Whether rows16_direct() would run this call.
@@ -340,19 +353,20 @@ bool rows16_direct_takes(const void* W, int64_t w_pitch, int type, int M, int N,
 }
 
 // Q4_K, Q5_K (W and its row pitch 16-byte aligned) or Q6_K, at most 16 rows of X; GGUF_NOT_TAKEN otherwise.
+// gemv_sums: the GEMV operator's offset term (see GSUM) instead of the tile operator's.
 int rows16_direct(const void* W, const void* ws, void* Y, int dtype, int type, int M, int N, int K, float* partial, int64_t partial_bytes,
-                  hipStream_t s, const LinearArgs& la) {
+                  hipStream_t s, const LinearArgs& la, bool gemv_sums) {
   if (!rows16_direct_takes(W, la.w_pitch, type, M, N, K, partial_bytes)) return GGUF_NOT_TAKEN;
   const Direct16Plan p = direct16_plan(N, K, partial_bytes);
   if (type == T_Q6_K) {
-    GGUF_DISPATCH_DTYPE(dtype, return (rows16_direct_typed<scalar_t, DIRECT_Q6_K>(W, ws, Y, M, N, K, partial, p, s, la)));
+    GGUF_DISPATCH_DTYPE(dtype, return (rows16_direct_typed<scalar_t, DIRECT_Q6_K>(W, ws, Y, M, N, K, partial, p, s, la, gemv_sums)));
     return GGUF_ERR_DTYPE;
   }
   if (type == T_Q5_K) {
-    GGUF_DISPATCH_DTYPE(dtype, return (rows16_direct_typed<scalar_t, DIRECT_Q5_K>(W, ws, Y, M, N, K, partial, p, s, la)));
+    GGUF_DISPATCH_DTYPE(dtype, return (rows16_direct_typed<scalar_t, DIRECT_Q5_K>(W, ws, Y, M, N, K, partial, p, s, la, gemv_sums)));
     return GGUF_ERR_DTYPE;
   }
-  GGUF_DISPATCH_DTYPE(dtype, return (rows16_direct_typed<scalar_t, DIRECT_Q4_K>(W, ws, Y, M, N, K, partial, p, s, la)));
+  GGUF_DISPATCH_DTYPE(dtype, return (rows16_direct_typed<scalar_t, DIRECT_Q4_K>(W, ws, Y, M, N, K, partial, p, s, la, gemv_sums)));
   return GGUF_ERR_DTYPE;
 }
 
