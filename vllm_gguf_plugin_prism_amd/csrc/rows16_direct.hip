@@ -140,9 +140,10 @@ __global__ __launch_bounds__(64 * KSPL, 4) void rows16_direct_kernel(const uint8
 #pragma unroll
   for (int i = 0; i < SI; ++i) {
     // d8 and s8 are half-precision values widened to fp32 by the quantizer: the narrowing is exact.  du is not one, but
-    // du / d8 = sum(q8) is an integer of at most 13 bits, exact as a quotient and as a half; the product is formed again
-    // where it is used.
-    const float second = GSUM ? (dreg[i] != 0.0f ? sreg[i] / dreg[i] : 0.0f) : sreg[i];
+    // du / d8 = sum(q8) is an integer of at most 13 bits, exact as a quotient and as a half; d8 multiplies it again
+    // together with the block sum.
+    // (the quotient is an integer below 4065 in magnitude: the hardware reciprocal's last-bit error rounds away)
+    const float second = GSUM ? (dreg[i] != 0.0f ? __builtin_rintf(sreg[i] * __builtin_amdgcn_rcpf(dreg[i])) : 0.0f) : sreg[i];
     xsc[min(at + TPR * i, spr - 1) * 16 + am] = (h2_d){(_Float16)dreg[i], (_Float16)second};
   }
   if constexpr (Q6)
@@ -234,9 +235,13 @@ __global__ __launch_bounds__(64 * KSPL, 4) void rows16_direct_kernel(const uint8
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
               const h2_d hh = __builtin_bit_cast(h2_d, scw[r]);
-              acc[q][r] = __builtin_fmaf(seeded_times(S[r], w, nsw), (float)hh[0], acc[q][r]);
-              const float sx = GSUM ? (float)hh[0] * (float)hh[1] : (float)hh[1];
-              acc[q][r] = __builtin_fmaf(sx, nm, acc[q][r]);
+              if constexpr (GSUM) {   // d8 * (S * dw - m * sum(q8)): the offset joins the block sum before d8 is applied
+                const float u = __builtin_fmaf((float)hh[1], nm, seeded_times(S[r], w, nsw));
+                acc[q][r] = __builtin_fmaf(u, (float)hh[0], acc[q][r]);
+              } else {
+                acc[q][r] = __builtin_fmaf(seeded_times(S[r], w, nsw), (float)hh[0], acc[q][r]);
+                acc[q][r] = __builtin_fmaf((float)hh[1], nm, acc[q][r]);
+              }
             }
           }
         }
