@@ -513,9 +513,9 @@ def test_mmq_nine_to_32_rows(qtype, dt):
 
 
 @pytest.mark.parametrize("dt", ["f32", "f16", "bf16"])
-@pytest.mark.parametrize("qtype", [o.Q4_K, o.Q5_K, o.Q6_K])
-def test_mmq_k_quants_up_to_16_rows_from_packed_blocks(qtype, dt):
-    """Q4_K, Q5_K and Q6_K with at most 16 rows of X build their MFMA operands straight from the packed blocks, K split over the waves
+@pytest.mark.parametrize("qtype", [o.Q4_K, o.Q5_K, o.Q6_K, o.Q4_0, o.Q8_0])
+def test_mmq_up_to_16_rows_from_packed_blocks(qtype, dt):
+    """Q4_K, Q5_K, Q6_K (and Q4_0, Q8_0 from nine rows on) with at most 16 rows of X build their MFMA operands straight from the packed blocks, K split over the waves
     of a workgroup: one super-block of K, a stretch that fills LDS (K = 4096), K beyond it (split over workgroups as
     well, and the same call without room for partial tiles), few columns (split down to a super-block per wave), the
     two-column-tile variant of wide outputs with a ragged last tile, a row slice of a wider weight tensor with bias
@@ -545,7 +545,7 @@ def test_mmq_k_quants_up_to_16_rows_from_packed_blocks(qtype, dt):
     # shard of a merged layer: rows 8 .. 8 + n of a taller tensor whose rows are 32 bytes longer than the blocks,
     # bias, result columns 5 .. 5 + n of a wider tensor
     m, n, k = 14, 150, 1024
-    row_bytes = k // 256 * o.QUANT_SIZES[qtype][1]
+    row_bytes = k // o.QUANT_SIZES[qtype][0] * o.QUANT_SIZES[qtype][1]
     for pad, where in ((32, "aligned"), (2, "unaligned")):
         tall = rng.integers(0, 256, (n + 20, row_bytes + pad), dtype=np.uint8)
         w = o.make_weights(rng, qtype, n, k)

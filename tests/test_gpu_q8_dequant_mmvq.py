@@ -208,10 +208,10 @@ def test_config2_q4_k_full_size_batch_4_and_8(shape, m):
 
 
 @pytest.mark.parametrize("dt", ["f32", "f16"])
-@pytest.mark.parametrize("qtype", [o.Q4_K, o.Q5_K, o.Q6_K])
+@pytest.mark.parametrize("qtype", [o.Q4_K, o.Q5_K, o.Q6_K, o.Q4_0, o.Q8_0])
 def test_mmvq_five_rows_or_more_of_a_large_matrix(qtype, dt):
-    """From five rows on, a K-quant matrix of at least 8M weights runs the GEMV operator on 16-row MFMA tiles read from
-    the packed blocks (16 rows per launch), with the GEMV's arithmetic: for Q4_K / Q5_K the offset term multiplies
+    """From five rows on (nine for Q4_0 / Q8_0), a matrix of at least 8M weights runs the GEMV operator on 16-row MFMA
+    tiles read from the packed blocks (16 rows per launch), with the GEMV's arithmetic: for Q4_K / Q5_K the offset term multiplies
     d8 * sum(q8), not the stored block sum of the tile operator (the two differ by about 1e-2 on these weights).  A
     matrix below that size and K beyond 4096 (no room for partial tiles in this operator's workspace) stay on the
     streaming kernel; all must agree with the GEMV oracle."""

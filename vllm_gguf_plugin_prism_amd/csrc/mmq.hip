@@ -618,6 +618,7 @@ int mmq_rows16(const void* W, const void* ws, void* Y, int dtype, int type, int 
 int64_t mmq_rows16_partial_bytes(int M, int N, int K);
 // rows16_direct.hip: whether a call with at most 16 rows runs the kernel that reads Q4_K from the packed blocks
 bool rows16_direct_takes(const void* W, int64_t w_pitch, int type, int M, int N, int K, int64_t partial_bytes);
+bool rows16_direct_pays(int type, int M, int64_t N, int64_t K, bool against_gemv);
 
 // mmq_i.hip
 int mmq_int(const void* W, const void* ws, void* Y, int dtype, int type, int M, int N, int K, float* partial,
@@ -673,11 +674,11 @@ int gguf::mmq_linear_impl(const void* W, int64_t w_row_pitch_bytes, const void* 
   if (!W || !x || !q8_workspace || !Y) return GGUF_ERR_NULL;
   if (((uintptr_t)W & 1) || (w_row_pitch_bytes & 1)) return GGUF_ERR_SHAPE;  // packed blocks sit at even addresses
   hipStream_t s = (hipStream_t)stream;
-  // (the 16-row tile kernel that reads Q4_K / Q5_K straight from the packed blocks takes the same time for 1 .. 16 rows
+  // (the 16-row tile kernel that reads the K-quants straight from the packed blocks takes the same time for 1 .. 16 rows
   // and passes the GEMV, which has one kernel for 5 .. 8 rows, there: Q4_K [14336,4096] 17 against 21 us at 6 rows,
-  // against 14 us at 4; below about 8M weights the GEMV's single launch wins, [1024,4096] 8 against 10 us)
+  // against 14 us at 4; see rows16_direct_pays)
   const int64_t partial_room = workspace_bytes - (rows_bytes < 0 ? mmq_rows_bytes(M, K) : rows_bytes);
-  const bool tiles_at_5 = M >= 5 && N * K >= (8 << 20) && rows16_direct_takes(W, w_row_pitch_bytes, type, (int)M, (int)N, (int)K, partial_room > 0 ? partial_room : 0);
+  const bool tiles_at_5 = M <= 16 && rows16_direct_pays(type, (int)M, N, K, true) && rows16_direct_takes(W, w_row_pitch_bytes, type, (int)M, (int)N, (int)K, partial_room > 0 ? partial_room : 0);
   if (engine == GGUF_MMQ_AUTO && M <= 8 && !tiles_at_5) {
     // a handful of rows: the streaming GEMV kernel with the tile kernels' offset sums reads W once at close to the
     // GEMV's rate and is exact in int8; it declines shapes it does not cover

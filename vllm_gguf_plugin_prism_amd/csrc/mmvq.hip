@@ -40,16 +40,17 @@ namespace gguf {
 // one GEMV call after validation; with la.tile_sums the result is GGUF_NOT_TAKEN where the streaming kernel does not apply
 // rows16_direct.hip: 16-row MFMA tiles read straight from the packed blocks (Q4_K, Q5_K, Q6_K)
 bool rows16_direct_takes(const void* W, int64_t w_pitch, int type, int M, int N, int K, int64_t partial_bytes);
+bool rows16_direct_pays(int type, int M, int64_t N, int64_t K, bool against_gemv);
 int rows16_direct(const void* W, const void* ws, void* Y, int dtype, int type, int M, int N, int K, float* partial, int64_t partial_bytes,
                   hipStream_t s, const LinearArgs& la, bool gemv_sums);
 
 int mmvq_any(int type, const void* W, const void* x, void* q8_workspace, void* Y, int xdtype, int64_t N, int64_t K, int64_t M,
              hipStream_t s, const LinearArgs& la) {
-  // Five rows or more of a matrix of at least 8M weights: the tile kernel's time does not grow with the rows (up to 16
-  // per launch), the streaming kernel's does (Q4_K [14336,4096] at 8 / 16 rows 22 / 42 us against 18 us, Q6_K 36 / 71
-  // against 27 us).  The operator's workspace holds the quantized rows and nothing else, so K up to 4096 (beyond that
+  // Five rows or more (nine for Q4_0 / Q8_0) of a matrix of at least 8M weights: the tile kernel's time does not grow
+  // with the rows (up to 16 per launch), the streaming kernel's does (Q4_K [14336,4096] at 8 / 16 rows 22 / 42 us
+  // against 17 us, Q6_K 36 / 71 against 27 us, Q4_0 at 16 rows 36 against 22 us).  The operator's workspace holds the quantized rows and nothing else, so K up to 4096 (beyond that
   // the tile kernel wants room for partial tiles).  The arithmetic stays the GEMV's (offset term on d8 * sum(q8)).
-  if (!la.tile_sums && M >= 5 && N * K >= (8 << 20) && N <= 0x7FFFFFF0LL && K <= 0x7FFFFFF0LL &&
+  if (!la.tile_sums && N <= 0x7FFFFFF0LL && K <= 0x7FFFFFF0LL && rows16_direct_pays(type, (int)(M < 16 ? M : 16), N, K, true) &&
       rows16_direct_takes(W, la.w_pitch, type, 16, (int)N, (int)K, 0)) {
     int rc = quantize_q8_1(x, xdtype, q8_workspace, M, K, s);
     if (rc != GGUF_OK) return rc;

@@ -311,6 +311,7 @@ static int dense16_fmt(const void* W, const void* ws, void* Y, int dtype, int M,
 
 int rows16_direct(const void* W, const void* ws, void* Y, int dtype, int type, int M, int N, int K, float* partial, int64_t partial_bytes,
                   hipStream_t s, const LinearArgs& la, bool gemv_sums);   // rows16_direct.hip
+bool rows16_direct_pays(int type, int M, int64_t N, int64_t K, bool against_gemv);
 
 // q8_1(X) . W^T for a few rows of X (the quantized rows are in the workspace); GGUF_NOT_TAKEN for other formats.
 int mmq_rows16(const void* W, const void* ws, void* Y, int dtype, int type, int M, int N, int K, float* partial, int64_t partial_bytes,
@@ -318,7 +319,7 @@ int mmq_rows16(const void* W, const void* ws, void* Y, int dtype, int type, int 
   // the 16-deep formats pay two MFMAs and four vector instructions per result and block here as in the large tiles, and
   // with two 16-row tiles (17 .. 32 rows) the large tiles are as fast: Q6_K [14336,4096] 44 us either way
   if ((type == T_Q6_K || type == T_Q3_K) && M > 16) return GGUF_NOT_TAKEN;
-  {   // Q4_K, Q5_K, Q6_K with at most 16 rows: straight from the packed blocks
+  if (rows16_direct_pays(type, M, N, K, false)) {   // at most 16 rows: straight from the packed blocks
     const int rc = rows16_direct(W, ws, Y, dtype, type, M, N, K, partial, partial_bytes, s, la, false);
     if (rc != GGUF_NOT_TAKEN) return rc;
   }

@@ -1,4 +1,4 @@
-// The tile GEMM for up to 16 rows of X without LDS staging of the weights (Q4_K, Q5_K, Q6_K).
+// The tile GEMM for up to 16 rows of X without LDS staging of the weights (Q4_K, Q5_K, Q6_K, Q4_0, Q8_0).
 //
 // With at most 16 rows every weight is used by exactly one MFMA, so staging the decoded weights in LDS buys no reuse:
 // it only reshapes them into the MFMA operand layout, at the price of a barrier per step of K.  For these formats that
@@ -16,6 +16,9 @@
 //   activations of one k group and zeros for the other three.  The 210-byte blocks sit at even addresses, so most of
 //   the 16-byte loads are unaligned, which costs about 30 % (measured with the blocks moved to 208-byte spacing);
 //   fetching whole dwords from the boundary below and funnel-shifting recovers 4 % of that and was not kept.
+//   Q4_0, Q8_0: a lane owns whole 32-value blocks (18 and 34 bytes at even addresses: every 16-byte load unaligned),
+//   two MFMAs per block onto one sum, one k group active at a time; the block scales reach the other lanes of the
+//   column by two lane swaps.  These stream at 2.3 TB/s only and serve a narrower range (rows16_direct_pays).
 // Only the activations go through LDS.
 //
 // K is split over the eight waves of a workgroup, not over workgroups: a workgroup owns 16 or 32 columns, each wave
@@ -50,17 +53,19 @@ struct Direct16Args {
   float* partial;
 };
 
-enum { DIRECT_Q4_K = 0, DIRECT_Q5_K = 1, DIRECT_Q6_K = 2 };
+enum { DIRECT_Q4_K = 0, DIRECT_Q5_K = 1, DIRECT_Q6_K = 2, DIRECT_Q4_0 = 3, DIRECT_Q8_0 = 4 };
 
 // NP: 16-column tiles a wave takes in turn (the workgroup owns 16 NP columns).  GSUM (Q4_K, Q5_K): the offset term
 // multiplies d8 * sum(q8), the GEMV operator's arithmetic (vecdotq.cuh:328-351), instead of the stored block sum.
 template <typename T, int KSPL, int NP, int FMT, bool GSUM>
 __global__ __launch_bounds__(64 * KSPL, 4) void rows16_direct_kernel(const uint8_t* __restrict__ W, const char* __restrict__ ws,
                                                                       T* __restrict__ Y, const T* __restrict__ bias, Direct16Args a) {
-  constexpr bool Q5 = FMT == DIRECT_Q5_K, Q6 = FMT == DIRECT_Q6_K;
+  constexpr bool Q5 = FMT == DIRECT_Q5_K, Q6 = FMT == DIRECT_Q6_K, Q40 = FMT == DIRECT_Q4_0, Q80 = FMT == DIRECT_Q8_0;
+  constexpr bool B32 = Q40 || Q80;                       // 32-value blocks: eight of them stand for a super-block
   constexpr int NT = 64 * KSPL, N_T = 16 * NP;
-  constexpr int BS = Q6 ? 210 : Q5 ? 176 : 144, QS = Q5 ? 48 : 16;   // block bytes, offset of qs (Q4_K, Q5_K)
-  constexpr int XROWS = Q6 ? 17 : 16;                    // Q6_K: a row of zeros behind the 16 rows of X
+  constexpr int BS = Q6 ? 210 : Q5 ? 176 : Q40 ? 8 * 18 : Q80 ? 8 * 34 : 144;   // bytes of 256 values
+  constexpr int QS = Q5 ? 48 : 16;                       // offset of qs (Q4_K, Q5_K)
+  constexpr int XROWS = Q6 || B32 ? 17 : 16;             // a row of zeros behind the 16 rows of X
   constexpr int MAX_SB = kDirectMaxSb;
   extern __shared__ __align__(16) char smem[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -88,12 +93,25 @@ __global__ __launch_bounds__(64 * KSPL, 4) void rows16_direct_kernel(const uint8
   // Q6_K (loads of any alignment): per half n of the super-block a lane takes ql[64 n + 16 g ..] -- its low nibbles
   // are the 16-value scale group 8 n + g, its high nibbles group 8 n + 4 + g -- the 16 bytes of qh that hold their
   // upper two bits, and with all lanes of its column the 16 scales and d.
+  // Q4_0, Q8_0 (blocks of 18 and 34 bytes at even addresses): a lane owns whole blocks, 4 i + g of every eight, i = 0, 1
+  // -- the four lanes of a column read 72 or 136 contiguous bytes.  Values 0..15 of the block (Q4_0: the low nibbles)
+  // and 16..31 go through two MFMAs onto one sum.
   struct Blk4 { uint4 hdr; u4_d q[2]; u4_d qh; };
   struct Blk6 { u4_d ql[2], qh[2], sc; uint32_t d; };
-  using Blk = std::conditional_t<Q6, Blk6, Blk4>;
+  struct Blk32 { u4_d q[Q80 ? 4 : 2]; uint32_t d[2]; };
+  using Blk = std::conditional_t<Q6, Blk6, std::conditional_t<B32, Blk32, Blk4>>;
   auto fetch = [&](int q, int sb, Blk& b) {
     const uint8_t* p = wrow[q] + sb * BS;
-    if constexpr (Q6) {
+    if constexpr (B32) {
+      constexpr int BB = BS / 8;
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        const uint8_t* pb = p + (4 * i + lgrp) * BB;
+        b.d[i] = ld<uint16_t>(pb);
+        if constexpr (Q80) { b.q[2 * i] = ld<u4_d>(pb + 2); b.q[2 * i + 1] = ld<u4_d>(pb + 18); }
+        else b.q[i] = ld<u4_d>(pb + 2);
+      }
+    } else if constexpr (Q6) {
 #pragma unroll
       for (int n = 0; n < 2; ++n) {
         b.ql[n] = ld<u4_d>(p + 64 * n + 16 * lgrp);
@@ -146,7 +164,7 @@ __global__ __launch_bounds__(64 * KSPL, 4) void rows16_direct_kernel(const uint8
     const float second = GSUM ? (dreg[i] != 0.0f ? __builtin_rintf(sreg[i] * __builtin_amdgcn_rcpf(dreg[i])) : 0.0f) : sreg[i];
     xsc[min(at + TPR * i, spr - 1) * 16 + am] = (h2_d){(_Float16)dreg[i], (_Float16)second};
   }
-  if constexpr (Q6)
+  if constexpr (XROWS == 17)
     for (int i = tid; i < gpr; i += NT) *(u4_d*)(xq + 16 * pitch + 16 * i) = (u4_d){0u, 0u, 0u, 0u};
 
   float acc[NP][4];
@@ -159,7 +177,45 @@ __global__ __launch_bounds__(64 * KSPL, 4) void rows16_direct_kernel(const uint8
 
   // One super-block of column tile q.  (A super-block past the wave's stretch was re-read: it is scaled to nothing.)
   auto consume = [&](int q, int s, const Blk& b, bool valid) {
-    if constexpr (Q6) {
+    if constexpr (B32) {
+      // the activations of the block that k group t owns for the lanes of that group, the row of zeros for the others
+      const int8_t* xsel[4];
+#pragma unroll
+      for (int t = 0; t < 4; ++t) xsel[t] = xq + (lgrp == t ? lcol : 16) * pitch + s * 256 + 32 * lgrp;
+#pragma unroll
+      for (int i = 0; i < 2; ++i) {
+        // every lane of the column needs the scales of all four blocks: two lane swaps spread them (rows of 16 lanes
+        // g0 g1 g2 g3 -> g0 g1 g0 g1 and g2 g3 g2 g3 -> four registers that hold one block's scale in every lane)
+        const auto half01 = __builtin_amdgcn_permlane32_swap(b.d[i], b.d[i], false, false);
+        const auto d01 = __builtin_amdgcn_permlane16_swap(half01[0], half01[0], false, false);
+        const auto d23 = __builtin_amdgcn_permlane16_swap(half01[1], half01[1], false, false);
+        const uint32_t dbits[4] = {d01[0], d01[1], d23[0], d23[1]};
+#pragma unroll
+        for (int t = 0; t < 4; ++t) {
+          const int blk = 4 * i + t;
+          const v4i_d alo = *(const v4i_d*)(xsel[t] + 128 * i);
+          const v4i_d ahi = *(const v4i_d*)(xsel[t] + 128 * i + 16);
+          v4i_d blo, bhi;
+#pragma unroll
+          for (int e = 0; e < 4; ++e) {
+            if constexpr (Q80) { blo[e] = (int)b.q[2 * i][e]; bhi[e] = (int)b.q[2 * i + 1][e]; }
+            else { blo[e] = (int)(b.q[i][e] & 0x0F0F0F0Fu); bhi[e] = (int)((b.q[i][e] >> 4) & 0x0F0F0F0Fu); }
+          }
+          v4i_d S = __builtin_amdgcn_mfma_i32_16x16x64_i8(alo, blo, seed, 0, 0, 0);
+          S = __builtin_amdgcn_mfma_i32_16x16x64_i8(ahi, bhi, S, 0, 0, 0);
+          const float w = valid ? (float)__builtin_bit_cast(_Float16, (uint16_t)dbits[t]) : 0.0f;
+          const float nsw = -kSeed * w, nm = -8.0f * w;   // Q4_0: d * (q - 8), the 8 on the stored block sum (vecdotq.cuh:46-66)
+          const uint4 x4 = *(const uint4*)(xsc + (s * 8 + blk) * 16 + 4 * lgrp);
+          const uint32_t scw[4] = {x4.x, x4.y, x4.z, x4.w};
+#pragma unroll
+          for (int r = 0; r < 4; ++r) {
+            const h2_d hh = __builtin_bit_cast(h2_d, scw[r]);
+            acc[q][r] = __builtin_fmaf(seeded_times(S[r], w, nsw), (float)hh[0], acc[q][r]);
+            if constexpr (Q40) acc[q][r] = __builtin_fmaf((float)hh[1], nm, acc[q][r]);
+          }
+        }
+      }
+    } else if constexpr (Q6) {
       // the activations of k group t for the lanes of that group, the row of zeros for the others
       const int8_t* xsel[4];
 #pragma unroll
@@ -312,13 +368,16 @@ static Direct16Plan direct16_plan(int N, int K, int64_t partial_bytes_available)
 }
 int64_t rows16_direct_partial_bytes(int N, int K) { return K % 256 ? 0 : direct16_plan(N, K, INT64_MAX).partial_bytes(); }
 
-static inline int direct_block_bytes(int type) { return type == T_Q6_K ? 210 : type == T_Q5_K ? 176 : 144; }
+// bytes of 256 values
+static inline int direct_block_bytes(int type) {
+  return type == T_Q6_K ? 210 : type == T_Q5_K ? 176 : type == T_Q4_0 ? 8 * 18 : type == T_Q8_0 ? 8 * 34 : 144;
+}
 
 template <typename T, int NP, int FMT, bool GSUM>
 static int rows16_direct_launch(const void* W, const void* ws, void* Y, int M, int N, int K, float* partial, const Direct16Plan& p,
                                 hipStream_t stream, const LinearArgs& la) {
-  constexpr int KSPL = kDirectKspl, N_T = 16 * NP, XROWS = FMT == DIRECT_Q6_K ? 17 : 16;
-  constexpr int BS = FMT == DIRECT_Q6_K ? 210 : FMT == DIRECT_Q5_K ? 176 : 144;
+  constexpr int KSPL = kDirectKspl, N_T = 16 * NP, XROWS = FMT == DIRECT_Q4_K || FMT == DIRECT_Q5_K ? 16 : 17;
+  constexpr int BS = FMT == DIRECT_Q6_K ? 210 : FMT == DIRECT_Q5_K ? 176 : FMT == DIRECT_Q4_0 ? 8 * 18 : FMT == DIRECT_Q8_0 ? 8 * 34 : 144;
   const size_t act = (size_t)XROWS * (p.per_wg * 256 + 16) + (size_t)p.per_wg * 8 * 16 * 4, red = (size_t)KSPL * 16 * N_T * 4;
   const size_t lds = act > red ? act : red;
   auto kern = rows16_direct_kernel<T, KSPL, NP, FMT, GSUM>;
@@ -339,7 +398,7 @@ static int rows16_direct_launch(const void* W, const void* ws, void* Y, int M, i
 template <typename T, int FMT>
 static int rows16_direct_typed(const void* W, const void* ws, void* Y, int M, int N, int K, float* partial, const Direct16Plan& p,
                                hipStream_t stream, const LinearArgs& la, bool gemv_sums) {
-  if constexpr (FMT != DIRECT_Q6_K) {   // (Q6_K has no offset term: the two operators agree)
+  if constexpr (FMT == DIRECT_Q4_K || FMT == DIRECT_Q5_K) {   // (the two operators agree on the other formats)
     if (gemv_sums) {
       if (p.np == 2) return rows16_direct_launch<T, 2, FMT, true>(W, ws, Y, M, N, K, partial, p, stream, la);
       return rows16_direct_launch<T, 1, FMT, true>(W, ws, Y, M, N, K, partial, p, stream, la);
@@ -351,13 +410,29 @@ static int rows16_direct_typed(const void* W, const void* ws, void* Y, int M, in
 
 // Whether rows16_direct() would run this call.
 bool rows16_direct_takes(const void* W, int64_t w_pitch, int type, int M, int N, int K, int64_t partial_bytes) {
-  if ((type != T_Q4_K && type != T_Q5_K && type != T_Q6_K) || M > 16 || K % 256) return false;
+  if ((type != T_Q4_K && type != T_Q5_K && type != T_Q6_K && type != T_Q4_0 && type != T_Q8_0) || M > 16 || K % 256) return false;
   const int64_t pitch = w_pitch ? w_pitch : (int64_t)(K / 256) * direct_block_bytes(type);
-  if (type != T_Q6_K && (((uintptr_t)W & 15) || (pitch & 15))) return false;   // (Q6_K blocks are at even addresses anyway)
+  // (the blocks of the other formats are at even addresses anyway)
+  if ((type == T_Q4_K || type == T_Q5_K) && (((uintptr_t)W & 15) || (pitch & 15))) return false;
   return direct16_plan(N, K, partial_bytes).gsplits != 0;
 }
 
-// Q4_K, Q5_K (W and its row pitch 16-byte aligned) or Q6_K, at most 16 rows of X; GGUF_NOT_TAKEN otherwise.
+// Whether the kernel is the faster route for a call it can run.  The K-quants: always on the tile operator's side
+// (against the staged 16-row tiles), and from five rows on against the streaming GEMV when the matrix has at least 8M
+// weights (below that the GEMV's single launch wins: [1024,4096] 8 against 10 us).  Q4_0 and Q8_0, whose blocks make
+// every 16-byte load unaligned, stream at 2.3 TB/s only: from nine rows on against the GEMV (eight rows of
+// [14336,4096] take it 18 us, this kernel 22 and 30 us; sixteen rows 36 and 35 us), and against the staged tiles while
+// K is not split over workgroups (Q4_0 [14336,4096] 21.8 against 24.0 us, [4096,4096] 10.6 against 13.7 us, but
+// [28672,8192] 65 against 50 us) and, for Q8_0, up to 32M weights ([4096,4096] 12.1 against 14.2 us; [14336,4096] 30
+// against 27 us).
+bool rows16_direct_pays(int type, int M, int64_t N, int64_t K, bool against_gemv) {
+  const bool kquant = type == T_Q4_K || type == T_Q5_K || type == T_Q6_K;
+  if (against_gemv) return M >= (kquant ? 5 : 9) && N * K >= (8 << 20);
+  if (kquant) return true;
+  return M >= 9 && K <= 256 * kDirectMaxSb && (type != T_Q8_0 || N * K <= (32 << 20));
+}
+
+// Q4_K, Q5_K (W and its row pitch 16-byte aligned), Q6_K, Q4_0 or Q8_0, at most 16 rows of X; GGUF_NOT_TAKEN otherwise.
 // gemv_sums: the GEMV operator's offset term (see GSUM) instead of the tile operator's.
 int rows16_direct(const void* W, const void* ws, void* Y, int dtype, int type, int M, int N, int K, float* partial, int64_t partial_bytes,
                   hipStream_t s, const LinearArgs& la, bool gemv_sums) {
@@ -365,6 +440,14 @@ int rows16_direct(const void* W, const void* ws, void* Y, int dtype, int type, i
   const Direct16Plan p = direct16_plan(N, K, partial_bytes);
   if (type == T_Q6_K) {
     GGUF_DISPATCH_DTYPE(dtype, return (rows16_direct_typed<scalar_t, DIRECT_Q6_K>(W, ws, Y, M, N, K, partial, p, s, la, gemv_sums)));
+    return GGUF_ERR_DTYPE;
+  }
+  if (type == T_Q4_0) {
+    GGUF_DISPATCH_DTYPE(dtype, return (rows16_direct_typed<scalar_t, DIRECT_Q4_0>(W, ws, Y, M, N, K, partial, p, s, la, gemv_sums)));
+    return GGUF_ERR_DTYPE;
+  }
+  if (type == T_Q8_0) {
+    GGUF_DISPATCH_DTYPE(dtype, return (rows16_direct_typed<scalar_t, DIRECT_Q8_0>(W, ws, Y, M, N, K, partial, p, s, la, gemv_sums)));
     return GGUF_ERR_DTYPE;
   }
   if (type == T_Q5_K) {
