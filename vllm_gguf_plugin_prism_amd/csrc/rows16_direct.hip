@@ -91,13 +91,13 @@ __global__ __launch_bounds__(64 * KSPL, 4) void rows16_direct_kernel(const uint8
   // Q5_K: the fifth bits of values l and 32 + l .. 224 + l of the super-block are the bits of qh[l]; a piece covers
   // l = 16 (g % 2) .. + 15 of its blocks, so the lane takes that half of qh (bit number = block number).
   // Q6_K (loads of any alignment): per half n of the super-block a lane takes ql[64 n + 16 g ..] -- its low nibbles
-  // are the 16-value scale group 8 n + g, its high nibbles group 8 n + 4 + g -- the 16 bytes of qh that hold their
-  // upper two bits, and with all lanes of its column the 16 scales and d.
+  // are the 16-value scale group 8 n + g, its high nibbles group 8 n + 4 + g.  The upper two bits of both halves are
+  // in qh[32 n + 16 (g % 2) ..]; the lane fetches qh[16 g ..] and four of the 16 scales, and lane swaps complete both.
   // Q4_0, Q8_0 (blocks of 18 and 34 bytes at even addresses): a lane owns whole blocks, 4 i + g of every eight, i = 0, 1
   // -- the four lanes of a column read 72 or 136 contiguous bytes.  Values 0..15 of the block (Q4_0: the low nibbles)
   // and 16..31 go through two MFMAs onto one sum.
   struct Blk4 { uint4 hdr; u4_d q[2]; u4_d qh; };
-  struct Blk6 { u4_d ql[2], qh[2], sc; uint32_t d; };
+  struct Blk6 { u4_d ql[2], qh; uint32_t sc, d; };   // qh: piece g of the four; sc: scales 4 g .. 4 g + 3
   struct Blk32 { u4_d q[Q80 ? 4 : 2]; uint32_t d[2]; };
   using Blk = std::conditional_t<Q6, Blk6, std::conditional_t<B32, Blk32, Blk4>>;
   auto fetch = [&](int q, int sb, Blk& b) {
@@ -113,11 +113,9 @@ __global__ __launch_bounds__(64 * KSPL, 4) void rows16_direct_kernel(const uint8
       }
     } else if constexpr (Q6) {
 #pragma unroll
-      for (int n = 0; n < 2; ++n) {
-        b.ql[n] = ld<u4_d>(p + 64 * n + 16 * lgrp);
-        b.qh[n] = ld<u4_d>(p + 128 + 32 * n + 16 * (lgrp & 1));
-      }
-      b.sc = ld<u4_d>(p + 192);
+      for (int n = 0; n < 2; ++n) b.ql[n] = ld<u4_d>(p + 64 * n + 16 * lgrp);
+      b.qh = ld<u4_d>(p + 128 + 16 * lgrp);
+      b.sc = ld<uint32_t>(p + 192 + 4 * lgrp);
       b.d = ld<uint16_t>(p + 208);
     } else {
       b.hdr = *(const uint4*)p;
@@ -221,6 +219,20 @@ __global__ __launch_bounds__(64 * KSPL, 4) void rows16_direct_kernel(const uint8
 #pragma unroll
       for (int t = 0; t < 4; ++t) xsel[t] = xq + (lgrp == t ? lcol : 16) * pitch + s * 256 + 16 * lgrp;
       const float d = valid ? (float)__builtin_bit_cast(_Float16, (uint16_t)b.d) : 0.0f;
+      // Each of the four lanes of a column fetched one 16-byte piece of qh and four of the 16 scales; lane swaps hand
+      // every lane the two pieces (g % 2 of either half) and all the scales it needs: rows of 16 lanes g0 g1 g2 g3 ->
+      // g0 g1 g0 g1 and g2 g3 g2 g3, and once more -> one k group's register in every lane.
+      u4_d qh[2];
+#pragma unroll
+      for (int e = 0; e < 4; ++e) {
+        const auto sw = __builtin_amdgcn_permlane32_swap(b.qh[e], b.qh[e], false, false);
+        qh[0][e] = sw[0];
+        qh[1][e] = sw[1];
+      }
+      const auto sc_h = __builtin_amdgcn_permlane32_swap(b.sc, b.sc, false, false);
+      const auto sc01 = __builtin_amdgcn_permlane16_swap(sc_h[0], sc_h[0], false, false);
+      const auto sc23 = __builtin_amdgcn_permlane16_swap(sc_h[1], sc_h[1], false, false);
+      const uint32_t scs[4] = {sc01[0], sc01[1], sc23[0], sc23[1]};
 #pragma unroll
       for (int n = 0; n < 2; ++n)
 #pragma unroll
@@ -229,7 +241,7 @@ __global__ __launch_bounds__(64 * KSPL, 4) void rows16_direct_kernel(const uint8
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             const uint32_t lo = (h ? b.ql[n][e] >> 4 : b.ql[n][e]) & 0x0F0F0F0Fu;
-            const uint32_t hi = (b.qh[n][e] >> (4 * h + 2 * (lgrp >> 1))) & 0x03030303u;
+            const uint32_t hi = (qh[n][e] >> (4 * h + 2 * (lgrp >> 1))) & 0x03030303u;
             bv[e] = (int)sub_bytes(lo | (hi << 4), 0x20202020u);
           }
           const uint4 sc4 = *(const uint4*)(xsc + (s * 8 + 4 * n + 2 * h) * 16 + 4 * lgrp);       // block 4 n + 2 h
@@ -240,7 +252,7 @@ __global__ __launch_bounds__(64 * KSPL, 4) void rows16_direct_kernel(const uint8
             const int grp = 8 * n + 4 * h + t;             // 16 values 128 n + 64 h + 16 t .. of the super-block
             const v4i_d av = *(const v4i_d*)(xsel[t] + 128 * n + 64 * h);
             const v4i_d S = __builtin_amdgcn_mfma_i32_16x16x64_i8(av, bv, seed, 0, 0, 0);
-            const int sc = (int)(int8_t)((b.sc[grp >> 2] >> (8 * (grp & 3))) & 0xFF);
+            const int sc = (int)(int8_t)((scs[grp >> 2] >> (8 * (grp & 3))) & 0xFF);
             const float w = d * (float)sc, nsw = -kSeed * w;
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
