@@ -515,7 +515,7 @@ def test_mmq_nine_to_32_rows(qtype, dt):
 @pytest.mark.parametrize("dt", ["f32", "f16", "bf16"])
 @pytest.mark.parametrize("qtype", [o.Q4_K, o.Q5_K, o.Q6_K, o.Q4_0, o.Q8_0])
 def test_mmq_up_to_16_rows_from_packed_blocks(qtype, dt):
-    """Q4_K, Q5_K, Q6_K (and Q4_0, Q8_0 from nine rows on) with at most 16 rows of X build their MFMA operands straight from the packed blocks, K split over the waves
+    """Q4_K, Q5_K, Q6_K with at most 32 rows of X (and Q4_0, Q8_0 with nine to 16) build their MFMA operands straight from the packed blocks, K split over the waves
     of a workgroup: one super-block of K, a stretch that fills LDS (K = 4096), K beyond it (split over workgroups as
     well, and the same call without room for partial tiles), few columns (split down to a super-block per wave), the
     two-column-tile variant of wide outputs with a ragged last tile, a row slice of a wider weight tensor with bias
@@ -542,9 +542,17 @@ def test_mmq_up_to_16_rows_from_packed_blocks(qtype, dt):
                                  int(qtype), n, k, m, 1, nbytes, torch.cuda.current_stream().cuda_stream)
         assert rc == 0
         assert o.rel_l2(y2.float().cpu().numpy(), want) <= tol, (m, n, k, "minimum workspace")
+    if qtype in (o.Q4_K, o.Q5_K, o.Q6_K):
+        # 17 .. 32 rows: two 16-row tiles of X against every weight operand; 32 and 64 columns per workgroup for wide
+        # outputs (ragged last tiles), K beyond 4096 (split over workgroups too)
+        for m, n, k in [(17, 72, 256), (32, 200, 4096), (20, 4200, 512), (31, 8300, 256), (24, 40, 8192)]:
+            w = o.make_weights(rng, qtype, n, k)
+            xd, xv = _x(rng, m, k, dt)
+            y = ops.ggml_mul_mat_a8(_dev(w), xd, qtype, n)
+            assert o.rel_l2(y.float().cpu().numpy(), o.mul_mat_a8(w, xv, qtype, n, "mmq")) <= tol, (m, n, k)
     # shard of a merged layer: rows 8 .. 8 + n of a taller tensor whose rows are 32 bytes longer than the blocks,
     # bias, result columns 5 .. 5 + n of a wider tensor
-    m, n, k = 14, 150, 1024
+    m, n, k = (14 if qtype in (o.Q4_0, o.Q8_0) else 27), 150, 1024
     row_bytes = k // o.QUANT_SIZES[qtype][0] * o.QUANT_SIZES[qtype][1]
     for pad, where in ((32, "aligned"), (2, "unaligned")):
         tall = rng.integers(0, 256, (n + 20, row_bytes + pad), dtype=np.uint8)

@@ -218,7 +218,7 @@ def test_mmvq_five_rows_or_more_of_a_large_matrix(qtype, dt):
     ops = _ops()
     rng = np.random.default_rng(1600 + qtype)
     tol = 1e-5 if dt == "f32" else 1e-3
-    for n, k, ms in [(2048, 4096, (5, 16, 21)), (1100, 8192, (6,)), (300, 1024, (7,))]:
+    for n, k, ms in [(2048, 4096, (5, 16, 21, 40)), (1100, 8192, (6,)), (300, 1024, (7,))]:
         w = o.make_weights(rng, qtype, n, k)
         wd = _to_dev(w)
         for m in ms:

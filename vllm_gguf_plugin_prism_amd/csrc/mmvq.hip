@@ -47,7 +47,7 @@ int rows16_direct(const void* W, const void* ws, void* Y, int dtype, int type, i
 int mmvq_any(int type, const void* W, const void* x, void* q8_workspace, void* Y, int xdtype, int64_t N, int64_t K, int64_t M,
              hipStream_t s, const LinearArgs& la) {
   // Five rows or more (nine for Q4_0 / Q8_0) of a matrix of at least 8M weights: the tile kernel's time does not grow
-  // with the rows (up to 16 per launch), the streaming kernel's does (Q4_K [14336,4096] at 8 / 16 rows 22 / 42 us
+  // with the rows (up to 16 or 32 per launch), the streaming kernel's does (Q4_K [14336,4096] at 8 / 16 rows 22 / 42 us
   // against 17 us, Q6_K 36 / 71 against 27 us, Q4_0 at 16 rows 36 against 22 us).  The operator's workspace holds the quantized rows and nothing else, so K up to 4096 (beyond that
   // the tile kernel wants room for partial tiles).  The arithmetic stays the GEMV's (offset term on d8 * sum(q8)).
   if (!la.tile_sums && N <= 0x7FFFFFF0LL && K <= 0x7FFFFFF0LL && rows16_direct_pays(type, (int)(M < 16 ? M : 16), N, K, true) &&
@@ -55,8 +55,9 @@ int mmvq_any(int type, const void* W, const void* x, void* q8_workspace, void* Y
     int rc = quantize_q8_1(x, xdtype, q8_workspace, M, K, s);
     if (rc != GGUF_OK) return rc;
     const int64_t ldy = la.ldy ? la.ldy : N, esz = xdtype == GGUF_DTYPE_F32 ? 4 : 2;
-    for (int64_t m0 = 0; m0 < M; m0 += 16) {
-      const int rows = (int)(M - m0 < 16 ? M - m0 : 16);
+    const int step = rows16_direct_takes(W, la.w_pitch, type, 32, (int)N, (int)K, 0) ? 32 : 16;   // (the K-quants take 32 rows per launch)
+    for (int64_t m0 = 0; m0 < M; m0 += step) {
+      const int rows = (int)(M - m0 < step ? M - m0 : step);
       rc = rows16_direct(W, (const char*)q8_workspace + m0 * q8_row_bytes(K), (char*)Y + m0 * ldy * esz, xdtype, type, rows, (int)N, (int)K,
                          nullptr, 0, s, la, true);
       if (rc != GGUF_OK) return rc;

@@ -273,11 +273,11 @@ static inline int dense16_splits(int M, int N, int K, int64_t partial_bytes_avai
   if (s < 2) return 1;
   return tiles * s * (16 * 128 * 4) <= partial_bytes_available ? s : 1;
 }
-int64_t rows16_direct_partial_bytes(int N, int K);   // rows16_direct.hip
+int64_t rows16_direct_partial_bytes(int M, int N, int K);   // rows16_direct.hip
 int64_t mmq_rows16_partial_bytes(int M, int N, int K) {
   const int s = dense16_splits(M, N, K, INT64_MAX);
   const int64_t tiled = s > 1 ? (int64_t)((M + 15) / 16) * ((N + 127) / 128) * s * (16 * 128 * 4) : 0;
-  return M <= 16 ? std::max(tiled, rows16_direct_partial_bytes(N, K)) : tiled;
+  return std::max(tiled, rows16_direct_partial_bytes(M, N, K));
 }
 
 template <class F, typename T>
@@ -316,13 +316,13 @@ bool rows16_direct_pays(int type, int M, int64_t N, int64_t K, bool against_gemv
 // q8_1(X) . W^T for a few rows of X (the quantized rows are in the workspace); GGUF_NOT_TAKEN for other formats.
 int mmq_rows16(const void* W, const void* ws, void* Y, int dtype, int type, int M, int N, int K, float* partial, int64_t partial_bytes,
                hipStream_t s, const LinearArgs& la) {
-  // the 16-deep formats pay two MFMAs and four vector instructions per result and block here as in the large tiles, and
-  // with two 16-row tiles (17 .. 32 rows) the large tiles are as fast: Q6_K [14336,4096] 44 us either way
-  if ((type == T_Q6_K || type == T_Q3_K) && M > 16) return GGUF_NOT_TAKEN;
-  if (rows16_direct_pays(type, M, N, K, false)) {   // at most 16 rows: straight from the packed blocks
+  if (rows16_direct_pays(type, M, N, K, false)) {   // straight from the packed blocks (the K-quants up to 32 rows, Q4_0 / Q8_0 up to 16)
     const int rc = rows16_direct(W, ws, Y, dtype, type, M, N, K, partial, partial_bytes, s, la, false);
     if (rc != GGUF_NOT_TAKEN) return rc;
   }
+  // the 16-deep formats pay two MFMAs and four vector instructions per result and block on the staged tiles as in the
+  // large tiles, and with two 16-row tiles (17 .. 32 rows) the large tiles are as fast: Q3_K [14336,4096] 44 us either way
+  if ((type == T_Q6_K || type == T_Q3_K) && M > 16) return GGUF_NOT_TAKEN;
   switch (type) {
     case T_Q4_0: return dense16_fmt<MQ4_0>(W, ws, Y, dtype, M, N, K, partial, partial_bytes, s, la);
     case T_Q8_0: return dense16_fmt<MQ8_0>(W, ws, Y, dtype, M, N, K, partial, partial_bytes, s, la);

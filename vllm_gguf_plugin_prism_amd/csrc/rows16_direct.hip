@@ -1,6 +1,6 @@
-// The tile GEMM for up to 16 rows of X without LDS staging of the weights (Q4_K, Q5_K, Q6_K, Q4_0, Q8_0).
+// The tile GEMM for up to 32 rows of X without LDS staging of the weights (Q4_K, Q5_K, Q6_K; Q4_0, Q8_0 up to 16 rows).
 //
-// With at most 16 rows every weight is used by exactly one MFMA, so staging the decoded weights in LDS buys no reuse:
+// With so few rows every weight is used by one or two MFMAs, so staging the decoded weights in LDS buys no reuse:
 // it only reshapes them into the MFMA operand layout, at the price of a barrier per step of K.  For these formats that
 // layout can be read straight from the packed block.  The operand lane (column c, k group g) of a 64-deep int8 MFMA
 // supplies 16 values.
@@ -31,10 +31,12 @@
 // become free: the staged activations serve both, the second tile's loads overlap the first's arithmetic, and the
 // kernel keeps the registers of one tile (both tiles held at once: Q4_K [14336,4096] 16.8 against 15.3 us; four tiles
 // in turn gain nothing over two).
-// More than 16 rows as further passes of 16 over the weights a wave holds were measured and lose to the staged tiles:
-// every pass repeats the rescaling, which is what the kernel spends its arithmetic on ([14336,4096] at 32 rows 37
-// against 32 us, at 64 rows 60 against 37 us).  One workgroup per CU instead of two, so that the rounds of workgroups
-// overlap each other's phases, is slower too (19.5 against 16.8 us).
+// 17 to 32 rows (the K-quants): two 16-row tiles of X, every weight operand multiplied with both.  The 32 rows of a
+// 4096-value stretch fill LDS, so one workgroup runs per CU (with twice the registers) and owns up to 64 columns, so
+// that one round of workgroups covers the output: Q4_K [14336,4096] 32 -> 22 us, Q5_K 47 -> 24 us, Q6_K 45 -> 29 us
+// against the staged tiles.  Further rows as passes of 16 over the weights a wave holds, restaging the activations,
+// lose to the staged tiles ([14336,4096] at 32 rows 37 against 32 us, at 64 rows 60 against 37 us), and for 16 rows one
+// workgroup per CU instead of two is slower (19.5 against 16.8 us).
 // Arithmetic as in the other integer tile kernels (mmq.cuh:2-104, vecdotq.cuh:353-379, 467-491: exact int32 block
 // sums, `d*sc*d8*S - dmin*m*s8` with the stored block sums s8; Q6_K `d*sc*d8*S` per 16 values).
 #include "mmq_i_core.h"
@@ -57,15 +59,17 @@ enum { DIRECT_Q4_K = 0, DIRECT_Q5_K = 1, DIRECT_Q6_K = 2, DIRECT_Q4_0 = 3, DIREC
 
 // NP: 16-column tiles a wave takes in turn (the workgroup owns 16 NP columns).  GSUM (Q4_K, Q5_K): the offset term
 // multiplies d8 * sum(q8), the GEMV operator's arithmetic (vecdotq.cuh:328-351), instead of the stored block sum.
-template <typename T, int KSPL, int NP, int FMT, bool GSUM>
-__global__ __launch_bounds__(64 * KSPL, 4) void rows16_direct_kernel(const uint8_t* __restrict__ W, const char* __restrict__ ws,
+// RT: 16-row tiles of X (1 or 2).  With two, every weight operand meets both tiles' activations; the 32 rows of a
+// 4096-value stretch fill LDS, so one workgroup runs per CU, with twice the registers.
+template <typename T, int KSPL, int NP, int FMT, bool GSUM, int RT>
+__global__ __launch_bounds__(64 * KSPL, RT == 2 ? 2 : 4) void rows16_direct_kernel(const uint8_t* __restrict__ W, const char* __restrict__ ws,
                                                                       T* __restrict__ Y, const T* __restrict__ bias, Direct16Args a) {
   constexpr bool Q5 = FMT == DIRECT_Q5_K, Q6 = FMT == DIRECT_Q6_K, Q40 = FMT == DIRECT_Q4_0, Q80 = FMT == DIRECT_Q8_0;
   constexpr bool B32 = Q40 || Q80;                       // 32-value blocks: eight of them stand for a super-block
   constexpr int NT = 64 * KSPL, N_T = 16 * NP;
   constexpr int BS = Q6 ? 210 : Q5 ? 176 : Q40 ? 8 * 18 : Q80 ? 8 * 34 : 144;   // bytes of 256 values
   constexpr int QS = Q5 ? 48 : 16;                       // offset of qs (Q4_K, Q5_K)
-  constexpr int XROWS = Q6 || B32 ? 17 : 16;             // a row of zeros behind the 16 rows of X
+  constexpr int XR = 16 * RT, XROWS = Q6 || B32 ? XR + 1 : XR;   // rows of X in LDS; a row of zeros behind them
   constexpr int MAX_SB = kDirectMaxSb;
   extern __shared__ __align__(16) char smem[];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -135,41 +139,50 @@ __global__ __launch_bounds__(64 * KSPL, 4) void rows16_direct_kernel(const uint8
   h2_d* xsc = (h2_d*)(smem + XROWS * pitch);
   const int gpr = nmine * 16, spr = nmine * 8;             // 16-byte granules, blocks per row
   const int am = tid / TPR, at = tid % TPR;
-  const char* const arow = ws + (int64_t)min(am, a.M - 1) * a.ws_row_bytes;
-  const float* const asc = (const float*)(arow + a.Kp) + sb0 * 8;
-  u4_d areg[AI];
-  float dreg[SI], sreg[SI];
+  u4_d areg[RT][AI];
+  float dreg[RT][SI], sreg[RT][SI];
 #pragma unroll
-  for (int i = 0; i < AI; ++i) areg[i] = *(const u4_d*)(arow + sb0 * 256 + 16 * min(at + TPR * i, gpr - 1));
+  for (int rt = 0; rt < RT; ++rt) {
+    const char* const arow = ws + (int64_t)min(16 * rt + am, a.M - 1) * a.ws_row_bytes;
+    const float* const asc = (const float*)(arow + a.Kp) + sb0 * 8;
 #pragma unroll
-  for (int i = 0; i < SI; ++i) {
-    const int kb = min(at + TPR * i, spr - 1);
-    dreg[i] = asc[kb];
-    sreg[i] = asc[(GSUM ? 2 : 1) * (a.Kp / 32) + kb];   // the stored sum s8, or du = d8 * sum(q8)
+    for (int i = 0; i < AI; ++i) areg[rt][i] = *(const u4_d*)(arow + sb0 * 256 + 16 * min(at + TPR * i, gpr - 1));
+#pragma unroll
+    for (int i = 0; i < SI; ++i) {
+      const int kb = min(at + TPR * i, spr - 1);
+      dreg[rt][i] = asc[kb];
+      sreg[rt][i] = asc[(GSUM ? 2 : 1) * (a.Kp / 32) + kb];   // the stored sum s8, or du = d8 * sum(q8)
+    }
   }
   Blk cur, nxt;
   fetch(0, min(my0, nmine - 1), cur);
   fetch(0, min(my0 + 1, nmine - 1), nxt);
   // (threads past the end store the last piece once more: a guarded store would draw its load into the guard)
 #pragma unroll
-  for (int i = 0; i < AI; ++i) *(u4_d*)(xq + am * pitch + 16 * min(at + TPR * i, gpr - 1)) = areg[i];
+  for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+    for (int i = 0; i < AI; ++i) *(u4_d*)(xq + (16 * rt + am) * pitch + 16 * min(at + TPR * i, gpr - 1)) = areg[rt][i];
+#pragma unroll
+  for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
   for (int i = 0; i < SI; ++i) {
     // d8 and s8 are half-precision values widened to fp32 by the quantizer: the narrowing is exact.  du is not one, but
     // du / d8 = sum(q8) is an integer of at most 13 bits, exact as a quotient and as a half; d8 multiplies it again
     // together with the block sum.
     // (the quotient is an integer below 4065 in magnitude: the hardware reciprocal's last-bit error rounds away)
-    const float second = GSUM ? (dreg[i] != 0.0f ? __builtin_rintf(sreg[i] * __builtin_amdgcn_rcpf(dreg[i])) : 0.0f) : sreg[i];
-    xsc[min(at + TPR * i, spr - 1) * 16 + am] = (h2_d){(_Float16)dreg[i], (_Float16)second};
+    const float second = GSUM ? (dreg[rt][i] != 0.0f ? __builtin_rintf(sreg[rt][i] * __builtin_amdgcn_rcpf(dreg[rt][i])) : 0.0f) : sreg[rt][i];
+    xsc[min(at + TPR * i, spr - 1) * XR + 16 * rt + am] = (h2_d){(_Float16)dreg[rt][i], (_Float16)second};
   }
-  if constexpr (XROWS == 17)
-    for (int i = tid; i < gpr; i += NT) *(u4_d*)(xq + 16 * pitch + 16 * i) = (u4_d){0u, 0u, 0u, 0u};
+  if constexpr (XROWS > XR)
+    for (int i = tid; i < gpr; i += NT) *(u4_d*)(xq + XR * pitch + 16 * i) = (u4_d){0u, 0u, 0u, 0u};
 
-  float acc[NP][4];
+  float acc[RT][NP][4];
 #pragma unroll
-  for (int q = 0; q < NP; ++q)
+  for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-    for (int r = 0; r < 4; ++r) acc[q][r] = 0.0f;
+    for (int q = 0; q < NP; ++q)
+#pragma unroll
+      for (int r = 0; r < 4; ++r) acc[rt][q][r] = 0.0f;
   const v4i_d seed = {kSeedBits, kSeedBits, kSeedBits, kSeedBits};
   __syncthreads();
 
@@ -177,9 +190,11 @@ __global__ __launch_bounds__(64 * KSPL, 4) void rows16_direct_kernel(const uint8
   auto consume = [&](int q, int s, const Blk& b, bool valid) {
     if constexpr (B32) {
       // the activations of the block that k group t owns for the lanes of that group, the row of zeros for the others
-      const int8_t* xsel[4];
+      const int8_t* xsel[RT][4];
 #pragma unroll
-      for (int t = 0; t < 4; ++t) xsel[t] = xq + (lgrp == t ? lcol : 16) * pitch + s * 256 + 32 * lgrp;
+      for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int t = 0; t < 4; ++t) xsel[rt][t] = xq + (lgrp == t ? 16 * rt + lcol : XR) * pitch + s * 256 + 32 * lgrp;
 #pragma unroll
       for (int i = 0; i < 2; ++i) {
         // every lane of the column needs the scales of all four blocks: two lane swaps spread them (rows of 16 lanes
@@ -191,33 +206,38 @@ __global__ __launch_bounds__(64 * KSPL, 4) void rows16_direct_kernel(const uint8
 #pragma unroll
         for (int t = 0; t < 4; ++t) {
           const int blk = 4 * i + t;
-          const v4i_d alo = *(const v4i_d*)(xsel[t] + 128 * i);
-          const v4i_d ahi = *(const v4i_d*)(xsel[t] + 128 * i + 16);
           v4i_d blo, bhi;
 #pragma unroll
           for (int e = 0; e < 4; ++e) {
             if constexpr (Q80) { blo[e] = (int)b.q[2 * i][e]; bhi[e] = (int)b.q[2 * i + 1][e]; }
             else { blo[e] = (int)(b.q[i][e] & 0x0F0F0F0Fu); bhi[e] = (int)((b.q[i][e] >> 4) & 0x0F0F0F0Fu); }
           }
-          v4i_d S = __builtin_amdgcn_mfma_i32_16x16x64_i8(alo, blo, seed, 0, 0, 0);
-          S = __builtin_amdgcn_mfma_i32_16x16x64_i8(ahi, bhi, S, 0, 0, 0);
           const float w = valid ? (float)__builtin_bit_cast(_Float16, (uint16_t)dbits[t]) : 0.0f;
           const float nsw = -kSeed * w, nm = -8.0f * w;   // Q4_0: d * (q - 8), the 8 on the stored block sum (vecdotq.cuh:46-66)
-          const uint4 x4 = *(const uint4*)(xsc + (s * 8 + blk) * 16 + 4 * lgrp);
-          const uint32_t scw[4] = {x4.x, x4.y, x4.z, x4.w};
 #pragma unroll
-          for (int r = 0; r < 4; ++r) {
-            const h2_d hh = __builtin_bit_cast(h2_d, scw[r]);
-            acc[q][r] = __builtin_fmaf(seeded_times(S[r], w, nsw), (float)hh[0], acc[q][r]);
-            if constexpr (Q40) acc[q][r] = __builtin_fmaf((float)hh[1], nm, acc[q][r]);
+          for (int rt = 0; rt < RT; ++rt) {
+            const v4i_d alo = *(const v4i_d*)(xsel[rt][t] + 128 * i);
+            const v4i_d ahi = *(const v4i_d*)(xsel[rt][t] + 128 * i + 16);
+            v4i_d S = __builtin_amdgcn_mfma_i32_16x16x64_i8(alo, blo, seed, 0, 0, 0);
+            S = __builtin_amdgcn_mfma_i32_16x16x64_i8(ahi, bhi, S, 0, 0, 0);
+            const uint4 x4 = *(const uint4*)(xsc + (s * 8 + blk) * XR + 16 * rt + 4 * lgrp);
+            const uint32_t scw[4] = {x4.x, x4.y, x4.z, x4.w};
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+              const h2_d hh = __builtin_bit_cast(h2_d, scw[r]);
+              acc[rt][q][r] = __builtin_fmaf(seeded_times(S[r], w, nsw), (float)hh[0], acc[rt][q][r]);
+              if constexpr (Q40) acc[rt][q][r] = __builtin_fmaf((float)hh[1], nm, acc[rt][q][r]);
+            }
           }
         }
       }
     } else if constexpr (Q6) {
       // the activations of k group t for the lanes of that group, the row of zeros for the others
-      const int8_t* xsel[4];
+      const int8_t* xsel[RT][4];
 #pragma unroll
-      for (int t = 0; t < 4; ++t) xsel[t] = xq + (lgrp == t ? lcol : 16) * pitch + s * 256 + 16 * lgrp;
+      for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int t = 0; t < 4; ++t) xsel[rt][t] = xq + (lgrp == t ? 16 * rt + lcol : XR) * pitch + s * 256 + 16 * lgrp;
       const float d = valid ? (float)__builtin_bit_cast(_Float16, (uint16_t)b.d) : 0.0f;
       // Each of the four lanes of a column fetched one 16-byte piece of qh and four of the 16 scales; lane swaps hand
       // every lane the two pieces (g % 2 of either half) and all the scales it needs: rows of 16 lanes g0 g1 g2 g3 ->
@@ -244,25 +264,30 @@ __global__ __launch_bounds__(64 * KSPL, 4) void rows16_direct_kernel(const uint8
             const uint32_t hi = (qh[n][e] >> (4 * h + 2 * (lgrp >> 1))) & 0x03030303u;
             bv[e] = (int)sub_bytes(lo | (hi << 4), 0x20202020u);
           }
-          const uint4 sc4 = *(const uint4*)(xsc + (s * 8 + 4 * n + 2 * h) * 16 + 4 * lgrp);       // block 4 n + 2 h
-          const uint4 sc5 = *(const uint4*)(xsc + (s * 8 + 4 * n + 2 * h + 1) * 16 + 4 * lgrp);   // and the next
-          const uint32_t d8w[2][4] = {{sc4.x, sc4.y, sc4.z, sc4.w}, {sc5.x, sc5.y, sc5.z, sc5.w}};
 #pragma unroll
-          for (int t = 0; t < 4; ++t) {
-            const int grp = 8 * n + 4 * h + t;             // 16 values 128 n + 64 h + 16 t .. of the super-block
-            const v4i_d av = *(const v4i_d*)(xsel[t] + 128 * n + 64 * h);
-            const v4i_d S = __builtin_amdgcn_mfma_i32_16x16x64_i8(av, bv, seed, 0, 0, 0);
-            const int sc = (int)(int8_t)((scs[grp >> 2] >> (8 * (grp & 3))) & 0xFF);
-            const float w = d * (float)sc, nsw = -kSeed * w;
+          for (int rt = 0; rt < RT; ++rt) {
+            const uint4 sc4 = *(const uint4*)(xsc + (s * 8 + 4 * n + 2 * h) * XR + 16 * rt + 4 * lgrp);       // block 4 n + 2 h
+            const uint4 sc5 = *(const uint4*)(xsc + (s * 8 + 4 * n + 2 * h + 1) * XR + 16 * rt + 4 * lgrp);   // and the next
+            const uint32_t d8w[2][4] = {{sc4.x, sc4.y, sc4.z, sc4.w}, {sc5.x, sc5.y, sc5.z, sc5.w}};
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-              const h2_d hh = __builtin_bit_cast(h2_d, d8w[t >> 1][r]);
-              acc[q][r] = __builtin_fmaf(seeded_times(S[r], w, nsw), (float)hh[0], acc[q][r]);
+            for (int t = 0; t < 4; ++t) {
+              const int grp = 8 * n + 4 * h + t;             // 16 values 128 n + 64 h + 16 t .. of the super-block
+              const v4i_d av = *(const v4i_d*)(xsel[rt][t] + 128 * n + 64 * h);
+              const v4i_d S = __builtin_amdgcn_mfma_i32_16x16x64_i8(av, bv, seed, 0, 0, 0);
+              const int sc = (int)(int8_t)((scs[grp >> 2] >> (8 * (grp & 3))) & 0xFF);
+              const float w = d * (float)sc, nsw = -kSeed * w;
+#pragma unroll
+              for (int r = 0; r < 4; ++r) {
+                const h2_d hh = __builtin_bit_cast(h2_d, d8w[t >> 1][r]);
+                acc[rt][q][r] = __builtin_fmaf(seeded_times(S[r], w, nsw), (float)hh[0], acc[rt][q][r]);
+              }
             }
           }
         }
     } else {
-      const int8_t* xrow = xq + lcol * pitch + s * 256 + 64 * (lgrp >> 1) + 16 * (lgrp & 1);
+      const int8_t* xrow[RT];
+#pragma unroll
+      for (int rt = 0; rt < RT; ++rt) xrow[rt] = xq + (16 * rt + lcol) * pitch + s * 256 + 64 * (lgrp >> 1) + 16 * (lgrp & 1);
       // 6-bit scales and mins of the 8 sub-blocks (dequantize.cuh:156-163), times d and dmin
       float dw[8], mw[8];
       const uint32_t dm = valid ? b.hdr.x : 0u;
@@ -282,8 +307,6 @@ __global__ __launch_bounds__(64 * KSPL, 4) void rows16_direct_kernel(const uint8
       for (int i = 0; i < 2; ++i)
 #pragma unroll
         for (int h = 0; h < 2; ++h) {
-          // this lane's 16 activations of block 4 i + 2 (lgrp / 2) + h
-          const v4i_d av = *(const v4i_d*)(xrow + (4 * i + h) * 32);
           const v4i_d zero = {0, 0, 0, 0};
           v4i_d bv;
 #pragma unroll
@@ -293,22 +316,27 @@ __global__ __launch_bounds__(64 * KSPL, 4) void rows16_direct_kernel(const uint8
             bv[e] = (int)v;
           }
 #pragma unroll
-          for (int sel = 0; sel < 2; ++sel) {
-            const int blkno = 4 * i + 2 * sel + h;
-            const v4i_d asel = (lgrp >> 1) == sel ? av : zero;
-            const v4i_d S = __builtin_amdgcn_mfma_i32_16x16x64_i8(asel, bv, seed, 0, 0, 0);
-            const uint4 x4 = *(const uint4*)(xsc + (s * 8 + blkno) * 16 + 4 * lgrp);
-            const uint32_t scw[4] = {x4.x, x4.y, x4.z, x4.w};
-            const float w = dw[blkno], nsw = -kSeed * w, nm = -mw[blkno];
+          for (int rt = 0; rt < RT; ++rt) {
+            // this lane's 16 activations of block 4 i + 2 (lgrp / 2) + h
+            const v4i_d av = *(const v4i_d*)(xrow[rt] + (4 * i + h) * 32);
 #pragma unroll
-            for (int r = 0; r < 4; ++r) {
-              const h2_d hh = __builtin_bit_cast(h2_d, scw[r]);
-              if constexpr (GSUM) {   // d8 * (S * dw - m * sum(q8)): the offset joins the block sum before d8 is applied
-                const float u = __builtin_fmaf((float)hh[1], nm, seeded_times(S[r], w, nsw));
-                acc[q][r] = __builtin_fmaf(u, (float)hh[0], acc[q][r]);
-              } else {
-                acc[q][r] = __builtin_fmaf(seeded_times(S[r], w, nsw), (float)hh[0], acc[q][r]);
-                acc[q][r] = __builtin_fmaf((float)hh[1], nm, acc[q][r]);
+            for (int sel = 0; sel < 2; ++sel) {
+              const int blkno = 4 * i + 2 * sel + h;
+              const v4i_d asel = (lgrp >> 1) == sel ? av : zero;
+              const v4i_d S = __builtin_amdgcn_mfma_i32_16x16x64_i8(asel, bv, seed, 0, 0, 0);
+              const uint4 x4 = *(const uint4*)(xsc + (s * 8 + blkno) * XR + 16 * rt + 4 * lgrp);
+              const uint32_t scw[4] = {x4.x, x4.y, x4.z, x4.w};
+              const float w = dw[blkno], nsw = -kSeed * w, nm = -mw[blkno];
+#pragma unroll
+              for (int r = 0; r < 4; ++r) {
+                const h2_d hh = __builtin_bit_cast(h2_d, scw[r]);
+                if constexpr (GSUM) {   // d8 * (S * dw - m * sum(q8)): the offset joins the block sum before d8 is applied
+                  const float u = __builtin_fmaf((float)hh[1], nm, seeded_times(S[r], w, nsw));
+                  acc[rt][q][r] = __builtin_fmaf(u, (float)hh[0], acc[rt][q][r]);
+                } else {
+                  acc[rt][q][r] = __builtin_fmaf(seeded_times(S[r], w, nsw), (float)hh[0], acc[rt][q][r]);
+                  acc[rt][q][r] = __builtin_fmaf((float)hh[1], nm, acc[rt][q][r]);
+                }
               }
             }
           }
@@ -337,34 +365,41 @@ __global__ __launch_bounds__(64 * KSPL, 4) void rows16_direct_kernel(const uint8
 
   // ---- the KSPL partial tiles are added in the order of K
   __syncthreads();                                        // every wave is done with the activations
-  float* red = (float*)smem;                              // [KSPL][16][N_T]
+  float* red = (float*)smem;                              // [KSPL][XR][N_T]
 #pragma unroll
-  for (int r = 0; r < 4; ++r)
+  for (int rt = 0; rt < RT; ++rt)
 #pragma unroll
-    for (int q = 0; q < NP; ++q) red[(ks * 16 + 4 * lgrp + r) * N_T + 16 * q + lcol] = acc[q][r];
+    for (int r = 0; r < 4; ++r)
+#pragma unroll
+      for (int q = 0; q < NP; ++q) red[(ks * XR + 16 * rt + 4 * lgrp + r) * N_T + 16 * q + lcol] = acc[rt][q][r];
   __syncthreads();
-  float* const mine = a.gsplits > 1 ? a.partial + ((int64_t)tile * a.gsplits + gs) * (16 * N_T) : nullptr;
-  for (int e = tid; e < 16 * N_T; e += NT) {
+  float* const mine = a.gsplits > 1 ? a.partial + ((int64_t)tile * a.gsplits + gs) * (XR * N_T) : nullptr;
+  for (int e = tid; e < XR * N_T; e += NT) {
     float sum = red[e];
 #pragma unroll
-    for (int z = 1; z < KSPL; ++z) sum += red[z * 16 * N_T + e];
+    for (int z = 1; z < KSPL; ++z) sum += red[z * XR * N_T + e];
     const int m = e / N_T, nn = n_base + e % N_T;
     if (mine) mine[e] = sum;
     else if (m < a.M && nn < a.N) Y[(int64_t)m * a.ldy + nn] = finish<T>(sum, bias, nn);
   }
 }
 
-// How a call is laid out.  16 columns per workgroup until that gives 640 workgroups, 32 above (measured on Q4_K,
+// How a call is laid out.  Up to 16 rows: 16 columns per workgroup until that gives 640 workgroups, 32 above (measured on Q4_K,
 // K = 4096 at 16 rows: N = 4096 8.9 against 13.5 us, N = 8192 11.3, N = 14336 15.3 against 17.5 us).  Workgroups split K
 // between them when a stretch would not fit LDS (K > 4096), or down to one super-block per wave when the output has
 // fewer than 192 column groups.
 struct Direct16Plan {
-  int np, tiles, gsplits, per_wg;   // np: 16-column tiles per workgroup
-  int64_t partial_bytes() const { return gsplits > 1 ? (int64_t)tiles * gsplits * (16 * 16 * np * 4) : 0; }
+  int np, rt, tiles, gsplits, per_wg;   // np: 16-column tiles per workgroup; rt: 16-row tiles of X (1 or 2)
+  int64_t partial_bytes() const { return gsplits > 1 ? (int64_t)tiles * gsplits * (16 * rt * 16 * np * 4) : 0; }
 };
-static Direct16Plan direct16_plan(int N, int K, int64_t partial_bytes_available) {
+static Direct16Plan direct16_plan(int M, int N, int K, int64_t partial_bytes_available) {
   Direct16Plan p;
-  p.np = (N + 31) / 32 >= 320 ? 2 : 1;
+  p.rt = M > 16 ? 2 : 1;
+  const int tiles16 = (N + 15) / 16;
+  // 32 rows of X fill LDS, so one workgroup runs per CU: columns per workgroup so that one round of workgroups covers
+  // the output where it can (Q4_K [14336,4096] at 32 rows: 64 columns 22 us, 32 columns 26 us)
+  if (p.rt == 2) p.np = tiles16 <= 256 ? 1 : tiles16 <= 512 ? 2 : 4;
+  else p.np = (N + 31) / 32 >= 320 ? 2 : 1;
   p.tiles = (N + 16 * p.np - 1) / (16 * p.np);
   const int nsb = K / 256;
   p.gsplits = (nsb + kDirectMaxSb - 1) / kDirectMaxSb;
@@ -378,32 +413,32 @@ static Direct16Plan direct16_plan(int N, int K, int64_t partial_bytes_available)
   }
   return p;
 }
-int64_t rows16_direct_partial_bytes(int N, int K) { return K % 256 ? 0 : direct16_plan(N, K, INT64_MAX).partial_bytes(); }
+int64_t rows16_direct_partial_bytes(int M, int N, int K) { return K % 256 || M > 32 ? 0 : direct16_plan(M, N, K, INT64_MAX).partial_bytes(); }
 
 // bytes of 256 values
 static inline int direct_block_bytes(int type) {
   return type == T_Q6_K ? 210 : type == T_Q5_K ? 176 : type == T_Q4_0 ? 8 * 18 : type == T_Q8_0 ? 8 * 34 : 144;
 }
 
-template <typename T, int NP, int FMT, bool GSUM>
+template <typename T, int NP, int FMT, bool GSUM, int RT = 1>
 static int rows16_direct_launch(const void* W, const void* ws, void* Y, int M, int N, int K, float* partial, const Direct16Plan& p,
                                 hipStream_t stream, const LinearArgs& la) {
-  constexpr int KSPL = kDirectKspl, N_T = 16 * NP, XROWS = FMT == DIRECT_Q4_K || FMT == DIRECT_Q5_K ? 16 : 17;
+  constexpr int KSPL = kDirectKspl, N_T = 16 * NP, XROWS = FMT == DIRECT_Q4_K || FMT == DIRECT_Q5_K ? 16 * RT : 16 * RT + 1;
   constexpr int BS = FMT == DIRECT_Q6_K ? 210 : FMT == DIRECT_Q5_K ? 176 : FMT == DIRECT_Q4_0 ? 8 * 18 : FMT == DIRECT_Q8_0 ? 8 * 34 : 144;
-  const size_t act = (size_t)XROWS * (p.per_wg * 256 + 16) + (size_t)p.per_wg * 8 * 16 * 4, red = (size_t)KSPL * 16 * N_T * 4;
+  const size_t act = (size_t)XROWS * (p.per_wg * 256 + 16) + (size_t)p.per_wg * 8 * 16 * RT * 4, red = (size_t)KSPL * 16 * RT * N_T * 4;
   const size_t lds = act > red ? act : red;
-  auto kern = rows16_direct_kernel<T, KSPL, NP, FMT, GSUM>;
+  auto kern = rows16_direct_kernel<T, KSPL, NP, FMT, GSUM, RT>;
   if (lds > 65536) {
     static std::atomic<uint64_t> done{0};
-    allow_large_lds(kern, 80 * 1024, done);
+    allow_large_lds(kern, RT * 80 * 1024, done);
   }
   Direct16Args a = {M, N, K, (int)q8_kp(K), p.gsplits, p.per_wg, q8_row_bytes(K), la.w_pitch ? la.w_pitch : (int64_t)(K / 256) * BS,
                     la.ldy ? la.ldy : (int64_t)N, partial};
   hipLaunchKernelGGL(kern, dim3(p.tiles * p.gsplits), dim3(64 * KSPL), lds, stream, (const uint8_t*)W, (const char*)ws, (T*)Y,
                      (const T*)la.bias, a);
   if (p.gsplits > 1)
-    hipLaunchKernelGGL((mmqi_reduce_kernel<16, N_T, T>), dim3(p.tiles, 1), dim3(256), 0, stream, partial, (T*)Y, M, N, 1, 0, p.gsplits,
-                       a.ldy, (const T*)la.bias);
+    hipLaunchKernelGGL((mmqi_reduce_kernel<16 * RT, N_T, T>), dim3(p.tiles, 1), dim3(256), 0, stream, partial, (T*)Y, M, N, 1, 0,
+                       p.gsplits, a.ldy, (const T*)la.bias);
   return launch_status();
 }
 
@@ -412,8 +447,20 @@ static int rows16_direct_typed(const void* W, const void* ws, void* Y, int M, in
                                hipStream_t stream, const LinearArgs& la, bool gemv_sums) {
   if constexpr (FMT == DIRECT_Q4_K || FMT == DIRECT_Q5_K) {   // (the two operators agree on the other formats)
     if (gemv_sums) {
+      if (p.rt == 2) {   // 17 .. 32 rows
+        if (p.np == 4) return rows16_direct_launch<T, 4, FMT, true, 2>(W, ws, Y, M, N, K, partial, p, stream, la);
+        if (p.np == 2) return rows16_direct_launch<T, 2, FMT, true, 2>(W, ws, Y, M, N, K, partial, p, stream, la);
+        return rows16_direct_launch<T, 1, FMT, true, 2>(W, ws, Y, M, N, K, partial, p, stream, la);
+      }
       if (p.np == 2) return rows16_direct_launch<T, 2, FMT, true>(W, ws, Y, M, N, K, partial, p, stream, la);
       return rows16_direct_launch<T, 1, FMT, true>(W, ws, Y, M, N, K, partial, p, stream, la);
+    }
+  }
+  if constexpr (FMT == DIRECT_Q4_K || FMT == DIRECT_Q5_K || FMT == DIRECT_Q6_K) {
+    if (p.rt == 2) {   // 17 .. 32 rows
+      if (p.np == 4) return rows16_direct_launch<T, 4, FMT, false, 2>(W, ws, Y, M, N, K, partial, p, stream, la);
+      if (p.np == 2) return rows16_direct_launch<T, 2, FMT, false, 2>(W, ws, Y, M, N, K, partial, p, stream, la);
+      return rows16_direct_launch<T, 1, FMT, false, 2>(W, ws, Y, M, N, K, partial, p, stream, la);
     }
   }
   if (p.np == 2) return rows16_direct_launch<T, 2, FMT, false>(W, ws, Y, M, N, K, partial, p, stream, la);
@@ -422,11 +469,12 @@ static int rows16_direct_typed(const void* W, const void* ws, void* Y, int M, in
 
 // Whether rows16_direct() would run this call.
 bool rows16_direct_takes(const void* W, int64_t w_pitch, int type, int M, int N, int K, int64_t partial_bytes) {
-  if ((type != T_Q4_K && type != T_Q5_K && type != T_Q6_K && type != T_Q4_0 && type != T_Q8_0) || M > 16 || K % 256) return false;
+  const bool kquant = type == T_Q4_K || type == T_Q5_K || type == T_Q6_K;
+  if ((!kquant && type != T_Q4_0 && type != T_Q8_0) || M > (kquant ? 32 : 16) || K % 256) return false;
   const int64_t pitch = w_pitch ? w_pitch : (int64_t)(K / 256) * direct_block_bytes(type);
   // (the blocks of the other formats are at even addresses anyway)
   if ((type == T_Q4_K || type == T_Q5_K) && (((uintptr_t)W & 15) || (pitch & 15))) return false;
-  return direct16_plan(N, K, partial_bytes).gsplits != 0;
+  return direct16_plan(M, N, K, partial_bytes).gsplits != 0;
 }
 
 // Whether the kernel is the faster route for a call it can run.  The K-quants: always on the tile operator's side
@@ -444,12 +492,13 @@ bool rows16_direct_pays(int type, int M, int64_t N, int64_t K, bool against_gemv
   return M >= 9 && K <= 256 * kDirectMaxSb && (type != T_Q8_0 || N * K <= (32 << 20));
 }
 
-// Q4_K, Q5_K (W and its row pitch 16-byte aligned), Q6_K, Q4_0 or Q8_0, at most 16 rows of X; GGUF_NOT_TAKEN otherwise.
+// Q4_K, Q5_K (W and its row pitch 16-byte aligned), Q6_K with at most 32 rows of X, Q4_0 or Q8_0 with at most 16;
+// GGUF_NOT_TAKEN otherwise.
 // gemv_sums: the GEMV operator's offset term (see GSUM) instead of the tile operator's.
 int rows16_direct(const void* W, const void* ws, void* Y, int dtype, int type, int M, int N, int K, float* partial, int64_t partial_bytes,
                   hipStream_t s, const LinearArgs& la, bool gemv_sums) {
   if (!rows16_direct_takes(W, la.w_pitch, type, M, N, K, partial_bytes)) return GGUF_NOT_TAKEN;
-  const Direct16Plan p = direct16_plan(N, K, partial_bytes);
+  const Direct16Plan p = direct16_plan(M, N, K, partial_bytes);
   if (type == T_Q6_K) {
     GGUF_DISPATCH_DTYPE(dtype, return (rows16_direct_typed<scalar_t, DIRECT_Q6_K>(W, ws, Y, M, N, K, partial, p, s, la, gemv_sums)));
     return GGUF_ERR_DTYPE;
