@@ -238,6 +238,41 @@ def test_mmvq_five_rows_or_more_of_a_large_matrix(qtype, dt):
     assert torch.all(wide[:, :8] == 3.0)
 
 
+SPAN_TYPES = [o.Q4_0, o.Q4_1, o.Q5_0, o.Q5_1, o.Q8_0, o.Q2_K, o.Q3_K, o.Q4_K, o.Q5_K, o.Q6_K, o.IQ4_NL]
+
+
+@pytest.mark.parametrize("dt", ["f32", "f16"])
+@pytest.mark.parametrize("qtype", SPAN_TYPES)
+def test_mmvq_rows_of_whole_spans_through_lds(qtype, dt):
+    """One or two rows of X over a matrix whose rows are whole 16-byte pieces at 16-byte aligned addresses: a wave fetches
+    its 2048-value stretch of a row as 16-byte pieces, every byte once, and the lanes cut their blocks out of a copy in LDS
+    (at 2-byte alignment for the 18-, 22-, 34-, 110- and 210-byte blocks).  Shards whose rows are a wider pitch apart
+    take the same route when pitch and address are multiples of 16 and the per-lane loads when they are not; all must
+    agree with the GEMV oracle."""
+    ops = _ops()
+    rng = np.random.default_rng(1700 + qtype)
+    tol = 1e-5 if dt == "f32" else 1e-3
+    # one, two, three waves per row; then rows whose last wave has 48, 32 or 16 of its 64 blocks (a shorter last stretch),
+    # for the formats whose rows still are whole 16-byte pieces
+    for n, k in [(4608, 2048), (2400, 4096), (1300, 6144), (2400, 3584), (1500, 5120), (5000, 1024), (1536, 2560)]:
+        w = o.make_weights(rng, qtype, n, k)
+        wd = _to_dev(w)
+        for m in (1, 2):
+            xd, xv = _x(rng, m, k, dt)
+            y = ops.ggml_mul_mat_vec_a8(wd, xd, qtype, n)
+            assert o.rel_l2(y.float().cpu().numpy(), o.mul_mat_a8(w, xv, qtype, n, "mmvq")) <= tol, (o.TYPE_NAMES[qtype], n, k, m)
+    # a shard inside a wider tensor: rows `extra` bytes further apart, starting `lead` bytes in
+    n, k = 2400, 4096
+    w = o.make_weights(rng, qtype, n, k)
+    xd, xv = _x(rng, 1, k, dt)
+    want = o.mul_mat_a8(w, xv, qtype, n, "mmvq")
+    for lead, extra in [(32, 48), (6, 48), (32, 10)]:
+        wide = torch.zeros((n, lead + w.shape[1] + extra), dtype=torch.uint8, device="cuda")
+        wide[:, lead:lead + w.shape[1]] = _to_dev(w)
+        y = ops.ggml_mul_mat_vec_a8(wide[:, lead:lead + w.shape[1]], xd, qtype, n)
+        assert o.rel_l2(y.float().cpu().numpy(), want) <= tol, (o.TYPE_NAMES[qtype], lead, extra)
+
+
 def test_empty_and_errors():
     ops = _ops()
     rng = np.random.default_rng(3)

@@ -94,6 +94,21 @@ __device__ __forceinline__ uint32_t ld_block_dwords(const uint8_t* p, uint32_t (
 __device__ __forceinline__ uint32_t funnel(uint32_t lo, uint32_t hi, uint32_t bits) {
   return (uint32_t)((((uint64_t)hi << 32) | lo) >> bits);
 }
+// The same cut from a copy of the blocks in LDS: the ND dwords from the dword boundary at or below byte off (even) of
+// base (16-byte aligned); returns the bit offset of that byte inside w[0].
+template <int ND>
+__device__ __forceinline__ uint32_t lds_block_dwords(const char* base, int off, uint32_t (&w)[ND]) {
+  const uint32_t* q = (const uint32_t*)(base + (off & ~3));
+#pragma unroll
+  for (int i = 0; i < ND; ++i) w[i] = q[i];
+  return (uint32_t)(off & 2) * 8;
+}
+// eight bytes at an even offset of such a copy (touches the dword behind them when the offset is a multiple of four)
+__device__ __forceinline__ uint2 lds_cut8(const char* base, int off) {
+  uint32_t w[3];
+  const uint32_t sh = lds_block_dwords(base, off, w);
+  return make_uint2(funnel(w[0], w[1], sh), funnel(w[1], w[2], sh));
+}
 __device__ __forceinline__ float ld_f16(const void* p) { return (float)ld<_Float16>(p); }
 __device__ __forceinline__ _Float16 ld_h(const void* p) { return ld<_Float16>(p); }
 

@@ -293,20 +293,37 @@ __device__ unsigned long long g_mmvq_phases[1024 * 2 * 8];
 // streaming kernel as plain 16-byte pieces, lane after lane, every byte requested once, and handed to the lanes
 // through LDS.  Requests that never meet a second request for the same cache line can carry the non-temporal hint,
 // which the memory system rewards (a plain streaming read of 33 MB: 6.7 us with the hint, 7.3 us without).
+#ifndef MMVQ_STAGED_MT
+#define MMVQ_STAGED_MT 2
+#endif
 template <class F, class = void> struct SpanOf { static constexpr int value = 0; };
 template <class F> struct SpanOf<F, std::void_t<decltype(F::SPAN)>> { static constexpr int value = F::SPAN; };
+template <class F, class = void> struct SpanSlack { static constexpr int value = 0; };   // bytes a reader may touch behind the last span
+template <class F> struct SpanSlack<F, std::void_t<decltype(F::SPAN_SLACK)>> { static constexpr int value = F::SPAN_SLACK; };
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
+// Orders this wave's LDS accesses before the call against those after it, for data that lanes hand to each other
+// through LDS without a workgroup barrier (the hardware keeps one wave's LDS accesses in order).
+__device__ __forceinline__ void wave_lds_fence() {
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
 template <int SPAN> struct SpanRegs {
-  static_assert(SPAN > 1024 && SPAN <= 2048 && SPAN % 16 == 0, "one full piece per lane and a tail of fewer than 64 pieces");
-  u32x4_t a, b;   // pieces lane and 64 + lane % TAIL of the span
-  static constexpr int TAIL = (SPAN - 1024) / 16;
-  __device__ __forceinline__ void load(const uint8_t* span, int lane) {
-    a = __builtin_nontemporal_load((const u32x4_t*)(span + 16 * lane));
-    b = __builtin_nontemporal_load((const u32x4_t*)(span + 1024 + 16 * (lane % TAIL)));
+  static_assert(SPAN % 16 == 0 && SPAN > 0, "whole 16-byte pieces");
+  static constexpr int PIECES = SPAN / 16, NR = (PIECES + 63) / 64, TAIL = PIECES - 64 * (NR - 1);
+  u32x4_t r[NR];   // pieces lane, 64 + lane, ...; the last set has TAIL pieces (idle lanes repeat one of them)
+  // `valid` pieces of the span belong to the row (the last stretch of a row may be shorter): later ones repeat the last
+  __device__ __forceinline__ void load(const uint8_t* span, int lane, int valid) {
+#pragma unroll
+    for (int i = 0; i < NR; ++i) {
+      const int p = 64 * i + ((i < NR - 1 || TAIL == 64) ? lane : lane % TAIL);
+      r[i] = __builtin_nontemporal_load((const u32x4_t*)(span + 16 * min(p, valid - 1)));
+    }
   }
   __device__ __forceinline__ void store(char* lds, int lane) const {
-    *(u32x4_t*)(lds + 16 * lane) = a;
-    if (lane < TAIL) *(u32x4_t*)(lds + 1024 + 16 * lane) = b;
+#pragma unroll
+    for (int i = 0; i < NR; ++i)
+      if (i < NR - 1 || TAIL == 64 || lane < TAIL) *(u32x4_t*)(lds + 1024 * i + 16 * lane) = r[i];
   }
 };
 
@@ -378,11 +395,13 @@ __device__ __forceinline__ void mmvq_stream_body(const uint8_t* __restrict__ W, 
   // Loads are issued unconditionally (row index clamped into the band) so that every iteration issues the
   // same number of loads and the hardware load counter can be waited on exactly, slot by slot.
   const uint8_t* wbase = W + (int64_t)r_begin * rowbytes;
+  // pieces of this wave's stretch that lie inside the row
+  const int span_valid = STAGED ? max(1, min(SPAN / 16, (K / F::QK) * F::BS / 16 - (wave_on ? step : 0) * (SPAN / 16))) : 0;
   auto load_row = [&](int i) {
     const int row = min(slot + slots * i, nrows - 1);
-    if constexpr (STAGED) {   // (the host takes this variant only for rows that are whole spans)
+    if constexpr (STAGED) {   // (the host takes this variant only for rows of whole 16-byte pieces at aligned addresses)
       SpanRegs<SPAN> r;
-      r.load(wbase + (int64_t)row * rowbytes + (int64_t)(wave_on ? step : 0) * SPAN, lane);
+      r.load(wbase + (int64_t)row * rowbytes + (int64_t)(wave_on ? step : 0) * SPAN, lane, span_valid);
       return r;
     } else {
       return F::load(wbase + (int64_t)row * rowbytes, 0, u, tab);
@@ -507,9 +526,14 @@ __device__ __forceinline__ void mmvq_stream_body(const uint8_t* __restrict__ W, 
       if constexpr (STAGED) {
         // through LDS to the lanes that use the bytes (one wave's LDS accesses keep their order: no barrier), and the
         // slot is free for the next request before the arithmetic starts
+        // (The fences are for the compiler, which reasons about one lane and would otherwise keep a value read from
+        //  the previous row's copy where this lane's own stores cannot reach it, or move the next row's stores above
+        //  these reads; they cost no instruction.)
         pre[d].store(stage, lane);
+        wave_lds_fence();
         pre[d] = load_row(i + D);
         cur = F::from_span(stage, lane);
+        wave_lds_fence();
       } else {
         cur = pre[d];
       }
@@ -598,11 +622,13 @@ static bool launch_stream(const void* W, const T* X, T* Y, int N, int K, hipStre
   const auto go = [&](auto full) {
     constexpr bool FULL = decltype(full)::value;
     if constexpr (MT <= 4) {
-      if constexpr (MT == 1 && NW == MMVQ_NW && SpanOf<F>::value > 0) {
-        // rows that are whole spans of 16-byte aligned pieces: every byte is requested once (see SpanRegs)
+      // (for Q4_K, whose per-lane loads are aligned 16-byte pieces already, the trip through LDS costs the 8-wave kernel
+      //  of the small matrices as much as it gains; [4096,4096]: Q8_0 6.4 -> 5.1 us, Q4_0 5.1 -> 4.4 us, Q6_K 6.2 -> 5.4 us)
+      if constexpr (MT <= MMVQ_STAGED_MT && (NW == MMVQ_NW || !std::is_same<F, FmtQ4_K>::value) && SpanOf<F>::value > 0) {
+        // rows of whole 16-byte pieces at aligned addresses: every byte is requested once (see SpanRegs)
         const int64_t pitch = la.w_pitch ? la.w_pitch : (int64_t)(K / F::QK) * F::BS;
-        const size_t lds_staged = lds + (size_t)NW * SpanOf<F>::value;
-        if (per_wave >= MMVQ_DEPTH && nb % 64 == 0 && pitch % 16 == 0 && (uintptr_t)W % 16 == 0 && lds_staged <= 160 * 1024) {
+        const size_t lds_staged = lds + (size_t)NW * SpanOf<F>::value + SpanSlack<F>::value;
+        if (per_wave >= MMVQ_DEPTH && (int64_t)(K / F::QK) * F::BS % 16 == 0 && pitch % 16 == 0 && (uintptr_t)W % 16 == 0 && lds_staged <= 160 * 1024) {
           launch_stream_d<F, MT, MMVQ_DEPTH, T, TILE, FULL, NW, true>(W, X, Y, N, K, rows_per_wg, grid, lds_staged, la, stream, m_act);
           return;
         }
@@ -646,9 +672,11 @@ static bool launch_stream_moe(const void* W, const T* X, T* Y, int N, int K, con
     }
     hipLaunchKernelGGL(kern, dim3(grid, pairs), dim3(64 * NW), bytes, stream, (const uint8_t*)W, X, Y, moe, geom);
   };
-  if constexpr (SpanOf<F>::value > 0) {
-    const size_t lds_staged = lds + (size_t)NW * SpanOf<F>::value;
-    if (per_wave >= MMVQ_DEPTH && nb % 64 == 0 && pitch % 16 == 0 && (uintptr_t)W % 16 == 0 && lds_staged <= 160 * 1024) {
+  // (experts shared between pairs come from the caches at more than the HBM rate, and there the trip through LDS costs
+  //  more than the tidier requests gain: Q4_0, 64 experts [2048,2048], 8 tokens 45 -> 48 us; Q4_K keeps it)
+  if constexpr (std::is_same<F, FmtQ4_K>::value) {
+    const size_t lds_staged = lds + (size_t)NW * SpanOf<F>::value + SpanSlack<F>::value;
+    if (per_wave >= MMVQ_DEPTH && (int64_t)(K / F::QK) * F::BS % 16 == 0 && pitch % 16 == 0 && (uintptr_t)W % 16 == 0 && lds_staged <= 160 * 1024) {
       go(mmvq_stream_moe_kernel<F, NW, MMVQ_DEPTH, T, true, GATED>, lds_staged);
       return true;
     }

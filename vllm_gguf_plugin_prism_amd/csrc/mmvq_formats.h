@@ -12,11 +12,23 @@ struct FmtQ4_0 {
   static __device__ __forceinline__ void init_tables(char*) {}
   static __device__ __forceinline__ Regs load(const uint8_t* row, int u0, int u, const char*) {
     uint32_t w[5];
-    const uint32_t sh = ld_block_dwords(row + (int64_t)(u0 + u) * BS, w), shq = sh + 16;
+    const uint32_t sh = ld_block_dwords(row + (int64_t)(u0 + u) * BS, w);
+    return cut(w, sh);
+  }
+  static __device__ __forceinline__ Regs cut(const uint32_t (&w)[5], uint32_t sh) {
+    const uint32_t shq = sh + 16;
     Regs r;
     r.d = (uint16_t)(w[0] >> sh);
     r.q = make_uint4(funnel(w[0], w[1], shq), funnel(w[1], w[2], shq), funnel(w[2], w[3], shq), funnel(w[3], w[4], shq));
     return r;
+  }
+  // The 64 blocks a wave covers, 1152 contiguous bytes, copied to LDS: lane l cuts block l out of the dwords that cover
+  // it (the last block may touch the dword behind the span).
+  static constexpr int SPAN = 64 * BS, SPAN_SLACK = 16;
+  static __device__ __forceinline__ Regs from_span(const char* span, int lane) {
+    uint32_t w[5];
+    const uint32_t sh = lds_block_dwords(span, lane * BS, w);
+    return cut(w, sh);
   }
   struct ActRegs { int4 lo, hi; float d, a; };
   static __device__ __forceinline__ ActRegs load_act(const Act& x, int u) {
@@ -46,12 +58,22 @@ struct FmtQ8_0 {
   static __device__ __forceinline__ void init_tables(char*) {}
   static __device__ __forceinline__ Regs load(const uint8_t* row, int u0, int u, const char*) {
     uint32_t w[9];
-    const uint32_t sh = ld_block_dwords(row + (int64_t)(u0 + u) * BS, w), shq = sh + 16;
+    const uint32_t sh = ld_block_dwords(row + (int64_t)(u0 + u) * BS, w);
+    return cut(w, sh);
+  }
+  static __device__ __forceinline__ Regs cut(const uint32_t (&w)[9], uint32_t sh) {
+    const uint32_t shq = sh + 16;
     Regs r;
     r.d = (uint16_t)(w[0] >> sh);
     r.q0 = make_uint4(funnel(w[0], w[1], shq), funnel(w[1], w[2], shq), funnel(w[2], w[3], shq), funnel(w[3], w[4], shq));
     r.q1 = make_uint4(funnel(w[4], w[5], shq), funnel(w[5], w[6], shq), funnel(w[6], w[7], shq), funnel(w[7], w[8], shq));
     return r;
+  }
+  static constexpr int SPAN = 64 * BS, SPAN_SLACK = 16;   // 2176 bytes: three pieces for the first eight lanes
+  static __device__ __forceinline__ Regs from_span(const char* span, int lane) {
+    uint32_t w[9];
+    const uint32_t sh = lds_block_dwords(span, lane * BS, w);
+    return cut(w, sh);
   }
   struct ActRegs { int4 a0, a1; float d; };
   static __device__ __forceinline__ ActRegs load_act(const Act& x, int u) {
@@ -145,6 +167,22 @@ struct FmtQ6_K {
     r.qh = ld<uint2>(b + 128 + 32 * h + 8 * cc);
     r.sc = ld<uint2>(b + 192 + 8 * h);
     r.d = ld<uint16_t>(b + 208);
+    return r;
+  }
+  // The 64 units a wave covers are 8 whole blocks, 1680 contiguous bytes.  In the copy of them in LDS the blocks with
+  // an odd number start two bytes into a dword (210 = 4 * 52 + 2): a lane reads the dwords that cover a field and
+  // cuts it out with funnel shifts.  (The last field of the last block may touch the dword behind the span.)
+  static constexpr int SPAN = 8 * BS, SPAN_SLACK = 16;
+  static __device__ __forceinline__ Regs from_span(const char* span, int lane) {
+    const int c = lane & 7, h = c >> 2, cc = c & 3, b = (lane >> 3) * BS;
+    Regs r;
+    r.qla = lds_cut8(span, b + 64 * h + 8 * cc);
+    r.qlb = lds_cut8(span, b + 64 * h + 32 + 8 * cc);
+    r.qh = lds_cut8(span, b + 128 + 32 * h + 8 * cc);
+    r.sc = lds_cut8(span, b + 192 + 8 * h);
+    uint32_t w[1];
+    const uint32_t sh = lds_block_dwords(span, b + 208, w);
+    r.d = (uint16_t)(w[0] >> sh);
     return r;
   }
   struct ActRegs { int2 a[4]; float d8[4]; int ones[4]; };
@@ -355,6 +393,11 @@ struct FmtQ4_1 {
     const uint8_t* b = row + (int64_t)(u0 + u) * BS;
     Regs r; r.dm = ld<uint32_t>(b); r.q = ld<uint4>(b + 4); return r;
   }
+  static constexpr int SPAN = 64 * BS;
+  static __device__ __forceinline__ Regs from_span(const char* span, int lane) {
+    const uint32_t* w = (const uint32_t*)(span + lane * BS);
+    Regs r; r.dm = w[0]; r.q = make_uint4(w[1], w[2], w[3], w[4]); return r;
+  }
   typedef FmtQ4_0::ActRegs ActRegs;
   static __device__ __forceinline__ ActRegs load_act(const Act& x, int u) { return FmtQ4_0::load_act(x, u); }
   static __device__ __forceinline__ float dot(const Regs& r, const ActRegs& x, int u) {
@@ -386,10 +429,29 @@ struct FmtQ5 {
     if (HAS_M) { r.dm = ld<uint32_t>(b); r.qh = ld<uint32_t>(b + 4); r.q = ld<uint4>(b + 8); }
     else {
       uint32_t w[6];
-      const uint32_t sh = ld_block_dwords(b, w), shq = sh + 16;
-      r.dm = (w[0] >> sh) & 0xFFFFu;
-      r.qh = funnel(w[0], w[1], shq);
-      r.q = make_uint4(funnel(w[1], w[2], shq), funnel(w[2], w[3], shq), funnel(w[3], w[4], shq), funnel(w[4], w[5], shq));
+      const uint32_t sh = ld_block_dwords(b, w);
+      r = cut(w, sh);
+    }
+    return r;
+  }
+  static __device__ __forceinline__ Regs cut(const uint32_t (&w)[6], uint32_t sh) {
+    const uint32_t shq = sh + 16;
+    Regs r;
+    r.dm = (w[0] >> sh) & 0xFFFFu;
+    r.qh = funnel(w[0], w[1], shq);
+    r.q = make_uint4(funnel(w[1], w[2], shq), funnel(w[2], w[3], shq), funnel(w[3], w[4], shq), funnel(w[4], w[5], shq));
+    return r;
+  }
+  static constexpr int SPAN = 64 * BS, SPAN_SLACK = 16;
+  static __device__ __forceinline__ Regs from_span(const char* span, int lane) {
+    Regs r;
+    if (HAS_M) {
+      const uint32_t* w = (const uint32_t*)(span + lane * BS);
+      r.dm = w[0]; r.qh = w[1]; r.q = make_uint4(w[2], w[3], w[4], w[5]);
+    } else {
+      uint32_t w[6];
+      const uint32_t sh = lds_block_dwords(span, lane * BS, w);
+      r = cut(w, sh);
     }
     return r;
   }
@@ -422,6 +484,8 @@ struct FmtIQ4_NL {
   typedef FmtQ4_0::Regs Regs;
   static __device__ __forceinline__ void init_tables(char*) {}
   static __device__ __forceinline__ Regs load(const uint8_t* row, int u0, int u, const char* t) { return FmtQ4_0::load(row, u0, u, t); }
+  static constexpr int SPAN = FmtQ4_0::SPAN, SPAN_SLACK = FmtQ4_0::SPAN_SLACK;
+  static __device__ __forceinline__ Regs from_span(const char* span, int lane) { return FmtQ4_0::from_span(span, lane); }
   typedef FmtIQ4_XS::ActRegs ActRegs;
   static __device__ __forceinline__ ActRegs load_act(const Act& x, int u) { return FmtIQ4_XS::load_act(x, u); }
   static __device__ __forceinline__ float dot(const Regs& r, const ActRegs& x, int u) {
@@ -450,6 +514,14 @@ struct FmtQ2_K {
     const int uu = u0 + u, sb = uu >> 3, c = uu & 7, n = c >> 2, cc = c & 3;
     const uint8_t* b = row + (int64_t)sb * BS;
     Regs r; r.q = ld<uint2>(b + 16 + 32 * n + 8 * cc); r.sc = ld<uint2>(b + 8 * n); r.dm = ld<uint32_t>(b + 80); return r;
+  }
+  static constexpr int SPAN = 8 * BS;   // 8 blocks, 672 bytes, every field of the LDS copy at a dword boundary
+  static __device__ __forceinline__ Regs from_span(const char* span, int lane) {
+    const int c = lane & 7, n = c >> 2, cc = c & 3;
+    const uint32_t* w = (const uint32_t*)(span + (lane >> 3) * BS);
+    Regs r;
+    r.q = make_uint2(w[4 + 8 * n + 2 * cc], w[5 + 8 * n + 2 * cc]); r.sc = make_uint2(w[2 * n], w[2 * n + 1]); r.dm = w[20];
+    return r;
   }
   typedef FmtQ6_K::ActRegs ActRegs;
   static __device__ __forceinline__ ActRegs load_act(const Act& x, int u) { return FmtQ6_K::load_act(x, u); }
@@ -484,6 +556,17 @@ struct FmtQ3_K {
     r.sc01 = ld<uint2>(b + 96); r.sc2 = ld<uint32_t>(b + 104); r.d = ld<uint16_t>(b + 108);
     return r;
   }
+  static constexpr int SPAN = 8 * BS, SPAN_SLACK = 16;   // 8 blocks, 880 bytes, at 2-byte alignment in the LDS copy
+  static __device__ __forceinline__ Regs from_span(const char* span, int lane) {
+    const int c = lane & 7, n = c >> 2, cc = c & 3, b = (lane >> 3) * BS;
+    Regs r;
+    r.q = lds_cut8(span, b + 32 + 32 * n + 8 * cc); r.hm = lds_cut8(span, b + 8 * cc);
+    uint32_t w[5];    // bytes 96 .. 109: twelve of scales and d
+    const uint32_t sh = lds_block_dwords(span, b + 96, w);
+    r.sc01 = make_uint2(funnel(w[0], w[1], sh), funnel(w[1], w[2], sh)); r.sc2 = funnel(w[2], w[3], sh);
+    r.d = (uint16_t)(funnel(w[3], w[4], sh));
+    return r;
+  }
   typedef FmtQ6_K::ActRegs ActRegs;
   static __device__ __forceinline__ ActRegs load_act(const Act& x, int u) { return FmtQ6_K::load_act(x, u); }
   static __device__ __forceinline__ float dot(const Regs& r, const ActRegs& x, int u) {
@@ -515,6 +598,12 @@ struct FmtQ5_K {
     const int uu = u0 + u, sb = uu >> 3, c = uu & 7;
     const uint8_t* b = row + (int64_t)sb * BS;
     Regs r; r.hdr = ld<uint4>(b); r.q = ld<uint4>(b + 48 + 16 * c); r.qh = ld<uint4>(b + 16 + 16 * (c & 1)); return r;
+  }
+  static constexpr int SPAN = 8 * BS;   // 8 blocks, 1408 bytes
+  static __device__ __forceinline__ Regs from_span(const char* span, int lane) {
+    const char* b = span + (lane >> 3) * BS;
+    const int c = lane & 7;
+    Regs r; r.hdr = *(const uint4*)b; r.q = *(const uint4*)(b + 48 + 16 * c); r.qh = *(const uint4*)(b + 16 + 16 * (c & 1)); return r;
   }
   typedef FmtQ4_K::ActRegs ActRegs;
   static __device__ __forceinline__ ActRegs load_act(const Act& x, int u) { return FmtQ4_K::load_act(x, u); }
