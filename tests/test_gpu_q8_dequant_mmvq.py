@@ -247,8 +247,9 @@ def test_mmvq_rows_of_whole_spans_through_lds(qtype, dt):
     """One or two rows of X over a matrix whose rows are whole 16-byte pieces at 16-byte aligned addresses: a wave fetches
     its 2048-value stretch of a row as 16-byte pieces, every byte once, and the lanes cut their blocks out of a copy in LDS
     (at 2-byte alignment for the 18-, 22-, 34-, 110- and 210-byte blocks).  Shards whose rows are a wider pitch apart
-    take the same route when pitch and address are multiples of 16 and the per-lane loads when they are not; all must
-    agree with the GEMV oracle."""
+    take the same route when pitch and address are multiples of 16; when they are not, Q3_K and Q6_K (whose rows are
+    whole pieces only for K a multiple of 2048) fetch the pieces from the 16-byte boundary below each stretch and the
+    others load per lane; all must agree with the GEMV oracle."""
     ops = _ops()
     rng = np.random.default_rng(1700 + qtype)
     tol = 1e-5 if dt == "f32" else 1e-3

@@ -298,6 +298,11 @@ __device__ unsigned long long g_mmvq_phases[1024 * 2 * 8];
 #endif
 template <class F, class = void> struct SpanOf { static constexpr int value = 0; };
 template <class F> struct SpanOf<F, std::void_t<decltype(F::SPAN)>> { static constexpr int value = F::SPAN; };
+// STAGED: rows are fetched per lane (0), as whole 16-byte pieces from aligned stretches, or from stretches that start
+// at any even address
+constexpr int STAGED_ALIGNED = 1, STAGED_ANY = 2;
+template <class F, class = void> struct SpanAny { static constexpr bool value = false; };   // spans may start at any even address
+template <class F> struct SpanAny<F, std::void_t<decltype(F::SPAN_ANY)>> { static constexpr bool value = F::SPAN_ANY; };
 template <class F, class = void> struct SpanSlack { static constexpr int value = 0; };   // bytes a reader may touch behind the last span
 template <class F> struct SpanSlack<F, std::void_t<decltype(F::SPAN_SLACK)>> { static constexpr int value = F::SPAN_SLACK; };
 typedef uint32_t u32x4_t __attribute__((ext_vector_type(4)));
@@ -308,16 +313,18 @@ __device__ __forceinline__ void wave_lds_fence() {
   __builtin_amdgcn_wave_barrier();
   __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
-template <int SPAN> struct SpanRegs {
+template <int SPAN, bool ANY = false> struct SpanRegs {
   static_assert(SPAN % 16 == 0 && SPAN > 0, "whole 16-byte pieces");
-  static constexpr int PIECES = SPAN / 16, NR = (PIECES + 63) / 64, TAIL = PIECES - 64 * (NR - 1);
+  // ANY: the span starts anywhere inside its first piece, so it may reach into one piece more
+  static constexpr int PIECES = SPAN / 16 + (ANY ? 1 : 0), NR = (PIECES + 63) / 64, TAIL = PIECES - 64 * (NR - 1);
   u32x4_t r[NR];   // pieces lane, 64 + lane, ...; the last set has TAIL pieces (idle lanes repeat one of them)
-  // `valid` pieces of the span belong to the row (the last stretch of a row may be shorter): later ones repeat the last
-  __device__ __forceinline__ void load(const uint8_t* span, int lane, int valid) {
+  // `first` is the 16-byte boundary at or below the span; `valid` pieces from there hold bytes of the row (the last
+  // stretch of a row may be shorter): later ones repeat the last
+  __device__ __forceinline__ void load(const uint8_t* first, int lane, int valid) {
 #pragma unroll
     for (int i = 0; i < NR; ++i) {
       const int p = 64 * i + ((i < NR - 1 || TAIL == 64) ? lane : lane % TAIL);
-      r[i] = __builtin_nontemporal_load((const u32x4_t*)(span + 16 * min(p, valid - 1)));
+      r[i] = __builtin_nontemporal_load((const u32x4_t*)(first + 16 * min(p, valid - 1)));
     }
   }
   __device__ __forceinline__ void store(char* lds, int lane) const {
@@ -355,7 +362,7 @@ static inline StreamGeom stream_geom(int N, int K, int rows_per_wg, int64_t w_pi
 
 // GATED (one activation row only): the row of X is [gate | up], K values each, and what is quantized is
 // T(T(act(gate)) * up), the values a separate act-and-multiply kernel would have stored (fused_moe.py:44-51,80).
-template <class F, int MT, int NW, int D, typename T, bool TILE, bool FULL, bool STAGED, bool GATED>
+template <class F, int MT, int NW, int D, typename T, bool TILE, bool FULL, int STAGED, bool GATED>
 __device__ __forceinline__ void mmvq_stream_body(const uint8_t* __restrict__ W, const T* __restrict__ X, T* __restrict__ Y,
                                                  const T* __restrict__ bias, int64_t ldy, const StreamGeom& geom, int act_fn) {
   static_assert(!GATED || MT == 1, "the gated variant quantizes one row");
@@ -395,20 +402,30 @@ __device__ __forceinline__ void mmvq_stream_body(const uint8_t* __restrict__ W, 
   // Loads are issued unconditionally (row index clamped into the band) so that every iteration issues the
   // same number of loads and the hardware load counter can be waited on exactly, slot by slot.
   const uint8_t* wbase = W + (int64_t)r_begin * rowbytes;
-  // pieces of this wave's stretch that lie inside the row
-  const int span_valid = STAGED ? max(1, min(SPAN / 16, (K / F::QK) * F::BS / 16 - (wave_on ? step : 0) * (SPAN / 16))) : 0;
-  auto load_row = [&](int i) {
+  // bytes of this wave's stretch that lie inside the row
+  constexpr bool ANY = STAGED == STAGED_ANY;
+  const int span_bytes = STAGED ? max(16, min(SPAN, (K / F::QK) * F::BS - (wave_on ? step : 0) * SPAN)) : 0;
+  typedef SpanRegs<STAGED ? SPAN : 16, ANY> Span;
+  [[maybe_unused]] uint32_t mis[D];   // ANY: where in its first 16-byte piece the stretch of each row in flight starts
+  auto load_row = [&](int i, [[maybe_unused]] uint32_t& m16) {
     const int row = min(slot + slots * i, nrows - 1);
-    if constexpr (STAGED) {   // (the host takes this variant only for rows of whole 16-byte pieces at aligned addresses)
-      SpanRegs<SPAN> r;
-      r.load(wbase + (int64_t)row * rowbytes + (int64_t)(wave_on ? step : 0) * SPAN, lane, span_valid);
+    if constexpr (STAGED) {   // (the host takes this variant only for rows it can fetch as whole 16-byte pieces)
+      Span r;
+      const uint8_t* a = wbase + (int64_t)row * rowbytes + (int64_t)(wave_on ? step : 0) * SPAN;
+      if constexpr (ANY) {
+        m16 = (uint32_t)(uintptr_t)a & 15u;
+        r.load(a - m16, lane, (int)(m16 + span_bytes + 15) >> 4);
+      } else {
+        r.load(a, lane, span_bytes >> 4);
+      }
       return r;
     } else {
       return F::load(wbase + (int64_t)row * rowbytes, 0, u, tab);
     }
   };
   // this wave's staging area for one span, behind the partial sums
-  char* stage = (char*)(part + (size_t)rows_per_wg * S * 4 * MT) + (STAGED ? wave * SPAN : 0);
+  constexpr int STAGE_BYTES = STAGED ? 16 * Span::PIECES : 0;
+  char* stage = (char*)(part + (size_t)rows_per_wg * S * 4 * MT) + wave * STAGE_BYTES;
 
   // Prologue, in one basic block per variant: request this thread's first QG groups of activation values,
   // then the weights of the first D rows, then quantize the activations into LDS (four lanes per 32-value
@@ -420,7 +437,7 @@ __device__ __forceinline__ void mmvq_stream_body(const uint8_t* __restrict__ W, 
   // computed on whatever the LDS holds and never stored.
   const int rows_x = FULL ? MT : m_act;
   const int qtotal = rows_x * g8;  // a multiple of 4, so quads stay whole
-  std::conditional_t<STAGED, SpanRegs<STAGED ? SPAN : 1040>, typename F::Regs> pre[D];
+  std::conditional_t<STAGED != 0, Span, typename F::Regs> pre[D];
   const auto row_of_group = [&](int qc) { return MT == 1 ? 0 : (int)__umulhi((unsigned)qc, geom.g8_inv); };  // qc / g8
   auto quantize_group = [&](const raw8<T>& raw, const raw8<T>& up, int q) {
     const int qc = min(q, qtotal - 1);
@@ -449,7 +466,7 @@ __device__ __forceinline__ void mmvq_stream_body(const uint8_t* __restrict__ W, 
       if (qtotal <= NT) __builtin_amdgcn_s_barrier();   // (see below: the others' activation requests go first)
       GGUF_PHASE(6);
 #pragma unroll
-      for (int d = 0; d < D; ++d) pre[d] = load_row(d);
+      for (int d = 0; d < D; ++d) pre[d] = load_row(d, mis[d]);
       __builtin_amdgcn_sched_barrier(0);
       GGUF_PHASE(7);
       return;
@@ -472,7 +489,7 @@ __device__ __forceinline__ void mmvq_stream_body(const uint8_t* __restrict__ W, 
     }
     GGUF_PHASE(6);                             // activation requests are out (every wave's, where one request covers them)
 #pragma unroll
-    for (int d = 0; d < D; ++d) pre[d] = load_row(d);
+    for (int d = 0; d < D; ++d) pre[d] = load_row(d, mis[d]);
     __builtin_amdgcn_sched_barrier(0);
     GGUF_PHASE(7);                             // weight requests of the first rows are out
 #pragma unroll
@@ -516,7 +533,9 @@ __device__ __forceinline__ void mmvq_stream_body(const uint8_t* __restrict__ W, 
     act[m] = F::load_act(x, u);
   }
 
-  for (int i0 = 0; i0 < max_rows; i0 += D) {
+  // (a wave without a slot -- NW is not always a multiple of the waves a row takes -- has quantized its share of the
+  //  activations and waits at the barrier behind the loop)
+  for (int i0 = 0; wave_on && i0 < max_rows; i0 += D) {
 #pragma unroll
     for (int d = 0; d < D; ++d) {
       const int i = i0 + d;
@@ -531,8 +550,14 @@ __device__ __forceinline__ void mmvq_stream_body(const uint8_t* __restrict__ W, 
         //  these reads; they cost no instruction.)
         pre[d].store(stage, lane);
         wave_lds_fence();
-        pre[d] = load_row(i + D);
-        cur = F::from_span(stage, lane);
+        if constexpr (ANY) {
+          const int at = (int)mis[d];
+          pre[d] = load_row(i + D, mis[d]);
+          cur = F::from_span(stage, lane, at);
+        } else {
+          pre[d] = load_row(i + D, mis[d]);
+          cur = F::from_span(stage, lane);
+        }
         wave_lds_fence();
       } else {
         cur = pre[d];
@@ -542,7 +567,7 @@ __device__ __forceinline__ void mmvq_stream_body(const uint8_t* __restrict__ W, 
         const float v = F::dot(cur, act[m], u);
         acc[m] = lane_on ? v : 0.0f;
       }
-      if constexpr (!STAGED) pre[d] = load_row(i + D);  // refill the slot: D - 1 other slots are still in flight
+      if constexpr (!STAGED) pre[d] = load_row(i + D, mis[d]);  // refill the slot: D - 1 other slots are still in flight
       // The MT sums over the wave are formed together: after log2(MT) exchange steps in which a lane keeps the value
       // of the class (lane mod MT) it belongs to and hands the other to its partner, one value per lane is left to
       // add up over lanes of equal class, instead of MT values over all lanes.  Rotations by 4 and 8 inside a row of 16
@@ -562,7 +587,7 @@ __device__ __forceinline__ void mmvq_stream_body(const uint8_t* __restrict__ W, 
   GGUF_PHASE(4);                               // results stored
 }
 
-template <class F, int MT, int NW, int D, typename T, bool TILE = false, bool FULL = true, bool STAGED = false>
+template <class F, int MT, int NW, int D, typename T, bool TILE = false, bool FULL = true, int STAGED = 0>
 __global__ __launch_bounds__(64 * NW) void mmvq_stream_kernel(const uint8_t* __restrict__ W, const T* __restrict__ X,
                                                                T* __restrict__ Y, const T* __restrict__ bias, int64_t ldy,
                                                                StreamGeom geom) {
@@ -579,7 +604,7 @@ struct MoeStreamArgs {
   int64_t x_pitch;        // elements between activation rows: K, or 2 K for [gate | up] rows
   int top_k, num_experts, act;
 };
-template <class F, int NW, int D, typename T, bool STAGED, bool GATED>
+template <class F, int NW, int D, typename T, int STAGED, bool GATED>
 __global__ __launch_bounds__(64 * NW) void mmvq_stream_moe_kernel(const uint8_t* __restrict__ W, const T* __restrict__ X,
                                                                    T* __restrict__ Y, MoeStreamArgs moe, StreamGeom geom) {
   const int z = blockIdx.y;
@@ -589,7 +614,16 @@ __global__ __launch_bounds__(64 * NW) void mmvq_stream_moe_kernel(const uint8_t*
                                                                Y + (int64_t)z * geom.N, nullptr, (int64_t)geom.N, geom, moe.act);
 }
 
-template <class F, int MT, int D, typename T, bool TILE, bool FULL, int NW, bool STAGED = false>
+// Whether the rows of W are whole 16-byte pieces at 16-byte aligned addresses.  Q3_K and Q6_K, whose rows are that only
+// when K is a multiple of 2048, have a second variant for any even address and pitch: its pieces start at the 16-byte
+// boundary below a stretch and the readers cut their fields out of the LDS copy from wherever it starts (nothing outside
+// the 16-byte granules that hold bytes of W is read).
+template <class F>
+static bool span_aligned(const void* W, int64_t pitch, int K) {
+  return (int64_t)(K / F::QK) * F::BS % 16 == 0 && pitch % 16 == 0 && (uintptr_t)W % 16 == 0;
+}
+
+template <class F, int MT, int D, typename T, bool TILE, bool FULL, int NW, int STAGED = 0>
 static void launch_stream_d(const void* W, const T* X, T* Y, int N, int K, int rows_per_wg, int grid, size_t lds, const LinearArgs& la,
                             hipStream_t stream, int m_act) {
   auto kern = mmvq_stream_kernel<F, MT, NW, D, T, TILE, FULL, STAGED>;
@@ -627,10 +661,18 @@ static bool launch_stream(const void* W, const T* X, T* Y, int N, int K, hipStre
       if constexpr (MT <= MMVQ_STAGED_MT && (NW == MMVQ_NW || !std::is_same<F, FmtQ4_K>::value) && SpanOf<F>::value > 0) {
         // rows of whole 16-byte pieces at aligned addresses: every byte is requested once (see SpanRegs)
         const int64_t pitch = la.w_pitch ? la.w_pitch : (int64_t)(K / F::QK) * F::BS;
-        const size_t lds_staged = lds + (size_t)NW * SpanOf<F>::value + SpanSlack<F>::value;
-        if (per_wave >= MMVQ_DEPTH && (int64_t)(K / F::QK) * F::BS % 16 == 0 && pitch % 16 == 0 && (uintptr_t)W % 16 == 0 && lds_staged <= 160 * 1024) {
-          launch_stream_d<F, MT, MMVQ_DEPTH, T, TILE, FULL, NW, true>(W, X, Y, N, K, rows_per_wg, grid, lds_staged, la, stream, m_act);
-          return;
+        const size_t lds_staged = lds + (size_t)NW * 16 * SpanRegs<SpanOf<F>::value, SpanAny<F>::value>::PIECES + SpanSlack<F>::value;
+        if (per_wave >= MMVQ_DEPTH && lds_staged <= 160 * 1024) {
+          if (span_aligned<F>(W, pitch, K)) {
+            launch_stream_d<F, MT, MMVQ_DEPTH, T, TILE, FULL, NW, STAGED_ALIGNED>(W, X, Y, N, K, rows_per_wg, grid, lds_staged, la, stream, m_act);
+            return;
+          }
+          if constexpr (SpanAny<F>::value) {
+            if (pitch % 2 == 0 && (uintptr_t)W % 2 == 0) {
+              launch_stream_d<F, MT, MMVQ_DEPTH, T, TILE, FULL, NW, STAGED_ANY>(W, X, Y, N, K, rows_per_wg, grid, lds_staged, la, stream, m_act);
+              return;
+            }
+          }
         }
       }
       if (per_wave >= MMVQ_DEPTH) { launch_stream_d<F, MT, MMVQ_DEPTH, T, TILE, FULL, NW>(W, X, Y, N, K, rows_per_wg, grid, lds, la, stream, m_act); return; }
@@ -675,14 +717,14 @@ static bool launch_stream_moe(const void* W, const T* X, T* Y, int N, int K, con
   // (experts shared between pairs come from the caches at more than the HBM rate, and there the trip through LDS costs
   //  more than the tidier requests gain: Q4_0, 64 experts [2048,2048], 8 tokens 45 -> 48 us; Q4_K keeps it)
   if constexpr (std::is_same<F, FmtQ4_K>::value) {
-    const size_t lds_staged = lds + (size_t)NW * SpanOf<F>::value + SpanSlack<F>::value;
-    if (per_wave >= MMVQ_DEPTH && (int64_t)(K / F::QK) * F::BS % 16 == 0 && pitch % 16 == 0 && (uintptr_t)W % 16 == 0 && lds_staged <= 160 * 1024) {
-      go(mmvq_stream_moe_kernel<F, NW, MMVQ_DEPTH, T, true, GATED>, lds_staged);
+    const size_t lds_staged = lds + (size_t)NW * 16 * SpanRegs<SpanOf<F>::value, SpanAny<F>::value>::PIECES + SpanSlack<F>::value;
+    if (per_wave >= MMVQ_DEPTH && span_aligned<F>(W, pitch, K) && lds_staged <= 160 * 1024) {
+      go(mmvq_stream_moe_kernel<F, NW, MMVQ_DEPTH, T, STAGED_ALIGNED, GATED>, lds_staged);
       return true;
     }
   }
-  if (per_wave >= MMVQ_DEPTH) go(mmvq_stream_moe_kernel<F, NW, MMVQ_DEPTH, T, false, GATED>, lds);
-  else go(mmvq_stream_moe_kernel<F, NW, 1, T, false, GATED>, lds);
+  if (per_wave >= MMVQ_DEPTH) go(mmvq_stream_moe_kernel<F, NW, MMVQ_DEPTH, T, 0, GATED>, lds);
+  else go(mmvq_stream_moe_kernel<F, NW, 1, T, 0, GATED>, lds);
   return true;
 }
 

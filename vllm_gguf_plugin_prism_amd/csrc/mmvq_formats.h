@@ -173,8 +173,9 @@ struct FmtQ6_K {
   // an odd number start two bytes into a dword (210 = 4 * 52 + 2): a lane reads the dwords that cover a field and
   // cuts it out with funnel shifts.  (The last field of the last block may touch the dword behind the span.)
   static constexpr int SPAN = 8 * BS, SPAN_SLACK = 16;
-  static __device__ __forceinline__ Regs from_span(const char* span, int lane) {
-    const int c = lane & 7, h = c >> 2, cc = c & 3, b = (lane >> 3) * BS;
+  static constexpr bool SPAN_ANY = true;   // the copy may start at any even offset `at` of its first 16 bytes
+  static __device__ __forceinline__ Regs from_span(const char* span, int lane, int at = 0) {
+    const int c = lane & 7, h = c >> 2, cc = c & 3, b = at + (lane >> 3) * BS;
     Regs r;
     r.qla = lds_cut8(span, b + 64 * h + 8 * cc);
     r.qlb = lds_cut8(span, b + 64 * h + 32 + 8 * cc);
@@ -557,8 +558,9 @@ struct FmtQ3_K {
     return r;
   }
   static constexpr int SPAN = 8 * BS, SPAN_SLACK = 16;   // 8 blocks, 880 bytes, at 2-byte alignment in the LDS copy
-  static __device__ __forceinline__ Regs from_span(const char* span, int lane) {
-    const int c = lane & 7, n = c >> 2, cc = c & 3, b = (lane >> 3) * BS;
+  static constexpr bool SPAN_ANY = true;
+  static __device__ __forceinline__ Regs from_span(const char* span, int lane, int at = 0) {
+    const int c = lane & 7, n = c >> 2, cc = c & 3, b = at + (lane >> 3) * BS;
     Regs r;
     r.q = lds_cut8(span, b + 32 + 32 * n + 8 * cc); r.hm = lds_cut8(span, b + 8 * cc);
     uint32_t w[5];    // bytes 96 .. 109: twelve of scales and d
