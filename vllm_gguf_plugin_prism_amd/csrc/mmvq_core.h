@@ -298,9 +298,10 @@ __device__ unsigned long long g_mmvq_phases[1024 * 2 * 8];
 #endif
 template <class F, class = void> struct SpanOf { static constexpr int value = 0; };
 template <class F> struct SpanOf<F, std::void_t<decltype(F::SPAN)>> { static constexpr int value = F::SPAN; };
-// STAGED: rows are fetched per lane (0), as whole 16-byte pieces from aligned stretches, or from stretches that start
-// at any even address
-constexpr int STAGED_ALIGNED = 1, STAGED_ANY = 2;
+// STAGED: rows are fetched per lane (0) or as whole 16-byte pieces: from aligned stretches of rows that are whole
+// stretches (K a multiple of 2048: nothing to clamp), from stretches that start at any even address, or from aligned
+// stretches of rows whose last stretch is shorter
+constexpr int STAGED_ALIGNED = 1, STAGED_ANY = 2, STAGED_PART = 3;
 template <class F, class = void> struct SpanAny { static constexpr bool value = false; };   // spans may start at any even address
 template <class F> struct SpanAny<F, std::void_t<decltype(F::SPAN_ANY)>> { static constexpr bool value = F::SPAN_ANY; };
 template <class F, class = void> struct SpanSlack { static constexpr int value = 0; };   // bytes a reader may touch behind the last span
@@ -325,6 +326,13 @@ template <int SPAN, bool ANY = false> struct SpanRegs {
     for (int i = 0; i < NR; ++i) {
       const int p = 64 * i + ((i < NR - 1 || TAIL == 64) ? lane : lane % TAIL);
       r[i] = __builtin_nontemporal_load((const u32x4_t*)(first + 16 * min(p, valid - 1)));
+    }
+  }
+  __device__ __forceinline__ void load(const uint8_t* first, int lane) {   // a whole stretch
+#pragma unroll
+    for (int i = 0; i < NR; ++i) {
+      const int p = 64 * i + ((i < NR - 1 || TAIL == 64) ? lane : lane % TAIL);
+      r[i] = __builtin_nontemporal_load((const u32x4_t*)(first + 16 * p));
     }
   }
   __device__ __forceinline__ void store(char* lds, int lane) const {
@@ -404,7 +412,7 @@ __device__ __forceinline__ void mmvq_stream_body(const uint8_t* __restrict__ W, 
   const uint8_t* wbase = W + (int64_t)r_begin * rowbytes;
   // bytes of this wave's stretch that lie inside the row
   constexpr bool ANY = STAGED == STAGED_ANY;
-  const int span_bytes = STAGED ? max(16, min(SPAN, (K / F::QK) * F::BS - (wave_on ? step : 0) * SPAN)) : 0;
+  const int span_bytes = STAGED == STAGED_ALIGNED ? SPAN : STAGED ? max(16, min(SPAN, (K / F::QK) * F::BS - (wave_on ? step : 0) * SPAN)) : 0;
   typedef SpanRegs<STAGED ? SPAN : 16, ANY> Span;
   [[maybe_unused]] uint32_t mis[D];   // ANY: where in its first 16-byte piece the stretch of each row in flight starts
   auto load_row = [&](int i, [[maybe_unused]] uint32_t& m16) {
@@ -415,8 +423,10 @@ __device__ __forceinline__ void mmvq_stream_body(const uint8_t* __restrict__ W, 
       if constexpr (ANY) {
         m16 = (uint32_t)(uintptr_t)a & 15u;
         r.load(a - m16, lane, (int)(m16 + span_bytes + 15) >> 4);
-      } else {
+      } else if constexpr (STAGED == STAGED_PART) {
         r.load(a, lane, span_bytes >> 4);
+      } else {
+        r.load(a, lane);
       }
       return r;
     } else {
@@ -662,9 +672,12 @@ static bool launch_stream(const void* W, const T* X, T* Y, int N, int K, hipStre
         // rows of whole 16-byte pieces at aligned addresses: every byte is requested once (see SpanRegs)
         const int64_t pitch = la.w_pitch ? la.w_pitch : (int64_t)(K / F::QK) * F::BS;
         const size_t lds_staged = lds + (size_t)NW * 16 * SpanRegs<SpanOf<F>::value, SpanAny<F>::value>::PIECES + SpanSlack<F>::value;
-        if (per_wave >= MMVQ_DEPTH && lds_staged <= 160 * 1024) {
+        // (a row shorter than one stretch leaves half the lanes of its wave without a block: not worth the trip through LDS,
+        //  Q8_0 [3072,1024] 3.3 -> 3.8 us)
+        if (per_wave >= MMVQ_DEPTH && nb >= 64 && lds_staged <= 160 * 1024) {
           if (span_aligned<F>(W, pitch, K)) {
-            launch_stream_d<F, MT, MMVQ_DEPTH, T, TILE, FULL, NW, STAGED_ALIGNED>(W, X, Y, N, K, rows_per_wg, grid, lds_staged, la, stream, m_act);
+            if (nb % 64 == 0) launch_stream_d<F, MT, MMVQ_DEPTH, T, TILE, FULL, NW, STAGED_ALIGNED>(W, X, Y, N, K, rows_per_wg, grid, lds_staged, la, stream, m_act);
+            else launch_stream_d<F, MT, MMVQ_DEPTH, T, TILE, FULL, NW, SpanAny<F>::value ? STAGED_ANY : STAGED_PART>(W, X, Y, N, K, rows_per_wg, grid, lds_staged, la, stream, m_act);
             return;
           }
           if constexpr (SpanAny<F>::value) {
@@ -718,7 +731,7 @@ static bool launch_stream_moe(const void* W, const T* X, T* Y, int N, int K, con
   //  more than the tidier requests gain: Q4_0, 64 experts [2048,2048], 8 tokens 45 -> 48 us; Q4_K keeps it)
   if constexpr (std::is_same<F, FmtQ4_K>::value) {
     const size_t lds_staged = lds + (size_t)NW * 16 * SpanRegs<SpanOf<F>::value, SpanAny<F>::value>::PIECES + SpanSlack<F>::value;
-    if (per_wave >= MMVQ_DEPTH && span_aligned<F>(W, pitch, K) && lds_staged <= 160 * 1024) {
+    if (per_wave >= MMVQ_DEPTH && nb % 64 == 0 && span_aligned<F>(W, pitch, K) && lds_staged <= 160 * 1024) {
       go(mmvq_stream_moe_kernel<F, NW, MMVQ_DEPTH, T, STAGED_ALIGNED, GATED>, lds_staged);
       return true;
     }
