@@ -274,6 +274,20 @@ def test_mmvq_rows_of_whole_spans_through_lds(qtype, dt):
         assert o.rel_l2(y.float().cpu().numpy(), want) <= tol, (o.TYPE_NAMES[qtype], lead, extra)
 
 
+@pytest.mark.parametrize("qtype", ALL)
+def test_mmvq_rows_handed_out_to_half_waves(qtype):
+    """One row of X over rows of 32, 80 or 160 units (K = 1024, 2560, 5120): a row takes one, three or five half-waves of
+    32 lanes, so the kernel hands rows out to half-waves (32, 10 or 6 rows side by side in a 16-wave workgroup) -- unless
+    the format fetches such rows as whole 16-byte pieces, which comes first.  Both must agree with the GEMV oracle."""
+    ops = _ops()
+    rng = np.random.default_rng(1800 + qtype)
+    for n, k in [(3000, 1024), (9000, 1024), (2600, 2560), (1700, 5120), (5200, 5120)]:   # (the first is too small: whole waves)
+        w = o.make_weights(rng, qtype, n, k)
+        xd, xv = _x(rng, 1, k, "f32")
+        y = ops.ggml_mul_mat_vec_a8(_to_dev(w), xd, qtype, n)
+        assert o.rel_l2(y.float().cpu().numpy(), o.mul_mat_a8(w, xv, qtype, n, "mmvq")) <= 1e-5, (o.TYPE_NAMES[qtype], n, k)
+
+
 def test_empty_and_errors():
     ops = _ops()
     rng = np.random.default_rng(3)

@@ -302,6 +302,10 @@ template <class F> struct SpanOf<F, std::void_t<decltype(F::SPAN)>> { static con
 // stretches (K a multiple of 2048: nothing to clamp), from stretches that start at any even address, or from aligned
 // stretches of rows whose last stretch is shorter
 constexpr int STAGED_ALIGNED = 1, STAGED_ANY = 2, STAGED_PART = 3;
+// A fourth way to run the kernel, with per-lane loads: rows are handed out to half-waves of 32 lanes.  A row of 160
+// units (K = 5120) takes five half-waves instead of three waves, so six rows instead of five run side by side and no
+// lane is without a unit (five waves of sixteen were half or wholly empty); K = 1024 fills a wave with two rows.
+constexpr int LANES_HALF = 4;
 template <class F, class = void> struct SpanAny { static constexpr bool value = false; };   // spans may start at any even address
 template <class F> struct SpanAny<F, std::void_t<decltype(F::SPAN_ANY)>> { static constexpr bool value = F::SPAN_ANY; };
 template <class F, class = void> struct SpanSlack { static constexpr int value = 0; };   // bytes a reader may touch behind the last span
@@ -345,25 +349,28 @@ template <int SPAN, bool ANY = false> struct SpanRegs {
 // What the streaming kernel needs before its first memory requests, worked out on the host so that the kernel starts
 // without a division, and packed so that all of its arguments fit the first 64 bytes of the argument block (one
 // fetch).  The quotients by S and by K/8 are taken by multiplication with a rounded-up reciprocal, exact for the small
-// numerators here: wave < 16 with S <= 16, and group index * K/8 < 2^32 because K <= 32768 for this kernel.
+// numerators here: wave < 16 with S <= 16 (half-wave < 32 with S <= 32), and group index * K/8 < 2^32 because
+// K <= 32768 for this kernel.
 struct StreamGeom {
   uint32_t w_pitch;       // bytes between rows of W
   int N, K, rows_per_wg;
-  uint32_t packed;        // m_act | S << 4 | slots << 9 | (4096 / S + 1) << 14
+  uint32_t packed;        // m_act | S << 4 | slots << 10 | (4096 / S + 1) << 16
   uint32_t g8_inv;        // 2^32 / (K / 8) + 1
   __device__ __forceinline__ int m_act() const { return packed & 15; }
-  __device__ __forceinline__ int S() const { return (packed >> 4) & 31; }          // waves per row: ceil(K / 32 / 64)
-  __device__ __forceinline__ int slots() const { return (packed >> 9) & 31; }      // rows side by side: NW / S (>= 1)
-  __device__ __forceinline__ int slot_of(int wave) const { return (int)(((unsigned)wave * (packed >> 14)) >> 12); }  // wave / S
+  __device__ __forceinline__ int S() const { return (packed >> 4) & 63; }          // waves (half-waves) per row
+  __device__ __forceinline__ int slots() const { return (packed >> 10) & 63; }     // rows side by side (>= 1)
+  __device__ __forceinline__ int slot_of(int w) const { return (int)(((unsigned)w * (packed >> 16)) >> 12); }  // w / S for w < 32
 };
-static inline StreamGeom stream_geom(int N, int K, int rows_per_wg, int64_t w_pitch, int m_act, int nw) {
+// `half`: rows are handed out to half-waves of 32 lanes instead of waves (LANES_HALF)
+static inline StreamGeom stream_geom(int N, int K, int rows_per_wg, int64_t w_pitch, int m_act, int nw, bool half = false) {
   StreamGeom g;
-  const int S = (K / 32 + 63) / 64;
+  const int per = half ? 32 : 64;
+  const int S = (K / 32 + per - 1) / per;
   g.w_pitch = (uint32_t)w_pitch;
   g.N = N;
   g.K = K;
   g.rows_per_wg = rows_per_wg;
-  g.packed = (uint32_t)m_act | (uint32_t)S << 4 | (uint32_t)(nw / S) << 9 | (4096u / (uint32_t)S + 1u) << 14;
+  g.packed = (uint32_t)m_act | (uint32_t)S << 4 | (uint32_t)((half ? 2 * nw : nw) / S) << 10 | (4096u / (uint32_t)S + 1u) << 16;
   g.g8_inv = (uint32_t)((1ull << 32) / (uint32_t)(K / 8)) + 1u;
   return g;
 }
@@ -386,8 +393,9 @@ __device__ __forceinline__ void mmvq_stream_body(const uint8_t* __restrict__ W, 
   float* ldv = (float*)(smem + (size_t)MT * K);  // [MT][nb]
   float* lav = ldv + MT * nb;                  // [MT][nb]
   char* tab = (char*)(lav + (F::AUX != AUX_NONE ? MT * nb : 0));
-  float* part = (float*)(tab + F::TABLE_BYTES);  // [rows_per_wg][S][4 rows of 16 lanes][MT]
-  constexpr int SPAN = STAGED ? SpanOf<F>::value : 0;
+  float* part = (float*)(tab + F::TABLE_BYTES);  // [rows_per_wg][S][4 (HALF: 2) groups of 16 lanes][MT]
+  constexpr bool HALF = STAGED == LANES_HALF, SPANS = STAGED != 0 && !HALF;
+  constexpr int SPAN = SPANS ? SpanOf<F>::value : 0;
 
   const int r_begin = blockIdx.x * rows_per_wg;   // (the host launches ceil(N / rows_per_wg) workgroups: r_begin < N)
   const int r_end = min(N, r_begin + rows_per_wg);
@@ -396,9 +404,13 @@ __device__ __forceinline__ void mmvq_stream_body(const uint8_t* __restrict__ W, 
   const int64_t rowbytes = geom.w_pitch;   // bytes between rows: the dense row size unless the caller's tensor is padded
 
   // this wave: slot (which of the side-by-side rows) and step (which 64-unit stretch of the row)
-  const int slot = geom.slot_of(wave), step = wave - slot * S;   // wave / S, wave % S
+  // (HALF: the same per half-wave, so these are per-lane values there)
+  const int wh = HALF ? 2 * wave + (lane >> 5) : wave;
+  const int slot = geom.slot_of(wh), step = wh - slot * S;   // wh / S, wh % S
   const bool wave_on = slot < slots;           // NW - slots*S waves have no weights to fetch; they still quantize
-  const int u_raw = step * 64 + lane;
+  const int u_raw = HALF ? step * 32 + (lane & 31) : step * 64 + lane;
+  constexpr int GW = HALF ? 2 : 4;             // 16-lane groups of a wave (half-wave): each leaves one partial sum per row
+  const int G = GW * S;                        // partial sums per row
   const bool lane_on = wave_on && u_raw < nb;
   const int u = min(u_raw, nb - 1);
 
@@ -412,12 +424,12 @@ __device__ __forceinline__ void mmvq_stream_body(const uint8_t* __restrict__ W, 
   const uint8_t* wbase = W + (int64_t)r_begin * rowbytes;
   // bytes of this wave's stretch that lie inside the row
   constexpr bool ANY = STAGED == STAGED_ANY;
-  const int span_bytes = STAGED == STAGED_ALIGNED ? SPAN : STAGED ? max(16, min(SPAN, (K / F::QK) * F::BS - (wave_on ? step : 0) * SPAN)) : 0;
-  typedef SpanRegs<STAGED ? SPAN : 16, ANY> Span;
+  const int span_bytes = STAGED == STAGED_ALIGNED ? SPAN : SPANS ? max(16, min(SPAN, (K / F::QK) * F::BS - (wave_on ? step : 0) * SPAN)) : 0;
+  typedef SpanRegs<SPANS ? SPAN : 16, ANY> Span;
   [[maybe_unused]] uint32_t mis[D];   // ANY: where in its first 16-byte piece the stretch of each row in flight starts
   auto load_row = [&](int i, [[maybe_unused]] uint32_t& m16) {
     const int row = min(slot + slots * i, nrows - 1);
-    if constexpr (STAGED) {   // (the host takes this variant only for rows it can fetch as whole 16-byte pieces)
+    if constexpr (SPANS) {   // (the host takes this variant only for rows it can fetch as whole 16-byte pieces)
       Span r;
       const uint8_t* a = wbase + (int64_t)row * rowbytes + (int64_t)(wave_on ? step : 0) * SPAN;
       if constexpr (ANY) {
@@ -434,8 +446,8 @@ __device__ __forceinline__ void mmvq_stream_body(const uint8_t* __restrict__ W, 
     }
   };
   // this wave's staging area for one span, behind the partial sums
-  constexpr int STAGE_BYTES = STAGED ? 16 * Span::PIECES : 0;
-  char* stage = (char*)(part + (size_t)rows_per_wg * S * 4 * MT) + wave * STAGE_BYTES;
+  constexpr int STAGE_BYTES = SPANS ? 16 * Span::PIECES : 0;
+  char* stage = (char*)(part + (size_t)rows_per_wg * G * MT) + wave * STAGE_BYTES;
 
   // Prologue, in one basic block per variant: request this thread's first QG groups of activation values,
   // then the weights of the first D rows, then quantize the activations into LDS (four lanes per 32-value
@@ -447,7 +459,7 @@ __device__ __forceinline__ void mmvq_stream_body(const uint8_t* __restrict__ W, 
   // computed on whatever the LDS holds and never stored.
   const int rows_x = FULL ? MT : m_act;
   const int qtotal = rows_x * g8;  // a multiple of 4, so quads stay whole
-  std::conditional_t<STAGED != 0, Span, typename F::Regs> pre[D];
+  std::conditional_t<SPANS, Span, typename F::Regs> pre[D];
   const auto row_of_group = [&](int qc) { return MT == 1 ? 0 : (int)__umulhi((unsigned)qc, geom.g8_inv); };  // qc / g8
   auto quantize_group = [&](const raw8<T>& raw, const raw8<T>& up, int q) {
     const int qc = min(q, qtotal - 1);
@@ -545,14 +557,14 @@ __device__ __forceinline__ void mmvq_stream_body(const uint8_t* __restrict__ W, 
 
   // (a wave without a slot -- NW is not always a multiple of the waves a row takes -- has quantized its share of the
   //  activations and waits at the barrier behind the loop)
-  for (int i0 = 0; wave_on && i0 < max_rows; i0 += D) {
+  for (int i0 = 0; (HALF || wave_on) && i0 < max_rows; i0 += D) {
 #pragma unroll
     for (int d = 0; d < D; ++d) {
       const int i = i0 + d;
       const bool row_ok = i < my_rows;
       float acc[MT];
       typename F::Regs cur;
-      if constexpr (STAGED) {
+      if constexpr (SPANS) {
         // through LDS to the lanes that use the bytes (one wave's LDS accesses keep their order: no barrier), and the
         // slot is free for the next request before the arithmetic starts
         // (The fences are for the compiler, which reasons about one lane and would otherwise keep a value read from
@@ -577,13 +589,13 @@ __device__ __forceinline__ void mmvq_stream_body(const uint8_t* __restrict__ W, 
         const float v = F::dot(cur, act[m], u);
         acc[m] = lane_on ? v : 0.0f;
       }
-      if constexpr (!STAGED) pre[d] = load_row(i + D, mis[d]);  // refill the slot: D - 1 other slots are still in flight
+      if constexpr (!SPANS) pre[d] = load_row(i + D, mis[d]);  // refill the slot: D - 1 other slots are still in flight
       // The MT sums over the wave are formed together: after log2(MT) exchange steps in which a lane keeps the value
       // of the class (lane mod MT) it belongs to and hands the other to its partner, one value per lane is left to
       // add up over lanes of equal class, instead of MT values over all lanes.  Rotations by 4 and 8 inside a row of 16
       // lanes finish that; the four rows of the wave leave their totals in LDS for the adder below.
       const float v = rows16_sums<MT>(acc, lane);
-      if ((lane & 15) < MT && row_ok) part[(((slot + slots * i) * S + step) * 4 + (lane >> 4)) * MT + (lane & 15)] = v;
+      if ((lane & 15) < MT && row_ok) part[((slot + slots * i) * G + step * GW + ((lane >> 4) & (GW - 1))) * MT + (lane & 15)] = v;
     }
   }
   GGUF_PHASE(3);                               // own rows walked
@@ -591,7 +603,7 @@ __device__ __forceinline__ void mmvq_stream_body(const uint8_t* __restrict__ W, 
   for (int i = tid; i < nrows * MT; i += 64 * NW) {
     const int row = i / MT, m = i - row * MT;
     float v = 0.0f;
-    for (int st = 0; st < 4 * S; ++st) v += part[(row * 4 * S + st) * MT + m];
+    for (int st = 0; st < G; ++st) v += part[(row * G + st) * MT + m];
     if (FULL || m < m_act) Y[(int64_t)m * ldy + r_begin + row] = finish<T>(v, bias, r_begin + row);
   }
   GGUF_PHASE(4);                               // results stored
@@ -643,7 +655,7 @@ static void launch_stream_d(const void* W, const T* X, T* Y, int N, int K, int r
   }
   const int64_t w_pitch = la.w_pitch ? la.w_pitch : (int64_t)(K / F::QK) * F::BS;
   hipLaunchKernelGGL(kern, dim3(grid), dim3(64 * NW), lds, stream, (const uint8_t*)W, X, Y, (const T*)la.bias,
-                     la.ldy ? la.ldy : (int64_t)N, stream_geom(N, K, rows_per_wg, w_pitch, m_act, NW));
+                     la.ldy ? la.ldy : (int64_t)N, stream_geom(N, K, rows_per_wg, w_pitch, m_act, NW, STAGED == LANES_HALF));
 }
 
 // Returns false when the shape does not fit the streaming kernel (a row longer than NW waves, or activations
@@ -685,6 +697,20 @@ static bool launch_stream(const void* W, const T* X, T* Y, int N, int K, hipStre
               launch_stream_d<F, MT, MMVQ_DEPTH, T, TILE, FULL, NW, STAGED_ANY>(W, X, Y, N, K, rows_per_wg, grid, lds_staged, la, stream, m_act);
               return;
             }
+          }
+        }
+      }
+      if constexpr (MT == 1) {
+        // rows handed out to half-waves where that puts more rows side by side (K = 5120: six instead of five)
+        const int sh = (nb + 31) / 32, slots_h = sh <= 2 * NW ? 2 * NW / sh : 0;
+        // (not where that would take more rows per workgroup and so fewer workgroups than the chip has CUs, and only
+        //  where a half-wave then walks fewer rows than a wave did: 20 rows per workgroup are four turns either way)
+        if (nb % 32 == 0 && slots_h > slots && rows_per_wg >= slots_h && (rows_per_wg + slots_h - 1) / slots_h < per_wave) {
+          const int rows_h = rows_per_wg;
+          const size_t lds_h = (size_t)K + (size_t)nb * 4 * (F::AUX != AUX_NONE ? 2 : 1) + F::TABLE_BYTES + (size_t)rows_h * sh * 2 * 4;
+          if ((rows_h + slots_h - 1) / slots_h >= MMVQ_DEPTH && lds_h <= 160 * 1024) {
+            launch_stream_d<F, MT, MMVQ_DEPTH, T, TILE, FULL, NW, LANES_HALF>(W, X, Y, N, K, rows_h, (N + rows_h - 1) / rows_h, lds_h, la, stream, m_act);
+            return;
           }
         }
       }
