@@ -294,7 +294,7 @@ __device__ unsigned long long g_mmvq_phases[1024 * 2 * 8];
 // through LDS.  Requests that never meet a second request for the same cache line can carry the non-temporal hint,
 // which the memory system rewards (a plain streaming read of 33 MB: 6.7 us with the hint, 7.3 us without).
 #ifndef MMVQ_STAGED_MT
-#define MMVQ_STAGED_MT 2
+#define MMVQ_STAGED_MT 2   // rows of X up to which rows of W are fetched this way (at four the gain is gone)
 #endif
 template <class F, class = void> struct SpanOf { static constexpr int value = 0; };
 template <class F> struct SpanOf<F, std::void_t<decltype(F::SPAN)>> { static constexpr int value = F::SPAN; };
@@ -304,7 +304,7 @@ template <class F> struct SpanOf<F, std::void_t<decltype(F::SPAN)>> { static con
 constexpr int STAGED_ALIGNED = 1, STAGED_ANY = 2, STAGED_PART = 3;
 // A fourth way to run the kernel, with per-lane loads: rows are handed out to half-waves of 32 lanes.  A row of 160
 // units (K = 5120) takes five half-waves instead of three waves, so six rows instead of five run side by side and no
-// lane is without a unit (five waves of sixteen were half or wholly empty); K = 1024 fills a wave with two rows.
+// lane is without a unit (of sixteen waves five were half empty and one had no row); K = 1024 fills a wave with two rows.
 constexpr int LANES_HALF = 4;
 template <class F, class = void> struct SpanAny { static constexpr bool value = false; };   // spans may start at any even address
 template <class F> struct SpanAny<F, std::void_t<decltype(F::SPAN_ANY)>> { static constexpr bool value = F::SPAN_ANY; };
