@@ -762,6 +762,23 @@ static bool launch_stream_moe(const void* W, const T* X, T* Y, int N, int K, con
       return true;
     }
   }
+  {
+    // rows handed out to half-waves where that saves turns of the row loop (K = 1024, the second expert GEMM of a layer
+    // with 1024 intermediate features: two rows per wave)
+    const int sh = (nb + 31) / 32, slots_h = sh <= 2 * NW ? 2 * NW / sh : 0;
+    if (nb % 32 == 0 && slots_h > slots && rows_per_wg >= slots_h && (rows_per_wg + slots_h - 1) / slots_h < per_wave &&
+        (rows_per_wg + slots_h - 1) / slots_h >= MMVQ_DEPTH) {
+      const size_t lds_h = (size_t)K + (size_t)nb * 4 * (F::AUX != AUX_NONE ? 2 : 1) + F::TABLE_BYTES + (size_t)rows_per_wg * sh * 2 * 4;
+      const StreamGeom geom_h = stream_geom(N, K, rows_per_wg, pitch, 1, NW, true);
+      auto kern = mmvq_stream_moe_kernel<F, NW, MMVQ_DEPTH, T, LANES_HALF, GATED>;
+      if (lds_h > 64 * 1024) {
+        static std::atomic<uint64_t> done{0};
+        allow_large_lds(kern, 160 * 1024, done);
+      }
+      hipLaunchKernelGGL(kern, dim3(grid, pairs), dim3(64 * NW), lds_h, stream, (const uint8_t*)W, X, Y, moe, geom_h);
+      return true;
+    }
+  }
   if (per_wave >= MMVQ_DEPTH) go(mmvq_stream_moe_kernel<F, NW, MMVQ_DEPTH, T, 0, GATED>, lds);
   else go(mmvq_stream_moe_kernel<F, NW, 1, T, 0, GATED>, lds);
   return true;
