@@ -433,11 +433,13 @@ def test_moe_vec_few_pairs_stream_each_expert(qtype, dt):
     """With fewer than two pairs per expert every pair walks its expert's matrix on the streaming GEMV kernel, which
     quantizes the pair's token itself: rows that are whole 2048-value spans (the staged loads of Q4_K) and shorter
     ones, an output that does not divide into the workgroups' bands, the gated activation of the layer's second GEMM
-    folded into the quantisation, and an expert id outside the table (left out, the others unaffected)."""
+    folded into the quantisation, an expert id outside the table (left out, the others unaffected), and rows short
+    enough for two of them to share a wave."""
     ops = _ops()
     rng = np.random.default_rng(1500 + qtype)
     tol = {"f32": 1e-5, "f16": 1e-3, "bf16": 8e-3}[dt]
-    for t, top_k, e, n, k in [(1, 8, 64, 200, 2048), (3, 2, 8, 77, 512), (5, 1, 16, 300, 1024)]:
+    # (the last: rows of 32 units and bands of 66 rows, which half-waves walk in three turns where waves take five)
+    for t, top_k, e, n, k in [(1, 8, 64, 200, 2048), (3, 2, 8, 77, 512), (5, 1, 16, 300, 1024), (2, 4, 8, 2100, 1024)]:
         w = np.stack([o.make_weights(rng, qtype, n, k) for _ in range(e)])
         xd, xv = _x(rng, t, k, dt)
         ids, _ = _routing(rng, t, e, top_k)
