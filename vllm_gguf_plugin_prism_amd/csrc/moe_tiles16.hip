@@ -253,9 +253,34 @@ static int moe16_typed(const void* W, const void* ws, void* Y, int N, int K, int
     static std::atomic<uint64_t> done{0};
     allow_large_lds(kern, lds, done);
   }
-  const int tiles_m = num_sorted / 16, tiles = tiles_m * ((N + N_T - 1) / N_T);
+  const int tiles_n = (N + N_T - 1) / N_T, tiles_m = num_sorted / 16, tiles = tiles_m * tiles_n;
   if (tiles == 0) return GGUF_OK;
-  hipLaunchKernelGGL(kern, dim3(tiles), dim3(64 * NW), lds, stream, (const uint8_t*)W, (const char*)ws, q8_row_bytes(K), (T*)Y, N, K,
+  // Three workgroups fit a CU.  When the blocks that hold pairs make a little more than one round of those (how many
+  // there are is known on the device only: the estimate takes the pairs as spread over the experts at random), the
+  // second round's few workgroups land three to a CU where the first finished first and take as long as the first
+  // round; with two per CU the same tiles make two full rounds, which is shorter: Q4_0, 64 experts [2048,2048], 32
+  // tokens top-8, 62 blocks of 64: 63 -> 55 us; 70 blocks the other way round, 64 against 71 us.  A larger LDS request
+  // is what limits a CU to two.
+  size_t lds_req = lds;
+  if (OCC == 3) {
+    const double experts = (double)(num_sorted - moe.num_pairs) / 15.0;   // the sorted array has room for 15 padding slots per expert
+    if (experts >= 1.0) {
+      const double lam = (double)moe.num_pairs / experts;
+      double blocks = 0.0, term = exp(-lam), cdf = 0.0, one_block = 0.0;   // sum over j >= 0 of P(pairs of an expert > 16 j)
+      for (int c = 0; c <= 64; ++c) {
+        cdf += term;
+        if (c % 16 == 0) blocks += 1.0 - cdf;
+        if (c == 16) one_block = cdf - exp(-lam);          // P(1 .. 16 pairs): the expert has exactly one block
+        term *= lam / (c + 1);
+      }
+      const double est = blocks * experts * tiles_n, cus = (double)num_cus();
+      // (exactly four tiles per CU is the one case in which three per CU do finish as three and one: 53 us above, and
+      //  the layer's second GEMM 28 against 31 us -- kept when every expert is likely to have exactly one block)
+      const bool four_each = (int)(experts + 0.5) * tiles_n == 4 * (int)cus && pow(one_block, experts) >= 0.8;
+      if (est > 3.0 * cus && est <= 4.0 * cus && !four_each) lds_req = 54 * 1024;
+    }
+  }
+  hipLaunchKernelGGL(kern, dim3(tiles), dim3(64 * NW), lds_req, stream, (const uint8_t*)W, (const char*)ws, q8_row_bytes(K), (T*)Y, N, K,
                      (int)q8_kp(K), tiles_m, tiles, moe, Dense16{}, (const T*)nullptr);
   return launch_status();
 }
