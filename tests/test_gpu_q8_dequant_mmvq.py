@@ -258,7 +258,7 @@ def test_mmvq_rows_of_whole_spans_through_lds(qtype, dt):
     for n, k in [(4608, 2048), (2400, 4096), (1300, 6144), (2400, 3584), (1500, 5120), (5000, 1024), (1536, 2560)]:
         w = o.make_weights(rng, qtype, n, k)
         wd = _to_dev(w)
-        for m in (1, 2):
+        for m in (1, 2, 3, 4) if qtype == o.Q8_0 else (1, 2):   # (Q8_0 fetches whole pieces up to four rows of X)
             xd, xv = _x(rng, m, k, dt)
             y = ops.ggml_mul_mat_vec_a8(wd, xd, qtype, n)
             assert o.rel_l2(y.float().cpu().numpy(), o.mul_mat_a8(w, xv, qtype, n, "mmvq")) <= tol, (o.TYPE_NAMES[qtype], n, k, m)

@@ -680,7 +680,8 @@ static bool launch_stream(const void* W, const T* X, T* Y, int N, int K, hipStre
     if constexpr (MT <= 4) {
       // (for Q4_K, whose per-lane loads are aligned 16-byte pieces already, the trip through LDS costs the 8-wave kernel
       //  of the small matrices as much as it gains; [4096,4096]: Q8_0 6.4 -> 5.1 us, Q4_0 5.1 -> 4.4 us, Q6_K 6.2 -> 5.4 us)
-      if constexpr (MT <= MMVQ_STAGED_MT && (NW == MMVQ_NW || !std::is_same<F, FmtQ4_K>::value) && SpanOf<F>::value > 0) {
+      // (Q8_0, most bytes per weight, still gains at four rows: [14336,4096] 16.6 -> 15.4 us)
+      if constexpr (MT <= (std::is_same<F, FmtQ8_0>::value ? 4 : MMVQ_STAGED_MT) && (NW == MMVQ_NW || !std::is_same<F, FmtQ4_K>::value) && SpanOf<F>::value > 0) {
         // rows of whole 16-byte pieces at aligned addresses: every byte is requested once (see SpanRegs)
         const int64_t pitch = la.w_pitch ? la.w_pitch : (int64_t)(K / F::QK) * F::BS;
         const size_t lds_staged = lds + (size_t)NW * 16 * SpanRegs<SpanOf<F>::value, SpanAny<F>::value>::PIECES + SpanSlack<F>::value;
