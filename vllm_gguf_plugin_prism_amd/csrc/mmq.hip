@@ -550,9 +550,9 @@ static bool mmq_type_ok(int type) {
 // group of pairs on the vector ALUs.  Results keep the GEMV's semantics: Q4_K / Q5_K take their offset term from the
 // quant sums (MoeArgs::gemv_sums); Q5_0 is the one tile format whose tile arithmetic differs from its GEMV
 // (vecdotq.cuh:98-125 against :668-749) and stays on the vector kernel.
-bool moe_vec_tiles_ok(int type, int64_t pairs, int64_t num_experts) {
+bool moe_vec_tiles_ok(int type, int64_t pairs, int64_t num_experts, int64_t expert_bytes) {
   if (!mmq_type_ok(type) || type == T_Q5_0) return false;
-  return num_experts > 0 && num_experts <= 256 && pairs >= 2 * num_experts;  // the tile kernel takes expert ids 0..255 (moe.cuh:33)
+  return num_experts > 0 && num_experts <= 256 && moe_share_pays(pairs, num_experts, expert_bytes);  // the tile kernel takes expert ids 0..255 (moe.cuh:33)
 }
 
 int64_t moe_vec_tiles_workspace(int64_t tokens, int64_t top_k, int64_t K, int64_t num_experts) {

@@ -123,7 +123,7 @@ extern "C" int gguf_moe_vec_act(const void* X, int xdtype, void* q8_workspace, c
 
 namespace gguf {
 // mmq.hip: the same operator on the grouped tile kernel, for calls whose experts are shared by enough pairs
-bool moe_vec_tiles_ok(int type, int64_t pairs, int64_t num_experts);
+bool moe_vec_tiles_ok(int type, int64_t pairs, int64_t num_experts, int64_t expert_bytes);
 int64_t moe_vec_tiles_workspace(int64_t tokens, int64_t top_k, int64_t K, int64_t num_experts);
 int moe_vec_tiles(const void* X, int xdtype, void* workspace, const void* W, const int32_t* topk_ids, void* Y, int type, int N,
                   int K, int top_k, int tokens, int act, int num_experts, hipStream_t s);
@@ -161,7 +161,7 @@ extern "C" int gguf_moe_vec_act(const void* X, int xdtype, void* q8_workspace, c
   const int ne = num_experts > 0 && num_experts <= 1024 ? (int)num_experts : 0;
   // the workspace holds at least the quantized activations; a caller that provides more says so
   const int64_t scratch_bytes = workspace_bytes > tokens * q8_row_bytes(K) ? workspace_bytes : tokens * q8_row_bytes(K);
-  if (ne > 0 && moe_vec_tiles_ok(type, pairs, ne) &&
+  if (ne > 0 && moe_vec_tiles_ok(type, pairs, ne, N * (K / qk) * block_bytes(type)) &&
       scratch_bytes >= moe_vec_tiles_workspace(tokens, top_k, K, ne))
     return moe_vec_tiles(X, xdtype, q8_workspace, W, topk_ids, Y, type, (int)N, (int)K, (int)top_k, (int)tokens, act, ne, s);
   switch (type) {

@@ -737,10 +737,20 @@ static bool launch_stream_moe(const void* W, const T* X, T* Y, int N, int K, con
   const int64_t pitch = (int64_t)(K / F::QK) * F::BS;
   if (pitch > (int64_t)UINT32_MAX) return false;
   const int slots = NW / S;
+  // Bands of rows per pair such that the workgroups (one per CU at a time) make whole rounds: N * pairs / CUs rows each
+  // would give 3 bands x 96 pairs = 288 workgroups for 12 tokens top-8 of [2048,2048], a full round and an eighth.
+  // Cost of a choice: rounds x (rows of a band + what a workgroup spends before its first row, about sixteen turns).
   const int64_t target = num_cus();
-  int rows_per_wg = (int)(((int64_t)N * pairs + target - 1) / target);
-  if (rows_per_wg < slots) rows_per_wg = slots;
-  if (rows_per_wg > N) rows_per_wg = N;
+  int rows_per_wg = N;
+  int64_t best = INT64_MAX;
+  for (int b = 1; b <= 64; ++b) {
+    const int rows = (N + b - 1) / b;
+    if (rows < slots && b > 1) break;
+    const int64_t wgs = (int64_t)((N + rows - 1) / rows) * pairs, rounds = (wgs + target - 1) / target;
+    const int64_t cost = rounds * (rows + 16 * slots);
+    if (cost < best) { best = cost; rows_per_wg = rows; }
+  }
+  if (rows_per_wg < slots) rows_per_wg = slots < N ? slots : N;
   const int grid = (N + rows_per_wg - 1) / rows_per_wg;
   const size_t lds = (size_t)K + (size_t)nb * 4 * (F::AUX != AUX_NONE ? 2 : 1) + F::TABLE_BYTES + (size_t)rows_per_wg * S * 4 * 4;
   if (lds > 160 * 1024) return false;
@@ -900,8 +910,9 @@ static int moe_vec_typed(const void* W, const char* x, void* Y, int xdtype, int 
   const int64_t sorted_cap = (int64_t)pairs + (int64_t)num_experts * (MOE_VEC_GROUP - 1);
   const int64_t block_cap = (sorted_cap + MOE_VEC_GROUP - 1) / MOE_VEC_GROUP;
   const int64_t need = q8_bytes + (sorted_cap + block_cap + 1) * (int64_t)sizeof(int32_t);
-  // grouping pays once experts are shared: at least two pairs per expert on average
-  if (num_experts > 0 && num_experts <= 1024 && pairs >= 2 * num_experts && block_cap <= 65535 && need <= scratch_bytes) {
+  // grouping pays once experts are shared
+  if (num_experts > 0 && num_experts <= 1024 && moe_share_pays(pairs, num_experts, (int64_t)N * (K / F::QK) * F::BS) && block_cap <= 65535 &&
+      need <= scratch_bytes) {
     int rc = quantize_q8_1(x, xdtype, scratch, tokens, K, stream, act);
     if (rc != GGUF_OK) return rc;
     int32_t* sorted = (int32_t*)((char*)scratch + q8_bytes);  // q8 rows are a multiple of 4 bytes long
