@@ -277,7 +277,7 @@ static int moe16_typed(const void* W, const void* ws, void* Y, int N, int K, int
       // (exactly four tiles per CU is the one case in which three per CU do finish as three and one: 53 us above, and
       //  the layer's second GEMM 28 against 31 us -- kept when every expert is likely to have exactly one block)
       const bool four_each = (int)(experts + 0.5) * tiles_n == 4 * (int)cus && pow(one_block, experts) >= 0.8;
-      if (est > 3.0 * cus && est <= 4.0 * cus && !four_each) lds_req = 54 * 1024;
+      if (est > 3.0 * cus && est <= 4.0 * cus && !four_each && lds < 54 * 1024) lds_req = 54 * 1024;
     }
   }
   hipLaunchKernelGGL(kern, dim3(tiles), dim3(64 * NW), lds_req, stream, (const uint8_t*)W, (const char*)ws, q8_row_bytes(K), (T*)Y, N, K,
