@@ -739,11 +739,19 @@ def moe_a8_vec(x, w, topk_ids, top_k, qtype, n, tokens):
     return y
 
 
-def silu_and_mul(x: np.ndarray) -> np.ndarray:
-    """SiLU(x[:, :d]) * x[:, d:] in fp64."""
+def silu_and_mul(x: np.ndarray, stored=None) -> np.ndarray:
+    """SiLU(x[:, :d]) * x[:, d:] in fp64.
+
+    With ``stored`` (np.float16) the result is what the layer holds between its two expert GEMMs
+    (quantization/fused_moe.py:44-51,80: the activation kernel rounds act(gate) to the tensor's dtype and multiplies in
+    that dtype): ``T(T(silu(gate)) * up)``, two roundings; the product of two halves is exact in fp32."""
     d = x.shape[-1] // 2
     a = x[..., :d].astype(np.float64)
-    return a / (1.0 + np.exp(-a)) * x[..., d:].astype(np.float64)
+    act = a / (1.0 + np.exp(-a))
+    if stored is None:
+        return act * x[..., d:].astype(np.float64)
+    assert stored == np.float16
+    return (act.astype(np.float16).astype(np.float32) * x[..., d:].astype(np.float16).astype(np.float32)).astype(np.float16)
 
 
 # ----------------------------------------------------------------------------

@@ -272,7 +272,7 @@ def test_mmq_and_mmvq_agree():
         assert o.rel_l2(a, b) <= (2e-2 if qtype == o.Q4_K else 1e-5), o.TYPE_NAMES[qtype]
 
 
-@pytest.mark.parametrize("m", [128, 512])
+@pytest.mark.parametrize("m", [128, 512, 2048])
 def test_config3_q6_k_qwen_mlp_slices(m):
     # Qwen2.5-7B MLP shapes at full K; N is cut to 1024 rows so the fp64 oracle stays in seconds
     ops = _ops()

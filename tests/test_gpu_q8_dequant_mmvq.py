@@ -238,6 +238,29 @@ def test_mmvq_five_rows_or_more_of_a_large_matrix(qtype, dt):
     assert torch.all(wide[:, :8] == 3.0)
 
 
+@pytest.mark.parametrize("qtype", [o.Q4_K, o.Q5_K])
+@pytest.mark.parametrize("kind", ["offset", "positive", "negative"])
+def test_mmvq_tile_route_keeps_large_block_sums_exact(qtype, kind):
+    """Activations with a common sign give q8_1 block sums far from zero (up to 32 * 127 = 4064 in magnitude, odd ones
+    included), which a half cannot hold exactly beyond 2048.  The offset term of Q4_K / Q5_K on the GEMV operator is
+    dmin * m * d8 * sum(q8) in exact integer arithmetic (vecdotq.cuh:328-351), so the tile route for five rows or more
+    must carry the sum as an integer: fp32 results within 1e-5 of the GEMV oracle, as for centred activations."""
+    ops = _ops()
+    rng = np.random.default_rng(1700 + qtype)
+    n, k = 2048, 4096
+    w = o.make_weights(rng, qtype, n, k)
+    wd = _to_dev(w)
+    for m in (5, 16, 32):
+        base = rng.standard_normal((m, k)).astype(np.float32)
+        x32 = {"offset": 1.0 + 0.3 * base, "positive": np.abs(base) + 0.5, "negative": -np.abs(base) - 0.5}[kind].astype(np.float32)
+        q = o.quantize_q8_1(x32)[0]
+        sums = np.abs(np.asarray(q, dtype=np.int64).reshape(m, -1, 32).sum(-1))
+        assert (sums > 2048).any() and (sums[sums > 2048] % 2 == 1).any()        # the case a half would round
+        y = ops.ggml_mul_mat_vec_a8(wd, torch.from_numpy(x32).cuda(), qtype, n)
+        want = o.mul_mat_a8(w, x32, qtype, n, "mmvq")
+        assert o.rel_l2(y.cpu().numpy(), want) <= 1e-5, (o.TYPE_NAMES[qtype], kind, m)
+
+
 SPAN_TYPES = [o.Q4_0, o.Q4_1, o.Q5_0, o.Q5_1, o.Q8_0, o.Q2_K, o.Q3_K, o.Q4_K, o.Q5_K, o.Q6_K, o.IQ4_NL]
 
 

@@ -286,3 +286,22 @@ def test_silu_and_mul():
     out = o.silu_and_mul(x)
     exp = np.array([[0.0 * 3.0, 1 / (1 + np.exp(-1.0)) * 4.0, -2 / (1 + np.exp(2.0)) * 5.0]])
     assert np.allclose(out, exp)
+
+
+def test_silu_and_mul_as_stored_in_half_matches_the_library_sequence():
+    """The intermediate of the MoE layer is act(gate) rounded to half, times up, rounded again (fused_moe.py:44-51).
+    torch's CPU half kernels do exactly that sequence (silu evaluated in fp32, stored as half; half product rounded
+    once), an implementation that shares nothing with the oracle."""
+    import torch
+
+    rng = np.random.default_rng(77)
+    x = (rng.standard_normal((64, 512)) * 4).astype(np.float16)
+    got = o.silu_and_mul(x, stored=np.float16)
+    t = torch.from_numpy(x)
+    want = (torch.nn.functional.silu(t[:, :256]) * t[:, 256:]).numpy()
+    assert got.dtype == np.float16
+    mism = np.count_nonzero(got.view(np.uint16) != want.view(np.uint16))
+    assert mism <= got.size // 2000      # fp64 against fp32 evaluation of exp: a last-place tie now and then
+    assert np.allclose(got.astype(np.float32), want.astype(np.float32), rtol=2e-3, atol=1e-7)
+    single = o.silu_and_mul(x.astype(np.float64)).astype(np.float16)
+    assert np.count_nonzero(single.view(np.uint16) != got.view(np.uint16)) > got.size // 20   # one rounding is a different function

@@ -60,6 +60,9 @@ int mmvq_any(int type, const void* W, const void* x, void* q8_workspace, void* Y
       const int rows = (int)(M - m0 < step ? M - m0 : step);
       rc = rows16_direct(W, (const char*)q8_workspace + m0 * q8_row_bytes(K), (char*)Y + m0 * ldy * esz, xdtype, type, rows, (int)N, (int)K,
                          nullptr, 0, s, la, true);
+      // takes() was asked for a full chunk above; a chunk the tile kernel then declines is a planning error, never a
+      // result the caller should see as the internal "not taken" code with part of Y written
+      if (rc == GGUF_NOT_TAKEN) return GGUF_ERR_LAUNCH;
       if (rc != GGUF_OK) return rc;
     }
     return GGUF_OK;

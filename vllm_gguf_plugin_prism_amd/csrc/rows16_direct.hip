@@ -167,11 +167,17 @@ __global__ __launch_bounds__(64 * KSPL, RT == 2 ? 2 : 4) void rows16_direct_kern
 #pragma unroll
   for (int i = 0; i < SI; ++i) {
     // d8 and s8 are half-precision values widened to fp32 by the quantizer: the narrowing is exact.  du is not one, but
-    // du / d8 = sum(q8) is an integer of at most 13 bits, exact as a quotient and as a half; d8 multiplies it again
-    // together with the block sum.
-    // (the quotient is an integer below 4065 in magnitude: the hardware reciprocal's last-bit error rounds away)
-    const float second = GSUM ? (dreg[rt][i] != 0.0f ? __builtin_rintf(sreg[rt][i] * __builtin_amdgcn_rcpf(dreg[rt][i])) : 0.0f) : sreg[rt][i];
-    xsc[min(at + TPR * i, spr - 1) * XR + 16 * rt + am] = (h2_d){(_Float16)dreg[rt][i], (_Float16)second};
+    // du / d8 = sum(q8) is an integer of at most 13 bits (|sum| <= 32 * 127 = 4064), exact as a quotient; a half holds
+    // integers exactly only up to 2048, so the sum travels as a 16-bit integer in the place of the second half and is
+    // widened again where d8 multiplies it together with the block sum.
+    // (the hardware reciprocal's last-bit error rounds away: the quotient lies within 4065 * 2^-22 of an integer)
+    h2_d pair = {(_Float16)dreg[rt][i], (_Float16)sreg[rt][i]};
+    if constexpr (GSUM) {
+      const int qsum = dreg[rt][i] != 0.0f ? (int)__builtin_rintf(sreg[rt][i] * __builtin_amdgcn_rcpf(dreg[rt][i])) : 0;
+      const uint32_t bits = (uint32_t)__builtin_bit_cast(uint16_t, pair[0]) | ((uint32_t)qsum << 16);
+      pair = __builtin_bit_cast(h2_d, bits);
+    }
+    xsc[min(at + TPR * i, spr - 1) * XR + 16 * rt + am] = pair;
   }
   if constexpr (XROWS > XR)
     for (int i = tid; i < gpr; i += NT) *(u4_d*)(xq + XR * pitch + 16 * i) = (u4_d){0u, 0u, 0u, 0u};
@@ -331,7 +337,8 @@ __global__ __launch_bounds__(64 * KSPL, RT == 2 ? 2 : 4) void rows16_direct_kern
               for (int r = 0; r < 4; ++r) {
                 const h2_d hh = __builtin_bit_cast(h2_d, scw[r]);
                 if constexpr (GSUM) {   // d8 * (S * dw - m * sum(q8)): the offset joins the block sum before d8 is applied
-                  const float u = __builtin_fmaf((float)hh[1], nm, seeded_times(S[r], w, nsw));
+                  const float qsum = (float)((int)scw[r] >> 16);   // the 16-bit integer staged in place of the second half
+                  const float u = __builtin_fmaf(qsum, nm, seeded_times(S[r], w, nsw));
                   acc[rt][q][r] = __builtin_fmaf(u, (float)hh[0], acc[rt][q][r]);
                 } else {
                   acc[rt][q][r] = __builtin_fmaf(seeded_times(S[r], w, nsw), (float)hh[0], acc[rt][q][r]);
