@@ -5,27 +5,30 @@
 
 namespace gguf {
 
-// Tile shape and the hand-out of tiles to workgroups for one launch (see MmqiPlan).  Two workgroups fit a CU, so the
-// chip holds 512 at once.
-//   * 128 x 64 tiles (the packed blocks of 64 weight rows are decoded once per 128 token rows); 64 x 128 for M <= 64.
-//   * Fewer tiles than the chip holds: every tile is split along K as far as that fills it (three ways when the
-//     tiles fill between half and two thirds of it).
-//   * More: whole rounds of tiles run unsplit, and the tiles of the last, partly filled round are split so that the
-//     round is short instead of sparse.
-// Splitting needs fp32 scratch behind the quantized rows; without it the plan falls back to whole tiles.
-MmqiPlan mmq_int_plan(int M, int N, int K, int64_t avail) {
-  constexpr int SLOTS = 512;
-  const int cfg = M > 64 ? 0 : 1;
-  const int mt = cfg == 0 ? 128 : 64, nt = cfg == 0 ? 64 : 128;
-  const int64_t t = (int64_t)((M + mt - 1) / mt) * ((N + nt - 1) / nt);
+// Tile shape and the hand-out of tiles to workgroups for one launch (see MmqiPlan).
+//   * Four shapes.  128 x 64 on four waves, two workgroups per CU (the packed blocks of 64 weight rows are decoded once
+//     per 128 token rows); 64 x 128 for M <= 64; 256 x 128 on eight waves, one workgroup per CU, a wave owning 32 x 128:
+//     the activation scales a wave reads from LDS per block serve four column tiles instead of two and the weights are
+//     decoded once per 256 rows (Q6_K [18944,3584] at 512 rows 229 -> 207 us, Q8_0 [14336,4096] 129 -> 112 us, IQ4_XS
+//     130 -> 108 us; Q5_K's kernel of that shape spills and is left out); 128 x 64 on eight waves, one workgroup per CU,
+//     for 65 .. 128 rows, where the larger tiles leave CUs without work.
+//   * How a shape's tiles fall into rounds of the workgroups the chip holds decides between them: fewer tiles than the
+//     chip holds are split along K as far as that fills it (three ways when they fill between half and two thirds of
+//     it); with more, whole rounds of tiles run unsplit and the tiles of the last, partly filled round are split so
+//     that the round is short instead of sparse.  The estimate is rounds x (steps of K + a start-up of about a step
+//     and a half), weighted by what a step of the shape was measured to take.
+// Splitting needs fp32 scratch behind the quantized rows; without it a plan falls back to whole tiles.
+static MmqiPlan plan_for(int cfg, int slots, int M, int N, int K, int64_t avail) {
+  MmqiPlan whole = {cfg, 0, 0, 1};
+  const int64_t t = (int64_t)((M + whole.mt() - 1) / whole.mt()) * ((N + whole.nt() - 1) / whole.nt());
   const int nsteps = (K + MMQI_KS - 1) / MMQI_KS;
-  const MmqiPlan whole = {cfg, (int)t, 0, 1};
-  const int rest = (int)(t % SLOTS);
+  whole.whole = (int)t;
+  const int rest = (int)(t % slots);
   if (rest == 0 || t <= 0) return whole;
-  int s = SLOTS / rest;
+  int s = slots / rest;
   // a round between half and two thirds full: split three ways it becomes two full rounds of a third the length
-  // (Q6_K [18944,3584] at 128 rows, 296 tiles: 85.5 -> 78 us; four ways 77, five 82 us)
-  if (s == 1 && 3 * rest <= 2 * SLOTS) s = 3;
+  // (Q6_K [18944,3584] at 128 rows, 296 tiles of 128 x 64: 85.5 -> 78 us; four ways 77, five 82 us)
+  if (s == 1 && 3 * rest <= 2 * slots) s = 3;
   if (s > nsteps / 4) s = nsteps / 4;   // a stretch of K shorter than four steps is mostly prologue
   if (s > 8) s = 8;
   if (s < 2) return whole;
@@ -33,7 +36,37 @@ MmqiPlan mmq_int_plan(int M, int N, int K, int64_t avail) {
   return p.partial_bytes() <= avail ? p : whole;
 }
 
-int64_t mmq_int_partial_bytes(int M, int N, int K) { return mmq_int_plan(M, N, K, INT64_MAX).partial_bytes(); }
+static double plan_cost(const MmqiPlan& p, int slots, double step_cost, int K) {
+  const int nsteps = (K + MMQI_KS - 1) / MMQI_KS;
+  constexpr double START = 1.5;   // pipeline fill, result or partial-tile store: in steps
+  double c = (double)((p.whole + slots - 1) / slots) * (nsteps + START);
+  if (p.shared > 0) c += (double)((p.shared * p.splits + slots - 1) / slots) * ((nsteps + p.splits - 1) / p.splits + START) + 1.0;
+  return c * step_cost;
+}
+
+MmqiPlan mmq_int_plan(int M, int N, int K, int64_t avail, bool wide_ok) {
+  // workgroups the chip holds, and what a step of K costs relative to the 128 x 64 tiles (two workgroups share a CU
+  // there: the figure is per round of workgroups)
+  struct Shape { int cfg, slots; double step_cost; };
+  if (M <= 64) return plan_for(1, 512, M, N, K, avail);
+  MmqiPlan best = plan_for(0, 512, M, N, K, avail);
+  double best_cost = plan_cost(best, 512, 1.0, K);
+  auto consider = [&](const Shape& sh) {
+    const MmqiPlan p = plan_for(sh.cfg, sh.slots, M, N, K, avail);
+    const double c = plan_cost(p, sh.slots, sh.step_cost, K);
+    if (c < 0.97 * best_cost) { best = p; best_cost = c; }
+  };
+  if (M <= 128) consider({3, 256, 0.6});
+  // 256-row tiles when the rows fill them (M = 384 would multiply 128 rows of padding)
+  if (wide_ok && M >= 448 && 20 * M >= 17 * ((M + 255) / 256 * 256)) consider({2, 256, 1.8});
+  return best;
+}
+
+// (the workspace is sized without knowing the format: room for whichever shape a format may take)
+int64_t mmq_int_partial_bytes(int M, int N, int K) {
+  const int64_t a = mmq_int_plan(M, N, K, INT64_MAX, true).partial_bytes(), b = mmq_int_plan(M, N, K, INT64_MAX, false).partial_bytes();
+  return a > b ? a : b;
+}
 
 template <class F>
 static int mmqi_fmt(const void* W, const void* ws, void* Y, int dtype, int M, int N, int K, float* partial, int64_t partial_bytes,

@@ -340,11 +340,14 @@ __global__ __launch_bounds__(256) void mmqi_reduce_kernel(const float* __restric
 // How the tiles of one launch are handed out: `whole` tiles get a workgroup each, the remaining `shared` tiles are
 // split `splits` ways along K.  partial_bytes() is the fp32 scratch the shared tiles need.
 struct MmqiPlan {
-  int cfg;            // 0: 128 x 64 tiles, 1: 64 x 128
+  int cfg;            // 0: 128 x 64 tiles, four waves; 1: 64 x 128, four waves; 2: 256 x 128, eight waves; 3: 128 x 64, eight waves
   int whole, shared, splits;
-  int64_t partial_bytes() const { return (int64_t)shared * splits * (128 * 64) * 4; }
+  int mt() const { return cfg == 1 ? 64 : cfg == 2 ? 256 : 128; }
+  int nt() const { return cfg == 1 || cfg == 2 ? 128 : 64; }
+  int64_t partial_bytes() const { return (int64_t)shared * splits * mt() * nt() * 4; }
 };
-MmqiPlan mmq_int_plan(int M, int N, int K, int64_t partial_bytes_available);  // mmq_i.hip
+// `wide_ok`: the format's 256 x 128 kernel keeps its registers (Q5_K's does not)
+MmqiPlan mmq_int_plan(int M, int N, int K, int64_t partial_bytes_available, bool wide_ok);  // mmq_i.hip
 
 template <class F, int WM, int WN, int TN, typename T>
 static void launch_mmqi(const void* W, const void* ws, void* Y, int M, int N, int K, hipStream_t stream, const MmqiPlan& p, float* partial,
@@ -366,12 +369,18 @@ static void launch_mmqi(const void* W, const void* ws, void* Y, int M, int N, in
                        tiles_m, p.whole, p.splits, ldy, (const T*)la.bias);
 }
 
+// Formats whose 256 x 128 kernel fits the register file without scratch worth mentioning.
+template <class F> struct MmqiWide { static constexpr bool ok = true; };
+template <> struct MmqiWide<MQ5_K> { static constexpr bool ok = false; };
+
 template <class F, typename T>
 static int mmqi_typed(const void* W, const void* ws, void* Y, int M, int N, int K, float* partial, int64_t partial_bytes,
                       hipStream_t stream, const LinearArgs& la) {
-  const MmqiPlan p = mmq_int_plan(M, N, K, partial_bytes);
-  if (p.cfg == 0) launch_mmqi<F, 4, 1, 2, T>(W, ws, Y, M, N, K, stream, p, partial, la);   // 128 x 64
-  else launch_mmqi<F, 2, 2, 2, T>(W, ws, Y, M, N, K, stream, p, partial, la);              // 64 x 128
+  const MmqiPlan p = mmq_int_plan(M, N, K, partial_bytes, MmqiWide<F>::ok);
+  if (p.cfg == 0) launch_mmqi<F, 4, 1, 2, T>(W, ws, Y, M, N, K, stream, p, partial, la);        // 128 x 64
+  else if (p.cfg == 1) launch_mmqi<F, 2, 2, 2, T>(W, ws, Y, M, N, K, stream, p, partial, la);   // 64 x 128
+  else if (p.cfg == 3) launch_mmqi<F, 4, 2, 1, T>(W, ws, Y, M, N, K, stream, p, partial, la);   // 128 x 64, eight waves
+  else if constexpr (MmqiWide<F>::ok) launch_mmqi<F, 8, 1, 4, T>(W, ws, Y, M, N, K, stream, p, partial, la);   // 256 x 128
   return launch_status();
 }
 
