@@ -306,6 +306,15 @@ constexpr int STAGED_ALIGNED = 1, STAGED_ANY = 2, STAGED_PART = 3;
 // units (K = 5120) takes five half-waves instead of three waves, so six rows instead of five run side by side and no
 // lane is without a unit (of sixteen waves five were half empty and one had no row); K = 1024 fills a wave with two rows.
 constexpr int LANES_HALF = 4;
+// A fifth: whole aligned stretches as under STAGED_ALIGNED, but requested with loads that write LDS directly, into a
+// ring of D stretches per wave: no registers hold the rows in flight and no store carries them to LDS.  What it
+// does not buy is depth: a wave's whole share requested at once (its 7 or 8 rows fit LDS for the [14336,4096] and
+// [4096,14336] matrices) ran 16 % slower, because requests beyond what the CU's memory pipeline accepts block the wave
+// that issues them, and the activations, which every wave needs first, were quantized 3 us later.
+constexpr int STAGED_DMA = 5;
+#ifndef MMVQ_DMA_DEPTH
+#define MMVQ_DMA_DEPTH 2   // (3 and 4 stretches in flight per wave, and a wave's whole share at once, measured slower: requests
+#endif                     //  beyond what the CU's memory pipeline holds block the waves that issue them)
 template <class F, class = void> struct SpanAny { static constexpr bool value = false; };   // spans may start at any even address
 template <class F> struct SpanAny<F, std::void_t<decltype(F::SPAN_ANY)>> { static constexpr bool value = F::SPAN_ANY; };
 template <class F, class = void> struct SpanSlack { static constexpr int value = 0; };   // bytes a reader may touch behind the last span
@@ -345,6 +354,12 @@ template <int SPAN, bool ANY = false> struct SpanRegs {
       if (i < NR - 1 || TAIL == 64 || lane < TAIL) *(u32x4_t*)(lds + 1024 * i + 16 * lane) = r[i];
   }
 };
+
+// Waits until at most N of this wave's vector-memory loads are outstanding; a compiler barrier for memory as well, so
+// that reads of LDS filled by such loads stay behind it.
+__device__ __forceinline__ void wait_vm_upto(int n) {   // n must fold to a constant (it is the instruction's immediate)
+  asm volatile("s_waitcnt vmcnt(%0)" ::"n"(n) : "memory");
+}
 
 // What the streaming kernel needs before its first memory requests, worked out on the host so that the kernel starts
 // without a division, and packed so that all of its arguments fit the first 64 bytes of the argument block (one
@@ -394,7 +409,7 @@ __device__ __forceinline__ void mmvq_stream_body(const uint8_t* __restrict__ W, 
   float* lav = ldv + MT * nb;                  // [MT][nb]
   char* tab = (char*)(lav + (F::AUX != AUX_NONE ? MT * nb : 0));
   float* part = (float*)(tab + F::TABLE_BYTES);  // [rows_per_wg][S][4 (HALF: 2) groups of 16 lanes][MT]
-  constexpr bool HALF = STAGED == LANES_HALF, SPANS = STAGED != 0 && !HALF;
+  constexpr bool HALF = STAGED == LANES_HALF, SPANS = STAGED != 0 && !HALF, DMA = STAGED == STAGED_DMA;
   constexpr int SPAN = SPANS ? SpanOf<F>::value : 0;
 
   const int r_begin = blockIdx.x * rows_per_wg;   // (the host launches ceil(N / rows_per_wg) workgroups: r_begin < N)
@@ -424,7 +439,7 @@ __device__ __forceinline__ void mmvq_stream_body(const uint8_t* __restrict__ W, 
   const uint8_t* wbase = W + (int64_t)r_begin * rowbytes;
   // bytes of this wave's stretch that lie inside the row
   constexpr bool ANY = STAGED == STAGED_ANY;
-  const int span_bytes = STAGED == STAGED_ALIGNED ? SPAN : SPANS ? max(16, min(SPAN, (K / F::QK) * F::BS - (wave_on ? step : 0) * SPAN)) : 0;
+  const int span_bytes = STAGED == STAGED_ALIGNED || DMA ? SPAN : SPANS ? max(16, min(SPAN, (K / F::QK) * F::BS - (wave_on ? step : 0) * SPAN)) : 0;
   typedef SpanRegs<SPANS ? SPAN : 16, ANY> Span;
   [[maybe_unused]] uint32_t mis[D];   // ANY: where in its first 16-byte piece the stretch of each row in flight starts
   auto load_row = [&](int i, [[maybe_unused]] uint32_t& m16) {
@@ -445,10 +460,27 @@ __device__ __forceinline__ void mmvq_stream_body(const uint8_t* __restrict__ W, 
       return F::load(wbase + (int64_t)row * rowbytes, 0, u, tab);
     }
   };
-  // this wave's staging area for one span, behind the partial sums
+  // this wave's staging area for one span (DMA: a ring of D), behind the partial sums
   constexpr int STAGE_BYTES = SPANS ? 16 * Span::PIECES : 0;
-  char* stage = (char*)(part + (size_t)rows_per_wg * G * MT) + wave * STAGE_BYTES;
-
+  char* stage = (char*)(part + (size_t)rows_per_wg * G * MT) + wave * (DMA ? D * 1024 * Span::NR : STAGE_BYTES);
+  // DMA: row i of this wave's share -> ring slot r, 16 bytes per lane and instruction straight into LDS (the LDS address is
+  // the instruction's base plus 16 x lane).  Span::NR instructions per row with every lane at work -- lanes past the last
+  // piece fetch it once more, into the padding of the slot, which is a whole number of KB -- so that no branch surrounds
+  // a load: the kernel counts the loads in flight itself (see the waits), and code the compiler moves or copies around
+  // a branch would not match the count.
+  constexpr int DMA_SLOT = 1024 * Span::NR, DMA_INSTRS = DMA ? D * Span::NR : 0;   // (the loads of the first D rows)
+  [[maybe_unused]] auto dma_row = [&](int i, int r) {
+    if constexpr (DMA) {
+      typedef const __attribute__((address_space(1))) void* gptr_t;
+      typedef __attribute__((address_space(3))) void* lptr_t;
+      const int row = min(slot + slots * i, nrows - 1);
+      const uint8_t* a = wbase + (int64_t)row * rowbytes + (int64_t)step * SPAN;
+      char* dst = stage + r * DMA_SLOT;
+#pragma unroll
+      for (int j = 0; j < Span::NR; ++j)
+        __builtin_amdgcn_global_load_lds((gptr_t)(a + 16 * min(64 * j + lane, Span::PIECES - 1)), (lptr_t)(dst + 1024 * j), 16, 0, 2);
+    }
+  };
   // Prologue, in one basic block per variant: request this thread's first QG groups of activation values,
   // then the weights of the first D rows, then quantize the activations into LDS (four lanes per 32-value
   // block) while the weights fly.  The activation loads go first so that waiting for them does not also
@@ -459,7 +491,20 @@ __device__ __forceinline__ void mmvq_stream_body(const uint8_t* __restrict__ W, 
   // computed on whatever the LDS holds and never stored.
   const int rows_x = FULL ? MT : m_act;
   const int qtotal = rows_x * g8;  // a multiple of 4, so quads stay whole
-  std::conditional_t<SPANS, Span, typename F::Regs> pre[D];
+  std::conditional_t<DMA, int, std::conditional_t<SPANS, Span, typename F::Regs>> pre[DMA ? 1 : D];
+  // the first D rows of this wave's share: D load slots in registers, or (DMA) all of the share; a fixed number of loads,
+  // rows past the share clamped, so that the loads behind the activation requests can be counted
+  auto first_rows = [&](auto on_tag) {
+    if constexpr (DMA) {
+      if constexpr (decltype(on_tag)::value) {
+#pragma unroll
+        for (int d = 0; d < D; ++d) dma_row(d, d);
+      }
+    } else {
+#pragma unroll
+      for (int d = 0; d < D; ++d) pre[d] = load_row(d, mis[d]);
+    }
+  };
   const auto row_of_group = [&](int qc) { return MT == 1 ? 0 : (int)__umulhi((unsigned)qc, geom.g8_inv); };  // qc / g8
   auto quantize_group = [&](const raw8<T>& raw, const raw8<T>& up, int q) {
     const int qc = min(q, qtotal - 1);
@@ -482,13 +527,12 @@ __device__ __forceinline__ void mmvq_stream_body(const uint8_t* __restrict__ W, 
       }
     }
   };
-  auto prologue = [&](auto qg_tag) {
+  auto prologue = [&](auto qg_tag, auto on_tag) {
     constexpr int QG = decltype(qg_tag)::value;
     if constexpr (QG == 0) {   // a wave with no activation values to quantize: its weights only
       if (qtotal <= NT) __builtin_amdgcn_s_barrier();   // (see below: the others' activation requests go first)
       GGUF_PHASE(6);
-#pragma unroll
-      for (int d = 0; d < D; ++d) pre[d] = load_row(d, mis[d]);
+      first_rows(on_tag);
       __builtin_amdgcn_sched_barrier(0);
       GGUF_PHASE(7);
       return;
@@ -498,8 +542,13 @@ __device__ __forceinline__ void mmvq_stream_body(const uint8_t* __restrict__ W, 
     for (int g = 0; g < QG; ++g) {
       const int qc = min(tid + g * NT, qtotal - 1);
       const int m = row_of_group(qc), j = qc - m * g8;
-      xraw[g].load(X + (int64_t)m * K + 8 * j);
-      if constexpr (GATED) xup[g].load(X + K + 8 * j);
+      if constexpr (DMA) {   // (not counted by the compiler: see the wait below)
+        xraw[g].load_uncounted(X + (int64_t)m * K + 8 * j);
+        if constexpr (GATED) xup[g].load_uncounted(X + K + 8 * j);
+      } else {
+        xraw[g].load(X + (int64_t)m * K + 8 * j);
+        if constexpr (GATED) xup[g].load(X + K + 8 * j);
+      }
     }
     __builtin_amdgcn_sched_barrier(0);
     if constexpr (QG == 1) {
@@ -510,24 +559,38 @@ __device__ __forceinline__ void mmvq_stream_body(const uint8_t* __restrict__ W, 
       __builtin_amdgcn_sched_barrier(0);
     }
     GGUF_PHASE(6);                             // activation requests are out (every wave's, where one request covers them)
-#pragma unroll
-    for (int d = 0; d < D; ++d) pre[d] = load_row(d, mis[d]);
+    first_rows(on_tag);
     __builtin_amdgcn_sched_barrier(0);
     GGUF_PHASE(7);                             // weight requests of the first rows are out
 #pragma unroll
     for (int g = 0; g < QG; ++g) {   // (keeps the conversions below from moving above the weight requests)
-      xraw[g].hold();
-      if constexpr (GATED) xup[g].hold();
+      if constexpr (DMA) {
+        // The compiler orders loads that write LDS like flat accesses and would wait for every load in flight, the
+        // weights included, before the first use of an activation value.  The activation loads are older than the
+        // weight loads and loads return in order: they have landed when no more than the weight loads are outstanding.
+        constexpr int BEHIND = decltype(on_tag)::value ? DMA_INSTRS : 0;
+        xraw[g].template landed<BEHIND>();
+        if constexpr (GATED) xup[g].template landed<BEHIND>();
+      } else {
+        xraw[g].hold();
+        if constexpr (GATED) xup[g].hold();
+      }
     }
 #pragma unroll
     for (int g = 0; g < QG; ++g) quantize_group(xraw[g], xup[GATED ? g : 0], tid + g * NT);
   };
   // (wave-uniform: a wave whose first lane is past the last group takes no part in the quantisation and reaches the
   // barrier as soon as its weight requests are out, instead of after a load and a quantisation nobody uses)
-  if (wave * 64 >= qtotal) prologue(std::integral_constant<int, 0>{});
-  else if (qtotal <= NT) prologue(std::integral_constant<int, 1>{});
-  else if (qtotal <= 2 * NT) prologue(std::integral_constant<int, 2>{});
-  else prologue(std::integral_constant<int, 4>{});
+  auto prologue_for = [&](auto on_tag) {
+    if (wave * 64 >= qtotal) prologue(std::integral_constant<int, 0>{}, on_tag);
+    else if (qtotal <= NT) prologue(std::integral_constant<int, 1>{}, on_tag);
+    else if (qtotal <= 2 * NT) prologue(std::integral_constant<int, 2>{}, on_tag);
+    else prologue(std::integral_constant<int, 4>{}, on_tag);
+  };
+  // (DMA: a wave without a slot asks for no weights; its prologue is a copy of its own, so that the one with the
+  //  requests has them outside any branch and the wait for the activations can count them)
+  if (DMA && !wave_on) prologue_for(std::false_type{});
+  else prologue_for(std::true_type{});
   for (int q = tid + 4 * NT; q - tid < qtotal; q += NT) {  // uniform trip count; only for K * MT > 32 * NT
     const int qc = min(q, qtotal - 1);
     const int m2 = row_of_group(qc), j2 = qc - m2 * g8;
@@ -557,6 +620,39 @@ __device__ __forceinline__ void mmvq_stream_body(const uint8_t* __restrict__ W, 
 
   // (a wave without a slot -- NW is not always a multiple of the waves a row takes -- has quantized its share of the
   //  activations and waits at the barrier behind the loop)
+  // one row's dot products -> its partial sums in LDS
+  auto finish_row = [&](const typename F::Regs& cur, int i, bool row_ok) {
+    float acc[MT];
+#pragma unroll
+    for (int m = 0; m < MT; ++m) {
+      const float v = F::dot(cur, act[m], u);
+      acc[m] = lane_on ? v : 0.0f;
+    }
+    const float v = rows16_sums<MT>(acc, lane);
+    if ((lane & 15) < MT && row_ok) part[((slot + slots * i) * G + step * GW + ((lane >> 4) & (GW - 1))) * MT + (lane & 15)] = v;
+  };
+  if constexpr (DMA) {
+    // Loads return in order: row i has landed once no more loads are outstanding than those of the rows requested
+    // behind it, `ahead` of them (the counter's operand is an immediate: one case per count).
+    constexpr int NRI = Span::NR;
+    int r = 0;
+    for (int i = 0; wave_on && i < max_rows; ++i) {
+      const int ahead = min(D - 1, max_rows - 1 - i);
+      if (ahead >= D - 1) wait_vm_upto((D - 1) * NRI);
+      else if (D > 2 && ahead == D - 2) wait_vm_upto((D > 2 ? D - 2 : 0) * NRI);
+      else if (D > 3 && ahead == D - 3) wait_vm_upto((D > 3 ? D - 3 : 0) * NRI);
+      else wait_vm_upto(0);
+      const typename F::Regs cur = F::from_span(stage + r * DMA_SLOT, lane);
+      if (i + D < max_rows) {
+        // the slot is asked for again only after this lane's reads of it have returned
+        asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+        dma_row(i + D, r);
+      }
+      finish_row(cur, i, i < my_rows);
+      r = r + 1 == D ? 0 : r + 1;
+    }
+  }
+  if constexpr (!DMA)
   for (int i0 = 0; (HALF || wave_on) && i0 < max_rows; i0 += D) {
 #pragma unroll
     for (int d = 0; d < D; ++d) {
@@ -645,6 +741,9 @@ static bool span_aligned(const void* W, int64_t pitch, int K) {
   return (int64_t)(K / F::QK) * F::BS % 16 == 0 && pitch % 16 == 0 && (uintptr_t)W % 16 == 0;
 }
 
+// Formats whose aligned stretches the streaming kernel fetches straight into LDS (STAGED_DMA)
+template <class F> struct DmaRing { static constexpr bool on = SpanOf<F>::value > 0; };
+
 template <class F, int MT, int D, typename T, bool TILE, bool FULL, int NW, int STAGED = 0>
 static void launch_stream_d(const void* W, const T* X, T* Y, int N, int K, int rows_per_wg, int grid, size_t lds, const LinearArgs& la,
                             hipStream_t stream, int m_act) {
@@ -681,22 +780,36 @@ static bool launch_stream(const void* W, const T* X, T* Y, int N, int K, hipStre
       // (for Q4_K, whose per-lane loads are aligned 16-byte pieces already, the trip through LDS costs the 8-wave kernel
       //  of the small matrices as much as it gains; [4096,4096]: Q8_0 6.4 -> 5.1 us, Q4_0 5.1 -> 4.4 us, Q6_K 6.2 -> 5.4 us)
       // (Q8_0, most bytes per weight, still gains at four rows: [14336,4096] 16.6 -> 15.4 us)
-      if constexpr (MT <= (std::is_same<F, FmtQ8_0>::value ? 4 : MMVQ_STAGED_MT) && (NW == MMVQ_NW || !std::is_same<F, FmtQ4_K>::value) && SpanOf<F>::value > 0) {
+      if constexpr (MT <= (std::is_same<F, FmtQ8_0>::value ? 4 : MMVQ_STAGED_MT) && (NW == MMVQ_NW || !std::is_same<F, FmtQ4_K>::value || DmaRing<F>::on) && SpanOf<F>::value > 0) {
         // rows of whole 16-byte pieces at aligned addresses: every byte is requested once (see SpanRegs)
         const int64_t pitch = la.w_pitch ? la.w_pitch : (int64_t)(K / F::QK) * F::BS;
         const size_t lds_staged = lds + (size_t)NW * 16 * SpanRegs<SpanOf<F>::value, SpanAny<F>::value>::PIECES + SpanSlack<F>::value;
         // (a row shorter than one stretch leaves half the lanes of its wave without a block: not worth the trip through LDS,
         //  Q8_0 [3072,1024] 3.3 -> 3.8 us)
         if (per_wave >= MMVQ_DEPTH && nb >= 64 && lds_staged <= 160 * 1024) {
-          if (span_aligned<F>(W, pitch, K)) {
-            if (nb % 64 == 0) launch_stream_d<F, MT, MMVQ_DEPTH, T, TILE, FULL, NW, STAGED_ALIGNED>(W, X, Y, N, K, rows_per_wg, grid, lds_staged, la, stream, m_act);
-            else launch_stream_d<F, MT, MMVQ_DEPTH, T, TILE, FULL, NW, SpanAny<F>::value ? STAGED_ANY : STAGED_PART>(W, X, Y, N, K, rows_per_wg, grid, lds_staged, la, stream, m_act);
-            return;
+          if constexpr (DmaRing<F>::on && MT <= 2) {
+            // whole aligned stretches straight into a ring in LDS, as deep as the rows a wave walks where LDS has the room
+            // (the activations must be quantized by the prologue's straight-line code: its loads are counted)
+            const size_t slot = 1024 * SpanRegs<SpanOf<F>::value>::NR;
+            const auto fits = [&](int d) { return per_wave >= d && lds + (size_t)NW * d * slot <= 160 * 1024; };
+            // (rows of up to two stretches on the 16-wave kernel: Q4_K [14336,4096] 8.9 -> 8.5 us; longer rows and the 8-wave
+            //  kernel of small matrices lose a little)
+            if (NW == MMVQ_NW && S <= 2 && nb % 64 == 0 && span_aligned<F>(W, pitch, K) && (size_t)MT * K <= 32 * 64 * NW) {
+              if (fits(MMVQ_DMA_DEPTH)) { launch_stream_d<F, MT, MMVQ_DMA_DEPTH, T, TILE, FULL, NW, STAGED_DMA>(W, X, Y, N, K, rows_per_wg, grid, lds + (size_t)NW * MMVQ_DMA_DEPTH * slot, la, stream, m_act); return; }
+            }
           }
-          if constexpr (SpanAny<F>::value) {
-            if (pitch % 2 == 0 && (uintptr_t)W % 2 == 0) {
-              launch_stream_d<F, MT, MMVQ_DEPTH, T, TILE, FULL, NW, STAGED_ANY>(W, X, Y, N, K, rows_per_wg, grid, lds_staged, la, stream, m_act);
+          // (through registers the trip costs the 8-wave kernel of Q4_K as much as it gains: per-lane loads below)
+          if constexpr (NW == MMVQ_NW || !std::is_same<F, FmtQ4_K>::value) {
+            if (span_aligned<F>(W, pitch, K)) {
+              if (nb % 64 == 0) launch_stream_d<F, MT, MMVQ_DEPTH, T, TILE, FULL, NW, STAGED_ALIGNED>(W, X, Y, N, K, rows_per_wg, grid, lds_staged, la, stream, m_act);
+              else launch_stream_d<F, MT, MMVQ_DEPTH, T, TILE, FULL, NW, SpanAny<F>::value ? STAGED_ANY : STAGED_PART>(W, X, Y, N, K, rows_per_wg, grid, lds_staged, la, stream, m_act);
               return;
+            }
+            if constexpr (SpanAny<F>::value) {
+              if (pitch % 2 == 0 && (uintptr_t)W % 2 == 0) {
+                launch_stream_d<F, MT, MMVQ_DEPTH, T, TILE, FULL, NW, STAGED_ANY>(W, X, Y, N, K, rows_per_wg, grid, lds_staged, la, stream, m_act);
+                return;
+              }
             }
           }
         }

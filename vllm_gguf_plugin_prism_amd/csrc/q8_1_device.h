@@ -15,9 +15,19 @@ namespace gguf {
 // Eight consecutive activation values: raw8<T>::load only issues the global load (so it can be hoisted
 // above other loads without forcing a wait), cvt widens to fp32.
 template <typename T> struct raw8;
+typedef float raw_f32x4 __attribute__((ext_vector_type(4)));      // (plain vector types: a register tuple the inline
+typedef uint32_t raw_u32x4 __attribute__((ext_vector_type(4)));   //  assembly below can name as one operand)
 template <> struct raw8<float> {
-  float4 a, b;
-  __device__ __forceinline__ void load(const float* p) { a = *(const float4*)p; b = *(const float4*)(p + 4); }
+  raw_f32x4 a, b;
+  __device__ __forceinline__ void load(const float* p) { a = *(const raw_f32x4*)p; b = *(const raw_f32x4*)(p + 4); }
+  // The same load kept from the compiler's count of loads in flight, for a kernel that has loads outstanding which the
+  // values need not wait for: landed() waits until at most `behind` younger loads are outstanding (loads return in order).
+  __device__ __forceinline__ void load_uncounted(const float* p) {
+    asm volatile("global_load_dwordx4 %0, %2, off\n\tglobal_load_dwordx4 %1, %2, off offset:16" : "=&v"(a), "=&v"(b) : "v"(p) : "memory");
+  }
+  template <int BEHIND> __device__ __forceinline__ void landed() {
+    asm volatile("s_waitcnt vmcnt(%2)" : "+v"(a), "+v"(b) : "n"(BEHIND) : "memory");
+  }
   // Nothing that uses the loaded values may be scheduled before this point (and the wait for them comes here).
   __device__ __forceinline__ void hold() {
     asm volatile("" : "+v"(a.x), "+v"(a.y), "+v"(a.z), "+v"(a.w), "+v"(b.x), "+v"(b.y), "+v"(b.z), "+v"(b.w));
@@ -27,8 +37,10 @@ template <> struct raw8<float> {
   }
 };
 template <> struct raw8<_Float16> {
-  uint4 a;
-  __device__ __forceinline__ void load(const _Float16* p) { a = *(const uint4*)p; }
+  raw_u32x4 a;
+  __device__ __forceinline__ void load(const _Float16* p) { a = *(const raw_u32x4*)p; }
+  __device__ __forceinline__ void load_uncounted(const _Float16* p) { asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(a) : "v"(p) : "memory"); }
+  template <int BEHIND> __device__ __forceinline__ void landed() { asm volatile("s_waitcnt vmcnt(%1)" : "+v"(a) : "n"(BEHIND) : "memory"); }
   __device__ __forceinline__ void hold() { asm volatile("" : "+v"(a.x), "+v"(a.y), "+v"(a.z), "+v"(a.w)); }
   __device__ __forceinline__ void cvt(float (&v)[8]) const {
     const uint32_t w[4] = {a.x, a.y, a.z, a.w};
@@ -40,8 +52,10 @@ template <> struct raw8<_Float16> {
   }
 };
 template <> struct raw8<bf16_t> {
-  uint4 a;
-  __device__ __forceinline__ void load(const bf16_t* p) { a = *(const uint4*)p; }
+  raw_u32x4 a;
+  __device__ __forceinline__ void load(const bf16_t* p) { a = *(const raw_u32x4*)p; }
+  __device__ __forceinline__ void load_uncounted(const bf16_t* p) { asm volatile("global_load_dwordx4 %0, %1, off" : "=&v"(a) : "v"(p) : "memory"); }
+  template <int BEHIND> __device__ __forceinline__ void landed() { asm volatile("s_waitcnt vmcnt(%1)" : "+v"(a) : "n"(BEHIND) : "memory"); }
   __device__ __forceinline__ void hold() { asm volatile("" : "+v"(a.x), "+v"(a.y), "+v"(a.z), "+v"(a.w)); }
   __device__ __forceinline__ void cvt(float (&v)[8]) const {
     const uint32_t w[4] = {a.x, a.y, a.z, a.w};
