@@ -53,10 +53,11 @@ int gguf_block_bytes(int type);
 
 /* Bytes of activation workspace per row of X for inner dimension K.
  * The reference sizes its workspace as int32[M, roundup(K,512)/32*9]
- * (gguf_kernel.cu:114-115); this library's private layout needs 108 bytes per 32
- * values instead of 36 (the quantized rows, and room for their dequantized half-precision
- * copy that the half-MFMA engine of gguf_mmq reads), so callers must size the workspace
- * with this function. */
+ * (gguf_kernel.cu:114-115); this library's private layout needs 44 bytes per 32
+ * values instead of 36 (int8 quants, then fp32 planes of the scale, the stored sum and
+ * scale x quant sum), so callers must size the workspace with this function.  The
+ * half-MFMA engine of gguf_mmq keeps a half-precision copy of the rows as well: its
+ * callers size the workspace with gguf_mmq_workspace_bytes_engine(..., GGUF_MMQ_HALF). */
 int64_t gguf_q8_1_row_bytes(int64_t K);
 
 /* q8_1 activation quantizer: M rows of K values -> workspace.
@@ -106,7 +107,12 @@ int gguf_mmq(const void* W, const void* x, int xdtype, void* q8_workspace, void*
 #define GGUF_MMQ_AUTO 0
 #define GGUF_MMQ_INT8 1
 #define GGUF_MMQ_HALF 2
-int64_t gguf_mmq_workspace_bytes(int64_t M, int64_t N, int64_t K);
+int64_t gguf_mmq_workspace_bytes(int64_t M, int64_t N, int64_t K);   /* room for either engine */
+/* The same for one engine (GGUF_MMQ_AUTO counts as GGUF_MMQ_INT8): only the half engine pays for the half-precision
+ * copy of the rows (64 bytes per 32 values on top of the 44).  GGUF_MMQ_HALF needs at least its row region,
+ * M * (gguf_q8_1_row_bytes(K) + 2 * (roundup(K, 512) + 128)) bytes, and returns GGUF_ERR_WORKSPACE below that; for it
+ * workspace_bytes = 0 is not accepted. */
+int64_t gguf_mmq_workspace_bytes_engine(int64_t M, int64_t N, int64_t K, int engine);
 int gguf_mmq_engine(const void* W, const void* x, int xdtype, void* q8_workspace, void* Y, int type, int64_t N, int64_t K,
                     int64_t M, int engine, int64_t workspace_bytes, gguf_stream_t stream);
 
@@ -146,8 +152,8 @@ int gguf_mmq_linear(const void* W, int64_t w_row_pitch_bytes, const void* x, int
  * batch sizes without an a8 kernel, ggml_dequantize followed by x @ weight.T (quantization/linear.py:50-58,
  * diffusion_config.py:21-30), which writes and re-reads the dense weights.  The weights take the half-precision
  * values the reference's dequantize kernels produce; X is converted to half.  X / Y dtype: fp16 or bf16.  Types: the
- * twelve standard and K formats plus IQ4_XS and IQ2_XXS.  Workspace: gguf_mmq_workspace_bytes(M, N, K) (or at least
- * M * gguf_q8_1_row_bytes(K), without the K split for small outputs). */
+ * twelve standard and K formats plus IQ4_XS and IQ2_XXS.  Workspace: gguf_mmq_workspace_bytes_engine(M, N, K,
+ * GGUF_MMQ_HALF); GGUF_ERR_WORKSPACE below the half engine's row region. */
 int gguf_dequant_gemm(const void* W, const void* x, int xdtype, void* workspace, void* Y, int type, int64_t N, int64_t K,
                       int64_t M, int64_t workspace_bytes, gguf_stream_t stream);
 
@@ -170,12 +176,14 @@ int gguf_moe_vec(const void* X, int xdtype, void* q8_workspace, const void* W, c
  * activation kernel would have stored it (quantization/fused_moe.py:44-51,80,92: act() between the two GEMMs).
  * act: 0 = none (X has K columns, same as the plain entry points), 1 = SiLU, 2 = GELU (erf).
  * gguf_moe_vec_act also takes the number of experts in W (0 = unknown) and the size of the workspace (0 = the
- * minimum, tokens * gguf_q8_1_row_bytes(K)).  When tokens*top_k >= 2*num_experts and the workspace has room for the
- * routing sort as well -- gguf_moe_vec_workspace_bytes() -- the pairs are sorted by expert, the activations quantized
- * once, and the pairs of an expert share each pass over its weights, so a shared expert is read about once per call
- * rather than once per pair (the reference's grid re-reads it per pair, moe_vec.cuh:3-53): 32 pairs per pass on the
- * grouped int8-MFMA kernel for the formats that have tiles (up to 256 experts; Q5_0 excepted), four per pass on the
- * vector kernel for the others.  The operator's arithmetic is the GEMV's on every route (Q4_K / Q5_K offsets from the
+ * minimum, tokens * gguf_q8_1_row_bytes(K)).  When experts are shared -- tokens*top_k >= 2*num_experts, or >= 2.5 *
+ * num_experts while all experts together are at most 192 MiB and so stay in the last-level cache, where the per-pair
+ * kernel reads them from -- and the workspace has room for the routing sort as well, gguf_moe_vec_workspace_bytes(),
+ * the pairs are sorted by expert, the activations quantized once, and the pairs of an expert share each pass over its
+ * weights, so a shared expert is read about once per call rather than once per pair (the reference's grid re-reads it
+ * per pair, moe_vec.cuh:3-53): on the grouped int8-MFMA kernels for the formats that have tiles (up to 256 experts;
+ * Q5_0 excepted) -- blocks of 16 slots while tokens*top_k <= 16*num_experts (Q4_0, Q8_0, Q3_K, Q4_K, Q5_K, Q6_K,
+ * IQ4_XS, IQ2_XXS), blocks of 32 above -- and four pairs per pass on the vector kernel for the others.  The operator's arithmetic is the GEMV's on every route (Q4_K / Q5_K offsets from the
  * quant sums); results agree to fp32 summation order. */
 int64_t gguf_moe_vec_workspace_bytes(int64_t tokens, int64_t top_k, int64_t K, int64_t num_experts);
 int gguf_moe_mmq_act(const void* X, int xdtype, void* q8_workspace, const void* W, int64_t expert_stride_bytes,
@@ -189,6 +197,20 @@ int gguf_moe_vec_act(const void* X, int xdtype, void* q8_workspace, const void* 
 /* Token-tile size that moe_align_block_size must pad expert groups to; 0 for unknown types.
  * Replaces ggml_moe_get_block_size (gguf_kernel.cu:532-566). */
 int gguf_moe_block_size(int type);
+
+/* The grouped operator with the block size of the routing sort stated by the caller, 32 or 16, and the number of
+ * experts in W (0 = not stated).  The reference tiles 4 or 8 tokens (moe.cuh:131-139, gguf_kernel.cu:532-566); here
+ * blocks of 32 slots suit experts with many pairs and blocks of 16 (int8 MFMA 16x16 tiles; Q4_0, Q8_0, Q3_K, Q4_K,
+ * Q5_K, Q6_K, IQ4_XS, IQ2_XXS, GGUF_ERR_TYPE otherwise) suit a layer whose experts see 16 pairs or fewer on average, where most
+ * of a 32-slot block would be padding: gguf_moe_block_size_for(type, tokens * top_k, num_experts) returns the one to
+ * sort with.  Arithmetic is the tile operator's either way (offset terms on the stored block sums).  num_experts above
+ * 256 is GGUF_ERR_SHAPE: the kernels keep the reference's guard that skips blocks of experts above 255 (moe.cuh:33),
+ * and a caller who states the count is told instead of receiving rows of zeros.  act as for gguf_moe_mmq_act. */
+int gguf_moe_block_size_for(int type, int64_t pairs, int64_t num_experts);
+int gguf_moe_mmq_block(const void* X, int xdtype, void* q8_workspace, const void* W, int64_t expert_stride_bytes,
+                       const int32_t* sorted_token_ids, const int32_t* expert_ids, const int32_t* num_tokens_post_padded,
+                       int64_t num_sorted, void* Y, int type, int64_t N, int64_t K, int64_t top_k, int64_t tokens, int act,
+                       int64_t block, int64_t num_experts, gguf_stream_t stream);
 
 /* Routing sort for the grouped kernel: pairs (flat index token*top_k + choice) grouped by expert in ascending index
  * order, every expert's run padded to a multiple of `block` with the value `numel`; one expert id per block (-1 past

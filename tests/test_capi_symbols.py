@@ -35,7 +35,7 @@ def handle():
 
 def test_header_declares_the_bound_entry_points():
     assert declared_symbols() == sorted(_lib.EXPORTS)
-    assert len(declared_symbols()) == 25
+    assert len(declared_symbols()) == 28
 
 
 def test_every_declared_symbol_is_exported(handle):
@@ -56,10 +56,10 @@ def test_block_sizes_match_the_format_table(handle):
 
 
 def test_workspace_row_bytes(handle):
-    # per 32 values of K rounded up to 512: int8 quants + three fp32 (44 bytes), and the half-precision copy (64 bytes) plus 256 bytes of row padding
-    assert handle.gguf_q8_1_row_bytes(4096) == 4096 // 32 * 108 + 256
-    assert handle.gguf_q8_1_row_bytes(256) == 512 // 32 * 108 + 256
-    assert handle.gguf_q8_1_row_bytes(14336) == 14336 // 32 * 108 + 256
+    # per 32 values of K rounded up to 512: int8 quants + three fp32 planes (44 bytes)
+    assert handle.gguf_q8_1_row_bytes(4096) == 4096 // 32 * 44
+    assert handle.gguf_q8_1_row_bytes(256) == 512 // 32 * 44
+    assert handle.gguf_q8_1_row_bytes(14336) == 14336 // 32 * 44
     assert handle.gguf_q8_1_row_bytes(0) == 0
 
 
@@ -67,6 +67,36 @@ def test_moe_block_size(handle):
     for qt in (2, 8, 12, 14):
         assert handle.gguf_moe_block_size(qt) == 32
     assert handle.gguf_moe_block_size(99) == 0
+    # blocks of 16 slots while an expert sees at most 16 pairs on average, for the formats that have such tiles
+    assert handle.gguf_moe_block_size_for(2, 64 * 16, 64) == 16
+    assert handle.gguf_moe_block_size_for(2, 64 * 16 + 1, 64) == 32
+    assert handle.gguf_moe_block_size_for(2, 8, 0) == 32                  # expert count not stated
+    assert handle.gguf_moe_block_size_for(3, 8, 64) == 32                 # Q4_1 has no 16-slot tiles
+    assert handle.gguf_moe_block_size_for(99, 8, 64) == 0
+
+
+def test_grouped_moe_states_its_limits_before_any_launch(handle):
+    """More than 256 stated experts, a block other than 16 or 32, or blocks of 16 for a format without such tiles are
+    refused by return code (the kernels would skip blocks of experts above 255 as moe.cuh:33 does)."""
+    args = lambda qt, block, experts: (None, 1, None, None, 0, None, None, None, 64, None, qt, 128, 256, 2, 4, 0, block, experts, None)
+    assert handle.gguf_moe_mmq_block(*args(2, 32, 257)) == -3
+    assert handle.gguf_moe_mmq_block(*args(2, 8, 64)) == -3
+    assert handle.gguf_moe_mmq_block(*args(3, 16, 64)) == -1
+    assert handle.gguf_moe_mmq_block(*args(2, 16, 64)) == -4              # passes the checks; null pointers next
+
+
+def test_workspace_sizes_by_engine(handle):
+    m, n, k = 2048, 18944, 18944
+    kp = (k + 511) // 512 * 512
+    assert handle.gguf_q8_1_row_bytes(k) == kp // 32 * 44
+    int8 = handle.gguf_mmq_workspace_bytes_engine(m, n, k, 1)
+    half = handle.gguf_mmq_workspace_bytes_engine(m, n, k, 2)
+    assert handle.gguf_mmq_workspace_bytes_engine(m, n, k, 0) == int8     # auto is the integer engine
+    rows = m * kp // 32 * 44
+    assert rows <= int8 < rows + (80 << 20)                                # quantized rows, then fp32 partial tiles
+    assert half >= rows + m * 2 * (kp + 128)                               # only the half engine keeps half-precision rows
+    assert handle.gguf_mmq_workspace_bytes(m, n, k) == max(int8, half)
+    assert handle.gguf_mmq_workspace_bytes_engine(m, n, k, 3) == 0
 
 
 def test_argument_validation_needs_no_gpu(handle):

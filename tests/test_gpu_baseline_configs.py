@@ -188,7 +188,12 @@ def test_config5_moe_layer_full_size(tokens, moe_weights):
     y = o.moe_a8_vec(a.astype(np.float32), w2, ids_s.reshape(-1), 1, qt, H, len(sample) * top_k)
     y = y.astype(np.float16).astype(np.float64).reshape(len(sample), top_k, H)
     want = (y * tw_s.astype(np.float16).astype(np.float64)[:, :, None]).astype(np.float16).astype(np.float64).sum(1)
-    # fp16 storage between the stages and the re-quantization of a slightly different intermediate bound the error
+    # What separates the two: (i) the layer's result is rounded to half once more than `want` (2^-11 / sqrt(3) = 2.8e-4
+    # at most, about 1.7e-4 on these values); (ii) fp32 against fp64 sums flip the half rounding of about one intermediate
+    # value in 2^13, each flip moves one of 1024 inputs of the second product by 2^-11 of its size -- below 1e-5 of the
+    # result; (iii) such a flip seldom moves a q8_1 code (probability about 127 * 2^-11 * |a| / amax per flipped value)
+    # and then by one step of amax / 127: also below 1e-5.  So the stated tolerance of the operators holds for the whole
+    # layer; measured 2.0e-4 to 2.3e-4 at 1, 64 and 512 tokens.
     err = o.rel_l2(got[sample].float().cpu().numpy(), want)
     print(f"config5 layer T={tokens}: rel-L2 of the layer against the per-token definition {err:.3e}")
-    assert err <= 1e-2
+    assert err <= 1e-3

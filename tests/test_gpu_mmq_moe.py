@@ -223,11 +223,17 @@ def test_mmq_half_engine_splits_the_last_round():
     ref = ops.ggml_mul_mat_a8(w, xd.float(), o.Q6_K, n).double()          # integer engine, fp32 result
     err = ((y.double() - ref).norm(dim=0) / ref.norm(dim=0))               # per output column: every tile is looked at
     assert float(err.max()) <= 1.5e-3 and float((y.double() - ref).norm() / ref.norm()) <= 6e-4
-    ws = torch.empty(m * _lib.lib().gguf_q8_1_row_bytes(k), dtype=torch.uint8, device="cuda")
+    # the half engine's row region and nothing behind it: no room for partial tiles, no split
+    kp = (k + 511) // 512 * 512
+    ws = torch.empty(m * (_lib.lib().gguf_q8_1_row_bytes(k) + 2 * (kp + 128)), dtype=torch.uint8, device="cuda")
     y_plain = torch.empty_like(y, dtype=torch.float16)
     rc = _lib.lib().gguf_mmq_engine(w.data_ptr(), xd.data_ptr(), 1, ws.data_ptr(), y_plain.data_ptr(), o.Q6_K, n, k, m,
                                     ops.MMQ_ENGINES["half"], ws.numel(), torch.cuda.current_stream().cuda_stream)
     assert rc == 0
+    # a workspace that holds the quantized rows only is too small for this engine, and says so
+    rc = _lib.lib().gguf_mmq_engine(w.data_ptr(), xd.data_ptr(), 1, ws.data_ptr(), y_plain.data_ptr(), o.Q6_K, n, k, m,
+                                    ops.MMQ_ENGINES["half"], m * _lib.lib().gguf_q8_1_row_bytes(k), torch.cuda.current_stream().cuda_stream)
+    assert rc == -6
     assert float((y_plain.double() - y.double()).norm() / ref.norm()) <= 4e-4
 
 
@@ -343,6 +349,33 @@ def test_moe_grouped_matches_oracle(qtype, t, top_k, e):
     y2 = ops.ggml_moe_a8(x2d, _dev(w), _dev(s), _dev(eids), _dev(npost), qtype, n, 1, t * top_k)
     exp2 = o.moe_a8(x2v, w, s, eids, npost, qtype, n, 1, t * top_k, blk)
     assert o.rel_l2(y2.cpu().numpy(), exp2) <= 1e-5
+
+
+@pytest.mark.parametrize("qtype", [o.Q4_0, o.Q8_0, o.Q3_K, o.Q4_K, o.Q5_K, o.Q6_K, o.IQ4_XS, o.IQ2_XXS])
+@pytest.mark.parametrize("t,top_k,e", [(7, 2, 8), (83, 4, 32), (100, 8, 64)])
+def test_moe_grouped_blocks_of_16_slots(qtype, t, top_k, e):
+    """The grouped operator on a routing sorted with blocks of 16 slots (ggml_moe_a8(..., block_size=16)): the tile
+    operator's arithmetic (stored block sums for the offset terms of Q4_K / Q5_K) on 16-row tiles, both stages of the
+    layer, against the oracle's per-pair definition; rows that no slot names stay zero."""
+    ops = _ops()
+    rng = np.random.default_rng(740 + qtype + t)
+    n, k = 160, 512
+    assert ops.moe_block_size_for(qtype, t * top_k, e) == (16 if t * top_k <= 16 * e else 32)
+    w = np.stack([o.make_weights(rng, qtype, n, k) for _ in range(e)])
+    xd, xv = _x(rng, t, k, "f32")
+    ids, _ = _routing(rng, t, e, top_k)
+    s, eids, npost = o.moe_align_block_size(ids, 16, e)
+    y = ops.ggml_moe_a8(xd, _dev(w), _dev(s), _dev(eids), _dev(npost), qtype, n, top_k, t, block_size=16)
+    assert o.rel_l2(y.cpu().numpy(), o.moe_a8(xv, w, s, eids, npost, qtype, n, top_k, t, 16)) <= 1e-5
+    x2d, x2v = _x(rng, t * top_k, k, "f32")
+    y2 = ops.ggml_moe_a8(x2d, _dev(w), _dev(s), _dev(eids), _dev(npost), qtype, n, 1, t * top_k, block_size=16)
+    assert o.rel_l2(y2.cpu().numpy(), o.moe_a8(x2v, w, s, eids, npost, qtype, n, 1, t * top_k, 16)) <= 1e-5
+    # a routing that leaves pairs out: their rows are zero
+    s2 = s.copy()
+    dropped = s2[:16][s2[:16] < t * top_k]
+    s2[:16] = t * top_k
+    y3 = ops.ggml_moe_a8(xd, _dev(w), _dev(s2), _dev(eids), _dev(npost), qtype, n, top_k, t, block_size=16).cpu().numpy()
+    assert np.all(y3[dropped] == 0)
 
 
 @pytest.mark.parametrize("qtype", [o.Q4_0, o.Q4_K])

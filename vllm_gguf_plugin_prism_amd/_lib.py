@@ -39,6 +39,7 @@ _SIGNATURES = {
     "gguf_mmq_linear": (_c.c_int, [_c.c_void_p, _c.c_int64, _c.c_void_p, _c.c_int, _c.c_void_p, _c.c_void_p, _c.c_int64,
                                    _c.c_void_p, _c.c_int, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int, _c.c_int64, _c.c_void_p]),
     "gguf_mmq_workspace_bytes": (_c.c_int64, [_c.c_int64, _c.c_int64, _c.c_int64]),
+    "gguf_mmq_workspace_bytes_engine": (_c.c_int64, [_c.c_int64, _c.c_int64, _c.c_int64, _c.c_int]),
     "gguf_mmq_static_capacity": (_c.c_int64, []),
     "gguf_mmq_static": (_c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_int, _c.c_void_p, _c.c_int, _c.c_int64, _c.c_int64, _c.c_int64,
                                    _c.c_void_p]),
@@ -59,6 +60,10 @@ _SIGNATURES = {
                                     _c.c_void_p]),
     "gguf_moe_vec_workspace_bytes": (_c.c_int64, [_c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64]),
     "gguf_moe_block_size": (_c.c_int, [_c.c_int]),
+    "gguf_moe_block_size_for": (_c.c_int, [_c.c_int, _c.c_int64, _c.c_int64]),
+    "gguf_moe_mmq_block": (_c.c_int, [_c.c_void_p, _c.c_int, _c.c_void_p, _c.c_void_p, _c.c_int64, _c.c_void_p, _c.c_void_p,
+                                      _c.c_void_p, _c.c_int64, _c.c_void_p, _c.c_int, _c.c_int64, _c.c_int64, _c.c_int64,
+                                      _c.c_int64, _c.c_int, _c.c_int64, _c.c_int64, _c.c_void_p]),
     "gguf_moe_align_block_size": (_c.c_int, [_c.c_void_p, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_void_p, _c.c_int64,
                                              _c.c_void_p, _c.c_int64, _c.c_void_p, _c.c_void_p]),
     "gguf_moe_weighted_sum": (_c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int, _c.c_int64, _c.c_int64,

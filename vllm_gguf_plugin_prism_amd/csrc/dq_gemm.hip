@@ -54,6 +54,7 @@ extern "C" int gguf_dequant_gemm(const void* W, const void* x, int xdtype, void*
   hipStream_t s = (hipStream_t)stream;
   // same workspace layout as the a8 operator: the half rows sit behind the (here unused) quantized rows
   const int64_t rows_bytes = (M * (q8_row_bytes(K) + 2 * q8_half_pitch(K)) + 255) / 256 * 256;
+  if (workspace_bytes < M * (q8_row_bytes(K) + 2 * q8_half_pitch(K))) return GGUF_ERR_WORKSPACE;
   _Float16* xh = (_Float16*)((char*)workspace + M * q8_row_bytes(K));
   const int pitch = (int)q8_half_pitch(K);
   const unsigned gx = (unsigned)((pitch / 8 + 255) / 256);

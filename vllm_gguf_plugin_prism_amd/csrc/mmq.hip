@@ -627,15 +627,25 @@ int64_t mmq_int_partial_bytes(int M, int N, int K);
 
 }  // namespace gguf
 
-// bytes of the quantized rows and their half-precision copy, rounded up so that what follows is aligned
-static int64_t mmq_rows_bytes(int64_t M, int64_t K) { return (M * (gguf::q8_row_bytes(K) + 2 * gguf::q8_half_pitch(K)) + 255) / 256 * 256; }
+// Bytes of the row region of a workspace, rounded up so that what follows is aligned: the quantized rows, and for
+// the half engine their half-precision copy behind them.
+static int64_t mmq_rows_bytes(int64_t M, int64_t K, bool half_plane) {
+  return (M * (gguf::q8_row_bytes(K) + (half_plane ? 2 * gguf::q8_half_pitch(K) : 0)) + 255) / 256 * 256;
+}
 
-extern "C" int64_t gguf_mmq_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+extern "C" int64_t gguf_mmq_workspace_bytes_engine(int64_t M, int64_t N, int64_t K, int engine) {
   if (M <= 0 || N <= 0 || K <= 0 || M > 0x7FFFFFF0LL || N > 0x7FFFFFF0LL || K > 0x7FFFFFF0LL) return 0;
-  const int64_t ph = gguf::mmq_half_partial_bytes((int)M, (int)N, (int)K), pi = gguf::mmq_int_partial_bytes((int)M, (int)N, (int)K);
+  if (engine < GGUF_MMQ_AUTO || engine > GGUF_MMQ_HALF) return 0;
+  if (engine == GGUF_MMQ_HALF) return mmq_rows_bytes(M, K, true) + gguf::mmq_half_partial_bytes((int)M, (int)N, (int)K);
+  const int64_t pi = gguf::mmq_int_partial_bytes((int)M, (int)N, (int)K);
   const int64_t p16 = M <= gguf::MMQ_ROWS16_MAX ? gguf::mmq_rows16_partial_bytes((int)M, (int)N, (int)K) : 0;
-  const int64_t p = ph > pi ? ph : pi;
-  return mmq_rows_bytes(M, K) + (p > p16 ? p : p16);
+  return mmq_rows_bytes(M, K, false) + (pi > p16 ? pi : p16);
+}
+
+// room for either engine
+extern "C" int64_t gguf_mmq_workspace_bytes(int64_t M, int64_t N, int64_t K) {
+  const int64_t a = gguf_mmq_workspace_bytes_engine(M, N, K, GGUF_MMQ_INT8), b = gguf_mmq_workspace_bytes_engine(M, N, K, GGUF_MMQ_HALF);
+  return a > b ? a : b;
 }
 
 // gguf_mmq_linear with the size of the workspace's row region given by the caller: rows_bytes < 0 stands for the public
@@ -677,7 +687,13 @@ int gguf::mmq_linear_impl(const void* W, int64_t w_row_pitch_bytes, const void* 
   // (the 16-row tile kernel that reads the K-quants straight from the packed blocks takes the same time for 1 .. 16 rows
   // and passes the GEMV, which has one kernel for 5 .. 8 rows, there: Q4_K [14336,4096] 17 against 21 us at 6 rows,
   // against 14 us at 4; see rows16_direct_pays)
-  const int64_t partial_room = workspace_bytes - (rows_bytes < 0 ? mmq_rows_bytes(M, K) : rows_bytes);
+  // The row region: the quantized rows, for the half engine also their half-precision copy.  (A caller-given size is
+  // that of quantized rows only.)
+  if (rows_bytes >= 0 && engine == GGUF_MMQ_HALF) return GGUF_ERR_SHAPE;   // no room for the half-precision rows in that layout
+  if (rows_bytes < 0) rows_bytes = mmq_rows_bytes(M, K, engine == GGUF_MMQ_HALF);
+  if (workspace_bytes == 0 && engine != GGUF_MMQ_HALF) workspace_bytes = M * q8_row_bytes(K);   // the stated minimum
+  if (workspace_bytes < M * (q8_row_bytes(K) + (engine == GGUF_MMQ_HALF ? 2 * q8_half_pitch(K) : 0))) return GGUF_ERR_WORKSPACE;
+  const int64_t partial_room = workspace_bytes - rows_bytes;
   const bool tiles_at_5 = M <= 16 && rows16_direct_pays(type, (int)M, N, K, true) && rows16_direct_takes(W, w_row_pitch_bytes, type, (int)M, (int)N, (int)K, partial_room > 0 ? partial_room : 0);
   if (engine == GGUF_MMQ_AUTO && M <= 8 && !tiles_at_5) {
     // a handful of rows: the streaming GEMV kernel with the tile kernels' offset sums reads W once at close to the
@@ -688,8 +704,6 @@ int gguf::mmq_linear_impl(const void* W, int64_t w_row_pitch_bytes, const void* 
     if (rc != GGUF_NOT_TAKEN) return rc;
   }
   if (engine == GGUF_MMQ_AUTO) engine = GGUF_MMQ_INT8;   // the reference's arithmetic; the half engine is for callers that ask
-  if (rows_bytes < 0) rows_bytes = mmq_rows_bytes(M, K);
-  else if (engine == GGUF_MMQ_HALF) return GGUF_ERR_SHAPE;   // no room for the half-precision rows in this layout
   float* partial = (float*)((char*)q8_workspace + rows_bytes);
   const int64_t partial_bytes = workspace_bytes > rows_bytes ? workspace_bytes - rows_bytes : 0;
   if (engine == GGUF_MMQ_HALF) {
@@ -739,27 +753,41 @@ extern "C" int gguf_mmq(const void* W, const void* x, int xdtype, void* q8_works
 
 extern "C" int gguf_moe_block_size(int type) { return gguf::block_elems(type) ? 32 : 0; }
 
-extern "C" int gguf_moe_mmq_act(const void* X, int xdtype, void* q8_workspace, const void* W, int64_t expert_stride_bytes,
-                                const int32_t* sorted_token_ids, const int32_t* expert_ids,
-                                const int32_t* num_tokens_post_padded, int64_t num_sorted, void* Y, int type, int64_t N,
-                                int64_t K, int64_t top_k, int64_t tokens, int act, gguf_stream_t stream);
-
 extern "C" int gguf_moe_mmq(const void* X, int xdtype, void* q8_workspace, const void* W, int64_t expert_stride_bytes,
                             const int32_t* sorted_token_ids, const int32_t* expert_ids,
                             const int32_t* num_tokens_post_padded, int64_t num_sorted, void* Y, int type, int64_t N,
                             int64_t K, int64_t top_k, int64_t tokens, gguf_stream_t stream) {
-  return gguf_moe_mmq_act(X, xdtype, q8_workspace, W, expert_stride_bytes, sorted_token_ids, expert_ids, num_tokens_post_padded,
-                          num_sorted, Y, type, N, K, top_k, tokens, 0, stream);
+  return gguf_moe_mmq_block(X, xdtype, q8_workspace, W, expert_stride_bytes, sorted_token_ids, expert_ids, num_tokens_post_padded,
+                            num_sorted, Y, type, N, K, top_k, tokens, 0, 32, 0, stream);
 }
 
 extern "C" int gguf_moe_mmq_act(const void* X, int xdtype, void* q8_workspace, const void* W, int64_t expert_stride_bytes,
                                 const int32_t* sorted_token_ids, const int32_t* expert_ids,
                                 const int32_t* num_tokens_post_padded, int64_t num_sorted, void* Y, int type, int64_t N,
                                 int64_t K, int64_t top_k, int64_t tokens, int act, gguf_stream_t stream) {
+  return gguf_moe_mmq_block(X, xdtype, q8_workspace, W, expert_stride_bytes, sorted_token_ids, expert_ids, num_tokens_post_padded,
+                            num_sorted, Y, type, N, K, top_k, tokens, act, 32, 0, stream);
+}
+
+extern "C" int gguf_moe_block_size_for(int type, int64_t pairs, int64_t num_experts) {
+  if (!gguf::block_elems(type)) return 0;
+  return num_experts > 0 && pairs <= 16 * num_experts && gguf::moe_tiles16_ok(type) ? 16 : 32;
+}
+
+extern "C" int gguf_moe_mmq_block(const void* X, int xdtype, void* q8_workspace, const void* W, int64_t expert_stride_bytes,
+                                  const int32_t* sorted_token_ids, const int32_t* expert_ids,
+                                  const int32_t* num_tokens_post_padded, int64_t num_sorted, void* Y, int type, int64_t N,
+                                  int64_t K, int64_t top_k, int64_t tokens, int act, int64_t block, int64_t num_experts,
+                                  gguf_stream_t stream) {
   using namespace gguf;
   if (act < 0 || act > 2) return GGUF_ERR_SHAPE;
   const int qk = block_elems(type);
   if (qk == 0 || !mmq_type_ok(type)) return GGUF_ERR_TYPE;
+  if (block != 32 && block != 16) return GGUF_ERR_SHAPE;
+  if (block == 16 && !moe_tiles16_ok(type)) return GGUF_ERR_TYPE;
+  // the kernels keep the reference's guard on expert ids (moe.cuh:33: blocks of experts above 255 are skipped); a
+  // caller that says how many experts there are is told so instead of receiving rows of zeros
+  if (num_experts < 0 || num_experts > 256) return GGUF_ERR_SHAPE;
   if (N < 0 || tokens < 0 || top_k <= 0 || num_sorted < 0 || K <= 0 || K % qk != 0 || expert_stride_bytes < 0 ||
       tokens * top_k > 0x7FFFFFF0LL || N > 0x7FFFFFF0LL)
     return GGUF_ERR_SHAPE;
@@ -774,8 +802,9 @@ extern "C" int gguf_moe_mmq_act(const void* X, int xdtype, void* q8_workspace, c
   const int rc = quantize_q8_1(X, xdtype, q8_workspace, tokens, K, s, act);
   if (rc != GGUF_OK) return rc;
   MoeArgs moe = {sorted_token_ids, expert_ids, num_tokens_post_padded, expert_stride_bytes, (int)top_k, (int)(tokens * top_k), 0};
-  const int ns = (int)(num_sorted / 32 * 32);  // a trailing partial block is ignored, like the reference's integer division
+  const int ns = (int)(num_sorted / block * block);  // a trailing partial block is ignored, like the reference's integer division
   if (ns == 0) return launch_status();
+  if (block == 16) return moe_tiles16(W, q8_workspace, Y, xdtype, type, (int)N, (int)K, ns, moe, s);
   switch (type) {
     case T_Q4_0: return moe_fmt<MQ4_0>(W, q8_workspace, Y, xdtype, (int)N, (int)K, ns, moe, s);
     case T_Q4_1: return moe_fmt<MQ4_1>(W, q8_workspace, Y, xdtype, (int)N, (int)K, ns, moe, s);

@@ -84,7 +84,7 @@ int quantize_q8_1(const void* x, int xdtype, void* ws, int64_t M, int64_t K, hip
 
 }  // namespace gguf
 
-extern "C" int64_t gguf_q8_1_row_bytes(int64_t K) { return K <= 0 ? 0 : gguf::q8_row_bytes(K) + 2 * gguf::q8_half_pitch(K); }
+extern "C" int64_t gguf_q8_1_row_bytes(int64_t K) { return K <= 0 ? 0 : gguf::q8_row_bytes(K); }
 
 extern "C" int gguf_quantize_q8_1(const void* x, int xdtype, void* ws, int64_t M, int64_t K, gguf_stream_t stream) {
   if (M < 0 || K <= 0 || K % 32 != 0) return GGUF_ERR_SHAPE;

@@ -190,12 +190,17 @@ def fused_moe_gguf(x, w1, w2, topk_weights, topk_ids, weight_type: int, weight_t
     topk_ids = topk_ids.to(torch.int32).contiguous()
     if path == "grouped":
         experts, rows, _ = w1.shape
-        block = ops.ggml_moe_get_block_size(weight_type)
+        # the reference sorts with ggml_moe_get_block_size(type); here a layer whose experts see few pairs each (65 .. 128
+        # tokens of a 64-expert top-8 layer) sorts with blocks of 16 slots where both formats have such tiles, so that the
+        # tiles are not mostly padding
+        block = min(ops.moe_block_size_for(weight_type, tokens * top_k, experts), ops.moe_block_size_for(weight_type2, tokens * top_k, experts))
+        if block != 16:
+            block = ops.ggml_moe_get_block_size(weight_type)
         sorted_ids, expert_ids, post_padded = ops.moe_align_block_size(topk_ids, block, experts)
-        out = ops.ggml_moe_a8(x, w1, sorted_ids, expert_ids, post_padded, weight_type, rows, top_k, tokens)
+        out = ops.ggml_moe_a8(x, w1, sorted_ids, expert_ids, post_padded, weight_type, rows, top_k, tokens, block_size=block)
         # act() of the reference is applied inside the second call, while its rows are quantized
         out = ops.ggml_moe_a8(out, w2, sorted_ids, expert_ids, post_padded, weight_type2, w2.shape[1], 1, tokens * top_k,
-                              activation=activation)
+                              activation=activation, block_size=block)
     elif path == "vec":
         rows = w1.shape[1]
         out = ops.ggml_moe_a8_vec(x, w1, topk_ids, top_k, weight_type, rows, tokens)

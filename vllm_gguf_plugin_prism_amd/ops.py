@@ -148,7 +148,8 @@ def ggml_mul_mat_a8(W: torch.Tensor, X: torch.Tensor, quant_type: int, row: int,
     out, w_pitch, ldy = _shard_args(W, X, quant_type, row, out, bias)
     vecs, col = X.shape
     with torch.cuda.device(X.device):
-        nbytes = max(_lib.lib().gguf_mmq_workspace_bytes(vecs, row, col), vecs * _lib.lib().gguf_q8_1_row_bytes(col), 16)
+        # (only the half engine pays for the half-precision copy of the rows)
+        nbytes = max(_lib.lib().gguf_mmq_workspace_bytes_engine(vecs, row, col, MMQ_ENGINES[engine]), 16)
         ws = torch.empty(nbytes, dtype=torch.uint8, device=X.device)
         rc = _lib.lib().gguf_mmq_linear(W.data_ptr(), w_pitch, X.data_ptr(), _code(X.dtype), ws.data_ptr(), out.data_ptr(), ldy,
                                         bias.data_ptr() if bias is not None else None, int(quant_type), row, col, vecs,
@@ -168,7 +169,7 @@ def ggml_dequant_gemm(W: torch.Tensor, X: torch.Tensor, quant_type: int, row: in
     vecs, col = X.shape
     with torch.cuda.device(X.device):
         out = torch.empty((vecs, row), dtype=X.dtype, device=W.device)
-        nbytes = max(_lib.lib().gguf_mmq_workspace_bytes(vecs, row, col), vecs * _lib.lib().gguf_q8_1_row_bytes(col), 16)
+        nbytes = max(_lib.lib().gguf_mmq_workspace_bytes_engine(vecs, row, col, MMQ_ENGINES["half"]), 16)
         ws = torch.empty(nbytes, dtype=torch.uint8, device=X.device)
         rc = _lib.lib().gguf_dequant_gemm(W.data_ptr(), X.data_ptr(), _code(X.dtype), ws.data_ptr(), out.data_ptr(),
                                           int(quant_type), row, col, vecs, nbytes, _stream(X))
@@ -191,11 +192,14 @@ def ggml_moe_a8(
     tokens: int,
     *,
     activation: str | None = None,
+    block_size: int | None = None,
 ) -> torch.Tensor:
     """Grouped MoE GEMM -> ``[tokens * top_k, row]`` (reference: gguf_kernel.cu:292-393).
 
     ``activation`` ("silu" / "gelu") is an extension: X then holds ``[gate | up]`` rows of twice the inner dimension and
-    the gated activation is applied while the rows are quantized, instead of by a separate kernel beforehand."""
+    the gated activation is applied while the rows are quantized, instead of by a separate kernel beforehand.
+    ``block_size`` is the block the routing was sorted with when it is not ``ggml_moe_get_block_size(quant_type)``:
+    :func:`moe_block_size_for` picks blocks of 16 slots for a layer whose experts see few pairs each."""
     _check_inputs(X, W, sorted_token_ids, expert_ids, num_tokens_post_padded)
     for t in (sorted_token_ids, expert_ids, num_tokens_post_padded):
         if t.dtype != torch.int32:
@@ -209,12 +213,19 @@ def ggml_moe_a8(
     with torch.cuda.device(X.device):
         out = torch.empty((tokens * top_k, row), dtype=X.dtype, device=W.device)
         ws = _workspace(X, tokens, col)
-        rc = _lib.lib().gguf_moe_mmq_act(
+        rc = _lib.lib().gguf_moe_mmq_block(
             X.data_ptr(), _code(X.dtype), ws.data_ptr(), W.data_ptr(), W.stride(0) * W.element_size(),
             sorted_token_ids.data_ptr(), expert_ids.data_ptr(), num_tokens_post_padded.data_ptr(),
-            sorted_token_ids.shape[0], out.data_ptr(), int(quant_type), row, col, top_k, tokens, act, _stream(X))
+            sorted_token_ids.shape[0], out.data_ptr(), int(quant_type), row, col, top_k, tokens, act,
+            int(block_size) if block_size else ggml_moe_get_block_size(quant_type), W.shape[0] if W.dim() == 3 else 0, _stream(X))
     _lib.check(rc, "ggml_moe_a8")
     return out
+
+
+def moe_block_size_for(quant_type: int, pairs: int, num_experts: int) -> int:
+    """Block size to sort the routing with for :func:`ggml_moe_a8` (``block_size=``): 16 while an expert sees 16 pairs or
+    fewer on average and the format has 16-slot tiles, else ``ggml_moe_get_block_size(quant_type)``; 0 for unknown types."""
+    return int(_lib.lib().gguf_moe_block_size_for(int(quant_type), int(pairs), int(num_experts)))
 
 
 def ggml_moe_a8_vec(
