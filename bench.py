@@ -35,7 +35,11 @@ ROOT = os.path.dirname(os.path.abspath(__file__))
 sys.path.insert(0, ROOT)
 
 HBM_PEAK_GBS = 8000.0          # MI355X HBM3E
-INT8_PEAK_TOPS = 5033.0        # dense int8 MFMA, K=32/64 shapes (256 CU x 8192 op/clk x 2.4 GHz)
+INT8_PEAK_TOPS = 5033.0        # dense int8 MFMA, double-K shapes v_mfma_i32_32x32x32_i8 / 16x16x64_i8 (256 CU x 8192 op/clk x 2.4 GHz)
+INT8_LEGACY_PEAK_TOPS = 2516.0 # the legacy-K shapes (v_mfma_i32_32x32x16_i8, 16x16x32_i8) run at half of it
+# the matrix instruction the integer engine issues per format: formats whose weight scale changes every 16 values
+# multiply 16 values at a time
+MMQ_INSTRUCTION = {14: "v_mfma_i32_32x32x16_i8", 11: "v_mfma_i32_32x32x16_i8"}
 F16_PEAK_TFLOPS = 2516.0       # dense half-precision MFMA
 Q4_K, Q6_K = 12, 14
 CFG2_SHAPES = [(4096, 4096), (14336, 4096), (4096, 14336)]
@@ -182,7 +186,38 @@ def _other_configs(rng, dev, w_14336x4096):
         res[f"config5_moe_q4_0_T{t}"] = {"path": dispatch.select_moe_path(Q4_0, Q4_0, t), "us": ms * 1e3,
                                          "TOPS": 2.0 * t * top_k * 3 * I * H / (ms * 1e-3) / 1e12,
                                          "distinct_expert_GBps": distinct * expert_bytes / (ms * 1e-3) / 1e9}
+    # every entry against the roofline its operator is bound by: HBM for dequantize / GEMV / per-pair MoE (algorithmic
+    # bytes; for the MoE layer each distinct expert once), int8 MFMA for the a8 tile GEMMs, half-precision MFMA for the
+    # library GEMM of the dequantize-then-GEMM route
+    for v in res.values():
+        if "GBps" in v:
+            v["roofline"] = {"bound": "hbm", "peak_GBps": HBM_PEAK_GBS, "frac": v["GBps"] / HBM_PEAK_GBS}
+        elif v.get("path") == "vec" and "distinct_expert_GBps" in v:   # the per-pair MoE operator: weights read, each distinct expert once
+            v["roofline"] = {"bound": "hbm (distinct experts once)", "peak_GBps": HBM_PEAK_GBS, "frac": v["distinct_expert_GBps"] / HBM_PEAK_GBS}
+        elif "TOPS" in v:
+            v["roofline"] = {"bound": "mfma int8", "peak_TOPS": INT8_PEAK_TOPS, "frac": v["TOPS"] / INT8_PEAK_TOPS}
+        elif "TFLOPS" in v:
+            v["roofline"] = {"bound": "mfma f16", "peak_TFLOPS": F16_PEAK_TFLOPS, "frac": v["TFLOPS"] / F16_PEAK_TFLOPS}
     return res
+
+
+def _errors(got, want):
+    """max-abs, rel-L2 and max-rel (over elements whose reference exceeds 1e-3 of the largest) of got against want."""
+    got, want = np.asarray(got, dtype=np.float64), np.asarray(want, dtype=np.float64)
+    d = np.abs(got - want)
+    big = np.abs(want) >= 1e-3 * np.abs(want).max()
+    return {"max_abs": float(d.max()), "rel_l2": float(np.linalg.norm(got - want) / np.linalg.norm(want)),
+            "max_rel": float((d[big] / np.abs(want[big])).max())}
+
+
+def _cpu_model():
+    try:
+        for line in open("/proc/cpuinfo"):
+            if line.lower().startswith("model name"):
+                return line.split(":", 1)[1].strip()
+    except OSError:
+        pass
+    return "unknown"
 
 
 def _probes(rng, dev):
@@ -380,7 +415,8 @@ def main() -> int:
                     call = lambda i, engine=engine: ops.ggml_mul_mat_a8(wd, x, Q6_K, n, engine=engine)  # noqa: E731
                     ms = _timed_ms(call, 20, eager=args.profile)
                     tops = 2.0 * m * n * k / (ms * 1e-3) / 1e12
-                    table[f"{n}x{k}@M{m}"] = {"ms": ms, "TOPS": tops, "frac_int8_peak": tops / INT8_PEAK_TOPS}
+                    table[f"{n}x{k}@M{m}"] = {"ms": ms, "TOPS": tops, "frac_int8_peak": tops / INT8_PEAK_TOPS,
+                                              "frac_int8_legacy_k_peak": tops / INT8_LEGACY_PEAK_TOPS}
             del wd
         ops_total = sum(2.0 * 512 * n * k for n, k in CFG3_SHAPES)
 
@@ -391,10 +427,16 @@ def main() -> int:
         tops512, half512 = at_m512(tables["auto"]), at_m512(tables["half"])
         out["mmq"] = {
             "metric": "Q6_K MMQ int8 TOPS @M=512", "value": tops512, "unit": "TOPS",
-            "engine": "gguf_mmq's default: exact int8 dot products on v_mfma_i32_32x32x32_i8, fp32 block scales",
+            "engine": "gguf_mmq's default: exact int8 dot products per block on int8 MFMA, fp32 block scales",
+            "matrix_instruction": MMQ_INSTRUCTION.get(Q6_K, "v_mfma_i32_32x32x32_i8")
+                                  + " (Q6_K's weight scale changes every 16 values: the legacy-K shape, whose own peak is half the chip's)",
             "dtype": "int8 products, int32 sums per block, fp32 accumulation",
             "roofline": {"bound": "mfma", "achieved": tops512, "peak": INT8_PEAK_TOPS, "unit": "TOP/s",
                          "frac": tops512 / INT8_PEAK_TOPS,
+                         "denominators": {"double_k_int8_peak_TOPS": INT8_PEAK_TOPS, "frac_of_double_k_peak": tops512 / INT8_PEAK_TOPS,
+                                          "legacy_k_int8_peak_TOPS": INT8_LEGACY_PEAK_TOPS,
+                                          "frac_of_legacy_k_peak": tops512 / INT8_LEGACY_PEAK_TOPS,
+                                          "used_for_frac": "double_k_int8_peak_TOPS (the chip's dense int8 peak)"},
                          "traffic": {f"{n}x{k}": _traffic(f"mmqi_q6_k_{n}x{k}_m512") for n, k in CFG3_SHAPES}},
             "per_shape": tables["auto"],
             "half_engine": {"value": half512, "unit": "TOPS", "frac_of_f16_mfma_peak": half512 / F16_PEAK_TFLOPS,
@@ -411,27 +453,39 @@ def main() -> int:
 
         n, k = CFG2_SHAPES[0]
         w = host_w[(n, k)]
-        x32 = torch.from_numpy(rng.standard_normal((1, k)).astype(np.float32))
+        x16 = torch.from_numpy(rng.standard_normal((1, k)).astype(np.float32)).to(torch.float16)
+        x32 = x16.float()
         threads_before = torch.get_num_threads()
         torch.set_num_threads(1)           # numpy's block decode is one thread; the matmul leg is held to the same
         best = None
         t_end = time.perf_counter() + 20.0
         reps = 0
-        while reps < 2 or (time.perf_counter() < t_end and reps < 8):
+        while reps < 6 or (time.perf_counter() < t_end and reps < 8):
             t0 = time.perf_counter()
             wd = oracle.dequantize(w, Q4_K, "f32", flavour="f32").reshape(n, k)
             t1 = time.perf_counter()
-            _ = x32 @ torch.from_numpy(wd).T
+            y_cpu = x32 @ torch.from_numpy(wd).T
             t2 = time.perf_counter()
             if reps > 0 and (best is None or t2 - t0 < best[0]):
                 best = (t2 - t0, t1 - t0, t2 - t1)
             reps += 1
         torch.set_num_threads(threads_before)
         qbytes = n * (k // 256) * 144
+        # the GPU result on the same bytes against this CPU result (unquantized activations: q8_1 noise, about 5e-3
+        # expected) and against the a8 oracle (the same q8_1 activations, exact integer dots)
+        y_gpu = ops.ggml_mul_mat_vec_a8(torch.from_numpy(w).to(dev), x16.to(dev), Q4_K, n).float().cpu().numpy()
+        y_a8 = oracle.mul_mat_a8(w, x32.numpy(), Q4_K, n, "mmvq")
+        print(f"CPU baseline on 1 of {os.cpu_count()} cores ({_cpu_model()}; torch threads {threads_before} -> 1 for the timed leg)",
+              file=sys.stderr)
         out["cpu_baseline"] = {
             "value": qbytes / best[0] / 1e9, "unit": "GB/s", "cores": 1, "kind": "port",
             "sample": f"Q4_K [{n},{k}] batch 1 on one thread: numpy fp32 block dequantize ({best[1] * 1e3:.1f} ms) + torch fp32 "
                       f"matmul ({best[2] * 1e3:.1f} ms), best of {reps - 1} after 1 warm-up",
+            "t_dequant_ms": best[1] * 1e3, "t_matmul_ms": best[2] * 1e3, "t_total_ms": best[0] * 1e3,
+            "effective_GOPS": 2.0 * n * k / best[0] / 1e9,
+            "cpu_model": _cpu_model(), "os_cpu_count": os.cpu_count(), "torch_num_threads": threads_before,
+            "gpu_vs_cpu_unquantized_activations": _errors(y_gpu, y_cpu.numpy()),
+            "gpu_vs_a8_oracle": _errors(y_gpu, y_a8),
         }
 
     if not args.no_other:
