@@ -201,7 +201,7 @@ int gguf_moe_block_size(int type);
 /* The grouped operator with the block size of the routing sort stated by the caller, 32 or 16, and the number of
  * experts in W (0 = not stated).  The reference tiles 4 or 8 tokens (moe.cuh:131-139, gguf_kernel.cu:532-566); here
  * blocks of 32 slots suit experts with many pairs and blocks of 16 (int8 MFMA 16x16 tiles; Q4_0, Q8_0, Q3_K, Q4_K,
- * Q5_K, Q6_K, IQ4_XS, IQ2_XXS, GGUF_ERR_TYPE otherwise) suit a layer whose experts see 16 pairs or fewer on average, where most
+ * Q5_K, Q6_K, IQ4_XS, IQ2_XXS, GGUF_ERR_TYPE otherwise) suit a layer whose experts see 12 pairs or fewer on average, where most
  * of a 32-slot block would be padding: gguf_moe_block_size_for(type, tokens * top_k, num_experts) returns the one to
  * sort with.  Arithmetic is the tile operator's either way (offset terms on the stored block sums).  num_experts above
  * 256 is GGUF_ERR_SHAPE: the kernels keep the reference's guard that skips blocks of experts above 255 (moe.cuh:33),

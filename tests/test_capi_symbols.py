@@ -67,9 +67,9 @@ def test_moe_block_size(handle):
     for qt in (2, 8, 12, 14):
         assert handle.gguf_moe_block_size(qt) == 32
     assert handle.gguf_moe_block_size(99) == 0
-    # blocks of 16 slots while an expert sees at most 16 pairs on average, for the formats that have such tiles
-    assert handle.gguf_moe_block_size_for(2, 64 * 16, 64) == 16
-    assert handle.gguf_moe_block_size_for(2, 64 * 16 + 1, 64) == 32
+    # blocks of 16 slots while an expert sees at most 12 pairs on average, for the formats that have such tiles
+    assert handle.gguf_moe_block_size_for(2, 64 * 12, 64) == 16
+    assert handle.gguf_moe_block_size_for(2, 64 * 12 + 1, 64) == 32
     assert handle.gguf_moe_block_size_for(2, 8, 0) == 32                  # expert count not stated
     assert handle.gguf_moe_block_size_for(3, 8, 64) == 32                 # Q4_1 has no 16-slot tiles
     assert handle.gguf_moe_block_size_for(99, 8, 64) == 0

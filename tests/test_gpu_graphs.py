@@ -65,3 +65,38 @@ def test_replays_match_eager(case):
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(out, eager), case
+
+
+@pytest.mark.parametrize("case", ["split_k", "few_rows"])
+def test_entry_point_without_workspace_replays_match_eager(case):
+    """gguf_mmq_static is meant for callers under graph capture: gguf_mmq_static_capacity() is called once beforehand
+    (it looks up the address of the library's scratch array), after which a captured call must do no set-up of its own.
+    One shape whose K is split (fp32 partial tiles and the second launch go through the array) and one that takes the
+    streaming kernel for a handful of rows; two replays each with eager work in between, against the eager result and
+    against gguf_mmq_engine."""
+    from vllm_gguf_plugin_prism_amd import _lib, ops
+    h = _lib.lib()
+    assert h.gguf_mmq_static_capacity() == 32 << 20           # before any capture
+    rng = np.random.default_rng(77)
+    qtype, m, n, k = {"split_k": (o.Q6_K, 200, 1792, 4096), "few_rows": (o.Q4_K, 3, 384, 1024)}[case]
+    w = _dev(o.make_weights(rng, qtype, n, k))
+    xs = [torch.randn(m, k, dtype=torch.float16, device="cuda") for _ in range(3)]
+    x = xs[0].clone()
+    y = torch.empty((m, n), dtype=torch.float16, device="cuda")
+
+    def fn():
+        rc = h.gguf_mmq_static(w.data_ptr(), x.data_ptr(), ops._code(x.dtype), y.data_ptr(), qtype, n, k, m,
+                               torch.cuda.current_stream().cuda_stream)
+        assert rc == 0
+        return y
+
+    graph, out = _capture(fn)
+    for xi in xs:
+        x.copy_(xi)
+        eager = fn().clone()
+        torch.cuda.synchronize()
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager), case
+        assert o.rel_l2(out.float().cpu().numpy(), ops.ggml_mul_mat_a8(w, x, qtype, n).float().cpu().numpy()) <= 1e-3

@@ -360,7 +360,7 @@ def test_moe_grouped_blocks_of_16_slots(qtype, t, top_k, e):
     ops = _ops()
     rng = np.random.default_rng(740 + qtype + t)
     n, k = 160, 512
-    assert ops.moe_block_size_for(qtype, t * top_k, e) == (16 if t * top_k <= 16 * e else 32)
+    assert ops.moe_block_size_for(qtype, t * top_k, e) == (16 if t * top_k <= 12 * e else 32)
     w = np.stack([o.make_weights(rng, qtype, n, k) for _ in range(e)])
     xd, xv = _x(rng, t, k, "f32")
     ids, _ = _routing(rng, t, e, top_k)

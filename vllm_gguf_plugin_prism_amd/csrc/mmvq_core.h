@@ -856,7 +856,10 @@ static bool launch_stream_moe(const void* W, const T* X, T* Y, int N, int K, con
   const int64_t target = num_cus();
   int rows_per_wg = N;
   int64_t best = INT64_MAX;
-  for (int b = 1; b <= 64; ++b) {
+  // (up to as many bands as put a workgroup on every CU: with one to three pairs, the batch-1 decode of a top-2 layer,
+  //  64 bands a pair would leave most of the chip idle)
+  const int max_bands = (int)(pairs > 0 && (target + pairs - 1) / pairs > 64 ? (target + pairs - 1) / pairs : 64);
+  for (int b = 1; b <= max_bands; ++b) {
     const int rows = (N + b - 1) / b;
     if (rows < slots && b > 1) break;
     const int64_t wgs = (int64_t)((N + rows - 1) / rows) * pairs, rounds = (wgs + target - 1) / target;

@@ -223,7 +223,7 @@ def ggml_moe_a8(
 
 
 def moe_block_size_for(quant_type: int, pairs: int, num_experts: int) -> int:
-    """Block size to sort the routing with for :func:`ggml_moe_a8` (``block_size=``): 16 while an expert sees 16 pairs or
+    """Block size to sort the routing with for :func:`ggml_moe_a8` (``block_size=``): 16 while an expert sees 12 pairs or
     fewer on average and the format has 16-slot tiles, else ``ggml_moe_get_block_size(quant_type)``; 0 for unknown types."""
     return int(_lib.lib().gguf_moe_block_size_for(int(quant_type), int(pairs), int(num_experts)))
 
