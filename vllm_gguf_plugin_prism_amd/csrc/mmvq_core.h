@@ -312,6 +312,9 @@ constexpr int LANES_HALF = 4;
 // [4096,14336] matrices) ran 16 % slower, because requests beyond what the CU's memory pipeline accepts block the wave
 // that issues them, and the activations, which every wave needs first, were quantized 3 us later.
 constexpr int STAGED_DMA = 5;
+#ifndef MMVQ_DMA_MT
+#define MMVQ_DMA_MT 4   // rows of X up to which the ring serves
+#endif
 #ifndef MMVQ_DMA_DEPTH
 #define MMVQ_DMA_DEPTH 2   // (3 and 4 stretches in flight per wave, and a wave's whole share at once, measured slower: requests
 #endif                     //  beyond what the CU's memory pipeline holds block the waves that issue them)
@@ -780,26 +783,28 @@ static bool launch_stream(const void* W, const T* X, T* Y, int N, int K, hipStre
       // (for Q4_K, whose per-lane loads are aligned 16-byte pieces already, the trip through LDS costs the 8-wave kernel
       //  of the small matrices as much as it gains; [4096,4096]: Q8_0 6.4 -> 5.1 us, Q4_0 5.1 -> 4.4 us, Q6_K 6.2 -> 5.4 us)
       // (Q8_0, most bytes per weight, still gains at four rows: [14336,4096] 16.6 -> 15.4 us)
-      if constexpr (MT <= (std::is_same<F, FmtQ8_0>::value ? 4 : MMVQ_STAGED_MT) && (NW == MMVQ_NW || !std::is_same<F, FmtQ4_K>::value || DmaRing<F>::on) && SpanOf<F>::value > 0) {
+      if constexpr (MT <= (std::is_same<F, FmtQ8_0>::value || DmaRing<F>::on ? 4 : MMVQ_STAGED_MT) && (NW == MMVQ_NW || !std::is_same<F, FmtQ4_K>::value || DmaRing<F>::on) && SpanOf<F>::value > 0) {
         // rows of whole 16-byte pieces at aligned addresses: every byte is requested once (see SpanRegs)
         const int64_t pitch = la.w_pitch ? la.w_pitch : (int64_t)(K / F::QK) * F::BS;
         const size_t lds_staged = lds + (size_t)NW * 16 * SpanRegs<SpanOf<F>::value, SpanAny<F>::value>::PIECES + SpanSlack<F>::value;
         // (a row shorter than one stretch leaves half the lanes of its wave without a block: not worth the trip through LDS,
         //  Q8_0 [3072,1024] 3.3 -> 3.8 us)
         if (per_wave >= MMVQ_DEPTH && nb >= 64 && lds_staged <= 160 * 1024) {
-          if constexpr (DmaRing<F>::on && MT <= 2) {
+          if constexpr (DmaRing<F>::on && MT <= MMVQ_DMA_MT) {
             // whole aligned stretches straight into a ring in LDS, as deep as the rows a wave walks where LDS has the room
             // (the activations must be quantized by the prologue's straight-line code: its loads are counted)
             const size_t slot = 1024 * SpanRegs<SpanOf<F>::value>::NR;
             const auto fits = [&](int d) { return per_wave >= d && lds + (size_t)NW * d * slot <= 160 * 1024; };
             // (rows of up to two stretches on the 16-wave kernel: Q4_K [14336,4096] 8.9 -> 8.5 us; longer rows and the 8-wave
-            //  kernel of small matrices lose a little)
-            if (NW == MMVQ_NW && S <= 2 && nb % 64 == 0 && span_aligned<F>(W, pitch, K) && (size_t)MT * K <= 32 * 64 * NW) {
+            //  kernel of small matrices lose a little; with three and four rows of X, [14336,4096] 13.5 -> 13.0 us but
+            //  [4096,4096] 7.1 -> 7.4 us, hence the floor on N)
+            if (NW == MMVQ_NW && S <= 2 && nb % 64 == 0 && span_aligned<F>(W, pitch, K) && (size_t)MT * K <= 32 * 64 * NW &&
+                (MT <= 2 || N >= 8192)) {
               if (fits(MMVQ_DMA_DEPTH)) { launch_stream_d<F, MT, MMVQ_DMA_DEPTH, T, TILE, FULL, NW, STAGED_DMA>(W, X, Y, N, K, rows_per_wg, grid, lds + (size_t)NW * MMVQ_DMA_DEPTH * slot, la, stream, m_act); return; }
             }
           }
           // (through registers the trip costs the 8-wave kernel of Q4_K as much as it gains: per-lane loads below)
-          if constexpr (NW == MMVQ_NW || !std::is_same<F, FmtQ4_K>::value) {
+          if constexpr ((NW == MMVQ_NW || !std::is_same<F, FmtQ4_K>::value) && MT <= (std::is_same<F, FmtQ8_0>::value ? 4 : MMVQ_STAGED_MT)) {
             if (span_aligned<F>(W, pitch, K)) {
               if (nb % 64 == 0) launch_stream_d<F, MT, MMVQ_DEPTH, T, TILE, FULL, NW, STAGED_ALIGNED>(W, X, Y, N, K, rows_per_wg, grid, lds_staged, la, stream, m_act);
               else launch_stream_d<F, MT, MMVQ_DEPTH, T, TILE, FULL, NW, SpanAny<F>::value ? STAGED_ANY : STAGED_PART>(W, X, Y, N, K, rows_per_wg, grid, lds_staged, la, stream, m_act);
