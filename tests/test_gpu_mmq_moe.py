@@ -378,6 +378,29 @@ def test_moe_grouped_blocks_of_16_slots(qtype, t, top_k, e):
     assert np.all(y3[dropped] == 0)
 
 
+def test_moe_16_slot_launch_geometry_does_not_change_results():
+    """The launcher of the 16-slot tiles guesses, from the length of the sorted array and the pair count, how the blocks
+    will fall into rounds of workgroups and asks for an LDS size that lets two or three of them share a CU.  That guess
+    moves time only: the same routing in a sorted array with room for twice the experts (more padding slots behind
+    num_tokens_post_padded, which no block reaches) lands on the other side of the estimate -- 64 experts x 16 feature
+    tiles at 4 pairs per expert is the 'two per CU' case, 128 apparent experts is not -- and must give the same bits."""
+    ops = _ops()
+    rng = np.random.default_rng(4242)
+    qtype, e, n, k, t, top_k = o.Q4_0, 64, 2048, 256, 32, 8
+    w = np.stack([o.make_weights(rng, qtype, n, k) for _ in range(e)])
+    wd = _dev(w)
+    xd, xv = _x(rng, t, k, "f32")
+    ids, _ = _routing(rng, t, e, top_k)
+    s, eids, npost = o.moe_align_block_size(ids, 16, e)
+    y = ops.ggml_moe_a8(xd, wd, _dev(s), _dev(eids), _dev(npost), qtype, n, top_k, t, block_size=16)
+    assert o.rel_l2(y.cpu().numpy(), o.moe_a8(xv, w, s, eids, npost, qtype, n, top_k, t, 16)) <= 1e-5
+    extra = 15 * e // 16 * 16
+    s_long = np.concatenate([s, np.full(extra, t * top_k, dtype=s.dtype)])
+    eids_long = np.concatenate([eids, np.zeros(extra // 16, dtype=eids.dtype)])
+    y_long = ops.ggml_moe_a8(xd, wd, _dev(s_long), _dev(eids_long), _dev(npost), qtype, n, top_k, t, block_size=16)
+    assert torch.equal(y, y_long)
+
+
 @pytest.mark.parametrize("qtype", [o.Q4_0, o.Q4_K])
 @pytest.mark.parametrize("t,top_k", [(2048, 8), (83, 4)])
 def test_moe_256_experts_as_the_reference_tests_them(qtype, t, top_k):
