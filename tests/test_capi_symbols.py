@@ -35,7 +35,7 @@ def handle():
 
 def test_header_declares_the_bound_entry_points():
     assert declared_symbols() == sorted(_lib.EXPORTS)
-    assert len(declared_symbols()) == 28
+    assert len(declared_symbols()) == 31
 
 
 def test_every_declared_symbol_is_exported(handle):
@@ -143,3 +143,19 @@ def test_ctypes_signatures_match_the_header_type_for_type():
         want_res, want_args = protos[name]
         assert res is want_res, (name, res, want_res)
         assert list(args) == want_args, (name, [a.__name__ for a in args], [a.__name__ for a in want_args])
+
+
+def test_two_launch_moe_layer_states_which_shapes_it_serves():
+    """gguf_moe_vec_layer_takes needs no GPU: the OLMoE-like layer at one token and a Mixtral-like one are served; top_k
+    times the waves a row takes beyond one workgroup, experts shared by many pairs, unknown types and inner sizes that
+    are not whole blocks are not.  The workspace holds one q8_1 row of the inner size per pair."""
+    h = _lib.lib()
+    assert h.gguf_moe_vec_layer_takes(2, 2, 2048, 1024, 2048, 8, 1, 64) == 1
+    assert h.gguf_moe_vec_layer_takes(12, 14, 4096, 14336, 4096, 2, 1, 8) == 1
+    assert h.gguf_moe_vec_layer_takes(2, 2, 2048, 8192, 2048, 8, 1, 64) == 0
+    assert h.gguf_moe_vec_layer_takes(2, 2, 2048, 1024, 2048, 8, 64, 64) == 0
+    assert h.gguf_moe_vec_layer_takes(1, 2, 2048, 1024, 2048, 8, 1, 64) == 0
+    assert h.gguf_moe_vec_layer_takes(2, 12, 2048, 1120, 2048, 8, 1, 64) == 0
+    assert h.gguf_moe_vec_layer_workspace_bytes(3, 8, 1024) == 24 * h.gguf_q8_1_row_bytes(1024)
+    assert h.gguf_moe_vec_layer(None, 1, None, 2, None, 2, None, None, None, None, 2048, 1024, 2048, 8, 1, 0, 64, None) == -3
+    assert h.gguf_moe_vec_layer(None, 1, None, 2, None, 2, None, None, None, None, 2048, 1024, 2048, 8, 1, 1, 64, None) == -4

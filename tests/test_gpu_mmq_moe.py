@@ -518,6 +518,64 @@ def test_moe_vec_few_pairs_stream_each_expert(qtype, dt):
         assert o.rel_l2(got.float().cpu().numpy(), ref) <= max(tol, 5e-4), (o.TYPE_NAMES[qtype], "gated", t, e, k)
 
 
+@pytest.mark.parametrize("dt", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("qtype", [q for q in sorted(o.QUANT_SIZES) if q != 9])      # (9 is q8_1, the activations' format)
+def test_moe_layer_in_two_launches_matches_the_separate_steps(qtype, dt):
+    """moe_vec_layer (first GEMV with the activation and the q8_1 quantisation in its epilogue; second GEMV with the
+    routing weights and the sum over the top-k axis) against ggml_moe_a8_vec, ggml_moe_a8_vec(..., activation=) and
+    moe_weighted_sum run one by one, to fp32 rounding -- the separate steps are held to the oracle by the tests above.
+    Rows of 32 units on half-waves and longer rows on waves, top-k from 1 to 8, inner sizes that leave the last band
+    short, a second format for the down projection, an expert id outside the table (that pair adds nothing), and shapes
+    the kernels decline."""
+    ops = _ops()
+    rng = np.random.default_rng(1700 + qtype)
+    qk = o.QUANT_SIZES[qtype][0]
+    other = o.Q8_0 if qk == 32 else o.Q4_0                 # the down projection in another format (32-value blocks)
+    # tokens, top_k, experts, hidden, inner
+    for case, (t, top_k, e, hid, inner) in enumerate([(1, 8, 16, 2048, 1024), (3, 2, 8, 512, 768), (2, 4, 8, 1024, 2048), (5, 1, 8, 256, 1280),
+                                                     (1, 2, 4, 4096, 512)]):
+        for qt2 in (qtype, other) if case < 2 else (qtype,):
+            if inner % o.QUANT_SIZES[qt2][0]:
+                continue
+            w13 = np.stack([o.make_weights(rng, qtype, 2 * inner, hid) for _ in range(e)])
+            w2 = np.stack([o.make_weights(rng, qt2, hid, inner) for _ in range(e)])
+            w13d, w2d = _dev(w13), _dev(w2)
+            ids, wts = _routing(rng, t, e, top_k)
+            pairs = t * top_k
+            assert ops.moe_vec_layer_takes(qtype, qt2, hid, inner, hid, top_k, t, e)
+            x = torch.randn(t, hid, device="cuda")
+            # (the random weights' scales are arbitrary: bring the first GEMV's results to a few units, so that the gated
+            #  products stay far below the half-precision range the q8_1 scales are stored in)
+            x = (x * (4.0 / ops.ggml_moe_a8_vec(x, w13d, _dev(ids), top_k, qtype, 2 * inner, t).abs().max())).to(TORCH_DT[dt])
+            for bad in (False, True):
+                if bad:
+                    ids = ids.copy()
+                    ids[0, top_k - 1] = e + 3
+                h = ops.ggml_moe_a8_vec(x, w13d, _dev(ids), top_k, qtype, 2 * inner, t)
+                y = ops.ggml_moe_a8_vec(h, w2d, _dev(ids.reshape(pairs, 1)), 1, qt2, hid, pairs, activation="silu")
+                if bad:
+                    y[top_k - 1].zero_()                   # the separate steps leave that pair's row unwritten
+                want = torch.empty((t, hid), dtype=x.dtype, device="cuda")
+                ops.moe_weighted_sum(y.reshape(t, top_k, hid), _dev(wts), want)
+                got = ops.moe_vec_layer(x, w13d, w2d, _dev(wts), _dev(ids), qtype, qt2, "silu")
+                assert not torch.isnan(want).any()
+                # (Most cases agree bit for bit.  Not all: the compiler contracts multiply-adds per kernel, so a sum or an
+                #  exponential may differ in its last bit and, about once in 10^5 values, move one quant of h by a step, which
+                #  shifts every output of that token by about 1e-4 of its size.)
+                err = o.rel_l2(got.float().cpu().numpy(), want.float().cpu().numpy())
+                assert err <= {"f32": 5e-4, "f16": 1e-3, "bf16": 4e-3}[dt], \
+                    f"{o.TYPE_NAMES[qtype]} {o.TYPE_NAMES[qt2]} {dt} t={t} top_k={top_k} hid={hid} inner={inner} bad={bad} rel-L2 {err}"
+    # top_k times the waves a row of the down projection takes exceed a workgroup; an inner size that is no multiple of 32
+    # blocks ... of its format; experts shared by many pairs (the grouped routes of the per-pair operator pay): declined
+    assert not ops.moe_vec_layer_takes(qtype, qtype, 2048, 8192, 2048, 8, 1, 64)
+    assert not ops.moe_vec_layer_takes(qtype, qtype, 2048, 1024, 2048, 8, 64, 64)
+    with pytest.raises(ValueError):
+        ops.moe_vec_layer(torch.zeros(64, 2048, device="cuda", dtype=TORCH_DT[dt]),
+                          _dev(np.zeros((64, 2048, 2048 // qk * o.QUANT_SIZES[qtype][1]), dtype=np.uint8)),
+                          _dev(np.zeros((64, 2048, 1024 // qk * o.QUANT_SIZES[qtype][1]), dtype=np.uint8)),
+                          _dev(np.ones((64, 8), dtype=np.float32)), _dev(np.zeros((64, 8), dtype=np.int32)), qtype, qtype, "silu")
+
+
 @pytest.mark.parametrize("dt", ["f32", "f16"])
 @pytest.mark.parametrize("qtype", MMQ_TYPES)
 def test_moe_vec_shared_experts_keep_gemv_semantics(qtype, dt):

@@ -79,12 +79,14 @@ __device__ __forceinline__ void load8(const T* p, float (&v)[8]) {
 enum { ACT_NONE = 0, ACT_SILU = 1, ACT_GELU = 2 };
 // g <- T(T(act(g)) * u) for eight values already widened to fp32
 template <typename T>
+__device__ __forceinline__ float gate1(float g, float u, int act) {
+  const float a = act == ACT_SILU ? g / (1.0f + expf(-g)) : g * 0.5f * (1.0f + erff(g * 0.70710678118654752440f));
+  return to_f32<T>(from_f32<T>(to_f32<T>(from_f32<T>(a)) * u));  // T x T products are exact in fp32, so one rounding each
+}
+template <typename T>
 __device__ __forceinline__ void gate8(float (&g)[8], const float (&u)[8], int act) {
 #pragma unroll
-  for (int i = 0; i < 8; ++i) {
-    const float a = act == ACT_SILU ? g[i] / (1.0f + expf(-g[i])) : g[i] * 0.5f * (1.0f + erff(g[i] * 0.70710678118654752440f));
-    g[i] = to_f32<T>(from_f32<T>(to_f32<T>(from_f32<T>(a)) * u[i]));  // T x T products are exact in fp32, so one rounding each
-  }
+  for (int i = 0; i < 8; ++i) g[i] = gate1<T>(g[i], u[i], act);
 }
 template <typename T>
 __device__ __forceinline__ void load8_gated(const T* gate, const T* up, int act, float (&v)[8]) {

@@ -309,6 +309,50 @@ def moe_align_block_size(topk_ids: torch.Tensor, block_size: int, num_experts: i
     return sorted_ids, expert_ids, post
 
 
+def moe_vec_layer_takes(quant_type: int, quant_type2: int, hidden: int, inner: int, out_features: int, top_k: int, tokens: int,
+                        num_experts: int) -> bool:
+    """Whether :func:`moe_vec_layer` serves a layer of this shape (a few tokens, experts not shared by many pairs)."""
+    return bool(_lib.lib().gguf_moe_vec_layer_takes(int(quant_type), int(quant_type2), int(hidden), int(inner), int(out_features),
+                                                    int(top_k), int(tokens), int(num_experts)))
+
+
+def moe_vec_layer(
+    X: torch.Tensor,
+    W13: torch.Tensor,
+    W2: torch.Tensor,
+    topk_weights: torch.Tensor,
+    topk_ids: torch.Tensor,
+    quant_type: int,
+    quant_type2: int,
+    activation: str,
+    output: torch.Tensor | None = None,
+) -> torch.Tensor:
+    """The reference's MoE layer on its per-pair operators (quantization/fused_moe.py:98-111) in two launches:
+    ``ggml_moe_a8_vec`` with ``act`` and the q8_1 quantisation of its result in the epilogue, then the second
+    ``ggml_moe_a8_vec`` with ``mul_`` by the routing weights and ``moe_sum`` -> ``[tokens, W2.shape[1]]``.  Same roundings as
+    those steps run one by one; raises ``ValueError`` for shapes :func:`moe_vec_layer_takes` declines."""
+    _check_inputs(X, W13, W2, topk_ids)
+    if topk_ids.dtype != torch.int32:
+        raise ValueError("topk_ids must be int32")
+    act = _act_code(activation)
+    if not act:
+        raise ValueError("moe_vec_layer needs an activation")
+    tokens, top_k = topk_ids.shape
+    hidden, inner, n_out = X.shape[1], W13.shape[1] // 2, W2.shape[1]
+    w = topk_weights.reshape(tokens, top_k)
+    if w.dtype != torch.float32 or not w.is_contiguous():
+        w = w.to(torch.float32).contiguous()
+    L = _lib.lib()
+    with torch.cuda.device(X.device):
+        out = output if output is not None else torch.empty((tokens, n_out), dtype=X.dtype, device=W2.device)
+        ws = torch.empty(max(16, L.gguf_moe_vec_layer_workspace_bytes(tokens, top_k, inner)), dtype=torch.uint8, device=X.device)
+        rc = L.gguf_moe_vec_layer(X.data_ptr(), _code(X.dtype), W13.data_ptr(), int(quant_type), W2.data_ptr(), int(quant_type2),
+                                  topk_ids.data_ptr(), w.data_ptr(), ws.data_ptr(), out.data_ptr(), hidden, inner, n_out, top_k, tokens,
+                                  act, W13.shape[0], _stream(X))
+    _lib.check(rc, "moe_vec_layer")
+    return out
+
+
 def moe_weighted_sum(expert_out: torch.Tensor, topk_weights: torch.Tensor, output: torch.Tensor) -> None:
     """``output[t] = sum_k expert_out[t, k] * topk_weights[t, k]``: the ``mul_`` by the routing weights and the
     ``moe_sum`` that end the reference's MoE layer (quantization/fused_moe.py:87-95), fused."""
