@@ -45,6 +45,10 @@ __device__ __forceinline__ float seeded_times(int bits, float dw, float neg_seed
   return __builtin_fmaf(__int_as_float(bits), dw, neg_seed_dw);
 }
 
+// LDS row pitch of this kernel: 16-byte operand reads (K=32 MFMA) want a 16-byte skew, the 8-byte reads of the K=16 form an
+// 8-byte skew, which spreads 16 consecutive rows over the banks.
+template <int G, int KS> struct OldPitch { static constexpr int value = G == 32 ? KS + 16 : KS + 8; };
+
 // acc += v[lane (l & ~3) + T] * c : a fused multiply-add whose first factor is taken from lane T of the caller's
 // quad by DPP.  In the 32x32 MFMA result layout register r of lane l is row 8*(r/4) + 4*(l/32) + r%4, so when lane l
 // holds a per-row factor for row 8*g + 4*(l/32) + l%4, the factor of register 4*g + T sits in lane T of every quad:
@@ -133,7 +137,7 @@ __host__ __device__ constexpr size_t mmq_group_lds_bytes() {
   constexpr int M_T = 32 * WM * TM, N_T = 32 * WN * TN, KB = KS / 32;
   constexpr int XA = !F::HAS_MIN ? 0 : F::MIN16 ? 2 * KB : KB;  // per-row offset factors: block sums, or 16-element quant sums
   constexpr int WMN = !F::HAS_MIN ? 0 : F::MIN16 ? KS / F::G : KB;
-  return (size_t)(M_T + N_T) * Pitch<F::G, KS>::value + (size_t)(KB + XA) * M_T * 4 + (size_t)(KS / F::G + WMN) * N_T * 4;
+  return (size_t)(M_T + N_T) * OldPitch<F::G, KS>::value + (size_t)(KB + XA) * M_T * 4 + (size_t)(KS / F::G + WMN) * N_T * 4;
 }
 
 // MODE selects how staging and contraction overlap:
@@ -153,7 +157,7 @@ __global__ __launch_bounds__(64 * WM * WN * (MODE == MODE_KSPLIT ? 2 : 1), OCC) 
   constexpr int NT = 64 * GW * KW;       // threads that stage one tile: the whole workgroup
   constexpr int KB = KS / 32;            // q8_1 blocks per step
   constexpr int GR = KS / 16;            // 16-byte granules per activation row and step
-  constexpr int LDK = Pitch<F::G, KS>::value;
+  constexpr int LDK = OldPitch<F::G, KS>::value;
   constexpr int M_T = 32 * WM * TM, N_T = 32 * WN * TN;
   constexpr int NG = KS / F::G;          // weight scales per row per step
   constexpr int AQ = (M_T * GR + NT - 1) / NT;  // activation granules per thread and step

@@ -49,9 +49,11 @@ __device__ __forceinline__ float seeded_times(int bits, float dw, float neg_seed
   return __builtin_fmaf(__int_as_float(bits), dw, neg_seed_dw);
 }
 
-// LDS row pitch in bytes.  K=32 operands are read 16 bytes per lane: a 16-byte skew (KS + 16) spreads 8 consecutive
-// rows over all banks.  K=16 operands are read 8 bytes per lane: an 8-byte skew (KS + 8) spreads 16 consecutive rows.
-template <int G, int KS> struct Pitch { static constexpr int value = G == 32 ? KS + 16 : KS + 8; };
+// LDS row pitch in bytes.  Operands are read 16 bytes per lane: a 16-byte skew (KS + 16) spreads 8 consecutive rows
+// over all banks.  The 16-deep formats multiply a 32-value block with two K=16 MFMAs, each of which wants 8 consecutive
+// k per lane half; their blocks are stored as [k 0-7 | k 16-23 | k 8-15 | k 24-31], so that the 16 bytes at 16 * lhalf
+// are this lane's operands of both MFMAs (one 16-byte read instead of two 8-byte reads at a pitch with bank conflicts).
+template <int G, int KS> struct Pitch { static constexpr int value = KS + 16; };
 
 constexpr int MMQI_KS = 128;  // values of K per step
 
@@ -147,11 +149,12 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void mmqi_kernel(const uint8_t* __
     for (int i = 0; i < AQ; ++i) {
       const int p = tid + NT * i, m = p / GR, g = p % GR;
       const uint4 v = r_aq[i];   // past K the padded row holds zeros, past Kp the scales below are zero
-      if (LDK % 16 == 0) {
+      if constexpr (F::G == 32) {
         *(uint4*)(xq + m * LDK + 16 * g) = v;
-      } else {
-        *(uint2*)(xq + m * LDK + 16 * g) = make_uint2(v.x, v.y);
-        *(uint2*)(xq + m * LDK + 16 * g + 8) = make_uint2(v.z, v.w);
+      } else {   // granule g holds k 0-15 (g even) or k 16-31 (g odd) of block g / 2: see Pitch
+        int8_t* blk = xq + m * LDK + 32 * (g >> 1) + 8 * (g & 1);
+        *(uint2*)blk = make_uint2(v.x, v.y);
+        *(uint2*)(blk + 16) = make_uint2(v.z, v.w);
       }
     }
     if (tid < M_T) {
@@ -170,12 +173,12 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void mmqi_kernel(const uint8_t* __
       float s0, s1, mn = 0.0f, mn1 = 0.0f;
       F::unpack(r_w[i], kb0 + kb, q, s0, s1, mn, mn1);
       if (kb0 + kb >= nkb_total) s0 = s1 = mn = 0.0f;
-      if (LDK % 16 == 0) {
+      if constexpr (F::G == 32) {
         *(uint4*)(wq + n * LDK + 32 * kb) = make_uint4(q[0], q[1], q[2], q[3]);
         *(uint4*)(wq + n * LDK + 32 * kb + 16) = make_uint4(q[4], q[5], q[6], q[7]);
       } else {
-#pragma unroll
-        for (int t2 = 0; t2 < 4; ++t2) *(uint2*)(wq + n * LDK + 32 * kb + 8 * t2) = make_uint2(q[2 * t2], q[2 * t2 + 1]);
+        *(uint4*)(wq + n * LDK + 32 * kb) = make_uint4(q[0], q[1], q[4], q[5]);
+        *(uint4*)(wq + n * LDK + 32 * kb + 16) = make_uint4(q[2], q[3], q[6], q[7]);
       }
       wsc[kb * N_T + n] = F::G == 32 ? (f32x2){s0, -mn} : (f32x2){s0, s1};
     }
@@ -206,23 +209,9 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void mmqi_kernel(const uint8_t* __
     const int8_t* xq = (const int8_t*)smem + buf * BUF;
     const int8_t* wq = xq + M_T * LDK;
     const int8_t* arow = xq + (32 * wm + lrow) * LDK + 32 * kb;
-    if constexpr (F::G == 32) {
-      o.a = *(const v4i*)(arow + 16 * lhalf);
-    } else {
-      // the K=16 MFMA wants 8 consecutive k per lane half: half h of the block is bytes [16h + 8 lhalf, +8)
-      const v2i lo = *(const v2i*)(arow + 8 * lhalf), hi = *(const v2i*)(arow + 16 + 8 * lhalf);
-      o.a = (v4i){lo[0], lo[1], hi[0], hi[1]};
-    }
+    o.a = *(const v4i*)(arow + 16 * lhalf);   // (16-deep formats: both halves' operands of this lane, see Pitch)
 #pragma unroll
-    for (int i = 0; i < TN; ++i) {
-      const int8_t* brow = wq + (32 * (wn * TN + i) + lrow) * LDK + 32 * kb;
-      if constexpr (F::G == 32) {
-        o.b[i] = *(const v4i*)(brow + 16 * lhalf);
-      } else {
-        const v2i lo = *(const v2i*)(brow + 8 * lhalf), hi = *(const v2i*)(brow + 16 + 8 * lhalf);
-        o.b[i] = (v4i){lo[0], lo[1], hi[0], hi[1]};
-      }
-    }
+    for (int i = 0; i < TN; ++i) o.b[i] = *(const v4i*)(wq + (32 * (wn * TN + i) + lrow) * LDK + 32 * kb + 16 * lhalf);
   };
   auto load_scales = [&](int buf, int kb, ScaleOps& o) {
     const float* xd = (const float*)(smem + buf * BUF + (M_T + N_T) * LDK);
