@@ -1,4 +1,5 @@
-// Prefill-path GEMM on packed GGUF weights with q8_1 activations, on gfx950 int8 MFMA.
+// The older integer tile kernel, kept for the grouped MoE contraction on blocks of 32 slots (the dense product of every
+// tile format runs on the pipelined kernel of mmq_i_core.h), and the C entry points of the tile operators.
 //
 //   Y[m, n] = sum_kb  d8[m, kb] * dw[n, kb] * S[m, n, kb]  ( - offset terms )
 //   S[m, n, kb] = sum over the 32 (or 16) elements of block kb of  xq[m, k] * wq[n, k]      (int32)
@@ -44,10 +45,6 @@ constexpr int kSeedBits = 0x4B400000;
 __device__ __forceinline__ float seeded_times(int bits, float dw, float neg_seed_dw) {
   return __builtin_fmaf(__int_as_float(bits), dw, neg_seed_dw);
 }
-
-// LDS row pitch of this kernel: 16-byte operand reads (K=32 MFMA) want a 16-byte skew, the 8-byte reads of the K=16 form an
-// 8-byte skew, which spreads 16 consecutive rows over the banks.
-template <int G, int KS> struct OldPitch { static constexpr int value = G == 32 ? KS + 16 : KS + 8; };
 
 // acc += v[lane (l & ~3) + T] * c : a fused multiply-add whose first factor is taken from lane T of the caller's
 // quad by DPP.  In the 32x32 MFMA result layout register r of lane l is row 8*(r/4) + 4*(l/32) + r%4, so when lane l
@@ -137,7 +134,7 @@ __host__ __device__ constexpr size_t mmq_group_lds_bytes() {
   constexpr int M_T = 32 * WM * TM, N_T = 32 * WN * TN, KB = KS / 32;
   constexpr int XA = !F::HAS_MIN ? 0 : F::MIN16 ? 2 * KB : KB;  // per-row offset factors: block sums, or 16-element quant sums
   constexpr int WMN = !F::HAS_MIN ? 0 : F::MIN16 ? KS / F::G : KB;
-  return (size_t)(M_T + N_T) * OldPitch<F::G, KS>::value + (size_t)(KB + XA) * M_T * 4 + (size_t)(KS / F::G + WMN) * N_T * 4;
+  return (size_t)(M_T + N_T) * Pitch<F::G, KS>::value + (size_t)(KB + XA) * M_T * 4 + (size_t)(KS / F::G + WMN) * N_T * 4;
 }
 
 // MODE selects how staging and contraction overlap:
@@ -157,7 +154,7 @@ __global__ __launch_bounds__(64 * WM * WN * (MODE == MODE_KSPLIT ? 2 : 1), OCC) 
   constexpr int NT = 64 * GW * KW;       // threads that stage one tile: the whole workgroup
   constexpr int KB = KS / 32;            // q8_1 blocks per step
   constexpr int GR = KS / 16;            // 16-byte granules per activation row and step
-  constexpr int LDK = OldPitch<F::G, KS>::value;
+  constexpr int LDK = Pitch<F::G, KS>::value;
   constexpr int M_T = 32 * WM * TM, N_T = 32 * WN * TN;
   constexpr int NG = KS / F::G;          // weight scales per row per step
   constexpr int AQ = (M_T * GR + NT - 1) / NT;  // activation granules per thread and step
@@ -490,35 +487,6 @@ static void launch_mmq(const void* W, const void* ws, void* Y, int M, int N, int
 
 
 
-// Tile choice.  The kernel is bound by vector-ALU issue, not by operand traffic, so small tiles cost little and what
-// matters is that every CU has several workgroups to overlap one group's load latency with another's arithmetic:
-//   large   128 x 128, 8 waves, two workgroups per CU      when that still gives every CU about two tiles
-//   small   64 x 64, 4 waves, four or more per CU          otherwise (few tokens, or a narrow N with a long K)
-//   split   64 x 64, 8 waves (MODE_KSPLIT)                 when even the small tiles leave CUs with two workgroups or fewer
-// Formats whose packed block is small keep the next step's loads in registers across the MFMA phase (PREFETCH);
-// for the others that would push the kernel past 128 registers and halve the waves per SIMD.
-template <class F, typename T>
-static int mmq_typed(const void* W, const void* ws, void* Y, int M, int N, int K, hipStream_t stream, const LinearArgs& la) {
-  MoeArgs none = {};
-  const int64_t large_tiles = (int64_t)((M + 127) / 128) * ((N + 127) / 128);
-  const int64_t small_tiles = (int64_t)((M + 63) / 64) * ((N + 63) / 64);
-  if (large_tiles >= 400) {
-    constexpr int MODE = F::LIGHT ? MODE_PREFETCH : MODE_PLAIN;
-    launch_mmq<F, 4, 2, 1, 2, 128, 4, MODE, T, false>(W, ws, Y, M, N, K, (M + 127) / 128, none, stream, la);
-  } else if (small_tiles > 512) {
-    launch_mmq<F, 2, 2, 1, 1, 128, 4, MODE_PLAIN, T, false>(W, ws, Y, M, N, K, (M + 63) / 64, none, stream, la);
-  } else {  // at most two workgroups per CU: double the waves of each by splitting the step's blocks
-    launch_mmq<F, 2, 2, 1, 1, 128, 4, MODE_KSPLIT, T, false>(W, ws, Y, M, N, K, (M + 63) / 64, none, stream, la);
-  }
-  return launch_status();
-}
-
-template <class F>
-static int mmq_fmt(const void* W, const void* ws, void* Y, int dtype, int M, int N, int K, hipStream_t s, const LinearArgs& la) {
-  GGUF_DISPATCH_DTYPE(dtype, return (mmq_typed<F, scalar_t>(W, ws, Y, M, N, K, s, la)));
-  return GGUF_ERR_DTYPE;
-}
-
 template <class F, typename T>
 static int moe_typed(const void* W, const void* ws, void* Y, int N, int K, int num_sorted, const MoeArgs& moe,
                      hipStream_t stream) {
@@ -722,23 +690,8 @@ int gguf::mmq_linear_impl(const void* W, int64_t w_row_pitch_bytes, const void* 
     rc = mmq_rows16(W, q8_workspace, Y, xdtype, type, (int)M, (int)N, (int)K, partial, partial_bytes, s, la);
     if (rc != GGUF_NOT_TAKEN) return rc;
   }
-  rc = mmq_int(W, q8_workspace, Y, xdtype, type, (int)M, (int)N, (int)K, partial, partial_bytes, s, la);
-  if (rc != GGUF_NOT_TAKEN) return rc;
-  switch (type) {
-    case T_Q4_0: return mmq_fmt<MQ4_0>(W, q8_workspace, Y, xdtype, (int)M, (int)N, (int)K, s, la);
-    case T_Q4_1: return mmq_fmt<MQ4_1>(W, q8_workspace, Y, xdtype, (int)M, (int)N, (int)K, s, la);
-    case T_Q5_0: return mmq_fmt<MQ5_0>(W, q8_workspace, Y, xdtype, (int)M, (int)N, (int)K, s, la);
-    case T_Q5_1: return mmq_fmt<MQ5_1>(W, q8_workspace, Y, xdtype, (int)M, (int)N, (int)K, s, la);
-    case T_Q2_K: return mmq_fmt<MQ2_K>(W, q8_workspace, Y, xdtype, (int)M, (int)N, (int)K, s, la);
-    case T_Q3_K: return mmq_fmt<MQ3_K>(W, q8_workspace, Y, xdtype, (int)M, (int)N, (int)K, s, la);
-    case T_Q5_K: return mmq_fmt<MQ5_K>(W, q8_workspace, Y, xdtype, (int)M, (int)N, (int)K, s, la);
-    case T_Q8_0: return mmq_fmt<MQ8_0>(W, q8_workspace, Y, xdtype, (int)M, (int)N, (int)K, s, la);
-    case T_Q4_K: return mmq_fmt<MQ4_K>(W, q8_workspace, Y, xdtype, (int)M, (int)N, (int)K, s, la);
-    case T_Q6_K: return mmq_fmt<MQ6_K>(W, q8_workspace, Y, xdtype, (int)M, (int)N, (int)K, s, la);
-    case T_IQ4_XS: return mmq_fmt<MIQ4_XS>(W, q8_workspace, Y, xdtype, (int)M, (int)N, (int)K, s, la);
-    case T_IQ2_XXS: return mmq_fmt<MIQ2_XXS>(W, q8_workspace, Y, xdtype, (int)M, (int)N, (int)K, s, la);
-  }
-  return GGUF_ERR_TYPE;
+  rc = mmq_int(W, q8_workspace, Y, xdtype, type, (int)M, (int)N, (int)K, partial, partial_bytes, s, la);   // every tile format
+  return rc == GGUF_NOT_TAKEN ? GGUF_ERR_TYPE : rc;
 }
 
 extern "C" int gguf_mmq_engine(const void* W, const void* x, int xdtype, void* q8_workspace, void* Y, int type, int64_t N,

@@ -75,12 +75,15 @@ static int mmqi_fmt(const void* W, const void* ws, void* Y, int dtype, int M, in
   return GGUF_ERR_DTYPE;
 }
 
-// The integer engine for one call; the workspace already holds the quantized rows.  GGUF_NOT_TAKEN for the formats
-// whose scale products follow other rules (Q4_1 / Q5_1: rounded to half; Q2_K: offsets per 16 values).
+// The integer engine for one call; the workspace already holds the quantized rows.  GGUF_NOT_TAKEN for types without
+// tiles.  (Q4_1 / Q5_1 round their scale products to half, Q2_K subtracts an offset per 16 values: see rescale.)
 int mmq_int(const void* W, const void* ws, void* Y, int dtype, int type, int M, int N, int K, float* partial,
             int64_t partial_bytes, hipStream_t s, const LinearArgs& la) {
   switch (type) {
     case T_Q4_0: return mmqi_fmt<MQ4_0>(W, ws, Y, dtype, M, N, K, partial, partial_bytes, s, la);
+    case T_Q4_1: return mmqi_fmt<MQ4_1>(W, ws, Y, dtype, M, N, K, partial, partial_bytes, s, la);
+    case T_Q5_1: return mmqi_fmt<MQ5_1>(W, ws, Y, dtype, M, N, K, partial, partial_bytes, s, la);
+    case T_Q2_K: return mmqi_fmt<MQ2_K>(W, ws, Y, dtype, M, N, K, partial, partial_bytes, s, la);
     case T_Q5_0: return mmqi_fmt<MQ5_0>(W, ws, Y, dtype, M, N, K, partial, partial_bytes, s, la);
     case T_Q8_0: return mmqi_fmt<MQ8_0>(W, ws, Y, dtype, M, N, K, partial, partial_bytes, s, la);
     case T_Q3_K: return mmqi_fmt<MQ3_K>(W, ws, Y, dtype, M, N, K, partial, partial_bytes, s, la);

@@ -60,7 +60,10 @@ constexpr int MMQI_KS = 128;  // values of K per step
 template <class F, int M_T, int N_T>
 __host__ __device__ constexpr size_t mmqi_buffer_bytes() {
   constexpr int KB = MMQI_KS / 32;
-  return (size_t)(M_T + N_T) * Pitch<F::G, MMQI_KS>::value + (size_t)KB * M_T * 4 * (F::HAS_MIN ? 2 : 1) + (size_t)KB * N_T * 8;
+  // activation planes of KB x M_T floats: the block scales, then the stored block sums (offset formats) or the quant
+  // sums of both 16-value groups of a block (MIN16); weight planes of KB x N_T float pairs: scales (and offset factors)
+  constexpr int XP = !F::HAS_MIN ? 1 : F::MIN16 ? 3 : 2, WPL = F::MIN16 ? 2 : 1;
+  return (size_t)(M_T + N_T) * Pitch<F::G, MMQI_KS>::value + (size_t)KB * M_T * 4 * XP + (size_t)KB * N_T * 8 * WPL;
 }
 
 template <class F, int WM, int WN, int TN, typename T>
@@ -129,7 +132,7 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void mmqi_kernel(const uint8_t* __
     for (int i = 0; i < AQ; ++i) r_aq[i] = *(const uint4*)(aq_src[i] + k0);   // q8 rows are padded to a multiple of 512
     if (tid < M_T) {
       r_ad = *(const f32x4*)(as_src + kb0);
-      if (F::HAS_MIN) r_as = *(const f32x4*)(as_src + Kp / 32 + kb0);
+      if (F::HAS_MIN && !F::MIN16) r_as = *(const f32x4*)(as_src + Kp / 32 + kb0);
     }
 #pragma unroll
     for (int i = 0; i < WP; ++i) {
@@ -144,11 +147,14 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void mmqi_kernel(const uint8_t* __
     int8_t* wq = xq + M_T * LDK;
     float* xd = (float*)(wq + N_T * LDK);
     float* xs = xd + KB * M_T;
-    f32x2* wsc = (f32x2*)(xd + KB * M_T * (F::HAS_MIN ? 2 : 1));
+    f32x2* wsc = (f32x2*)(xd + KB * M_T * (!F::HAS_MIN ? 1 : F::MIN16 ? 3 : 2));
+    f32x2* wmn = wsc + KB * N_T;   // MIN16: {-min of group 0, -min of group 1} per block
 #pragma unroll
     for (int i = 0; i < AQ; ++i) {
       const int p = tid + NT * i, m = p / GR, g = p % GR;
       const uint4 v = r_aq[i];   // past K the padded row holds zeros, past Kp the scales below are zero
+      if constexpr (F::MIN16)    // this granule is one 16-value group: the sum of its quants, for the per-group offset term
+        xs[g * M_T + m] = (float)dot4(0x01010101, (int)v.x, dot4(0x01010101, (int)v.y, dot4(0x01010101, (int)v.z, dot4(0x01010101, (int)v.w, 0))));
       if constexpr (F::G == 32) {
         *(uint4*)(xq + m * LDK + 16 * g) = v;
       } else {   // granule g holds k 0-15 (g even) or k 16-31 (g odd) of block g / 2: see Pitch
@@ -162,7 +168,7 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void mmqi_kernel(const uint8_t* __
       for (int kb = 0; kb < KB; ++kb) {
         const bool in = kb0 + kb < nkb_total;
         xd[kb * M_T + tid] = in ? r_ad[kb] : 0.0f;
-        if (F::HAS_MIN) xs[kb * M_T + tid] = in ? r_as[kb] : 0.0f;
+        if (F::HAS_MIN && !F::MIN16) xs[kb * M_T + tid] = in ? r_as[kb] : 0.0f;
       }
     }
 #pragma unroll
@@ -172,7 +178,7 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void mmqi_kernel(const uint8_t* __
       uint32_t q[8];
       float s0, s1, mn = 0.0f, mn1 = 0.0f;
       F::unpack(r_w[i], kb0 + kb, q, s0, s1, mn, mn1);
-      if (kb0 + kb >= nkb_total) s0 = s1 = mn = 0.0f;
+      if (kb0 + kb >= nkb_total) s0 = s1 = mn = mn1 = 0.0f;
       if constexpr (F::G == 32) {
         *(uint4*)(wq + n * LDK + 32 * kb) = make_uint4(q[0], q[1], q[2], q[3]);
         *(uint4*)(wq + n * LDK + 32 * kb + 16) = make_uint4(q[4], q[5], q[6], q[7]);
@@ -181,6 +187,7 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void mmqi_kernel(const uint8_t* __
         *(uint4*)(wq + n * LDK + 32 * kb + 16) = make_uint4(q[2], q[3], q[6], q[7]);
       }
       wsc[kb * N_T + n] = F::G == 32 ? (f32x2){s0, -mn} : (f32x2){s0, s1};
+      if constexpr (F::MIN16) wmn[kb * N_T + n] = (f32x2){-mn, -mn1};
     }
   };
 
@@ -203,7 +210,9 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void mmqi_kernel(const uint8_t* __
   };
   struct ScaleOps {
     f32x2 sc[TN];   // 32-deep: {dw, -offset factor}; 16-deep: {dw of half 0, dw of half 1}
-    f32x4 d8[4], s8[4];
+    f32x2 mn[F::MIN16 ? TN : 1];   // MIN16: {-min of half 0, -min of half 1}
+    f32x4 d8[4], s8[4];           // s8: the stored block sums; MIN16: d8 x the quant sum of half 0
+    f32x4 u8[F::MIN16 ? 4 : 1];   // MIN16: d8 x the quant sum of half 1
   };
   auto load_mma = [&](int buf, int kb, MmaOps& o) {
     const int8_t* xq = (const int8_t*)smem + buf * BUF;
@@ -216,13 +225,21 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void mmqi_kernel(const uint8_t* __
   auto load_scales = [&](int buf, int kb, ScaleOps& o) {
     const float* xd = (const float*)(smem + buf * BUF + (M_T + N_T) * LDK);
     const float* xs = xd + KB * M_T;
-    const f32x2* wsc = (const f32x2*)(xd + KB * M_T * (F::HAS_MIN ? 2 : 1));
+    const f32x2* wsc = (const f32x2*)(xd + KB * M_T * (!F::HAS_MIN ? 1 : F::MIN16 ? 3 : 2));
 #pragma unroll
-    for (int i = 0; i < TN; ++i) o.sc[i] = wsc[kb * N_T + 32 * (wn * TN + i) + lrow];
+    for (int i = 0; i < TN; ++i) {
+      o.sc[i] = wsc[kb * N_T + 32 * (wn * TN + i) + lrow];
+      if constexpr (F::MIN16) o.mn[i] = wsc[(KB + kb) * N_T + 32 * (wn * TN + i) + lrow];
+    }
 #pragma unroll
     for (int g = 0; g < 4; ++g) {
       o.d8[g] = *(const f32x4*)(xd + kb * M_T + 32 * wm + 8 * g + 4 * lhalf);
-      if constexpr (F::HAS_MIN) o.s8[g] = *(const f32x4*)(xs + kb * M_T + 32 * wm + 8 * g + 4 * lhalf);
+      if constexpr (F::MIN16) {   // d8 x the groups' quant sums, once per block and lane for all the tiles
+        o.s8[g] = o.d8[g] * *(const f32x4*)(xs + (2 * kb) * M_T + 32 * wm + 8 * g + 4 * lhalf);
+        o.u8[g] = o.d8[g] * *(const f32x4*)(xs + (2 * kb + 1) * M_T + 32 * wm + 8 * g + 4 * lhalf);
+      } else if constexpr (F::HAS_MIN) {
+        o.s8[g] = *(const f32x4*)(xs + kb * M_T + 32 * wm + 8 * g + 4 * lhalf);
+      }
     }
   };
   // A unit is one MFMA and the rescale of its 16 results per lane: a (block, tile) pair for the 32-deep formats, one
@@ -243,11 +260,27 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void mmqi_kernel(const uint8_t* __
     const int i = ub / H, h = ub % H;
     const float dw = F::G == 32 ? o.sc[i][0] : o.sc[i][h];
     const float nsd = -kSeed * dw;
+    if constexpr (F::HALFPROD) {
+      // Q4_1, Q5_1: S * half(d * d8) + half(m * s8), both products rounded to half precision as the reference's
+      // __hmul2 leaves them (vecdotq.cuh:179-198); d, d8, m and s8 are half values held in floats
+      const _Float16 dh = (_Float16)dw, mh = (_Float16)-o.sc[i][1];
 #pragma unroll
-    for (int r = 0; r < 16; ++r) {
-      const float c = seeded_times(s_in[r], dw, nsd);   // = RN(S * dw)
-      acc[i][r] = __builtin_fmaf(c, o.d8[r >> 2][r & 3], acc[i][r]);
-      if constexpr (F::HAS_MIN) acc[i][r] = __builtin_fmaf(o.s8[r >> 2][r & 3], o.sc[i][1], acc[i][r]);
+      for (int r = 0; r < 16; ++r) {
+        const _Float16 dd = dh * (_Float16)o.d8[r >> 2][r & 3];
+        const _Float16 ms = mh * (_Float16)o.s8[r >> 2][r & 3];
+        acc[i][r] += (__int_as_float(s_in[r]) - kSeed) * (float)dd + (float)ms;
+      }
+    } else {
+#pragma unroll
+      for (int r = 0; r < 16; ++r) {
+        const float c = seeded_times(s_in[r], dw, nsd);   // = RN(S * dw)
+        acc[i][r] = __builtin_fmaf(c, o.d8[r >> 2][r & 3], acc[i][r]);
+        if constexpr (F::MIN16) {   // Q2_K: the group's min times d8 x the sum of the group's activation quants
+          acc[i][r] = __builtin_fmaf(h ? o.u8[r >> 2][r & 3] : o.s8[r >> 2][r & 3], o.mn[i][h], acc[i][r]);
+        } else if constexpr (F::HAS_MIN) {
+          acc[i][r] = __builtin_fmaf(o.s8[r >> 2][r & 3], o.sc[i][1], acc[i][r]);
+        }
+      }
     }
   };
   // One step of K from buffer `buf`.  The matrix operands of block kb + 1 are requested while block kb is worked
@@ -361,6 +394,9 @@ static void launch_mmqi(const void* W, const void* ws, void* Y, int M, int N, in
 // Formats whose 256 x 128 kernel fits the register file without scratch worth mentioning.
 template <class F> struct MmqiWide { static constexpr bool ok = true; };
 template <> struct MmqiWide<MQ5_K> { static constexpr bool ok = false; };
+template <> struct MmqiWide<MQ2_K> { static constexpr bool ok = false; };   // (three activation planes per block in registers)
+template <> struct MmqiWide<MQ4_1> { static constexpr bool ok = false; };   // (the half-precision products' temporaries)
+template <> struct MmqiWide<MQ5_1> { static constexpr bool ok = false; };
 
 template <class F, typename T>
 static int mmqi_typed(const void* W, const void* ws, void* Y, int M, int N, int K, float* partial, int64_t partial_bytes,
