@@ -100,3 +100,27 @@ def test_entry_point_without_workspace_replays_match_eager(case):
         torch.cuda.synchronize()
         assert torch.equal(out, eager), case
         assert o.rel_l2(out.float().cpu().numpy(), ops.ggml_mul_mat_a8(w, x, qtype, n).float().cpu().numpy()) <= 1e-3
+
+
+def test_two_launch_moe_layer_replays_match_eager():
+    """dispatch.fused_moe_gguf at a few tokens (both expert GEMVs, activation, routing weights and top-k sum in two
+    launches with a workspace allocated per call) captured and replayed with eager work in between."""
+    from vllm_gguf_plugin_prism_amd import dispatch, ops
+    rng = np.random.default_rng(91)
+    e, hid, inner, t, top_k, qtype = 16, 1024, 512, 3, 4, o.Q4_K
+    w13 = _dev(np.stack([o.make_weights(rng, qtype, 2 * inner, hid) for _ in range(e)]))
+    w2 = _dev(np.stack([o.make_weights(rng, qtype, hid, inner) for _ in range(e)]))
+    assert ops.moe_vec_layer_takes(qtype, qtype, hid, inner, hid, top_k, t, e)
+    ids = _dev(np.stack([rng.choice(e, size=top_k, replace=False) for _ in range(t)]).astype(np.int32))
+    wts = torch.rand(t, top_k, device="cuda")
+    xs = [torch.randn(t, hid, dtype=torch.float16, device="cuda") * 0.05 for _ in range(3)]
+    x = xs[0].clone()
+    fn = lambda: dispatch.fused_moe_gguf(x, w13, w2, wts, ids, qtype, qtype, "silu")
+    graph, out = _capture(fn)
+    for xi in xs:
+        x.copy_(xi)
+        eager = fn().clone()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager)

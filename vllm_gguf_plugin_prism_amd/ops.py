@@ -26,7 +26,25 @@ def _code(dtype: torch.dtype) -> int:
 
 
 def _stream(t: torch.Tensor) -> int:
-    return torch.cuda.current_stream(t.device).cuda_stream
+    # (the raw handle of torch's current stream on the tensor's device: a Stream object per call costs 4 us)
+    return torch._C._cuda_getCurrentRawStream(t.device.index if t.device.index is not None else torch.cuda.current_device())
+
+
+class _NoSwitch:
+    def __enter__(self):
+        return None
+
+    def __exit__(self, *exc):
+        return False
+
+
+_NO_SWITCH = _NoSwitch()
+
+
+def _on_device_of(t: torch.Tensor):
+    """Context in which the tensor's device is current: nothing to do (and 3 us less to pay) when it already is."""
+    idx = t.device.index
+    return _NO_SWITCH if idx is None or idx == torch._C._cuda_getDevice() else torch.cuda.device(t.device)
 
 
 def _check_inputs(*tensors: torch.Tensor) -> None:
@@ -47,17 +65,29 @@ def _act_code(name: str | None) -> int:
         raise ValueError(f"unsupported MoE activation {name!r}; need 'silu' or 'gelu'") from None
 
 
+_ROW_BYTES: dict[int, int] = {}
+
+
 def _workspace(x: torch.Tensor, rows: int, k: int) -> torch.Tensor:
-    nbytes = rows * _lib.lib().gguf_q8_1_row_bytes(k)
-    return torch.empty(max(nbytes, 16), dtype=torch.uint8, device=x.device)
+    rb = _ROW_BYTES.get(k)
+    if rb is None:
+        rb = _ROW_BYTES[k] = _lib.lib().gguf_q8_1_row_bytes(k)
+    return torch.empty(max(rows * rb, 16), dtype=torch.uint8, device=x.device)
+
+
+_QUANT_SIZES: dict[int, tuple[int, int]] = {}
 
 
 def quant_sizes(quant_type: int) -> tuple[int, int]:
     """(elements, bytes) of one block; stands in for ``gguf.GGML_QUANT_SIZES`` (quantization/linear.py:51)."""
+    hit = _QUANT_SIZES.get(quant_type)
+    if hit is not None:
+        return hit
     L = _lib.lib()
     qk, bs = L.gguf_block_elems(int(quant_type)), L.gguf_block_bytes(int(quant_type))
     if qk == 0:
         raise NotImplementedError(f"Unsupported GGUF quantization type: {quant_type}")
+    _QUANT_SIZES[quant_type] = (qk, bs)
     return qk, bs
 
 
@@ -65,7 +95,7 @@ def ggml_dequantize(W: torch.Tensor, quant_type: int, m: int, n: int, dtype: tor
     """Dense ``[m, n]`` values of the packed tensor ``W`` (reference: gguf_kernel.cu:87-102)."""
     _check_inputs(W)
     out_dtype = dtype or torch.float16
-    with torch.cuda.device(W.device):
+    with _on_device_of(W):
         out = torch.empty((m, n), dtype=out_dtype, device=W.device)
         rc = _lib.lib().gguf_dequantize(W.data_ptr(), int(quant_type), out.data_ptr(), _code(out_dtype), m * n, _stream(W))
     _lib.check(rc, "ggml_dequantize")
@@ -79,7 +109,7 @@ def ggml_dequantize_rows(W: torch.Tensor, quant_type: int, row_ids: torch.Tensor
     _check_inputs(W, row_ids)
     out_dtype = dtype or torch.float16
     ids = row_ids.reshape(-1).to(torch.int64)
-    with torch.cuda.device(W.device):
+    with _on_device_of(W):
         out = torch.empty((ids.numel(), hidden_size), dtype=out_dtype, device=W.device)
         rc = _lib.lib().gguf_dequantize_rows(W.data_ptr(), int(quant_type), ids.data_ptr(), ids.numel(), W.shape[0],
                                              hidden_size, out.data_ptr(), _code(out_dtype), _stream(W))
@@ -125,7 +155,7 @@ def ggml_mul_mat_vec_a8(W: torch.Tensor, X: torch.Tensor, quant_type: int, row: 
     ``bias`` is added the way ``out.add_(bias)`` would (quantization/linear.py:243-262)."""
     out, w_pitch, ldy = _shard_args(W, X, quant_type, row, out, bias)
     vecs, col = X.shape
-    with torch.cuda.device(X.device):
+    with _on_device_of(X):
         ws = _workspace(X, vecs, col)
         rc = _lib.lib().gguf_mmvq_linear(W.data_ptr(), w_pitch, X.data_ptr(), _code(X.dtype), ws.data_ptr(), out.data_ptr(), ldy,
                                          bias.data_ptr() if bias is not None else None, int(quant_type), row, col, vecs,
@@ -147,7 +177,7 @@ def ggml_mul_mat_a8(W: torch.Tensor, X: torch.Tensor, quant_type: int, row: int,
     only).  ``out`` / ``bias`` / sliced ``W``: as for :func:`ggml_mul_mat_vec_a8`."""
     out, w_pitch, ldy = _shard_args(W, X, quant_type, row, out, bias)
     vecs, col = X.shape
-    with torch.cuda.device(X.device):
+    with _on_device_of(X):
         # (only the half engine pays for the half-precision copy of the rows)
         nbytes = max(_lib.lib().gguf_mmq_workspace_bytes_engine(vecs, row, col, MMQ_ENGINES[engine]), 16)
         ws = torch.empty(nbytes, dtype=torch.uint8, device=X.device)
@@ -167,7 +197,7 @@ def ggml_dequant_gemm(W: torch.Tensor, X: torch.Tensor, quant_type: int, row: in
     fp16 / bf16 only; raises ``NotImplementedError`` for types outside ``DEQUANT_GEMM_TYPES``."""
     _check_inputs(W, X)
     vecs, col = X.shape
-    with torch.cuda.device(X.device):
+    with _on_device_of(X):
         out = torch.empty((vecs, row), dtype=X.dtype, device=W.device)
         nbytes = max(_lib.lib().gguf_mmq_workspace_bytes_engine(vecs, row, col, MMQ_ENGINES["half"]), 16)
         ws = torch.empty(nbytes, dtype=torch.uint8, device=X.device)
@@ -210,7 +240,7 @@ def ggml_moe_a8(
         raise NotImplementedError(f"ggml_moe_a8 takes at most {MOE_GROUPED_MAX_EXPERTS} experts, got {W.shape[0]}")
     act = _act_code(activation)
     col = X.shape[1] // 2 if act else X.shape[1]
-    with torch.cuda.device(X.device):
+    with _on_device_of(X):
         out = torch.empty((tokens * top_k, row), dtype=X.dtype, device=W.device)
         ws = _workspace(X, tokens, col)
         rc = _lib.lib().gguf_moe_mmq_block(
@@ -247,7 +277,7 @@ def ggml_moe_a8_vec(
     act = _act_code(activation)
     col = X.shape[1] // 2 if act else X.shape[1]
     L = _lib.lib()
-    with torch.cuda.device(X.device):
+    with _on_device_of(X):
         out = torch.empty((tokens * top_k, row), dtype=X.dtype, device=W.device)
         nbytes = max(16, L.gguf_moe_vec_workspace_bytes(tokens, top_k, col, W.shape[0]))  # quantized rows + routing sort
         ws = torch.empty(nbytes, dtype=torch.uint8, device=X.device)
@@ -276,7 +306,7 @@ def quantize_q8_1(X: torch.Tensor) -> tuple[torch.Tensor, torch.Tensor]:
     _check_inputs(X)
     m, k = X.shape
     kp = (k + 511) // 512 * 512
-    with torch.cuda.device(X.device):
+    with _on_device_of(X):
         ws = _workspace(X, m, k)
         q = torch.empty((m, kp), dtype=torch.int8, device=X.device)
         ds = torch.empty((m, kp // 32, 2), dtype=torch.float32, device=X.device)
@@ -298,7 +328,7 @@ def moe_align_block_size(topk_ids: torch.Tensor, block_size: int, num_experts: i
     numel = ids.numel()
     capacity = numel + num_experts * (block_size - 1)
     nblocks = (capacity + block_size - 1) // block_size
-    with torch.cuda.device(ids.device):
+    with _on_device_of(ids):
         sorted_ids = torch.empty(capacity, dtype=torch.int32, device=ids.device)
         expert_ids = torch.empty(nblocks, dtype=torch.int32, device=ids.device)
         post = torch.empty(1, dtype=torch.int32, device=ids.device)
@@ -343,7 +373,7 @@ def moe_vec_layer(
     if w.dtype != torch.float32 or not w.is_contiguous():
         w = w.to(torch.float32).contiguous()
     L = _lib.lib()
-    with torch.cuda.device(X.device):
+    with _on_device_of(X):
         out = output if output is not None else torch.empty((tokens, n_out), dtype=X.dtype, device=W2.device)
         ws = torch.empty(max(16, L.gguf_moe_vec_layer_workspace_bytes(tokens, top_k, inner)), dtype=torch.uint8, device=X.device)
         rc = L.gguf_moe_vec_layer(X.data_ptr(), _code(X.dtype), W13.data_ptr(), int(quant_type), W2.data_ptr(), int(quant_type2),
@@ -359,7 +389,7 @@ def moe_weighted_sum(expert_out: torch.Tensor, topk_weights: torch.Tensor, outpu
     tokens, top_k, n = expert_out.shape
     _check_inputs(expert_out, output)
     w = topk_weights.reshape(tokens, top_k).to(torch.float32).contiguous()
-    with torch.cuda.device(expert_out.device):
+    with _on_device_of(expert_out):
         rc = _lib.lib().gguf_moe_weighted_sum(expert_out.data_ptr(), w.data_ptr(), output.data_ptr(), _code(expert_out.dtype),
                                               tokens, top_k, n, _stream(expert_out))
     _lib.check(rc, "moe_weighted_sum")
