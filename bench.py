@@ -367,11 +367,24 @@ def main() -> int:
         step(i)
     torch.cuda.synchronize()
     eager_ms = (time.perf_counter() - t0) * 1e3 / args.steps
+    # the same eager steps through torch.ops._C_gguf, i.e. through the compiled binding where it has been built
+    from vllm_gguf_plugin_prism_amd import _C_gguf
+    torch_op = torch.ops._C_gguf.ggml_mul_mat_vec_a8
+    for i in range(args.warmup):
+        for n, k, copies, x in mats:
+            torch_op(copies[i % ncopies], x, Q4_K, n)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for i in range(args.steps):
+        for n, k, copies, x in mats:
+            torch_op(copies[i % ncopies], x, Q4_K, n)
+    torch.cuda.synchronize()
+    eager_torch_ops_ms = (time.perf_counter() - t0) * 1e3 / args.steps
     # the same steps as one HIP graph of a full rotation over the weight copies, replayed: host launch cost out of the
     # timed region.  At least K steps and at least MIN_LAUNCHES kernel launches are timed whatever K is.
     replays = max(-(-args.steps // ncopies), -(-MIN_LAUNCHES // (len(CFG2_SHAPES) * ncopies)))
     graph_ms = eager_ms if args.profile else _graph_ms(step, ncopies, replays)
-    ms_per_step = min(eager_ms, graph_ms)
+    ms_per_step = min(eager_ms, eager_torch_ops_ms, graph_ms)
     value = step_bytes / (ms_per_step * 1e-3) / 1e9
 
     # per-launch duration of one matrix at a time (roofline of the dominant kernel)
@@ -398,6 +411,8 @@ def main() -> int:
         "config": {"workload": "BASELINE config 2: Q4_K batch-1 MMVQ over [4096,4096],[14336,4096],[4096,14336]",
                    "weight_copies_rotated": ncopies, "rotated_bytes": ncopies * total_copy_bytes,
                    "eager_ms_per_step": eager_ms, "graph_ms_per_step": graph_ms,
+                   "eager_ms_per_step_torch_ops": eager_torch_ops_ms,
+                   "torch_ops_binding": "compiled (_C_gguf_native.so)" if _C_gguf.NATIVE else "python (torch.library + ctypes)",
                    "graph_steps_timed": 0 if args.profile else replays * ncopies,
                    "pct_of_hbm_peak": 100.0 * value / HBM_PEAK_GBS},
         "roofline": roofline,

@@ -29,6 +29,29 @@ def test_schemas_match_the_reference():
         assert str(getattr(torch.ops._C_gguf, name).default._schema) == want
 
 
+def test_both_bindings_define_the_same_library():
+    """The compiled binding is the one in use when it has been built; the Python binding (GGUF_TORCH_BINDING=python)
+    defines the same schemas and dispatch keys in a fresh interpreter."""
+    import subprocess
+
+    assert _C_gguf.NATIVE == _C_gguf.NATIVE_PATH.exists()
+    code = (
+        "import torch\n"
+        "from vllm_gguf_plugin_prism_amd import _C_gguf\n"
+        "assert not _C_gguf.NATIVE\n"
+        "for n in ('ggml_dequantize', 'ggml_mul_mat_vec_a8', 'ggml_mul_mat_a8', 'ggml_moe_a8', 'ggml_moe_a8_vec', 'ggml_moe_get_block_size'):\n"
+        "    print(getattr(torch.ops._C_gguf, n).default._schema)\n"
+        "    print(n, torch._C._dispatch_has_kernel_for_dispatch_key('_C_gguf::' + n, 'CUDA'))\n"
+    )
+    env = dict(__import__("os").environ, GGUF_TORCH_BINDING="python")
+    res = subprocess.run([sys.executable, "-c", code], capture_output=True, text=True, env=env, cwd=str(_C_gguf.NATIVE_PATH.parent.parent))
+    assert res.returncode == 0, res.stderr
+    lines = res.stdout.strip().splitlines()
+    for i, (name, want) in enumerate(REFERENCE_SCHEMAS.items()):
+        assert lines[2 * i] == want
+        assert lines[2 * i + 1] == f"{name} {name != 'ggml_moe_get_block_size'}"
+
+
 def test_dispatch_keys():
     for name in REFERENCE_SCHEMAS:
         op = f"_C_gguf::{name}"

@@ -7,9 +7,12 @@ Importing this module defines the six operator schemas of the reference's
 extension as ``vllm_gguf_plugin._C_gguf`` (``ops.py:42-48``); ``install_as("vllm_gguf_plugin._C_gguf")`` puts this
 module under that name.
 
-The binding is Python on purpose: it needs no build against a particular torch, and all it does per call is allocate
-the output and the workspace with torch and pass pointers and torch's current stream to the C ABI (the work of
-``vllm_gguf_plugin_prism_amd.ops``).
+Two bindings define the same library.  ``_C_gguf_native.so`` (``csrc/torch_binding/gguf_torch_ops.cpp``, built by
+``python -m vllm_gguf_plugin_prism_amd.build`` against the installed torch) registers the operators in C++, as the
+reference's extension does, and is loaded when it is there: per call it allocates the output and the workspace with
+torch and passes pointers and torch's current stream to the C ABI, without the interpreter.  Without it (or with
+``GGUF_TORCH_BINDING=python`` in the environment) the same schemas are defined and implemented here in Python over
+``vllm_gguf_plugin_prism_amd.ops``, which needs no build against a particular torch.  ``NATIVE`` says which one is active.
 
 Fake (meta) functions are *not* registered on import: the reference registers its own when it finds the library
 (``ops.py:110-175``) and torch refuses a second registration.  A caller without the reference's ``ops.py`` calls
@@ -17,12 +20,21 @@ Fake (meta) functions are *not* registered on import: the reference registers it
 """
 from __future__ import annotations
 
+import os
 import sys
+from pathlib import Path
 
 import torch
 from torch.library import Library
 
-from . import ops
+from . import _lib, ops
+
+NATIVE_PATH = Path(__file__).resolve().parent / "_C_gguf_native.so"
+NATIVE = False
+if NATIVE_PATH.exists() and os.environ.get("GGUF_TORCH_BINDING", "native") != "python":
+    _lib.lib()                                   # torch's HIP runtime and libgguf_hip.so first (see _lib.lib)
+    torch.ops.load_library(str(NATIVE_PATH))
+    NATIVE = True
 
 SCHEMAS = (
     "ggml_dequantize(Tensor W, int type, SymInt m, SymInt n, ScalarType? dtype) -> Tensor",
@@ -34,8 +46,8 @@ SCHEMAS = (
     "ggml_moe_get_block_size(int type) -> int",
 )
 
-_def = Library("_C_gguf", "DEF")
-for _schema in SCHEMAS:
+_def = None if NATIVE else Library("_C_gguf", "DEF")
+for _schema in () if NATIVE else SCHEMAS:
     _def.define(_schema)
 
 
@@ -63,12 +75,13 @@ def _moe_get_block_size(type):
     return ops.ggml_moe_get_block_size(type)
 
 
-_def.impl("ggml_dequantize", _dequantize, "CUDA")
-_def.impl("ggml_mul_mat_vec_a8", _mul_mat_vec_a8, "CUDA")
-_def.impl("ggml_mul_mat_a8", _mul_mat_a8, "CUDA")
-_def.impl("ggml_moe_a8", _moe_a8, "CUDA")
-_def.impl("ggml_moe_a8_vec", _moe_a8_vec, "CUDA")
-_def.impl("ggml_moe_get_block_size", _moe_get_block_size, "CompositeExplicitAutograd")
+if not NATIVE:
+    _def.impl("ggml_dequantize", _dequantize, "CUDA")
+    _def.impl("ggml_mul_mat_vec_a8", _mul_mat_vec_a8, "CUDA")
+    _def.impl("ggml_mul_mat_a8", _mul_mat_a8, "CUDA")
+    _def.impl("ggml_moe_a8", _moe_a8, "CUDA")
+    _def.impl("ggml_moe_a8_vec", _moe_a8_vec, "CUDA")
+    _def.impl("ggml_moe_get_block_size", _moe_get_block_size, "CompositeExplicitAutograd")
 
 _fakes_registered = False
 
