@@ -226,28 +226,34 @@ int gguf_moe_align_block_size(const int32_t* topk_ids, int64_t numel, int64_t nu
 int gguf_moe_weighted_sum(const void* Y, const float* topk_weights, void* out, int dtype, int64_t tokens, int64_t top_k,
                           int64_t N, gguf_stream_t stream);
 
-/* A whole MoE layer for a few tokens in two launches: X[tokens][H] -> out[tokens][N_out] through
+/* A whole MoE layer on the per-pair operators' arithmetic in one call: X[tokens][H] -> out[tokens][N_out] through
  * W13[E][2 I][H packed] ([gate | up] rows) and W2[E][N_out][I packed], with topk_ids[tokens][top_k] and fp32
  * topk_weights[tokens][top_k] (ggml_moe_a8_vec, act(), ggml_moe_a8_vec, out.mul_(topk_weights), ops.moe_sum:
  * quantization/fused_moe.py:98-111; here gguf_moe_vec, gguf_moe_vec_act and gguf_moe_weighted_sum in sequence, whose
  * result it reproduces up to the last bit of the fp32 dot products -- every intermediate is rounded to the dtype where
- * those steps store it).  The first
- * kernel's workgroups own the same features in the gate and the up half, apply the activation and write h as q8_1 rows
- * into `workspace` (gguf_moe_vec_layer_workspace_bytes(tokens, top_k, I) bytes, layout private); the second kernel's
- * workgroups own a band of output features of one token, walk it in all top_k experts and form the weighted sum, so
- * neither [tokens*top_k][2 I] nor [tokens*top_k][N_out] exists in memory.  act: 1 = SiLU, 2 = GELU.  A pair whose expert
- * id is outside [0, num_experts) (num_experts > 0) adds nothing.  gguf_moe_vec_layer_takes says (1 / 0) whether the two
- * kernels serve a layer: I a multiple of 32 and of type2's block, top_k times the (half-)waves a row of W2 takes within
- * one workgroup, at most 65535 pairs, and experts not shared by so many pairs that the grouped routes of
- * gguf_moe_vec_act pay; gguf_moe_vec_layer returns GGUF_ERR_SHAPE where it does not.  No counterpart as one call in
- * the reference. */
+ * those steps store it).  No counterpart as one call in the reference.  gguf_moe_vec_layer_takes says how a layer is
+ * served:
+ *   1  a few tokens, experts not shared (fewer than 2 - 2.5 pairs per expert): two launches.  The first GEMV's workgroups
+ *      own the same features in the gate and the up half, apply the activation and write h as q8_1 rows into the
+ *      workspace; the second's own a band of output features of one token, walk it in all top_k experts and form the
+ *      weighted sum, so neither [tokens*top_k][2 I] nor [tokens*top_k][N_out] exists in memory.
+ *   2  experts shared by a few pairs each (at most 16 per expert on average, formats with 16-slot tiles, E <= 256): five
+ *      launches on the tile kernels -- quantize, one routing sort for both GEMMs, first GEMM with the activation and the
+ *      quantisation of its result in the epilogue, second GEMM from those rows, weighted sum -- where the separate
+ *      operators take seven.
+ *   0  not served (I no multiple of 32 or of type2's block, top_k times the waves a row of W2 takes beyond a workgroup,
+ *      more than 65535 pairs, experts shared by more pairs than that): gguf_moe_vec_layer returns GGUF_ERR_SHAPE.
+ * workspace: gguf_moe_vec_layer_workspace_bytes(...) bytes, layout private; GGUF_ERR_WORKSPACE if workspace_bytes is less
+ * than the route needs.  act: 1 = SiLU, 2 = GELU.  A pair whose expert id is outside [0, num_experts) (num_experts > 0)
+ * adds nothing on route 1. */
 int gguf_moe_vec_layer_takes(int type13, int type2, int64_t H, int64_t I, int64_t N_out, int64_t top_k, int64_t tokens,
                              int64_t num_experts);
-int64_t gguf_moe_vec_layer_workspace_bytes(int64_t tokens, int64_t top_k, int64_t I);
+int64_t gguf_moe_vec_layer_workspace_bytes(int64_t tokens, int64_t top_k, int64_t H, int64_t I, int64_t N_out,
+                                           int64_t num_experts, int xdtype);
 int gguf_moe_vec_layer(const void* X, int xdtype, const void* W13, int type13, const void* W2, int type2,
-                       const int32_t* topk_ids, const float* topk_weights, void* workspace, void* out, int64_t H,
-                       int64_t I, int64_t N_out, int64_t top_k, int64_t tokens, int act, int64_t num_experts,
-                       gguf_stream_t stream);
+                       const int32_t* topk_ids, const float* topk_weights, void* workspace, int64_t workspace_bytes,
+                       void* out, int64_t H, int64_t I, int64_t N_out, int64_t top_k, int64_t tokens, int act,
+                       int64_t num_experts, gguf_stream_t stream);
 
 #ifdef __cplusplus
 }

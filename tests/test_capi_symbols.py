@@ -147,15 +147,18 @@ def test_ctypes_signatures_match_the_header_type_for_type():
 
 def test_two_launch_moe_layer_states_which_shapes_it_serves():
     """gguf_moe_vec_layer_takes needs no GPU: the OLMoE-like layer at one token and a Mixtral-like one are served; top_k
-    times the waves a row takes beyond one workgroup, experts shared by many pairs, unknown types and inner sizes that
-    are not whole blocks are not.  The workspace holds one q8_1 row of the inner size per pair."""
+    times the waves a row takes beyond one workgroup, experts shared by more than 16 pairs each, unknown types and inner
+    sizes that are not whole blocks are not; experts shared by a few pairs each take the tile route.  The workspace holds
+    at least one q8_1 row of the inner size per pair and the quantized rows of X."""
     h = _lib.lib()
     assert h.gguf_moe_vec_layer_takes(2, 2, 2048, 1024, 2048, 8, 1, 64) == 1
     assert h.gguf_moe_vec_layer_takes(12, 14, 4096, 14336, 4096, 2, 1, 8) == 1
     assert h.gguf_moe_vec_layer_takes(2, 2, 2048, 8192, 2048, 8, 1, 64) == 0
-    assert h.gguf_moe_vec_layer_takes(2, 2, 2048, 1024, 2048, 8, 64, 64) == 0
+    assert h.gguf_moe_vec_layer_takes(2, 2, 2048, 1024, 2048, 8, 64, 64) == 2      # 8 pairs per expert: the tile route
+    assert h.gguf_moe_vec_layer_takes(2, 2, 2048, 1024, 2048, 8, 200, 64) == 0     # 25 pairs per expert: blocks of 32, not served
+    assert h.gguf_moe_vec_layer_takes(6, 6, 2048, 1024, 2048, 8, 64, 64) == 0       # Q5_0 has no 16-slot tiles with the GEMV's sums
     assert h.gguf_moe_vec_layer_takes(1, 2, 2048, 1024, 2048, 8, 1, 64) == 0
     assert h.gguf_moe_vec_layer_takes(2, 12, 2048, 1120, 2048, 8, 1, 64) == 0
-    assert h.gguf_moe_vec_layer_workspace_bytes(3, 8, 1024) == 24 * h.gguf_q8_1_row_bytes(1024)
-    assert h.gguf_moe_vec_layer(None, 1, None, 2, None, 2, None, None, None, None, 2048, 1024, 2048, 8, 1, 0, 64, None) == -3
-    assert h.gguf_moe_vec_layer(None, 1, None, 2, None, 2, None, None, None, None, 2048, 1024, 2048, 8, 1, 1, 64, None) == -4
+    assert h.gguf_moe_vec_layer_workspace_bytes(3, 8, 2048, 1024, 2048, 64, 1) >= 24 * h.gguf_q8_1_row_bytes(1024) + 3 * h.gguf_q8_1_row_bytes(2048)
+    assert h.gguf_moe_vec_layer(None, 1, None, 2, None, 2, None, None, None, 0, None, 2048, 1024, 2048, 8, 1, 0, 64, None) == -3
+    assert h.gguf_moe_vec_layer(None, 1, None, 2, None, 2, None, None, None, 0, None, 2048, 1024, 2048, 8, 1, 1, 64, None) == -4

@@ -569,12 +569,49 @@ def test_moe_layer_in_two_launches_matches_the_separate_steps(qtype, dt):
     # top_k times the waves a row of the down projection takes exceed a workgroup; an inner size that is no multiple of 32
     # blocks ... of its format; experts shared by many pairs (the grouped routes of the per-pair operator pay): declined
     assert not ops.moe_vec_layer_takes(qtype, qtype, 2048, 8192, 2048, 8, 1, 64)
-    assert not ops.moe_vec_layer_takes(qtype, qtype, 2048, 1024, 2048, 8, 64, 64)
+    assert not ops.moe_vec_layer_takes(qtype, qtype, 2048, 1024, 2048, 8, 200, 64)
     with pytest.raises(ValueError):
-        ops.moe_vec_layer(torch.zeros(64, 2048, device="cuda", dtype=TORCH_DT[dt]),
+        ops.moe_vec_layer(torch.zeros(200, 2048, device="cuda", dtype=TORCH_DT[dt]),
                           _dev(np.zeros((64, 2048, 2048 // qk * o.QUANT_SIZES[qtype][1]), dtype=np.uint8)),
                           _dev(np.zeros((64, 2048, 1024 // qk * o.QUANT_SIZES[qtype][1]), dtype=np.uint8)),
-                          _dev(np.ones((64, 8), dtype=np.float32)), _dev(np.zeros((64, 8), dtype=np.int32)), qtype, qtype, "silu")
+                          _dev(np.ones((200, 8), dtype=np.float32)), _dev(np.zeros((200, 8), dtype=np.int32)), qtype, qtype, "silu")
+
+
+@pytest.mark.parametrize("dt", ["f32", "f16", "bf16"])
+@pytest.mark.parametrize("qtype", [o.Q4_0, o.Q8_0, o.Q3_K, o.Q4_K, o.Q5_K, o.Q6_K, o.IQ4_XS, o.IQ2_XXS])
+def test_moe_layer_on_tiles_matches_the_separate_steps(qtype, dt):
+    """moe_vec_layer where a few pairs share each expert: quantize, one routing sort, first GEMM on 16-slot tiles with
+    the activation and the q8_1 quantisation in its epilogue, second GEMM from those rows, weighted sum -- against the
+    per-pair operator called twice and moe_weighted_sum (which take the same tile kernels with a sort and a quantize
+    launch more each).  Inner sizes that end inside a 128-column tile, an expert without pairs, a second format."""
+    ops = _ops()
+    rng = np.random.default_rng(1800 + qtype)
+    qk = o.QUANT_SIZES[qtype][0]
+    other = o.Q8_0 if qtype != o.Q8_0 else o.Q4_0
+    for case, (t, top_k, e, hid, inner) in enumerate([(24, 4, 8, 512, 768), (40, 2, 6, 256, 1280 if qk == 32 else 1024)]):
+        for qt2 in (qtype, other) if case == 0 else (qtype,):
+            w13 = np.stack([o.make_weights(rng, qtype, 2 * inner, hid) for _ in range(e)])
+            w2 = np.stack([o.make_weights(rng, qt2, hid, inner) for _ in range(e)])
+            w13d, w2d = _dev(w13), _dev(w2)
+            ids, wts = _routing(rng, t, e - 1, top_k)            # the last expert has no pairs
+            pairs = t * top_k
+            assert _lib_takes(ops, qtype, qt2, hid, inner, hid, top_k, t, e) == 2
+            x = torch.randn(t, hid, device="cuda")
+            x = (x * (4.0 / ops.ggml_moe_a8_vec(x, w13d, _dev(ids), top_k, qtype, 2 * inner, t).abs().max())).to(TORCH_DT[dt])
+            h = ops.ggml_moe_a8_vec(x, w13d, _dev(ids), top_k, qtype, 2 * inner, t)
+            y = ops.ggml_moe_a8_vec(h, w2d, _dev(ids.reshape(pairs, 1)), 1, qt2, hid, pairs, activation="silu")
+            want = torch.empty((t, hid), dtype=x.dtype, device="cuda")
+            ops.moe_weighted_sum(y.reshape(t, top_k, hid), _dev(wts), want)
+            got = ops.moe_vec_layer(x, w13d, w2d, _dev(wts), _dev(ids), qtype, qt2, "silu")
+            assert not torch.isnan(want).any()
+            # (as for the two-launch route: bit for bit in most cases, a quant of h may move by a step in rare ones)
+            err = o.rel_l2(got.float().cpu().numpy(), want.float().cpu().numpy())
+            assert err <= {"f32": 5e-4, "f16": 1e-3, "bf16": 4e-3}[dt], f"{o.TYPE_NAMES[qtype]} {o.TYPE_NAMES[qt2]} {dt} case {case} rel-L2 {err}"
+
+
+def _lib_takes(ops, *args):
+    from vllm_gguf_plugin_prism_amd import _lib
+    return _lib.lib().gguf_moe_vec_layer_takes(*[int(a) for a in args])
 
 
 @pytest.mark.parametrize("dt", ["f32", "f16"])

@@ -69,10 +69,10 @@ _SIGNATURES = {
     "gguf_moe_weighted_sum": (_c.c_int, [_c.c_void_p, _c.c_void_p, _c.c_void_p, _c.c_int, _c.c_int64, _c.c_int64,
                                          _c.c_int64, _c.c_void_p]),
     "gguf_moe_vec_layer_takes": (_c.c_int, [_c.c_int, _c.c_int, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64]),
-    "gguf_moe_vec_layer_workspace_bytes": (_c.c_int64, [_c.c_int64, _c.c_int64, _c.c_int64]),
+    "gguf_moe_vec_layer_workspace_bytes": (_c.c_int64, [_c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int]),
     "gguf_moe_vec_layer": (_c.c_int, [_c.c_void_p, _c.c_int, _c.c_void_p, _c.c_int, _c.c_void_p, _c.c_int, _c.c_void_p, _c.c_void_p,
-                                      _c.c_void_p, _c.c_void_p, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int,
-                                      _c.c_int64, _c.c_void_p]),
+                                      _c.c_void_p, _c.c_int64, _c.c_void_p, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64,
+                                      _c.c_int, _c.c_int64, _c.c_void_p]),
 }
 EXPORTS = tuple(_SIGNATURES)
 

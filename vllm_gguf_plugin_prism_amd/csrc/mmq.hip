@@ -572,6 +572,57 @@ int moe_vec_tiles(const void* X, int xdtype, void* workspace, const void* W, con
   return GGUF_ERR_TYPE;
 }
 
+// ---- A MoE layer on the tile kernels for experts shared by a few pairs each (blocks of 16 slots): quantize X, sort the
+// pairs once, first expert GEMM with the gated activation and the quantisation of its result in the epilogue, second
+// expert GEMM straight from those rows, weighted sum -- five launches where the separate operators take seven
+// (quantize, sort, GEMM, quantize with the activation, sort, GEMM, sum).  The arithmetic is the per-pair operator's on
+// both GEMMs (offset sums of the GEMV for Q4_K / Q5_K), every intermediate rounded where the separate steps store it.
+int moe_tiles16_gate(const void* W, const void* ws, void* q8h, int dtype, int type, int inner, int K, int num_sorted, const MoeArgs& moe,
+                     int act, hipStream_t s);
+}  // namespace gguf
+extern "C" int gguf_moe_weighted_sum(const void* Y, const float* topk_weights, void* out, int dtype, int64_t tokens, int64_t top_k,
+                                     int64_t N, gguf_stream_t stream);
+namespace gguf {
+
+static inline int64_t up16(int64_t v) { return (v + 15) / 16 * 16; }
+
+bool moe_tiles_layer_ok(int type13, int type2, int64_t pairs, int64_t num_experts, int64_t I) {
+  return moe_tiles16_ok(type13) && moe_tiles16_ok(type2) && type13 != T_Q5_0 && type2 != T_Q5_0 && num_experts > 0 && num_experts <= 256 &&
+         pairs <= 16 * num_experts && I % 32 == 0;
+}
+
+// [q8_1 rows of X][q8_1 rows of h][second GEMM's result, pairs x N_out][sorted ids, expert ids, padded total]
+int64_t moe_tiles_layer_workspace(int64_t tokens, int64_t top_k, int64_t H, int64_t I, int64_t N_out, int64_t num_experts, int elt) {
+  const int64_t pairs = tokens * top_k, sorted_cap = pairs + num_experts * 15;
+  return up16(tokens * q8_row_bytes(H)) + up16(pairs * q8_row_bytes(I)) + up16(pairs * N_out * elt) + (sorted_cap + sorted_cap / 16 + 2) * 4;
+}
+
+int moe_tiles_layer(const void* X, int xdtype, void* workspace, const void* W13, int type13, const void* W2, int type2, const int32_t* topk_ids,
+                    const float* topk_w, void* out, int H, int I, int N_out, int top_k, int tokens, int act, int num_experts, hipStream_t s) {
+  const int pairs = tokens * top_k, elt = xdtype == GGUF_DTYPE_F32 ? 4 : 2;
+  char* q8x = (char*)workspace;
+  char* q8h = q8x + up16((int64_t)tokens * q8_row_bytes(H));
+  char* y2 = q8h + up16((int64_t)pairs * q8_row_bytes(I));
+  const int64_t sorted_cap = (int64_t)pairs + (int64_t)num_experts * 15, block_cap = sorted_cap / 16 + 1;
+  int32_t* sorted = (int32_t*)(y2 + up16((int64_t)pairs * N_out * elt));
+  int32_t* experts = sorted + sorted_cap;
+  int32_t* post = experts + block_cap;
+  int rc = quantize_q8_1(X, xdtype, q8x, tokens, H, s);
+  if (rc != GGUF_OK) return rc;
+  rc = gguf_moe_align_block_size(topk_ids, pairs, num_experts, 16, sorted, sorted_cap, experts, block_cap, post, (gguf_stream_t)s);
+  if (rc != GGUF_OK) return rc;
+  const int ns = (int)(sorted_cap / 16 * 16);
+  const auto gemv_sums = [](int type) { return type == T_Q4_K || type == T_Q5_K ? 1 : 0; };
+  const MoeArgs m1 = {sorted, experts, post, (int64_t)2 * I * (H / block_elems(type13)) * block_bytes(type13), top_k, pairs, gemv_sums(type13)};
+  rc = moe_tiles16_gate(W13, q8x, q8h, xdtype, type13, I, H, ns, m1, act, s);
+  if (rc != GGUF_OK) return rc == GGUF_NOT_TAKEN ? GGUF_ERR_TYPE : rc;
+  // the second GEMM's rows are the pairs themselves: slot -> pair -> row pair of q8h
+  const MoeArgs m2 = {sorted, experts, post, (int64_t)N_out * (I / block_elems(type2)) * block_bytes(type2), 1, pairs, gemv_sums(type2)};
+  rc = moe_tiles16(W2, q8h, y2, xdtype, type2, N_out, I, ns, m2, s);
+  if (rc != GGUF_OK) return rc == GGUF_NOT_TAKEN ? GGUF_ERR_TYPE : rc;
+  return gguf_moe_weighted_sum(y2, topk_w, out, xdtype, tokens, top_k, N_out, (gguf_stream_t)s);
+}
+
 // mmvq.hip
 int mmvq_any(int type, const void* W, const void* x, void* q8_workspace, void* Y, int xdtype, int64_t N, int64_t K, int64_t M,
              hipStream_t s, const LinearArgs& la);

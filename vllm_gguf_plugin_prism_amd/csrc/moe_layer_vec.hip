@@ -17,9 +17,18 @@
 // Results are those of gguf_moe_vec, gguf_moe_vec_act and gguf_moe_weighted_sum in sequence up to the last bit of a dot
 // product (the compiler contracts multiply-adds per kernel): the same per-lane arithmetic, the same order of the partial
 // sums (ascending in K), the same quantizer and activation routines, every intermediate rounded where those steps store it.
+//
+// Where experts are shared by a few pairs each (the per-pair operator's tile route on blocks of 16 slots) the same entry
+// point runs the layer in five launches on the tile kernels instead (mmq.hip, moe_tiles_layer).
 #include "mmvq_core.h"
 
 namespace gguf {
+
+// mmq.hip
+bool moe_tiles_layer_ok(int type13, int type2, int64_t pairs, int64_t num_experts, int64_t I);
+int64_t moe_tiles_layer_workspace(int64_t tokens, int64_t top_k, int64_t H, int64_t I, int64_t N_out, int64_t num_experts, int elt);
+int moe_tiles_layer(const void* X, int xdtype, void* workspace, const void* W13, int type13, const void* W2, int type2, const int32_t* topk_ids,
+                    const float* topk_w, void* out, int H, int I, int N_out, int top_k, int tokens, int act, int num_experts, hipStream_t s);
 
 struct MoeUpArgs {
   const int32_t* topk_ids;
@@ -377,14 +386,15 @@ static int moe_sum_fmt(int dtype, const void* W, const void* ws, const int32_t* 
   CASE(T_IQ2_XXS, FmtIQ2_XXS) CASE(T_IQ2_XS, FmtIQ2_XS) CASE(T_IQ2_S, FmtIQ2_S) CASE(T_IQ3_XXS, FmtIQ3_XXS) CASE(T_IQ3_S, FmtIQ3_S) \
   CASE(T_IQ1_S, FmtIQ1_S) CASE(T_IQ1_M, FmtIQ1_M)
 
-static bool moe_layer_takes(int type13, int type2, int H, int I, int N_out, int top_k, int tokens, int num_experts) {
+// 0: not served; 1: the two launches above; 2: five launches on the tile kernels (experts shared by a few pairs each)
+static int moe_layer_takes(int type13, int type2, int H, int I, int N_out, int top_k, int tokens, int num_experts) {
   const int qk13 = block_elems(type13), qk2 = block_elems(type2);
-  if (qk13 == 0 || qk2 == 0 || H % qk13 != 0 || I % qk2 != 0 || I % 32 != 0) return false;
+  if (qk13 == 0 || qk2 == 0 || H % qk13 != 0 || I % qk2 != 0 || I % 32 != 0) return 0;
   // where experts are shared by enough pairs the per-pair operator reads each once per group of pairs instead
   const int64_t pairs = (int64_t)tokens * top_k;
-  if (num_experts > 0 && (moe_share_pays(pairs, num_experts, (int64_t)2 * I * (H / qk13) * block_bytes(type13)) ||
-                          moe_share_pays(pairs, num_experts, (int64_t)N_out * (I / qk2) * block_bytes(type2))))
-    return false;
+  const bool shared13 = num_experts > 0 && moe_share_pays(pairs, num_experts, (int64_t)2 * I * (H / qk13) * block_bytes(type13));
+  const bool shared2 = num_experts > 0 && moe_share_pays(pairs, num_experts, (int64_t)N_out * (I / qk2) * block_bytes(type2));
+  if (shared13 || shared2) return shared13 && shared2 && moe_tiles_layer_ok(type13, type2, pairs, num_experts, I) ? 2 : 0;
   bool up = false, down = false;
   switch (type13) {
 #define MOE_LAYER_CASE(ID, FMT) case ID: up = moe_up_plan<FMT>(H, I, (int)pairs).ok; break;
@@ -396,7 +406,7 @@ static bool moe_layer_takes(int type13, int type2, int H, int I, int N_out, int 
     GGUF_MOE_LAYER_FORMATS(MOE_LAYER_CASE)
 #undef MOE_LAYER_CASE
   }
-  return up && down;
+  return up && down ? 1 : 0;
 }
 
 }  // namespace gguf
@@ -410,16 +420,20 @@ extern "C" int gguf_moe_vec_layer_takes(int type13, int type2, int64_t H, int64_
                                         int64_t num_experts) {
   if (!moe_layer_sizes_ok(H, I, N_out, top_k, tokens)) return 0;
   return gguf::moe_layer_takes(type13, type2, (int)H, (int)I, (int)N_out, (int)top_k, (int)tokens,
-                               num_experts > 0 && num_experts <= 1024 ? (int)num_experts : 0) ? 1 : 0;
+                               num_experts > 0 && num_experts <= 1024 ? (int)num_experts : 0);
 }
 
-extern "C" int64_t gguf_moe_vec_layer_workspace_bytes(int64_t tokens, int64_t top_k, int64_t I) {
-  return tokens <= 0 || top_k <= 0 || I <= 0 ? 0 : tokens * top_k * gguf::q8_row_bytes(I);
+extern "C" int64_t gguf_moe_vec_layer_workspace_bytes(int64_t tokens, int64_t top_k, int64_t H, int64_t I, int64_t N_out, int64_t num_experts,
+                                                      int xdtype) {
+  if (tokens <= 0 || top_k <= 0 || H <= 0 || I <= 0 || N_out <= 0 || num_experts < 0) return 0;
+  const int64_t pair_rows = tokens * top_k * gguf::q8_row_bytes(I);
+  const int64_t tiles = gguf::moe_tiles_layer_workspace(tokens, top_k, H, I, N_out, num_experts, xdtype == GGUF_DTYPE_F32 ? 4 : 2);
+  return pair_rows > tiles ? pair_rows : tiles;
 }
 
 extern "C" int gguf_moe_vec_layer(const void* X, int xdtype, const void* W13, int type13, const void* W2, int type2, const int32_t* topk_ids,
-                                  const float* topk_weights, void* workspace, void* out, int64_t H, int64_t I, int64_t N_out, int64_t top_k,
-                                  int64_t tokens, int act, int64_t num_experts, gguf_stream_t stream) {
+                                  const float* topk_weights, void* workspace, int64_t workspace_bytes, void* out, int64_t H, int64_t I,
+                                  int64_t N_out, int64_t top_k, int64_t tokens, int act, int64_t num_experts, gguf_stream_t stream) {
   using namespace gguf;
   if (act != ACT_SILU && act != ACT_GELU) return GGUF_ERR_SHAPE;
   if (block_elems(type13) == 0 || block_elems(type2) == 0) return GGUF_ERR_TYPE;
@@ -429,8 +443,15 @@ extern "C" int gguf_moe_vec_layer(const void* X, int xdtype, const void* W13, in
   if (!X || !W13 || !W2 || !topk_ids || !topk_weights || !workspace || !out) return GGUF_ERR_NULL;
   if (((uintptr_t)W13 | (uintptr_t)W2) & 1) return GGUF_ERR_SHAPE;   // packed blocks sit at even addresses
   const int ne = num_experts > 0 && num_experts <= 1024 ? (int)num_experts : 0;
-  if (!moe_layer_takes(type13, type2, (int)H, (int)I, (int)N_out, (int)top_k, (int)tokens, ne)) return GGUF_ERR_SHAPE;
+  const int route = moe_layer_takes(type13, type2, (int)H, (int)I, (int)N_out, (int)top_k, (int)tokens, ne);
+  if (route == 0) return GGUF_ERR_SHAPE;
   hipStream_t s = (hipStream_t)stream;
+  if (route == 2) {
+    if (workspace_bytes < moe_tiles_layer_workspace(tokens, top_k, H, I, N_out, ne, xdtype == GGUF_DTYPE_F32 ? 4 : 2)) return GGUF_ERR_WORKSPACE;
+    return moe_tiles_layer(X, xdtype, workspace, W13, type13, W2, type2, topk_ids, topk_weights, out, (int)H, (int)I, (int)N_out, (int)top_k,
+                           (int)tokens, act, ne, s);
+  }
+  if (workspace_bytes < tokens * top_k * q8_row_bytes(I)) return GGUF_ERR_WORKSPACE;
   int rc = GGUF_ERR_TYPE;
   switch (type13) {
 #define MOE_LAYER_CASE(ID, FMT) \

@@ -14,6 +14,7 @@
 // wave owns 32 features = two 16 x 16 tiles.  The packed blocks of the weight rows are decoded once per step into LDS
 // (two buffers, one barrier per step); global loads run two steps ahead in registers (one for Q6_K / Q3_K).
 #include "mmq_i_core.h"
+#include "q8_1_device.h"
 
 namespace gguf {
 
@@ -29,10 +30,21 @@ struct Dense16 {
   float* partial;
 };
 
-template <class F, typename T, int NW, int OCC, bool MOE = true>
+// GATE (with MOE): the first expert GEMM of a layer with its seam.  The weight rows are [gate | up], inner features
+// each, and a tile's 128 columns are the SAME 64 features of both halves; the workgroup that has both finishes them --
+// y = T(sum), h = T(T(act(gate)) up), the q8_1 blocks of h -- and writes them into the pair's row of a second
+// activation workspace, which the second expert GEMM reads as it is (no [pairs][2 inner] tensor, no quantize launch).
+struct Gate16 {
+  char* rows;             // q8_1 rows of h, one per pair
+  int64_t row_bytes;
+  int inner, kp, act;     // features of each half; q8_kp(inner); ACT_SILU / ACT_GELU
+};
+
+template <class F, typename T, int NW, int OCC, bool MOE = true, bool GATE = false>
 __global__ __launch_bounds__(64 * NW, OCC) void moe16_kernel(const uint8_t* __restrict__ W, const char* __restrict__ ws, int64_t ws_row_bytes,
                                                         T* __restrict__ Y, int N, int K, int Kp, int tiles_m, int tiles, MoeArgs moe,
-                                                        Dense16 dn, const T* __restrict__ bias) {
+                                                        Dense16 dn, const T* __restrict__ bias, Gate16 gate) {
+  static_assert(!GATE || (MOE && NW == 4), "the gated epilogue pairs the halves of a 128-column tile");
   static_assert(!(F::G == 16 && F::HAS_MIN), "16-deep formats with per-group offsets keep the 32-row kernel");
   constexpr int NT = 64 * NW, KS = MMQI_KS, KB = KS / 32, GR = KS / 16, LDK = Pitch<32, KS>::value;
   constexpr int M_T = 16, CT = 2, N_T = 16 * CT * NW;   // two 16-feature tiles per wave
@@ -50,7 +62,7 @@ __global__ __launch_bounds__(64 * NW, OCC) void moe16_kernel(const uint8_t* __re
   const int total = tiles * nsplit, total8 = total & ~7;   // workgroups go to the 8 XCDs in turn: give each a contiguous run
   if (wg < total8) wg = (wg & 7) * (total8 >> 3) + (wg >> 3);
   const int tile = wg % tiles, split = wg / tiles;
-  const int block = tile % tiles_m, m_base = block * M_T, n_base = (tile / tiles_m) * N_T;
+  const int block = tile % tiles_m, m_base = block * M_T, n_base = (tile / tiles_m) * (GATE ? N_T / 2 : N_T);
   int64_t w_pitch = (int64_t)(K / F::QK) * F::BS;
   if constexpr (MOE) {
     if (m_base >= moe.num_tokens_post_padded[0]) return;
@@ -78,7 +90,12 @@ __global__ __launch_bounds__(64 * NW, OCC) void moe16_kernel(const uint8_t* __re
   const int sum_plane = (MOE && moe.gemv_sums ? 2 : 1) * (Kp / 32);
   const uint8_t* w_src[WP];
 #pragma unroll
-  for (int i = 0; i < WP; ++i) w_src[i] = W + (int64_t)min(n_base + (tid + NT * i) / KB, N - 1) * w_pitch;
+  for (int i = 0; i < WP; ++i) {
+    const int n = (tid + NT * i) / KB;   // column of the tile
+    // GATE: columns 0..63 are features n_base .. of the gate half, 64..127 the same features of the up half
+    const int row = GATE ? (n < N_T / 2 ? 0 : gate.inner) + min(n_base + (n & (N_T / 2 - 1)), gate.inner - 1) : min(n_base + n, N - 1);
+    w_src[i] = W + (int64_t)row * w_pitch;
+  }
 
   struct Stage {
     uint4 aq;
@@ -211,6 +228,37 @@ __global__ __launch_bounds__(64 * NW, OCC) void moe16_kernel(const uint8_t* __re
     }
   }
 
+  if constexpr (GATE) {
+    // ---- the tile's sums, rounded as the operator stores them, meet in LDS (the buffers are free: the loop ends on a
+    // barrier); then 8 threads per slot take 8 features each of both halves, and every four of them form one q8_1 block
+    float* yt = (float*)smem;   // [16][128]
+#pragma unroll
+    for (int r = 0; r < 4; ++r)
+#pragma unroll
+      for (int c = 0; c < CT; ++c) yt[(4 * lgrp + r) * N_T + 32 * wave + 16 * c + lcol] = to_f32<T>(from_f32<T>(acc[c][r]));
+    __syncthreads();
+    if (tid < 16 * 8) {
+      const int slot = tid >> 3, part = tid & 7;
+      float xv[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) xv[i] = gate1<T>(yt[slot * N_T + 8 * part + i], yt[slot * N_T + N_T / 2 + 8 * part + i], gate.act);
+      const Q8Quad qq = q8_1_quantize8(xv);
+      const int pair = moe.sorted_token_ids[m_base + slot];
+      const int f = n_base + 8 * part;
+      if (pair < moe.num_pairs && f < gate.inner) {     // (inner is a multiple of 32: blocks are whole)
+        char* row = gate.rows + (int64_t)pair * gate.row_bytes;
+        *(uint2*)(row + f) = qq.q;
+        if ((part & 3) == 0) {
+          float* fd = (float*)(row + gate.kp);
+          const int b = f >> 5, nbp = gate.kp >> 5;
+          fd[b] = qq.d;
+          fd[nbp + b] = qq.s;
+          fd[2 * nbp + b] = qq.du;
+        }
+      }
+    }
+    return;
+  }
   // ---- store: lane = one output feature of each of its tiles, four rows
   if constexpr (!MOE) {
     if (nsplit > 1) {   // the whole partial tile, edges included: the adder masks them
@@ -281,7 +329,29 @@ static int moe16_typed(const void* W, const void* ws, void* Y, int N, int K, int
     }
   }
   hipLaunchKernelGGL(kern, dim3(tiles), dim3(64 * NW), lds_req, stream, (const uint8_t*)W, (const char*)ws, q8_row_bytes(K), (T*)Y, N, K,
-                     (int)q8_kp(K), tiles_m, tiles, moe, Dense16{}, (const T*)nullptr);
+                     (int)q8_kp(K), tiles_m, tiles, moe, Dense16{}, (const T*)nullptr, Gate16{});
+  return launch_status();
+}
+
+// The first expert GEMM of a layer with the gated activation and the q8_1 quantisation of its result in the epilogue
+// (see Gate16): W is [experts][2 inner][K packed], the result goes to q8h.
+template <class F, typename T>
+static int moe16_gate_typed(const void* W, const void* ws, void* q8h, int inner, int K, int num_sorted, const MoeArgs& moe, int act,
+                            hipStream_t stream) {
+  constexpr int NW = 4, N_T = 32 * NW, OCC = sizeof(typename F::Raw) > 64 ? 2 : 3;
+  constexpr size_t BUF = (size_t)(16 + N_T) * Pitch<32, MMQI_KS>::value + (size_t)4 * 16 * 4 * (F::HAS_MIN ? 2 : 1) + (size_t)4 * N_T * 8;
+  constexpr size_t lds = 2 * BUF;
+  static_assert(lds >= 16 * N_T * 4, "the tile of sums fits the buffers");
+  auto kern = moe16_kernel<F, T, NW, OCC, true, true>;
+  if constexpr (lds > 65536) {
+    static std::atomic<uint64_t> done{0};
+    allow_large_lds(kern, lds, done);
+  }
+  const int tiles_n = (inner + N_T / 2 - 1) / (N_T / 2), tiles_m = num_sorted / 16, tiles = tiles_m * tiles_n;
+  if (tiles == 0) return GGUF_OK;
+  hipLaunchKernelGGL(kern, dim3(tiles), dim3(64 * NW), lds, stream, (const uint8_t*)W, (const char*)ws, q8_row_bytes(K), (T*)nullptr, 2 * inner, K,
+                     (int)q8_kp(K), tiles_m, tiles, moe, Dense16{}, (const T*)nullptr,
+                     Gate16{(char*)q8h, q8_row_bytes(inner), inner, (int)q8_kp(inner), act});
   return launch_status();
 }
 
@@ -320,7 +390,7 @@ static int dense16_typed(const void* W, const void* ws, void* Y, int M, int N, i
   const int splits = dense16_splits(M, N, K, partial_bytes);
   const int64_t w_pitch = la.w_pitch ? la.w_pitch : (int64_t)(K / F::QK) * F::BS, ldy = la.ldy ? la.ldy : (int64_t)N;
   hipLaunchKernelGGL(kern, dim3(tiles * splits), dim3(64 * NW), lds, stream, (const uint8_t*)W, (const char*)ws, q8_row_bytes(K), (T*)Y, N, K,
-                     (int)q8_kp(K), tiles_m, tiles, MoeArgs{}, Dense16{M, splits, w_pitch, ldy, partial}, (const T*)la.bias);
+                     (int)q8_kp(K), tiles_m, tiles, MoeArgs{}, Dense16{M, splits, w_pitch, ldy, partial}, (const T*)la.bias, Gate16{});
   if (splits > 1)
     hipLaunchKernelGGL((mmqi_reduce_kernel<16, N_T, T>), dim3(tiles, 2), dim3(256), 0, stream, partial, (T*)Y, M, N, tiles_m, 0, splits,
                        ldy, (const T*)la.bias);
@@ -373,6 +443,30 @@ bool moe_tiles16_ok(int type) {
     case T_Q4_0: case T_Q8_0: case T_Q3_K: case T_Q4_K: case T_Q5_K: case T_Q6_K: case T_IQ4_XS: case T_IQ2_XXS: return true;
     default: return false;   // formats with other scale rules (Q4_1, Q5_1, Q2_K; Q5_0 in the per-pair operator) keep the 32-slot kernel
   }
+}
+
+template <class F>
+static int moe16_gate_fmt(const void* W, const void* ws, void* q8h, int dtype, int inner, int K, int num_sorted, const MoeArgs& moe, int act,
+                          hipStream_t s) {
+  GGUF_DISPATCH_DTYPE(dtype, return (moe16_gate_typed<F, scalar_t>(W, ws, q8h, inner, K, num_sorted, moe, act, s)));
+  return GGUF_ERR_DTYPE;
+}
+
+// The first expert GEMM over blocks of 16 slots with the activation and the quantisation of its result inside; dtype is
+// the dtype the separate operator would have stored its result in.  GGUF_NOT_TAKEN for formats without 16-slot tiles.
+int moe_tiles16_gate(const void* W, const void* ws, void* q8h, int dtype, int type, int inner, int K, int num_sorted, const MoeArgs& moe,
+                     int act, hipStream_t s) {
+  switch (type) {
+    case T_Q4_0: return moe16_gate_fmt<MQ4_0>(W, ws, q8h, dtype, inner, K, num_sorted, moe, act, s);
+    case T_Q8_0: return moe16_gate_fmt<MQ8_0>(W, ws, q8h, dtype, inner, K, num_sorted, moe, act, s);
+    case T_Q3_K: return moe16_gate_fmt<MQ3_K>(W, ws, q8h, dtype, inner, K, num_sorted, moe, act, s);
+    case T_Q6_K: return moe16_gate_fmt<MQ6_K>(W, ws, q8h, dtype, inner, K, num_sorted, moe, act, s);
+    case T_Q4_K: return moe16_gate_fmt<MQ4_K>(W, ws, q8h, dtype, inner, K, num_sorted, moe, act, s);
+    case T_Q5_K: return moe16_gate_fmt<MQ5_K>(W, ws, q8h, dtype, inner, K, num_sorted, moe, act, s);
+    case T_IQ4_XS: return moe16_gate_fmt<MIQ4_XS>(W, ws, q8h, dtype, inner, K, num_sorted, moe, act, s);
+    case T_IQ2_XXS: return moe16_gate_fmt<MIQ2_XXS>(W, ws, q8h, dtype, inner, K, num_sorted, moe, act, s);
+  }
+  return GGUF_NOT_TAKEN;
 }
 
 // The contraction over blocks of 16 sorted slots (moe_align_block_size with block 16); GGUF_NOT_TAKEN for other formats.

@@ -205,8 +205,9 @@ def fused_moe_gguf(x, w1, w2, topk_weights, topk_ids, weight_type: int, weight_t
         rows = w1.shape[1]
         if activation in ("silu", "gelu") and w1.shape[0] == w2.shape[0] and ops.moe_vec_layer_takes(
                 weight_type, weight_type2, x.shape[1], rows // 2, w2.shape[1], top_k, tokens, w1.shape[0]):
-            # a few tokens, nothing shared between pairs: two launches, the activation in the first GEMV's epilogue and the
-            # routing weights and the sum over the top-k axis in the second's
+            # the layer in one call: two launches where nothing is shared between pairs (the activation in the first GEMV's
+            # epilogue, the routing weights and the sum over the top-k axis in the second's), five on the tile kernels where
+            # a few pairs share each expert (one routing sort, no separate activation-and-quantize launch)
             return ops.moe_vec_layer(x, w1, w2, topk_weights, topk_ids, weight_type, weight_type2, activation, out_hidden)
         out = ops.ggml_moe_a8_vec(x, w1, topk_ids, top_k, weight_type, rows, tokens)
         out = ops.ggml_moe_a8_vec(out, w2, topk_ids, 1, weight_type2, w2.shape[1], tokens * top_k, activation=activation)

@@ -341,7 +341,8 @@ def moe_align_block_size(topk_ids: torch.Tensor, block_size: int, num_experts: i
 
 def moe_vec_layer_takes(quant_type: int, quant_type2: int, hidden: int, inner: int, out_features: int, top_k: int, tokens: int,
                         num_experts: int) -> bool:
-    """Whether :func:`moe_vec_layer` serves a layer of this shape (a few tokens, experts not shared by many pairs)."""
+    """Whether :func:`moe_vec_layer` serves a layer of this shape: a few tokens whose experts are not shared (two
+    launches) or experts shared by at most 16 pairs each on average (five launches on the tile kernels)."""
     return bool(_lib.lib().gguf_moe_vec_layer_takes(int(quant_type), int(quant_type2), int(hidden), int(inner), int(out_features),
                                                     int(top_k), int(tokens), int(num_experts)))
 
@@ -357,10 +358,11 @@ def moe_vec_layer(
     activation: str,
     output: torch.Tensor | None = None,
 ) -> torch.Tensor:
-    """The reference's MoE layer on its per-pair operators (quantization/fused_moe.py:98-111) in two launches:
+    """The reference's MoE layer on its per-pair operators (quantization/fused_moe.py:98-111) in one call:
     ``ggml_moe_a8_vec`` with ``act`` and the q8_1 quantisation of its result in the epilogue, then the second
-    ``ggml_moe_a8_vec`` with ``mul_`` by the routing weights and ``moe_sum`` -> ``[tokens, W2.shape[1]]``.  Same roundings as
-    those steps run one by one; raises ``ValueError`` for shapes :func:`moe_vec_layer_takes` declines."""
+    ``ggml_moe_a8_vec`` with ``mul_`` by the routing weights and ``moe_sum`` -> ``[tokens, W2.shape[1]]`` (two launches
+    where experts are not shared, five on the tile kernels where a few pairs share each).  Same roundings as those steps
+    run one by one; raises ``ValueError`` for shapes :func:`moe_vec_layer_takes` declines."""
     _check_inputs(X, W13, W2, topk_ids)
     if topk_ids.dtype != torch.int32:
         raise ValueError("topk_ids must be int32")
@@ -375,10 +377,11 @@ def moe_vec_layer(
     L = _lib.lib()
     with _on_device_of(X):
         out = output if output is not None else torch.empty((tokens, n_out), dtype=X.dtype, device=W2.device)
-        ws = torch.empty(max(16, L.gguf_moe_vec_layer_workspace_bytes(tokens, top_k, inner)), dtype=torch.uint8, device=X.device)
+        nbytes = max(16, L.gguf_moe_vec_layer_workspace_bytes(tokens, top_k, hidden, inner, n_out, W13.shape[0], _code(X.dtype)))
+        ws = torch.empty(nbytes, dtype=torch.uint8, device=X.device)
         rc = L.gguf_moe_vec_layer(X.data_ptr(), _code(X.dtype), W13.data_ptr(), int(quant_type), W2.data_ptr(), int(quant_type2),
-                                  topk_ids.data_ptr(), w.data_ptr(), ws.data_ptr(), out.data_ptr(), hidden, inner, n_out, top_k, tokens,
-                                  act, W13.shape[0], _stream(X))
+                                  topk_ids.data_ptr(), w.data_ptr(), ws.data_ptr(), nbytes, out.data_ptr(), hidden, inner, n_out, top_k,
+                                  tokens, act, W13.shape[0], _stream(X))
     _lib.check(rc, "moe_vec_layer")
     return out
 
