@@ -33,8 +33,14 @@ NATIVE_PATH = Path(__file__).resolve().parent / "_C_gguf_native.so"
 NATIVE = False
 if NATIVE_PATH.exists() and os.environ.get("GGUF_TORCH_BINDING", "native") != "python":
     _lib.lib()                                   # torch's HIP runtime and libgguf_hip.so first (see _lib.lib)
-    torch.ops.load_library(str(NATIVE_PATH))
-    NATIVE = True
+    try:
+        torch.ops.load_library(str(NATIVE_PATH))
+        NATIVE = True
+    except OSError as exc:                       # built against another torch: the Python binding serves, and says why
+        import warnings
+
+        warnings.warn(f"{NATIVE_PATH.name} does not load with this torch ({exc}); rebuild it with "
+                      "`python -m vllm_gguf_plugin_prism_amd.build`.  Using the Python binding.", RuntimeWarning)
 
 SCHEMAS = (
     "ggml_dequantize(Tensor W, int type, SymInt m, SymInt n, ScalarType? dtype) -> Tensor",
