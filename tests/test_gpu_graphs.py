@@ -124,3 +124,31 @@ def test_two_launch_moe_layer_replays_match_eager():
         graph.replay()
         torch.cuda.synchronize()
         assert torch.equal(out, eager)
+
+
+def test_five_launch_moe_layer_replays_match_eager():
+    """dispatch.fused_moe_gguf above 64 tokens with few pairs per expert (quantize, routing sort, both expert GEMMs on
+    16-slot tiles and the weighted sum, all inside one call with a workspace allocated per call) captured and replayed
+    with eager work in between; the routing changes between replays as well."""
+    from vllm_gguf_plugin_prism_amd import dispatch, ops
+    rng = np.random.default_rng(92)
+    e, hid, inner, t, top_k, qtype = 16, 512, 256, 70, 2, o.Q4_K
+    w13 = _dev(np.stack([o.make_weights(rng, qtype, 2 * inner, hid) for _ in range(e)]))
+    w2 = _dev(np.stack([o.make_weights(rng, qtype, hid, inner) for _ in range(e)]))
+    assert ops.moe_mmq_layer_takes(qtype, qtype, hid, inner, hid, top_k, t, e)
+    routes = [_dev(np.stack([rng.choice(e, size=top_k, replace=False) for _ in range(t)]).astype(np.int32)) for _ in range(3)]
+    ids = routes[0].clone()
+    wts = torch.rand(t, top_k, device="cuda")
+    xs = [torch.randn(t, hid, dtype=torch.float16, device="cuda") * 0.05 for _ in range(3)]
+    x = xs[0].clone()
+    fn = lambda: dispatch.fused_moe_gguf(x, w13, w2, wts, ids, qtype, qtype, "silu")
+    graph, out = _capture(fn)
+    for xi, ri in zip(xs, routes):
+        x.copy_(xi)
+        ids.copy_(ri)
+        eager = fn().clone()
+        torch.cuda.synchronize()
+        out.zero_()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(out, eager)

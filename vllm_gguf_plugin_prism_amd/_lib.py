@@ -73,6 +73,10 @@ _SIGNATURES = {
     "gguf_moe_vec_layer": (_c.c_int, [_c.c_void_p, _c.c_int, _c.c_void_p, _c.c_int, _c.c_void_p, _c.c_int, _c.c_void_p, _c.c_void_p,
                                       _c.c_void_p, _c.c_int64, _c.c_void_p, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64,
                                       _c.c_int, _c.c_int64, _c.c_void_p]),
+    "gguf_moe_mmq_layer_takes": (_c.c_int, [_c.c_int, _c.c_int, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64]),
+    "gguf_moe_mmq_layer": (_c.c_int, [_c.c_void_p, _c.c_int, _c.c_void_p, _c.c_int, _c.c_void_p, _c.c_int, _c.c_void_p, _c.c_void_p,
+                                      _c.c_void_p, _c.c_int64, _c.c_void_p, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64,
+                                      _c.c_int, _c.c_int64, _c.c_void_p]),
 }
 EXPORTS = tuple(_SIGNATURES)
 

@@ -597,8 +597,12 @@ int64_t moe_tiles_layer_workspace(int64_t tokens, int64_t top_k, int64_t H, int6
   return up16(tokens * q8_row_bytes(H)) + up16(pairs * q8_row_bytes(I)) + up16(pairs * N_out * elt) + (sorted_cap + sorted_cap / 16 + 2) * 4;
 }
 
+int moe_weighted_sum_live(const void* Y, const float* topk_weights, const int32_t* topk_ids, int num_experts, void* out, int dtype,
+                          int64_t tokens, int64_t top_k, int64_t N, hipStream_t s);   // moe_aux.hip
+
 int moe_tiles_layer(const void* X, int xdtype, void* workspace, const void* W13, int type13, const void* W2, int type2, const int32_t* topk_ids,
-                    const float* topk_w, void* out, int H, int I, int N_out, int top_k, int tokens, int act, int num_experts, hipStream_t s) {
+                    const float* topk_w, void* out, int H, int I, int N_out, int top_k, int tokens, int act, int num_experts, bool vec_sums,
+                    hipStream_t s) {
   const int pairs = tokens * top_k, elt = xdtype == GGUF_DTYPE_F32 ? 4 : 2;
   char* q8x = (char*)workspace;
   char* q8h = q8x + up16((int64_t)tokens * q8_row_bytes(H));
@@ -612,7 +616,8 @@ int moe_tiles_layer(const void* X, int xdtype, void* workspace, const void* W13,
   rc = gguf_moe_align_block_size(topk_ids, pairs, num_experts, 16, sorted, sorted_cap, experts, block_cap, post, (gguf_stream_t)s);
   if (rc != GGUF_OK) return rc;
   const int ns = (int)(sorted_cap / 16 * 16);
-  const auto gemv_sums = [](int type) { return type == T_Q4_K || type == T_Q5_K ? 1 : 0; };
+  // vec_sums: the offset term of Q4_K / Q5_K as the per-pair operator forms it; else as the grouped operator does
+  const auto gemv_sums = [&](int type) { return vec_sums && (type == T_Q4_K || type == T_Q5_K) ? 1 : 0; };
   const MoeArgs m1 = {sorted, experts, post, (int64_t)2 * I * (H / block_elems(type13)) * block_bytes(type13), top_k, pairs, gemv_sums(type13)};
   rc = moe_tiles16_gate(W13, q8x, q8h, xdtype, type13, I, H, ns, m1, act, s);
   if (rc != GGUF_OK) return rc == GGUF_NOT_TAKEN ? GGUF_ERR_TYPE : rc;
@@ -620,7 +625,9 @@ int moe_tiles_layer(const void* X, int xdtype, void* workspace, const void* W13,
   const MoeArgs m2 = {sorted, experts, post, (int64_t)N_out * (I / block_elems(type2)) * block_bytes(type2), 1, pairs, gemv_sums(type2)};
   rc = moe_tiles16(W2, q8h, y2, xdtype, type2, N_out, I, ns, m2, s);
   if (rc != GGUF_OK) return rc == GGUF_NOT_TAKEN ? GGUF_ERR_TYPE : rc;
-  return gguf_moe_weighted_sum(y2, topk_w, out, xdtype, tokens, top_k, N_out, (gguf_stream_t)s);
+  // the grouped operator leaves the rows of pairs whose expert id names no expert at zero (the sort drops them): the
+  // sum takes them as zero instead of reading rows of y2 that nobody wrote
+  return moe_weighted_sum_live(y2, topk_w, vec_sums ? nullptr : topk_ids, num_experts, out, xdtype, tokens, top_k, N_out, s);
 }
 
 // mmvq.hip

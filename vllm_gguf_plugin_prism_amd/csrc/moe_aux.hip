@@ -106,16 +106,32 @@ __global__ __launch_bounds__(ALIGN_THREADS) void moe_align_kernel(const int32_t*
 // once: the in-place multiply by the routing weights followed by the sum over the top-k axis.
 template <typename T>
 __global__ __launch_bounds__(256) void moe_weighted_sum_kernel(const T* __restrict__ Y, const float* __restrict__ w,
-                                                               T* __restrict__ out, int top_k, int64_t N) {
+                                                               T* __restrict__ out, int top_k, int64_t N,
+                                                               const int32_t* __restrict__ ids, int num_experts) {
   const int64_t t = blockIdx.y;
   for (int64_t n = (int64_t)blockIdx.x * 256 + threadIdx.x; n < N; n += (int64_t)gridDim.x * 256) {
     float acc = 0.0f;
     for (int k = 0; k < top_k; ++k) {
-      const T p = from_f32<T>(to_f32<T>(Y[(t * top_k + k) * N + n]) * w[t * top_k + k]);
+      // (ids given: a pair whose id names no expert has a row of zeros, whatever Y holds there)
+      const bool live = !ids || (unsigned)ids[t * top_k + k] < (unsigned)num_experts;
+      const T p = from_f32<T>((live ? to_f32<T>(Y[(t * top_k + k) * N + n]) : 0.0f) * w[t * top_k + k]);
       acc += to_f32<T>(p);
     }
     out[t * N + n] = from_f32<T>(acc);
   }
+}
+
+int moe_weighted_sum_live(const void* Y, const float* topk_weights, const int32_t* topk_ids, int num_experts, void* out, int dtype,
+                          int64_t tokens, int64_t top_k, int64_t N, hipStream_t s) {
+  const unsigned gx = (unsigned)((N + 255) / 256 < 64 ? (N + 255) / 256 : 64);
+  for (int64_t t0 = 0; t0 < tokens; t0 += 65535) {
+    const unsigned gy = (unsigned)(tokens - t0 < 65535 ? tokens - t0 : 65535);
+    GGUF_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL((moe_weighted_sum_kernel<scalar_t>), dim3(gx, gy), dim3(256), 0, s,
+                                                  (const scalar_t*)Y + t0 * top_k * N, topk_weights + t0 * top_k,
+                                                  (scalar_t*)out + t0 * N, (int)top_k, N, topk_ids ? topk_ids + t0 * top_k : nullptr,
+                                                  num_experts));
+  }
+  return launch_status();
 }
 
 }  // namespace gguf
@@ -149,13 +165,5 @@ extern "C" int gguf_moe_weighted_sum(const void* Y, const float* topk_weights, v
   if (dtype < 0 || dtype > 2) return GGUF_ERR_DTYPE;
   if (tokens == 0 || N == 0) return GGUF_OK;
   if (!Y || !topk_weights || !out) return GGUF_ERR_NULL;
-  hipStream_t s = (hipStream_t)stream;
-  const unsigned gx = (unsigned)((N + 255) / 256 < 64 ? (N + 255) / 256 : 64);
-  for (int64_t t0 = 0; t0 < tokens; t0 += 65535) {
-    const unsigned gy = (unsigned)(tokens - t0 < 65535 ? tokens - t0 : 65535);
-    GGUF_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL((moe_weighted_sum_kernel<scalar_t>), dim3(gx, gy), dim3(256), 0, s,
-                                                  (const scalar_t*)Y + t0 * top_k * N, topk_weights + t0 * top_k,
-                                                  (scalar_t*)out + t0 * N, (int)top_k, N));
-  }
-  return launch_status();
+  return moe_weighted_sum_live(Y, topk_weights, nullptr, 0, out, dtype, tokens, top_k, N, (hipStream_t)stream);
 }

@@ -28,7 +28,8 @@ namespace gguf {
 bool moe_tiles_layer_ok(int type13, int type2, int64_t pairs, int64_t num_experts, int64_t I);
 int64_t moe_tiles_layer_workspace(int64_t tokens, int64_t top_k, int64_t H, int64_t I, int64_t N_out, int64_t num_experts, int elt);
 int moe_tiles_layer(const void* X, int xdtype, void* workspace, const void* W13, int type13, const void* W2, int type2, const int32_t* topk_ids,
-                    const float* topk_w, void* out, int H, int I, int N_out, int top_k, int tokens, int act, int num_experts, hipStream_t s);
+                    const float* topk_w, void* out, int H, int I, int N_out, int top_k, int tokens, int act, int num_experts, bool vec_sums,
+                    hipStream_t s);
 
 struct MoeUpArgs {
   const int32_t* topk_ids;
@@ -449,7 +450,7 @@ extern "C" int gguf_moe_vec_layer(const void* X, int xdtype, const void* W13, in
   if (route == 2) {
     if (workspace_bytes < moe_tiles_layer_workspace(tokens, top_k, H, I, N_out, ne, xdtype == GGUF_DTYPE_F32 ? 4 : 2)) return GGUF_ERR_WORKSPACE;
     return moe_tiles_layer(X, xdtype, workspace, W13, type13, W2, type2, topk_ids, topk_weights, out, (int)H, (int)I, (int)N_out, (int)top_k,
-                           (int)tokens, act, ne, s);
+                           (int)tokens, act, ne, true, s);
   }
   if (workspace_bytes < tokens * top_k * q8_row_bytes(I)) return GGUF_ERR_WORKSPACE;
   int rc = GGUF_ERR_TYPE;
@@ -467,4 +468,32 @@ extern "C" int gguf_moe_vec_layer(const void* X, int xdtype, const void* W13, in
 #undef MOE_LAYER_CASE
   }
   return GGUF_ERR_TYPE;
+}
+
+// The same five launches with the grouped operator's arithmetic (gguf_moe_mmq_block on blocks of 16 slots, twice, and the
+// weighted sum): what a layer with more than 64 tokens takes while its experts still see at most 16 pairs each on average.
+extern "C" int gguf_moe_mmq_layer_takes(int type13, int type2, int64_t H, int64_t I, int64_t N_out, int64_t top_k, int64_t tokens,
+                                        int64_t num_experts) {
+  using namespace gguf;
+  if (!moe_layer_sizes_ok(H, I, N_out, top_k, tokens)) return 0;
+  const int qk13 = block_elems(type13), qk2 = block_elems(type2);
+  if (qk13 == 0 || qk2 == 0 || H % qk13 != 0 || I % qk2 != 0) return 0;
+  return moe_tiles_layer_ok(type13, type2, tokens * top_k, num_experts, I) ? 1 : 0;
+}
+
+extern "C" int gguf_moe_mmq_layer(const void* X, int xdtype, const void* W13, int type13, const void* W2, int type2, const int32_t* topk_ids,
+                                  const float* topk_weights, void* workspace, int64_t workspace_bytes, void* out, int64_t H, int64_t I,
+                                  int64_t N_out, int64_t top_k, int64_t tokens, int act, int64_t num_experts, gguf_stream_t stream) {
+  using namespace gguf;
+  if (act != ACT_SILU && act != ACT_GELU) return GGUF_ERR_SHAPE;
+  if (block_elems(type13) == 0 || block_elems(type2) == 0) return GGUF_ERR_TYPE;
+  if (xdtype < 0 || xdtype > 2) return GGUF_ERR_DTYPE;
+  if (tokens == 0) return GGUF_OK;
+  if (!gguf_moe_mmq_layer_takes(type13, type2, H, I, N_out, top_k, tokens, num_experts)) return GGUF_ERR_SHAPE;
+  if (!X || !W13 || !W2 || !topk_ids || !topk_weights || !workspace || !out) return GGUF_ERR_NULL;
+  if (((uintptr_t)W13 | (uintptr_t)W2) & 1) return GGUF_ERR_SHAPE;   // packed blocks sit at even addresses
+  if (workspace_bytes < moe_tiles_layer_workspace(tokens, top_k, H, I, N_out, num_experts, xdtype == GGUF_DTYPE_F32 ? 4 : 2))
+    return GGUF_ERR_WORKSPACE;
+  return moe_tiles_layer(X, xdtype, workspace, W13, type13, W2, type2, topk_ids, topk_weights, out, (int)H, (int)I, (int)N_out, (int)top_k,
+                         (int)tokens, act, (int)num_experts, false, (hipStream_t)stream);
 }

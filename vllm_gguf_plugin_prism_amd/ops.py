@@ -347,6 +347,23 @@ def moe_vec_layer_takes(quant_type: int, quant_type2: int, hidden: int, inner: i
                                                     int(top_k), int(tokens), int(num_experts)))
 
 
+def moe_mmq_layer_takes(quant_type: int, quant_type2: int, hidden: int, inner: int, out_features: int, top_k: int, tokens: int,
+                        num_experts: int) -> bool:
+    """Whether :func:`moe_mmq_layer` serves a layer of this shape: experts that see at most 16 pairs each on average,
+    both formats with 16-slot tiles, at most 256 experts."""
+    return bool(_lib.lib().gguf_moe_mmq_layer_takes(int(quant_type), int(quant_type2), int(hidden), int(inner), int(out_features),
+                                                    int(top_k), int(tokens), int(num_experts)))
+
+
+def moe_mmq_layer(X, W13, W2, topk_weights, topk_ids, quant_type: int, quant_type2: int, activation: str,
+                  output: torch.Tensor | None = None) -> torch.Tensor:
+    """The reference's MoE layer on its grouped operator (quantization/fused_moe.py:62-95) in one call of five launches:
+    one routing sort on blocks of 16 slots for both ``ggml_moe_a8`` GEMMs, ``act`` and the q8_1 quantisation of its
+    result in the first one's epilogue, ``mul_`` by the routing weights and ``moe_sum`` -> ``[tokens, W2.shape[1]]``.
+    Same roundings as those steps run one by one; raises ``ValueError`` for shapes :func:`moe_mmq_layer_takes` declines."""
+    return _moe_layer("gguf_moe_mmq_layer", X, W13, W2, topk_weights, topk_ids, quant_type, quant_type2, activation, output)
+
+
 def moe_vec_layer(
     X: torch.Tensor,
     W13: torch.Tensor,
@@ -363,12 +380,16 @@ def moe_vec_layer(
     ``ggml_moe_a8_vec`` with ``mul_`` by the routing weights and ``moe_sum`` -> ``[tokens, W2.shape[1]]`` (two launches
     where experts are not shared, five on the tile kernels where a few pairs share each).  Same roundings as those steps
     run one by one; raises ``ValueError`` for shapes :func:`moe_vec_layer_takes` declines."""
+    return _moe_layer("gguf_moe_vec_layer", X, W13, W2, topk_weights, topk_ids, quant_type, quant_type2, activation, output)
+
+
+def _moe_layer(entry, X, W13, W2, topk_weights, topk_ids, quant_type, quant_type2, activation, output):
     _check_inputs(X, W13, W2, topk_ids)
     if topk_ids.dtype != torch.int32:
         raise ValueError("topk_ids must be int32")
     act = _act_code(activation)
     if not act:
-        raise ValueError("moe_vec_layer needs an activation")
+        raise ValueError("the layer entry points need an activation")
     tokens, top_k = topk_ids.shape
     hidden, inner, n_out = X.shape[1], W13.shape[1] // 2, W2.shape[1]
     w = topk_weights.reshape(tokens, top_k)
@@ -379,10 +400,10 @@ def moe_vec_layer(
         out = output if output is not None else torch.empty((tokens, n_out), dtype=X.dtype, device=W2.device)
         nbytes = max(16, L.gguf_moe_vec_layer_workspace_bytes(tokens, top_k, hidden, inner, n_out, W13.shape[0], _code(X.dtype)))
         ws = torch.empty(nbytes, dtype=torch.uint8, device=X.device)
-        rc = L.gguf_moe_vec_layer(X.data_ptr(), _code(X.dtype), W13.data_ptr(), int(quant_type), W2.data_ptr(), int(quant_type2),
-                                  topk_ids.data_ptr(), w.data_ptr(), ws.data_ptr(), nbytes, out.data_ptr(), hidden, inner, n_out, top_k,
-                                  tokens, act, W13.shape[0], _stream(X))
-    _lib.check(rc, "moe_vec_layer")
+        rc = getattr(L, entry)(X.data_ptr(), _code(X.dtype), W13.data_ptr(), int(quant_type), W2.data_ptr(), int(quant_type2),
+                               topk_ids.data_ptr(), w.data_ptr(), ws.data_ptr(), nbytes, out.data_ptr(), hidden, inner, n_out, top_k,
+                               tokens, act, W13.shape[0], _stream(X))
+    _lib.check(rc, entry[len("gguf_"):])
     return out
 
 
