@@ -237,10 +237,10 @@ int gguf_moe_weighted_sum(const void* Y, const float* topk_weights, void* out, i
  *      own the same features in the gate and the up half, apply the activation and write h as q8_1 rows into the
  *      workspace; the second's own a band of output features of one token, walk it in all top_k experts and form the
  *      weighted sum, so neither [tokens*top_k][2 I] nor [tokens*top_k][N_out] exists in memory.
- *   2  experts shared by a few pairs each (at most 16 per expert on average, formats with 16-slot tiles, E <= 256): five
- *      launches on the tile kernels -- quantize, one routing sort for both GEMMs, first GEMM with the activation and the
- *      quantisation of its result in the epilogue, second GEMM from those rows, weighted sum -- where the separate
- *      operators take seven.
+ *   2  experts shared by a few pairs each (at most 16 per expert on average, formats with 16-slot tiles, E <= 256): four
+ *      launches on the tile kernels -- one that quantizes X and sorts the routing for both GEMMs, first GEMM with the
+ *      activation and the quantisation of its result in the epilogue, second GEMM from those rows, weighted sum -- where
+ *      the separate operators take seven.
  *   0  not served (I no multiple of 32 or of type2's block, top_k times the waves a row of W2 takes beyond a workgroup,
  *      more than 65535 pairs, experts shared by more pairs than that): gguf_moe_vec_layer returns GGUF_ERR_SHAPE.
  * workspace: gguf_moe_vec_layer_workspace_bytes(...) bytes, layout private; GGUF_ERR_WORKSPACE if workspace_bytes is less
@@ -259,7 +259,7 @@ int gguf_moe_vec_layer(const void* X, int xdtype, const void* W13, int type13, c
  * out.mul_(topk_weights), ops.moe_sum: quantization/fused_moe.py:62-95; here gguf_moe_align_block_size with blocks of
  * 16 slots, gguf_moe_mmq_block, gguf_moe_mmq_block with act and gguf_moe_weighted_sum in sequence, whose result it
  * reproduces up to the last bit of the fp32 dot products), for layers with more than 64 tokens whose experts still see
- * at most 16 pairs each on average: the five launches of route 2 above where the separate operators take nine.  No
+ * at most 16 pairs each on average: the four launches of route 2 above where the separate operators take nine.  No
  * counterpart as one call in the reference.  gguf_moe_mmq_layer_takes: 1 where both formats have 16-slot tiles,
  * 0 < num_experts <= 256, tokens * top_k <= 16 num_experts (and <= 65535), I a multiple of 32 and of type2's block;
  * else 0, and gguf_moe_mmq_layer returns GGUF_ERR_SHAPE.  A pair whose expert id is outside [0, num_experts) adds

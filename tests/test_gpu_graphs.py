@@ -126,7 +126,7 @@ def test_two_launch_moe_layer_replays_match_eager():
         assert torch.equal(out, eager)
 
 
-def test_five_launch_moe_layer_replays_match_eager():
+def test_tile_route_moe_layer_replays_match_eager():
     """dispatch.fused_moe_gguf above 64 tokens with few pairs per expert (quantize, routing sort, both expert GEMMs on
     16-slot tiles and the weighted sum, all inside one call with a workspace allocated per call) captured and replayed
     with eager work in between; the routing changes between replays as well."""

@@ -580,7 +580,7 @@ def test_moe_layer_in_two_launches_matches_the_separate_steps(qtype, dt):
 @pytest.mark.parametrize("dt", ["f32", "f16", "bf16"])
 @pytest.mark.parametrize("qtype", [o.Q4_0, o.Q8_0, o.Q3_K, o.Q4_K, o.Q5_K, o.Q6_K, o.IQ4_XS, o.IQ2_XXS])
 def test_moe_layer_on_tiles_matches_the_separate_steps(qtype, dt):
-    """moe_vec_layer where a few pairs share each expert: quantize, one routing sort, first GEMM on 16-slot tiles with
+    """moe_vec_layer where a few pairs share each expert: quantize and one routing sort, first GEMM on 16-slot tiles with
     the activation and the q8_1 quantisation in its epilogue, second GEMM from those rows, weighted sum -- against the
     per-pair operator called twice and moe_weighted_sum (which take the same tile kernels with a sort and a quantize
     launch more each).  Inner sizes that end inside a 128-column tile, an expert without pairs, a second format."""
@@ -612,7 +612,7 @@ def test_moe_layer_on_tiles_matches_the_separate_steps(qtype, dt):
 @pytest.mark.parametrize("dt", ["f32", "f16", "bf16"])
 @pytest.mark.parametrize("qtype", [o.Q4_0, o.Q8_0, o.Q3_K, o.Q4_K, o.Q5_K, o.Q6_K, o.IQ4_XS, o.IQ2_XXS])
 def test_moe_layer_on_grouped_tiles_matches_the_separate_steps(qtype, dt):
-    """moe_mmq_layer (the five launches of the tile route with the grouped operator's arithmetic) against
+    """moe_mmq_layer (the four launches of the tile route with the grouped operator's arithmetic) against
     moe_align_block_size on blocks of 16, ggml_moe_a8 twice (the second with the activation) and moe_weighted_sum.
     More than 64 tokens, inner sizes that end inside a 128-column tile, an expert without pairs, a second format, and a
     pair whose expert id names no expert (it adds nothing in both)."""

@@ -199,7 +199,8 @@ __device__ __forceinline__ T finish(float v, const T* bias, int64_t n) {
 // From how many pairs on the per-pair MoE operator sorts its pairs by expert and reads a shared expert once per group
 // of them: two pairs per expert on average.  While all the experts together fit the last-level cache the per-pair
 // kernel, which has no sort and no second launch, reads shared experts from there and stays ahead a little longer
-// (Q4_0, 64 experts [2048,2048] top-8: 65 against 95 us at 16 tokens, 91 against 96 at 20, 101 against 95 at 24).
+// (Q4_0, 64 experts [2048,2048] top-8: 65 against 95 us at 16 tokens, 91 against 96 at 20, 101 against 95 at 24;
+// the whole layer on the tile kernels takes 85 us from there on).
 static inline bool moe_share_pays(int64_t pairs, int64_t num_experts, int64_t expert_bytes) {
   const bool cached = num_experts * expert_bytes <= (192ll << 20);
   return cached ? 2 * pairs >= 5 * num_experts : pairs >= 2 * num_experts;

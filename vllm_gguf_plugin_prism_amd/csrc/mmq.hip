@@ -572,9 +572,9 @@ int moe_vec_tiles(const void* X, int xdtype, void* workspace, const void* W, con
   return GGUF_ERR_TYPE;
 }
 
-// ---- A MoE layer on the tile kernels for experts shared by a few pairs each (blocks of 16 slots): quantize X, sort the
-// pairs once, first expert GEMM with the gated activation and the quantisation of its result in the epilogue, second
-// expert GEMM straight from those rows, weighted sum -- five launches where the separate operators take seven
+// ---- A MoE layer on the tile kernels for experts shared by a few pairs each (blocks of 16 slots): quantize X and sort
+// the pairs once (one launch), first expert GEMM with the gated activation and the quantisation of its result in the epilogue, second
+// expert GEMM straight from those rows, weighted sum -- four launches where the separate operators take seven
 // (quantize, sort, GEMM, quantize with the activation, sort, GEMM, sum).  The arithmetic is the per-pair operator's on
 // both GEMMs (offset sums of the GEMV for Q4_K / Q5_K), every intermediate rounded where the separate steps store it.
 int moe_tiles16_gate(const void* W, const void* ws, void* q8h, int dtype, int type, int inner, int K, int num_sorted, const MoeArgs& moe,
@@ -597,6 +597,9 @@ int64_t moe_tiles_layer_workspace(int64_t tokens, int64_t top_k, int64_t H, int6
   return up16(tokens * q8_row_bytes(H)) + up16(pairs * q8_row_bytes(I)) + up16(pairs * N_out * elt) + (sorted_cap + sorted_cap / 16 + 2) * 4;
 }
 
+int moe_prepare(const void* X, int xdtype, void* q8x, int tokens, int K, const int32_t* topk_ids, int numel, int num_experts, int block,
+                int32_t* sorted_ids, int sorted_capacity, int32_t* expert_ids, int expert_capacity, int32_t* num_post_padded,
+                hipStream_t s);   // moe_aux.hip
 int moe_weighted_sum_live(const void* Y, const float* topk_weights, const int32_t* topk_ids, int num_experts, void* out, int dtype,
                           int64_t tokens, int64_t top_k, int64_t N, hipStream_t s);   // moe_aux.hip
 
@@ -611,9 +614,13 @@ int moe_tiles_layer(const void* X, int xdtype, void* workspace, const void* W13,
   int32_t* sorted = (int32_t*)(y2 + up16((int64_t)pairs * N_out * elt));
   int32_t* experts = sorted + sorted_cap;
   int32_t* post = experts + block_cap;
-  int rc = quantize_q8_1(X, xdtype, q8x, tokens, H, s);
-  if (rc != GGUF_OK) return rc;
-  rc = gguf_moe_align_block_size(topk_ids, pairs, num_experts, 16, sorted, sorted_cap, experts, block_cap, post, (gguf_stream_t)s);
+  // the rows of X quantized and the routing sorted in one launch (two where the sort's histogram rows outgrow 64 KB of LDS)
+  int rc = moe_prepare(X, xdtype, q8x, tokens, H, topk_ids, pairs, num_experts, 16, sorted, (int)sorted_cap, experts, (int)block_cap, post, s);
+  if (rc == GGUF_NOT_TAKEN) {
+    rc = quantize_q8_1(X, xdtype, q8x, tokens, H, s);
+    if (rc != GGUF_OK) return rc;
+    rc = gguf_moe_align_block_size(topk_ids, pairs, num_experts, 16, sorted, sorted_cap, experts, block_cap, post, (gguf_stream_t)s);
+  }
   if (rc != GGUF_OK) return rc;
   const int ns = (int)(sorted_cap / 16 * 16);
   // vec_sums: the offset term of Q4_K / Q5_K as the per-pair operator forms it; else as the grouped operator does

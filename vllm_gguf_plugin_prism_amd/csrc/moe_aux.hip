@@ -3,7 +3,7 @@
 //
 // The reference takes both from vLLM (quantization/fused_moe.py:53-66: moe_align_block_size;
 // :87-95: out.mul_(topk_weights) then ops.moe_sum); they are not part of its own native code.
-#include "gguf_common.h"
+#include "q8_1_device.h"
 
 namespace gguf {
 
@@ -22,12 +22,10 @@ constexpr int ALIGN_MAX_EXPERTS = 1024;
 // walks the stretch again 64 pairs at a time, places every pair at its row's cursor plus the number of lanes below it
 // with the same expert, and moves the cursor on.  The lanes that share an expert are found with one ballot per bit
 // of the expert id.  A wave's LDS operations complete in order, so its row needs no barrier inside a pass.
-__global__ __launch_bounds__(ALIGN_THREADS) void moe_align_kernel(const int32_t* __restrict__ topk_ids, int numel,
-                                                                  int num_experts, int block,
-                                                                  int32_t* __restrict__ sorted_ids, int sorted_capacity,
-                                                                  int32_t* __restrict__ expert_ids, int expert_capacity,
-                                                                  int32_t* __restrict__ num_post_padded) {
-  extern __shared__ int lds[];
+__device__ __forceinline__ void moe_align_body(const int32_t* __restrict__ topk_ids, int numel, int num_experts, int block,
+                                               int32_t* __restrict__ sorted_ids, int sorted_capacity,
+                                               int32_t* __restrict__ expert_ids, int expert_capacity,
+                                               int32_t* __restrict__ num_post_padded, int* lds) {
   int* start = lds;                          // [E] pairs of the expert, then the first slot of its run
   int* cursor = lds + num_experts;           // [ALIGN_WAVES][E] per-wave counts, then per-wave cursors
   __shared__ int total_padded;
@@ -102,6 +100,36 @@ __global__ __launch_bounds__(ALIGN_THREADS) void moe_align_kernel(const int32_t*
   }
 }
 
+__global__ __launch_bounds__(ALIGN_THREADS) void moe_align_kernel(const int32_t* __restrict__ topk_ids, int numel,
+                                                                  int num_experts, int block,
+                                                                  int32_t* __restrict__ sorted_ids, int sorted_capacity,
+                                                                  int32_t* __restrict__ expert_ids, int expert_capacity,
+                                                                  int32_t* __restrict__ num_post_padded) {
+  extern __shared__ int lds[];
+  moe_align_body(topk_ids, numel, num_experts, block, sorted_ids, sorted_capacity, expert_ids, expert_capacity, num_post_padded, lds);
+}
+
+// The two preparations of a MoE layer on tiles in one launch: workgroup 0 sorts the routing, the others quantize the
+// rows of X (1024 threads, eight values each: 8192 values of the padded rows per workgroup, rows in turn).
+template <typename T>
+__global__ __launch_bounds__(ALIGN_THREADS) void moe_prepare_kernel(const T* __restrict__ x, char* __restrict__ ws, int K, int Kp,
+                                                                    int64_t row_bytes, int tokens, const int32_t* __restrict__ topk_ids,
+                                                                    int numel, int num_experts, int block,
+                                                                    int32_t* __restrict__ sorted_ids, int sorted_capacity,
+                                                                    int32_t* __restrict__ expert_ids, int expert_capacity,
+                                                                    int32_t* __restrict__ num_post_padded) {
+  extern __shared__ int lds[];
+  if (blockIdx.x == 0) {
+    moe_align_body(topk_ids, numel, num_experts, block, sorted_ids, sorted_capacity, expert_ids, expert_capacity, num_post_padded, lds);
+    return;
+  }
+  const int per_row = Kp / 8;                                   // threads a row takes
+  const int64_t g = (int64_t)(blockIdx.x - 1) * ALIGN_THREADS + threadIdx.x;
+  const int64_t m = g / per_row;
+  if (m >= tokens) return;                                      // (per_row is a multiple of 64: whole waves leave)
+  q8_1_quantize_thread<T>(x, ws, K, Kp, row_bytes, ACT_NONE, m, (int)(g % per_row), nullptr);
+}
+
 // out[t, n] = sum_k  T( float(Y[t, k, n]) * w[t, k] )   accumulated in fp32 in the order k = 0 .. top_k-1 and rounded
 // once: the in-place multiply by the routing weights followed by the sum over the top-k axis.
 template <typename T>
@@ -131,6 +159,21 @@ int moe_weighted_sum_live(const void* Y, const float* topk_weights, const int32_
                                                   (scalar_t*)out + t0 * N, (int)top_k, N, topk_ids ? topk_ids + t0 * top_k : nullptr,
                                                   num_experts));
   }
+  return launch_status();
+}
+
+// quantize_q8_1(X) and gguf_moe_align_block_size(topk_ids) in one launch (sizes checked by the caller)
+int moe_prepare(const void* X, int xdtype, void* q8x, int tokens, int K, const int32_t* topk_ids, int numel, int num_experts, int block,
+                int32_t* sorted_ids, int sorted_capacity, int32_t* expert_ids, int expert_capacity, int32_t* num_post_padded,
+                hipStream_t s) {
+  const int Kp = (int)q8_kp(K);
+  const size_t lds = (size_t)(1 + ALIGN_WAVES) * num_experts * sizeof(int);
+  if (lds > 65536) return GGUF_NOT_TAKEN;
+  const int64_t threads = (int64_t)tokens * (Kp / 8);
+  const unsigned grid = 1 + (unsigned)((threads + ALIGN_THREADS - 1) / ALIGN_THREADS);
+  GGUF_DISPATCH_DTYPE(xdtype, hipLaunchKernelGGL(moe_prepare_kernel<scalar_t>, dim3(grid), dim3(ALIGN_THREADS), lds, s, (const scalar_t*)X,
+                                                 (char*)q8x, K, Kp, q8_row_bytes(K), tokens, topk_ids, numel, num_experts, block, sorted_ids,
+                                                 sorted_capacity, expert_ids, expert_capacity, num_post_padded));
   return launch_status();
 }
 

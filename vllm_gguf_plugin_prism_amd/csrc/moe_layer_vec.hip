@@ -19,7 +19,7 @@
 // sums (ascending in K), the same quantizer and activation routines, every intermediate rounded where those steps store it.
 //
 // Where experts are shared by a few pairs each (the per-pair operator's tile route on blocks of 16 slots) the same entry
-// point runs the layer in five launches on the tile kernels instead (mmq.hip, moe_tiles_layer).
+// point runs the layer in four launches on the tile kernels instead (mmq.hip, moe_tiles_layer).
 #include "mmvq_core.h"
 
 namespace gguf {
@@ -387,7 +387,7 @@ static int moe_sum_fmt(int dtype, const void* W, const void* ws, const int32_t* 
   CASE(T_IQ2_XXS, FmtIQ2_XXS) CASE(T_IQ2_XS, FmtIQ2_XS) CASE(T_IQ2_S, FmtIQ2_S) CASE(T_IQ3_XXS, FmtIQ3_XXS) CASE(T_IQ3_S, FmtIQ3_S) \
   CASE(T_IQ1_S, FmtIQ1_S) CASE(T_IQ1_M, FmtIQ1_M)
 
-// 0: not served; 1: the two launches above; 2: five launches on the tile kernels (experts shared by a few pairs each)
+// 0: not served; 1: the two launches above; 2: four launches on the tile kernels (experts shared by a few pairs each)
 static int moe_layer_takes(int type13, int type2, int H, int I, int N_out, int top_k, int tokens, int num_experts) {
   const int qk13 = block_elems(type13), qk2 = block_elems(type2);
   if (qk13 == 0 || qk2 == 0 || H % qk13 != 0 || I % qk2 != 0 || I % 32 != 0) return 0;
@@ -470,7 +470,7 @@ extern "C" int gguf_moe_vec_layer(const void* X, int xdtype, const void* W13, in
   return GGUF_ERR_TYPE;
 }
 
-// The same five launches with the grouped operator's arithmetic (gguf_moe_mmq_block on blocks of 16 slots, twice, and the
+// The same four launches with the grouped operator's arithmetic (gguf_moe_mmq_block on blocks of 16 slots, twice, and the
 // weighted sum): what a layer with more than 64 tokens takes while its experts still see at most 16 pairs each on average.
 extern "C" int gguf_moe_mmq_layer_takes(int type13, int type2, int64_t H, int64_t I, int64_t N_out, int64_t top_k, int64_t tokens,
                                         int64_t num_experts) {

@@ -289,6 +289,30 @@ __global__ __launch_bounds__(64 * NW, OCC) void moe16_kernel(const uint8_t* __re
   }
 }
 
+// Three workgroups of the MoE tile kernel fit a CU.  When the blocks that hold pairs make a little more than one round
+// of those (how many there are is known on the device only: the estimate takes the pairs as spread over the experts at
+// random), the second round's few workgroups land three to a CU where the first finished first and take as long as the
+// first round; with two per CU the same tiles make two full rounds, which is shorter: Q4_0, 64 experts [2048,2048], 32
+// tokens top-8, 62 blocks of 64: 63 -> 55 us (the gated first GEMM of the layer 60 -> 51 us); 70 blocks the other way
+// round, 64 against 71 us.  A larger LDS request is what limits a CU to two: the bytes to ask for.
+static inline size_t moe16_lds_request(size_t lds, int num_sorted, int num_pairs, int tiles_n) {
+  const double experts = (double)(num_sorted - num_pairs) / 15.0;   // the sorted array has room for 15 padding slots per expert
+  if (experts < 1.0) return lds;
+  const double lam = (double)num_pairs / experts;
+  double blocks = 0.0, term = exp(-lam), cdf = 0.0, one_block = 0.0;   // sum over j >= 0 of P(pairs of an expert > 16 j)
+  for (int c = 0; c <= 64; ++c) {
+    cdf += term;
+    if (c % 16 == 0) blocks += 1.0 - cdf;
+    if (c == 16) one_block = cdf - exp(-lam);          // P(1 .. 16 pairs): the expert has exactly one block
+    term *= lam / (c + 1);
+  }
+  const double est = blocks * experts * tiles_n, cus = (double)num_cus();
+  // (exactly four tiles per CU is the one case in which three per CU do finish as three and one: 53 us above, and
+  //  the layer's second GEMM 28 against 31 us -- kept when every expert is likely to have exactly one block)
+  const bool four_each = (int)(experts + 0.5) * tiles_n == 4 * (int)cus && pow(one_block, experts) >= 0.8;
+  return est > 3.0 * cus && est <= 4.0 * cus && !four_each && lds < 54 * 1024 ? (size_t)54 * 1024 : lds;
+}
+
 template <class F, typename T>
 static int moe16_typed(const void* W, const void* ws, void* Y, int N, int K, int num_sorted, const MoeArgs& moe, hipStream_t stream) {
   // four waves, three workgroups per CU (two for Q5_K, whose packed block needs the registers); eight waves with one
@@ -303,31 +327,7 @@ static int moe16_typed(const void* W, const void* ws, void* Y, int N, int K, int
   }
   const int tiles_n = (N + N_T - 1) / N_T, tiles_m = num_sorted / 16, tiles = tiles_m * tiles_n;
   if (tiles == 0) return GGUF_OK;
-  // Three workgroups fit a CU.  When the blocks that hold pairs make a little more than one round of those (how many
-  // there are is known on the device only: the estimate takes the pairs as spread over the experts at random), the
-  // second round's few workgroups land three to a CU where the first finished first and take as long as the first
-  // round; with two per CU the same tiles make two full rounds, which is shorter: Q4_0, 64 experts [2048,2048], 32
-  // tokens top-8, 62 blocks of 64: 63 -> 55 us; 70 blocks the other way round, 64 against 71 us.  A larger LDS request
-  // is what limits a CU to two.
-  size_t lds_req = lds;
-  if (OCC == 3) {
-    const double experts = (double)(num_sorted - moe.num_pairs) / 15.0;   // the sorted array has room for 15 padding slots per expert
-    if (experts >= 1.0) {
-      const double lam = (double)moe.num_pairs / experts;
-      double blocks = 0.0, term = exp(-lam), cdf = 0.0, one_block = 0.0;   // sum over j >= 0 of P(pairs of an expert > 16 j)
-      for (int c = 0; c <= 64; ++c) {
-        cdf += term;
-        if (c % 16 == 0) blocks += 1.0 - cdf;
-        if (c == 16) one_block = cdf - exp(-lam);          // P(1 .. 16 pairs): the expert has exactly one block
-        term *= lam / (c + 1);
-      }
-      const double est = blocks * experts * tiles_n, cus = (double)num_cus();
-      // (exactly four tiles per CU is the one case in which three per CU do finish as three and one: 53 us above, and
-      //  the layer's second GEMM 28 against 31 us -- kept when every expert is likely to have exactly one block)
-      const bool four_each = (int)(experts + 0.5) * tiles_n == 4 * (int)cus && pow(one_block, experts) >= 0.8;
-      if (est > 3.0 * cus && est <= 4.0 * cus && !four_each && lds < 54 * 1024) lds_req = 54 * 1024;
-    }
-  }
+  const size_t lds_req = OCC == 3 ? moe16_lds_request(lds, num_sorted, moe.num_pairs, tiles_n) : lds;
   hipLaunchKernelGGL(kern, dim3(tiles), dim3(64 * NW), lds_req, stream, (const uint8_t*)W, (const char*)ws, q8_row_bytes(K), (T*)Y, N, K,
                      (int)q8_kp(K), tiles_m, tiles, moe, Dense16{}, (const T*)nullptr, Gate16{});
   return launch_status();
@@ -349,7 +349,8 @@ static int moe16_gate_typed(const void* W, const void* ws, void* q8h, int inner,
   }
   const int tiles_n = (inner + N_T / 2 - 1) / (N_T / 2), tiles_m = num_sorted / 16, tiles = tiles_m * tiles_n;
   if (tiles == 0) return GGUF_OK;
-  hipLaunchKernelGGL(kern, dim3(tiles), dim3(64 * NW), lds, stream, (const uint8_t*)W, (const char*)ws, q8_row_bytes(K), (T*)nullptr, 2 * inner, K,
+  const size_t lds_req = OCC == 3 ? moe16_lds_request(lds, num_sorted, moe.num_pairs, tiles_n) : lds;
+  hipLaunchKernelGGL(kern, dim3(tiles), dim3(64 * NW), lds_req, stream, (const uint8_t*)W, (const char*)ws, q8_row_bytes(K), (T*)nullptr, 2 * inner, K,
                      (int)q8_kp(K), tiles_m, tiles, moe, Dense16{}, (const T*)nullptr,
                      Gate16{(char*)q8h, q8_row_bytes(inner), inner, (int)q8_kp(inner), act});
   return launch_status();

@@ -19,38 +19,7 @@ __global__ __launch_bounds__(256) void quantize_q8_1_kernel(const T* __restrict_
                                                            _Float16* __restrict__ xh) {
   const int t = blockIdx.x * 256 + threadIdx.x;  // one thread per 8 values of the padded row
   if (t * 8 >= Kp) return;
-  const int64_t m = blockIdx.y;
-  const int e0 = t * 8;
-  float v[8];
-  if (e0 < K) {
-    if (act == ACT_NONE) load8<T>(x + m * (int64_t)K + e0, v);
-    else load8_gated<T>(x + m * (int64_t)(2 * K) + e0, x + m * (int64_t)(2 * K) + K + e0, act, v);  // rows are [gate | up]
-  } else {
-#pragma unroll
-    for (int i = 0; i < 8; ++i) v[i] = 0.0f;
-  }
-  const Q8Quad r = q8_1_quantize8(v);
-  char* row = ws + m * row_bytes;
-  *(uint2*)(row + e0) = r.q;
-  if (xh) {
-    // the dequantized row in half precision for the half-MFMA GEMM: RN16(d * q), d being the half-rounded scale.
-    // d * q is exact in fp32; magnitudes past the half range saturate (only reachable from bf16 / fp32 inputs).
-    union { _Float16 h[8]; uint4 v; } o;
-#pragma unroll
-    for (int i = 0; i < 8; ++i) {
-      const int q = (int)(int8_t)((i < 4 ? r.q.x >> (8 * i) : r.q.y >> (8 * (i - 4))) & 0xFF);
-      o.h[i] = (_Float16)fminf(fmaxf(r.d * (float)q, -65504.0f), 65504.0f);
-    }
-    *(uint4*)(xh + m * (int64_t)(Kp + 128) + e0) = o.v;   // row pitch: q8_half_pitch
-  }
-  if ((t & 3) == 0) {
-    const int b = t >> 2;
-    const int nb = Kp / 32;
-    float* fd = (float*)(row + Kp);
-    fd[b] = r.d;
-    fd[nb + b] = r.s;
-    fd[2 * nb + b] = r.du;
-  }
+  q8_1_quantize_thread<T>(x, ws, K, Kp, row_bytes, act, blockIdx.y, t, xh);
 }
 
 __global__ void q8_1_unpack_kernel(const char* __restrict__ ws, int8_t* __restrict__ q, float* __restrict__ ds, int Kp,

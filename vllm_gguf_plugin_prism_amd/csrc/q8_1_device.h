@@ -166,4 +166,45 @@ __device__ __forceinline__ Q8Quad q8_1_quantize8(const float (&v)[8]) {
   return r;
 }
 
+// One thread of the row quantizer: the eight values [8 t, 8 t + 8) of padded row m -> eight quants, and from the first
+// lane of each quad the block's d, s and d * sum(q) planes.  The four lanes of a quad must run together (the block's
+// amax and sum cross them).  act: rows of x are [gate | up] and the gated activation is quantized; xh: also the
+// dequantized row in half precision.
+template <typename T>
+__device__ __forceinline__ void q8_1_quantize_thread(const T* __restrict__ x, char* __restrict__ ws, int K, int Kp, int64_t row_bytes, int act,
+                                                     int64_t m, int t, _Float16* __restrict__ xh) {
+  const int e0 = t * 8;
+  float v[8];
+  if (e0 < K) {
+    if (act == ACT_NONE) load8<T>(x + m * (int64_t)K + e0, v);
+    else load8_gated<T>(x + m * (int64_t)(2 * K) + e0, x + m * (int64_t)(2 * K) + K + e0, act, v);  // rows are [gate | up]
+  } else {
+#pragma unroll
+    for (int i = 0; i < 8; ++i) v[i] = 0.0f;
+  }
+  const Q8Quad r = q8_1_quantize8(v);
+  char* row = ws + m * row_bytes;
+  *(uint2*)(row + e0) = r.q;
+  if (xh) {
+    // the dequantized row in half precision for the half-MFMA GEMM: RN16(d * q), d being the half-rounded scale.
+    // d * q is exact in fp32; magnitudes past the half range saturate (only reachable from bf16 / fp32 inputs).
+    union { _Float16 h[8]; uint4 v; } o;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+      const int q = (int)(int8_t)((i < 4 ? r.q.x >> (8 * i) : r.q.y >> (8 * (i - 4))) & 0xFF);
+      o.h[i] = (_Float16)fminf(fmaxf(r.d * (float)q, -65504.0f), 65504.0f);
+    }
+    *(uint4*)(xh + m * (int64_t)(Kp + 128) + e0) = o.v;   // row pitch: q8_half_pitch
+  }
+  if ((t & 3) == 0) {
+    const int b = t >> 2;
+    const int nb = Kp / 32;
+    float* fd = (float*)(row + Kp);
+    fd[b] = r.d;
+    fd[nb + b] = r.s;
+    fd[2 * nb + b] = r.du;
+  }
+}
+
+
 }  // namespace gguf

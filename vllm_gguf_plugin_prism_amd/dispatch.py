@@ -192,7 +192,7 @@ def fused_moe_gguf(x, w1, w2, topk_weights, topk_ids, weight_type: int, weight_t
         experts, rows, _ = w1.shape
         if activation in ("silu", "gelu") and w2.shape[0] == experts and ops.moe_mmq_layer_takes(
                 weight_type, weight_type2, x.shape[1], rows // 2, w2.shape[1], top_k, tokens, experts):
-            # experts that see at most 16 pairs each: the layer in one call of five launches on 16-slot tiles (one sort for
+            # experts that see at most 16 pairs each: the layer in one call of four launches on 16-slot tiles (one sort for
             # both GEMMs, the activation and the quantisation of its result in the first one's epilogue)
             return ops.moe_mmq_layer(x, w1, w2, topk_weights, topk_ids, weight_type, weight_type2, activation, out_hidden)
         # the reference sorts with ggml_moe_get_block_size(type); here a layer whose experts see few pairs each (65 .. 128
@@ -211,7 +211,7 @@ def fused_moe_gguf(x, w1, w2, topk_weights, topk_ids, weight_type: int, weight_t
         if activation in ("silu", "gelu") and w1.shape[0] == w2.shape[0] and ops.moe_vec_layer_takes(
                 weight_type, weight_type2, x.shape[1], rows // 2, w2.shape[1], top_k, tokens, w1.shape[0]):
             # the layer in one call: two launches where nothing is shared between pairs (the activation in the first GEMV's
-            # epilogue, the routing weights and the sum over the top-k axis in the second's), five on the tile kernels where
+            # epilogue, the routing weights and the sum over the top-k axis in the second's), four on the tile kernels where
             # a few pairs share each expert (one routing sort, no separate activation-and-quantize launch)
             return ops.moe_vec_layer(x, w1, w2, topk_weights, topk_ids, weight_type, weight_type2, activation, out_hidden)
         out = ops.ggml_moe_a8_vec(x, w1, topk_ids, top_k, weight_type, rows, tokens)

@@ -342,7 +342,7 @@ def moe_align_block_size(topk_ids: torch.Tensor, block_size: int, num_experts: i
 def moe_vec_layer_takes(quant_type: int, quant_type2: int, hidden: int, inner: int, out_features: int, top_k: int, tokens: int,
                         num_experts: int) -> bool:
     """Whether :func:`moe_vec_layer` serves a layer of this shape: a few tokens whose experts are not shared (two
-    launches) or experts shared by at most 16 pairs each on average (five launches on the tile kernels)."""
+    launches) or experts shared by at most 16 pairs each on average (four launches on the tile kernels)."""
     return bool(_lib.lib().gguf_moe_vec_layer_takes(int(quant_type), int(quant_type2), int(hidden), int(inner), int(out_features),
                                                     int(top_k), int(tokens), int(num_experts)))
 
@@ -357,7 +357,7 @@ def moe_mmq_layer_takes(quant_type: int, quant_type2: int, hidden: int, inner: i
 
 def moe_mmq_layer(X, W13, W2, topk_weights, topk_ids, quant_type: int, quant_type2: int, activation: str,
                   output: torch.Tensor | None = None) -> torch.Tensor:
-    """The reference's MoE layer on its grouped operator (quantization/fused_moe.py:62-95) in one call of five launches:
+    """The reference's MoE layer on its grouped operator (quantization/fused_moe.py:62-95) in one call of four launches:
     one routing sort on blocks of 16 slots for both ``ggml_moe_a8`` GEMMs, ``act`` and the q8_1 quantisation of its
     result in the first one's epilogue, ``mul_`` by the routing weights and ``moe_sum`` -> ``[tokens, W2.shape[1]]``.
     Same roundings as those steps run one by one; raises ``ValueError`` for shapes :func:`moe_mmq_layer_takes` declines."""
@@ -378,7 +378,7 @@ def moe_vec_layer(
     """The reference's MoE layer on its per-pair operators (quantization/fused_moe.py:98-111) in one call:
     ``ggml_moe_a8_vec`` with ``act`` and the q8_1 quantisation of its result in the epilogue, then the second
     ``ggml_moe_a8_vec`` with ``mul_`` by the routing weights and ``moe_sum`` -> ``[tokens, W2.shape[1]]`` (two launches
-    where experts are not shared, five on the tile kernels where a few pairs share each).  Same roundings as those steps
+    where experts are not shared, four on the tile kernels where a few pairs share each).  Same roundings as those steps
     run one by one; raises ``ValueError`` for shapes :func:`moe_vec_layer_takes` declines."""
     return _moe_layer("gguf_moe_vec_layer", X, W13, W2, topk_weights, topk_ids, quant_type, quant_type2, activation, output)
 
