@@ -257,13 +257,16 @@ int gguf_moe_vec_layer(const void* X, int xdtype, const void* W13, int type13, c
 
 /* The same layer on the grouped operator's arithmetic (moe_align_block_size, ggml_moe_a8, act(), ggml_moe_a8,
  * out.mul_(topk_weights), ops.moe_sum: quantization/fused_moe.py:62-95; here gguf_moe_align_block_size with blocks of
- * 16 slots, gguf_moe_mmq_block, gguf_moe_mmq_block with act and gguf_moe_weighted_sum in sequence, whose result it
- * reproduces up to the last bit of the fp32 dot products), for layers with more than 64 tokens whose experts still see
- * at most 16 pairs each on average: the four launches of route 2 above where the separate operators take nine.  No
- * counterpart as one call in the reference.  gguf_moe_mmq_layer_takes: 1 where both formats have 16-slot tiles,
- * 0 < num_experts <= 256, tokens * top_k <= 16 num_experts (and <= 65535), I a multiple of 32 and of type2's block;
- * else 0, and gguf_moe_mmq_layer returns GGUF_ERR_SHAPE.  A pair whose expert id is outside [0, num_experts) adds
- * nothing, like the rows the grouped operator leaves at zero.  Workspace: gguf_moe_vec_layer_workspace_bytes(...). */
+ * 16 or 32 slots, gguf_moe_mmq_block, gguf_moe_mmq_block with act and gguf_moe_weighted_sum in sequence, whose result it
+ * reproduces up to the last bit of the fp32 dot products), for layers with more than 64 tokens: the four launches of
+ * route 2 above where the separate operators take nine (sort; zero-fill, quantize and GEMM twice; weighted sum).  No
+ * counterpart as one call in the reference.  gguf_moe_mmq_layer_takes:
+ *   1  blocks of 16 slots: both formats have such tiles and tokens * top_k <= 16 num_experts;
+ *   2  the reference's blocks of 32 slots: every other layer of two tile formats (the twelve of ggml_moe_a8);
+ *   0  not served (num_experts outside 1..256, I no multiple of 32 or of type2's block, a format without tiles, more
+ *      than about two million pairs): gguf_moe_mmq_layer returns GGUF_ERR_SHAPE.
+ * A pair whose expert id is outside [0, num_experts) adds nothing, like the rows the grouped operator leaves at zero.
+ * Workspace: gguf_moe_vec_layer_workspace_bytes(...), which covers both entry points and every route. */
 int gguf_moe_mmq_layer_takes(int type13, int type2, int64_t H, int64_t I, int64_t N_out, int64_t top_k, int64_t tokens,
                              int64_t num_experts);
 int gguf_moe_mmq_layer(const void* X, int xdtype, const void* W13, int type13, const void* W2, int type2,

@@ -160,14 +160,18 @@ def test_two_launch_moe_layer_states_which_shapes_it_serves():
     assert h.gguf_moe_vec_layer_takes(1, 2, 2048, 1024, 2048, 8, 1, 64) == 0
     assert h.gguf_moe_vec_layer_takes(2, 12, 2048, 1120, 2048, 8, 1, 64) == 0
     assert h.gguf_moe_vec_layer_workspace_bytes(3, 8, 2048, 1024, 2048, 64, 1) >= 24 * h.gguf_q8_1_row_bytes(1024) + 3 * h.gguf_q8_1_row_bytes(2048)
-    # the grouped operator's arithmetic: up to 16 pairs per expert on average, at most 256 experts, formats with 16-slot tiles
+    # the grouped operator's arithmetic: 1 = blocks of 16 slots (up to 16 pairs per expert on average, formats with such
+    # tiles), 2 = blocks of 32; at most 256 experts
     assert h.gguf_moe_mmq_layer_takes(2, 2, 2048, 1024, 2048, 8, 96, 64) == 1
     assert h.gguf_moe_mmq_layer_takes(2, 2, 2048, 1024, 2048, 8, 128, 64) == 1
-    assert h.gguf_moe_mmq_layer_takes(2, 2, 2048, 1024, 2048, 8, 129, 64) == 0
-    assert h.gguf_moe_mmq_layer_takes(3, 2, 2048, 1024, 2048, 8, 96, 64) == 0       # Q4_1: blocks of 32 only
+    assert h.gguf_moe_mmq_layer_takes(2, 2, 2048, 1024, 2048, 8, 129, 64) == 2
+    assert h.gguf_moe_mmq_layer_takes(2, 2, 2048, 1024, 2048, 8, 2048, 64) == 2
+    assert h.gguf_moe_mmq_layer_takes(3, 2, 2048, 1024, 2048, 8, 96, 64) == 2       # Q4_1: blocks of 32 only
+    assert h.gguf_moe_mmq_layer_takes(20, 2, 2048, 1024, 2048, 8, 96, 64) == 0      # IQ4_NL has no tile kernel
     assert h.gguf_moe_mmq_layer_takes(2, 2, 2048, 1024, 2048, 8, 96, 300) == 0
     assert h.gguf_moe_mmq_layer_takes(2, 2, 2048, 1024, 2048, 8, 96, 0) == 0
+    assert h.gguf_moe_mmq_layer_takes(2, 2, 2048, 1000, 2048, 8, 96, 64) == 0       # inner size not in whole blocks
     assert h.gguf_moe_mmq_layer(None, 1, None, 2, None, 2, None, None, None, 0, None, 2048, 1024, 2048, 8, 96, 1, 64, None) == -4
-    assert h.gguf_moe_mmq_layer(None, 1, None, 2, None, 2, None, None, None, 0, None, 2048, 1024, 2048, 8, 200, 1, 64, None) == -3
+    assert h.gguf_moe_mmq_layer(None, 1, None, 2, None, 2, None, None, None, 0, None, 2048, 1024, 2048, 8, 200, 1, 300, None) == -3
     assert h.gguf_moe_vec_layer(None, 1, None, 2, None, 2, None, None, None, 0, None, 2048, 1024, 2048, 8, 1, 0, 64, None) == -3
     assert h.gguf_moe_vec_layer(None, 1, None, 2, None, 2, None, None, None, 0, None, 2048, 1024, 2048, 8, 1, 1, 64, None) == -4

@@ -609,32 +609,42 @@ def test_moe_layer_on_tiles_matches_the_separate_steps(qtype, dt):
             assert err <= {"f32": 5e-4, "f16": 1e-3, "bf16": 4e-3}[dt], f"{o.TYPE_NAMES[qtype]} {o.TYPE_NAMES[qt2]} {dt} case {case} rel-L2 {err}"
 
 
+TILE16_TYPES = [o.Q4_0, o.Q8_0, o.Q3_K, o.Q4_K, o.Q5_K, o.Q6_K, o.IQ4_XS, o.IQ2_XXS]
+
+
 @pytest.mark.parametrize("dt", ["f32", "f16", "bf16"])
-@pytest.mark.parametrize("qtype", [o.Q4_0, o.Q8_0, o.Q3_K, o.Q4_K, o.Q5_K, o.Q6_K, o.IQ4_XS, o.IQ2_XXS])
+@pytest.mark.parametrize("qtype", MMQ_TYPES)
 def test_moe_layer_on_grouped_tiles_matches_the_separate_steps(qtype, dt):
     """moe_mmq_layer (the four launches of the tile route with the grouped operator's arithmetic) against
-    moe_align_block_size on blocks of 16, ggml_moe_a8 twice (the second with the activation) and moe_weighted_sum.
-    More than 64 tokens, inner sizes that end inside a 128-column tile, an expert without pairs, a second format, and a
-    pair whose expert id names no expert (it adds nothing in both)."""
+    moe_align_block_size, ggml_moe_a8 twice (the second with the activation) and moe_weighted_sum on the same block
+    size: blocks of 16 slots where the experts see few pairs and the format has such tiles, else the reference's blocks
+    of 32.  More than 64 tokens, inner sizes that end inside a tile of features, an expert without pairs, a second
+    format, and a pair whose expert id names no expert (it adds nothing in both)."""
     ops = _ops()
+    from vllm_gguf_plugin_prism_amd import _lib, dispatch
     rng = np.random.default_rng(2100 + qtype)
     qk = o.QUANT_SIZES[qtype][0]
     other = o.Q8_0 if qtype != o.Q8_0 else o.Q4_0
-    for case, (t, top_k, e, hid, inner) in enumerate([(70, 2, 12, 512, 768), (24, 4, 8, 256, 1280 if qk == 32 else 1024)]):
-        for qt2 in (qtype, other) if case == 0 else (qtype,):
+    cases = [(70, 2, 12, 512, 768, 16), (24, 4, 8, 256, 1280 if qk == 32 else 1024, 16),
+             (70, 4, 8, 512, 768, 32), (40, 2, 3, 256, 1312 if qk == 32 else 1280, 32)]
+    for case, (t, top_k, e, hid, inner, block) in enumerate(cases):
+        if block == 16 and qtype not in TILE16_TYPES:
+            continue
+        for qt2 in (qtype, other) if case in (0, 2) else (qtype,):
             w13 = np.stack([o.make_weights(rng, qtype, 2 * inner, hid) for _ in range(e)])
             w2 = np.stack([o.make_weights(rng, qt2, hid, inner) for _ in range(e)])
             w13d, w2d = _dev(w13), _dev(w2)
             ids, wts = _routing(rng, t, e - 1, top_k)            # the last expert has no pairs
-            if case == 1:
+            if case % 2 == 1:
                 ids[5, 1] = e + 3
             pairs = t * top_k
-            assert ops.moe_mmq_layer_takes(qtype, qt2, hid, inner, hid, top_k, t, e)
-            sorted_ids, expert_ids, post = ops.moe_align_block_size(_dev(ids), 16, e)
+            route = _lib.lib().gguf_moe_mmq_layer_takes(int(qtype), int(qt2), hid, inner, hid, top_k, t, e)
+            assert route == (1 if block == 16 else 2), (case, route)
+            sorted_ids, expert_ids, post = ops.moe_align_block_size(_dev(ids), block, e)
 
             def separate(x):
-                h = ops.ggml_moe_a8(x, w13d, sorted_ids, expert_ids, post, qtype, 2 * inner, top_k, t, block_size=16)
-                y = ops.ggml_moe_a8(h, w2d, sorted_ids, expert_ids, post, qt2, hid, 1, pairs, activation="silu", block_size=16)
+                h = ops.ggml_moe_a8(x, w13d, sorted_ids, expert_ids, post, qtype, 2 * inner, top_k, t, block_size=block)
+                y = ops.ggml_moe_a8(h, w2d, sorted_ids, expert_ids, post, qt2, hid, 1, pairs, activation="silu", block_size=block)
                 want = torch.empty((t, hid), dtype=x.dtype, device="cuda")
                 ops.moe_weighted_sum(y.reshape(t, top_k, hid), _dev(wts), want)
                 return h, want
@@ -648,15 +658,13 @@ def test_moe_layer_on_grouped_tiles_matches_the_separate_steps(qtype, dt):
             #  differently in the two kernels)
             err = o.rel_l2(got.float().cpu().numpy(), want.float().cpu().numpy())
             assert err <= {"f32": 5e-4, "f16": 1e-3, "bf16": 4e-3}[dt], f"{o.TYPE_NAMES[qtype]} {o.TYPE_NAMES[qt2]} {dt} case {case} rel-L2 {err}"
-            # the layer through the dispatcher takes the same call
-            if t > 64:
-                from vllm_gguf_plugin_prism_amd import dispatch
+            if t > 64:   # the layer through the dispatcher takes the same call
                 assert torch.equal(dispatch.fused_moe_gguf(x, w13d, w2d, _dev(wts), _dev(ids), qtype, qt2, "silu"), got)
-    with pytest.raises(ValueError):     # 25 pairs per expert: blocks of 32, left to the separate operators
-        ops.moe_mmq_layer(torch.zeros(200, 2048, device="cuda", dtype=TORCH_DT[dt]),
-                          _dev(np.zeros((64, 2048, 2048 // qk * o.QUANT_SIZES[qtype][1]), dtype=np.uint8)),
-                          _dev(np.zeros((64, 2048, 1024 // qk * o.QUANT_SIZES[qtype][1]), dtype=np.uint8)),
-                          _dev(np.ones((200, 8), dtype=np.float32)), _dev(np.zeros((200, 8), dtype=np.int32)), qtype, qtype, "silu")
+    with pytest.raises(ValueError):     # more experts than the tile kernels' guard on expert ids admits
+        row = 256 // qk * o.QUANT_SIZES[qtype][1]
+        ops.moe_mmq_layer(torch.zeros(70, 256, device="cuda", dtype=TORCH_DT[dt]), _dev(np.zeros((300, 512, row), dtype=np.uint8)),
+                          _dev(np.zeros((300, 256, row), dtype=np.uint8)), _dev(np.ones((70, 2), dtype=np.float32)),
+                          _dev(np.zeros((70, 2), dtype=np.int32)), qtype, qtype, "silu")
 
 
 def _lib_takes(ops, *args):

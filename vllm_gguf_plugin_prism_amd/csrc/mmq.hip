@@ -26,6 +26,7 @@
 // token rows are gathered through sorted_token_ids, the weight base moves to the block's
 // expert, and results scatter to the rows the slots name.
 #include "mmq_formats.h"
+#include "q8_1_device.h"
 
 namespace gguf {
 
@@ -145,10 +146,11 @@ __host__ __device__ constexpr size_t mmq_group_lds_bytes() {
 //                  are added through LDS at the end.  For shapes with too few output tiles to fill the chip.
 enum { MODE_PREFETCH = 0, MODE_PLAIN = 1, MODE_KSPLIT = 3 };
 
-template <class F, int WM, int WN, int TM, int TN, int KS, int OCC, int MODE, typename T, bool MOE>
+template <class F, int WM, int WN, int TM, int TN, int KS, int OCC, int MODE, typename T, bool MOE, bool GATE = false>
 __global__ __launch_bounds__(64 * WM * WN * (MODE == MODE_KSPLIT ? 2 : 1), OCC) void mmq_kernel(const uint8_t* __restrict__ W, const char* __restrict__ ws,
                                                          T* __restrict__ Y, int M, int N, int K, int64_t ws_row_bytes,
-                                                         MoeArgs moe, int64_t w_pitch, int64_t ldy, const T* __restrict__ bias) {
+                                                         MoeArgs moe, int64_t w_pitch, int64_t ldy, const T* __restrict__ bias, Gate16 gate) {
+  static_assert(!GATE || (MOE && TM == 1 && WM == 1 && MODE == MODE_PREFETCH), "the gated epilogue is the MoE tile's");
   constexpr int GW = WM * WN;            // waves that share one set of accumulators' tile
   constexpr int KW = MODE == MODE_KSPLIT ? 2 : 1;  // wave sets splitting the 32-blocks of a step
   constexpr int NT = 64 * GW * KW;       // threads that stage one tile: the whole workgroup
@@ -173,7 +175,7 @@ __global__ __launch_bounds__(64 * WM * WN * (MODE == MODE_KSPLIT ? 2 : 1), OCC) 
   const int wm = wave / WN, wn = wave % WN;
   constexpr int KB_MINE = (KS / 32) / KW;                            // 32-blocks of a step this wave contracts
   const int m_base = blockIdx.y * M_T;
-  const int n_base = blockIdx.x * N_T;
+  const int n_base = blockIdx.x * (GATE ? N_T / 2 : N_T);   // GATE: in features of one half (see Gate16)
   const int Kp = (int)q8_kp(K);
   const int64_t rowbytes = w_pitch;   // bytes between rows of W: the dense row size unless the caller's tensor is padded
   const int nkb_total = K >> 5;
@@ -226,7 +228,9 @@ __global__ __launch_bounds__(64 * WM * WN * (MODE == MODE_KSPLIT ? 2 : 1), OCC) 
 #pragma unroll
   for (int i = 0; i < WP; ++i) {
     const int p = tid + NT * i, n = min(p / KB, N_T - 1);
-    w_src[i] = W + (int64_t)min(n_base + n, N - 1) * rowbytes;
+    // GATE: the first half of the columns are features n_base .. of the gate half, the second the same features of up
+    const int row = GATE ? (n < N_T / 2 ? 0 : gate.inner) + min(n_base + (n & (N_T / 2 - 1)), gate.inner - 1) : min(n_base + n, N - 1);
+    w_src[i] = W + (int64_t)row * rowbytes;
   }
 
   uint4 r_aq[AQ];
@@ -442,6 +446,42 @@ __global__ __launch_bounds__(64 * WM * WN * (MODE == MODE_KSPLIT ? 2 : 1), OCC) 
     }
   }
 
+  if constexpr (GATE) {
+    // ---- the tile's sums, rounded as the operator stores them, meet in LDS (the staging area is free: the loop ends on
+    // a barrier); then eight features of a slot per thread, both halves, and every four threads form one q8_1 block
+    static_assert((size_t)M_T * N_T * 4 <= mmq_group_lds_bytes<F, WM, WN, TM, TN, KS>(), "the tile of sums fits the staging area");
+    float* yt = (float*)smem;   // [M_T][N_T]
+#pragma unroll
+    for (int r = 0; r < 16; ++r)
+#pragma unroll
+      for (int i = 0; i < TN; ++i)
+        yt[(8 * (r >> 2) + 4 * lhalf + (r & 3)) * N_T + 32 * (wn * TN + i) + lrow] = to_f32<T>(from_f32<T>(acc[0][i][r]));
+    __syncthreads();
+    constexpr int PARTS = N_T / 2 / 8;   // threads per slot (a multiple of 4: quads stay whole)
+    static_assert((M_T * PARTS) % NT == 0 && PARTS % 4 == 0, "every thread takes the same number of (slot, part) items");
+#pragma unroll
+    for (int it = 0; it < M_T * PARTS / NT; ++it) {
+      const int item = tid + NT * it, slot = item / PARTS, part = item % PARTS;
+      float xv[8];
+#pragma unroll
+      for (int i = 0; i < 8; ++i) xv[i] = gate1<T>(yt[slot * N_T + 8 * part + i], yt[slot * N_T + N_T / 2 + 8 * part + i], gate.act);
+      const Q8Quad qq = q8_1_quantize8(xv);
+      const int pair = moe.sorted_token_ids[m_base + slot];
+      const int f = n_base + 8 * part;
+      if (pair < moe.num_pairs && f < gate.inner) {     // (inner is a multiple of 32: blocks are whole)
+        char* row = gate.rows + (int64_t)pair * gate.row_bytes;
+        *(uint2*)(row + f) = qq.q;
+        if ((part & 3) == 0) {
+          float* fd = (float*)(row + gate.kp);
+          const int b = f >> 5, nbp = gate.kp >> 5;
+          fd[b] = qq.d;
+          fd[nbp + b] = qq.s;
+          fd[2 * nbp + b] = qq.du;
+        }
+      }
+    }
+    return;
+  }
   // ---- store: lane = one output feature, 16 token rows per tile
 #pragma unroll
   for (int j = 0; j < TM; ++j) {
@@ -468,21 +508,22 @@ __global__ __launch_bounds__(64 * WM * WN * (MODE == MODE_KSPLIT ? 2 : 1), OCC) 
 }
 
 
-template <class F, int WM, int WN, int TM, int TN, int KS, int OCC, int MODE, typename T, bool MOE>
+template <class F, int WM, int WN, int TM, int TN, int KS, int OCC, int MODE, typename T, bool MOE, bool GATE = false>
 static void launch_mmq(const void* W, const void* ws, void* Y, int M, int N, int K, int m_tiles, const MoeArgs& moe,
-                       hipStream_t stream, const LinearArgs& la = LinearArgs()) {
+                       hipStream_t stream, const LinearArgs& la = LinearArgs(), const Gate16& gate = Gate16{}) {
   constexpr int KW = MODE == MODE_KSPLIT ? 2 : 1;
   constexpr int N_T = 32 * WN * TN;
   constexpr size_t lds = mmq_group_lds_bytes<F, WM, WN, TM, TN, KS>();
   static_assert(mmq_group_lds_bytes<F, WM, WN, TM, TN, KS>() % 16 == 0, "group tiles keep 16-byte alignment");
-  auto kern = mmq_kernel<F, WM, WN, TM, TN, KS, OCC, MODE, T, MOE>;
+  auto kern = mmq_kernel<F, WM, WN, TM, TN, KS, OCC, MODE, T, MOE, GATE>;
   if constexpr (lds > 65536) {
     static std::atomic<uint64_t> done{0};
     allow_large_lds(kern, lds, done);
   }
-  hipLaunchKernelGGL(kern, dim3((N + N_T - 1) / N_T, m_tiles), dim3(64 * WM * WN * KW), lds, stream, (const uint8_t*)W, (const char*)ws,
+  const int n_tiles = GATE ? (gate.inner + N_T / 2 - 1) / (N_T / 2) : (N + N_T - 1) / N_T;
+  hipLaunchKernelGGL(kern, dim3(n_tiles, m_tiles), dim3(64 * WM * WN * KW), lds, stream, (const uint8_t*)W, (const char*)ws,
                      (T*)Y, M, N, K, q8_row_bytes(K), moe, la.w_pitch ? la.w_pitch : (int64_t)(K / F::QK) * F::BS,
-                     la.ldy ? la.ldy : (int64_t)N, (const T*)la.bias);
+                     la.ldy ? la.ldy : (int64_t)N, (const T*)la.bias, gate);
 }
 
 
@@ -501,11 +542,46 @@ static int moe_fmt(const void* W, const void* ws, void* Y, int dtype, int N, int
   return GGUF_ERR_DTYPE;
 }
 
+// The first expert GEMM of a layer on blocks of 32 slots with the gated activation and the q8_1 quantisation of its
+// result in the epilogue (see Gate16): W is [experts][2 inner][K packed], a tile is 32 slots x 128 features of both halves.
+template <class F>
+static int moe_gate_fmt(const void* W, const void* ws, void* q8h, int dtype, int inner, int K, int num_sorted, const MoeArgs& moe, int act,
+                        hipStream_t s) {
+  const Gate16 gate{(char*)q8h, q8_row_bytes(inner), inner, (int)q8_kp(inner), act};
+  GGUF_DISPATCH_DTYPE(dtype, (launch_mmq<F, 1, 4, 1, 2, 128, 2, MODE_PREFETCH, scalar_t, true, true>(W, ws, nullptr, 0, 2 * inner, K, num_sorted / 32,
+                                                                                                   moe, s, LinearArgs(), gate));
+                      return launch_status());
+  return GGUF_ERR_DTYPE;
+}
+
 // nbytes of zeros from p (16-byte aligned): whole 16-byte words, then the last thread past them clears the odd bytes
 __global__ void zero_rows_kernel(uint4* __restrict__ p, int64_t nbytes) {
   const int64_t i = (int64_t)blockIdx.x * 256 + threadIdx.x, n16 = nbytes >> 4;
   if (i < n16) p[i] = make_uint4(0, 0, 0, 0);
   else if (i == n16) for (int64_t b = n16 << 4; b < nbytes; ++b) ((uint8_t*)p)[b] = 0;
+}
+
+#define GGUF_MOE32_FORMATS(CASE) \
+  CASE(T_Q4_0, MQ4_0) CASE(T_Q4_1, MQ4_1) CASE(T_Q5_0, MQ5_0) CASE(T_Q5_1, MQ5_1) CASE(T_Q8_0, MQ8_0) CASE(T_Q2_K, MQ2_K) \
+  CASE(T_Q3_K, MQ3_K) CASE(T_Q4_K, MQ4_K) CASE(T_Q5_K, MQ5_K) CASE(T_Q6_K, MQ6_K) CASE(T_IQ4_XS, MIQ4_XS) CASE(T_IQ2_XXS, MIQ2_XXS)
+
+// the grouped contraction on blocks of 32 slots, and the gated first GEMM of a layer on them
+static int moe_tiles32(const void* W, const void* ws, void* Y, int dtype, int type, int N, int K, int num_sorted, const MoeArgs& moe, hipStream_t s) {
+  switch (type) {
+#define MOE32_CASE(ID, FMT) case ID: return moe_fmt<FMT>(W, ws, Y, dtype, N, K, num_sorted, moe, s);
+    GGUF_MOE32_FORMATS(MOE32_CASE)
+#undef MOE32_CASE
+  }
+  return GGUF_ERR_TYPE;
+}
+static int moe_tiles32_gate(const void* W, const void* ws, void* q8h, int dtype, int type, int inner, int K, int num_sorted, const MoeArgs& moe,
+                            int act, hipStream_t s) {
+  switch (type) {
+#define MOE32_CASE(ID, FMT) case ID: return moe_gate_fmt<FMT>(W, ws, q8h, dtype, inner, K, num_sorted, moe, act, s);
+    GGUF_MOE32_FORMATS(MOE32_CASE)
+#undef MOE32_CASE
+  }
+  return GGUF_ERR_TYPE;
 }
 
 static bool mmq_type_ok(int type) {
@@ -586,15 +662,18 @@ namespace gguf {
 
 static inline int64_t up16(int64_t v) { return (v + 15) / 16 * 16; }
 
-bool moe_tiles_layer_ok(int type13, int type2, int64_t pairs, int64_t num_experts, int64_t I) {
-  return moe_tiles16_ok(type13) && moe_tiles16_ok(type2) && type13 != T_Q5_0 && type2 != T_Q5_0 && num_experts > 0 && num_experts <= 256 &&
-         pairs <= 16 * num_experts && I % 32 == 0;
+// 16: both formats have 16-slot tiles and the experts see at most 16 pairs each on average; 32: the layer runs on blocks of
+// 32 slots (grouped arithmetic only: the per-pair operator's differs there for Q5_0); 0: not on the tile kernels
+int moe_tiles_layer_block(int type13, int type2, int64_t pairs, int64_t num_experts, int64_t I, bool vec_sums) {
+  if (num_experts <= 0 || num_experts > 256 || I % 32 != 0) return 0;
+  if (moe_tiles16_ok(type13) && moe_tiles16_ok(type2) && type13 != T_Q5_0 && type2 != T_Q5_0 && pairs <= 16 * num_experts) return 16;
+  return !vec_sums && mmq_type_ok(type13) && mmq_type_ok(type2) ? 32 : 0;
 }
 
 // [q8_1 rows of X][q8_1 rows of h][second GEMM's result, pairs x N_out][sorted ids, expert ids, padded total]
-int64_t moe_tiles_layer_workspace(int64_t tokens, int64_t top_k, int64_t H, int64_t I, int64_t N_out, int64_t num_experts, int elt) {
-  const int64_t pairs = tokens * top_k, sorted_cap = pairs + num_experts * 15;
-  return up16(tokens * q8_row_bytes(H)) + up16(pairs * q8_row_bytes(I)) + up16(pairs * N_out * elt) + (sorted_cap + sorted_cap / 16 + 2) * 4;
+int64_t moe_tiles_layer_workspace(int64_t tokens, int64_t top_k, int64_t H, int64_t I, int64_t N_out, int64_t num_experts, int elt, int block) {
+  const int64_t pairs = tokens * top_k, sorted_cap = pairs + num_experts * (block - 1);
+  return up16(tokens * q8_row_bytes(H)) + up16(pairs * q8_row_bytes(I)) + up16(pairs * N_out * elt) + (sorted_cap + sorted_cap / block + 2) * 4;
 }
 
 int moe_prepare(const void* X, int xdtype, void* q8x, int tokens, int K, const int32_t* topk_ids, int numel, int num_experts, int block,
@@ -605,32 +684,33 @@ int moe_weighted_sum_live(const void* Y, const float* topk_weights, const int32_
 
 int moe_tiles_layer(const void* X, int xdtype, void* workspace, const void* W13, int type13, const void* W2, int type2, const int32_t* topk_ids,
                     const float* topk_w, void* out, int H, int I, int N_out, int top_k, int tokens, int act, int num_experts, bool vec_sums,
-                    hipStream_t s) {
+                    int block, hipStream_t s) {
   const int pairs = tokens * top_k, elt = xdtype == GGUF_DTYPE_F32 ? 4 : 2;
   char* q8x = (char*)workspace;
   char* q8h = q8x + up16((int64_t)tokens * q8_row_bytes(H));
   char* y2 = q8h + up16((int64_t)pairs * q8_row_bytes(I));
-  const int64_t sorted_cap = (int64_t)pairs + (int64_t)num_experts * 15, block_cap = sorted_cap / 16 + 1;
+  const int64_t sorted_cap = (int64_t)pairs + (int64_t)num_experts * (block - 1), block_cap = sorted_cap / block + 1;
   int32_t* sorted = (int32_t*)(y2 + up16((int64_t)pairs * N_out * elt));
   int32_t* experts = sorted + sorted_cap;
   int32_t* post = experts + block_cap;
   // the rows of X quantized and the routing sorted in one launch (two where the sort's histogram rows outgrow 64 KB of LDS)
-  int rc = moe_prepare(X, xdtype, q8x, tokens, H, topk_ids, pairs, num_experts, 16, sorted, (int)sorted_cap, experts, (int)block_cap, post, s);
+  int rc = moe_prepare(X, xdtype, q8x, tokens, H, topk_ids, pairs, num_experts, block, sorted, (int)sorted_cap, experts, (int)block_cap, post, s);
   if (rc == GGUF_NOT_TAKEN) {
     rc = quantize_q8_1(X, xdtype, q8x, tokens, H, s);
     if (rc != GGUF_OK) return rc;
-    rc = gguf_moe_align_block_size(topk_ids, pairs, num_experts, 16, sorted, sorted_cap, experts, block_cap, post, (gguf_stream_t)s);
+    rc = gguf_moe_align_block_size(topk_ids, pairs, num_experts, block, sorted, sorted_cap, experts, block_cap, post, (gguf_stream_t)s);
   }
   if (rc != GGUF_OK) return rc;
-  const int ns = (int)(sorted_cap / 16 * 16);
+  const int ns = (int)(sorted_cap / block * block);
   // vec_sums: the offset term of Q4_K / Q5_K as the per-pair operator forms it; else as the grouped operator does
   const auto gemv_sums = [&](int type) { return vec_sums && (type == T_Q4_K || type == T_Q5_K) ? 1 : 0; };
   const MoeArgs m1 = {sorted, experts, post, (int64_t)2 * I * (H / block_elems(type13)) * block_bytes(type13), top_k, pairs, gemv_sums(type13)};
-  rc = moe_tiles16_gate(W13, q8x, q8h, xdtype, type13, I, H, ns, m1, act, s);
+  rc = block == 16 ? moe_tiles16_gate(W13, q8x, q8h, xdtype, type13, I, H, ns, m1, act, s)
+                   : moe_tiles32_gate(W13, q8x, q8h, xdtype, type13, I, H, ns, m1, act, s);
   if (rc != GGUF_OK) return rc == GGUF_NOT_TAKEN ? GGUF_ERR_TYPE : rc;
   // the second GEMM's rows are the pairs themselves: slot -> pair -> row pair of q8h
   const MoeArgs m2 = {sorted, experts, post, (int64_t)N_out * (I / block_elems(type2)) * block_bytes(type2), 1, pairs, gemv_sums(type2)};
-  rc = moe_tiles16(W2, q8h, y2, xdtype, type2, N_out, I, ns, m2, s);
+  rc = block == 16 ? moe_tiles16(W2, q8h, y2, xdtype, type2, N_out, I, ns, m2, s) : moe_tiles32(W2, q8h, y2, xdtype, type2, N_out, I, ns, m2, s);
   if (rc != GGUF_OK) return rc == GGUF_NOT_TAKEN ? GGUF_ERR_TYPE : rc;
   // the grouped operator leaves the rows of pairs whose expert id names no expert at zero (the sort drops them): the
   // sum takes them as zero instead of reading rows of y2 that nobody wrote
@@ -829,19 +909,5 @@ extern "C" int gguf_moe_mmq_block(const void* X, int xdtype, void* q8_workspace,
   const int ns = (int)(num_sorted / block * block);  // a trailing partial block is ignored, like the reference's integer division
   if (ns == 0) return launch_status();
   if (block == 16) return moe_tiles16(W, q8_workspace, Y, xdtype, type, (int)N, (int)K, ns, moe, s);
-  switch (type) {
-    case T_Q4_0: return moe_fmt<MQ4_0>(W, q8_workspace, Y, xdtype, (int)N, (int)K, ns, moe, s);
-    case T_Q4_1: return moe_fmt<MQ4_1>(W, q8_workspace, Y, xdtype, (int)N, (int)K, ns, moe, s);
-    case T_Q5_0: return moe_fmt<MQ5_0>(W, q8_workspace, Y, xdtype, (int)N, (int)K, ns, moe, s);
-    case T_Q5_1: return moe_fmt<MQ5_1>(W, q8_workspace, Y, xdtype, (int)N, (int)K, ns, moe, s);
-    case T_Q2_K: return moe_fmt<MQ2_K>(W, q8_workspace, Y, xdtype, (int)N, (int)K, ns, moe, s);
-    case T_Q3_K: return moe_fmt<MQ3_K>(W, q8_workspace, Y, xdtype, (int)N, (int)K, ns, moe, s);
-    case T_Q5_K: return moe_fmt<MQ5_K>(W, q8_workspace, Y, xdtype, (int)N, (int)K, ns, moe, s);
-    case T_Q8_0: return moe_fmt<MQ8_0>(W, q8_workspace, Y, xdtype, (int)N, (int)K, ns, moe, s);
-    case T_Q4_K: return moe_fmt<MQ4_K>(W, q8_workspace, Y, xdtype, (int)N, (int)K, ns, moe, s);
-    case T_Q6_K: return moe_fmt<MQ6_K>(W, q8_workspace, Y, xdtype, (int)N, (int)K, ns, moe, s);
-    case T_IQ4_XS: return moe_fmt<MIQ4_XS>(W, q8_workspace, Y, xdtype, (int)N, (int)K, ns, moe, s);
-    case T_IQ2_XXS: return moe_fmt<MIQ2_XXS>(W, q8_workspace, Y, xdtype, (int)N, (int)K, ns, moe, s);
-  }
-  return GGUF_ERR_TYPE;
+  return moe_tiles32(W, q8_workspace, Y, xdtype, type, (int)N, (int)K, ns, moe, s);
 }

@@ -18,6 +18,17 @@ struct MoeArgs {
                           // vecdotq.cuh:369-372), 1 = times d8 * (sum of the quants) (its GEMV, vecdotq.cuh:328-351)
 };
 
+// The first expert GEMM of a layer with its seam.  The weight rows are [gate | up], inner features each, and a tile's
+// columns are the SAME features of both halves (the first half of the columns gate, the second up); the workgroup that
+// has both finishes them -- y = T(sum), h = T(T(act(gate)) up), the q8_1 blocks of h -- and writes them into the pair's
+// row of a second activation workspace, which the second expert GEMM reads as it is (no [pairs][2 inner] tensor, no
+// quantize launch).
+struct Gate16 {
+  char* rows;             // q8_1 rows of h, one per pair
+  int64_t row_bytes;
+  int inner, kp, act;     // features of each half; q8_kp(inner); ACT_SILU / ACT_GELU
+};
+
 // --------------------------------------------------------------------------------------------
 // Format policies: unpack one 32-element block of one weight row to int8 (8 dwords, element order)
 // plus fp32 scale(s) and, where the format has one, the fp32 offset factor multiplied by the

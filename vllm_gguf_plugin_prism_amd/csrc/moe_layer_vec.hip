@@ -25,11 +25,11 @@
 namespace gguf {
 
 // mmq.hip
-bool moe_tiles_layer_ok(int type13, int type2, int64_t pairs, int64_t num_experts, int64_t I);
-int64_t moe_tiles_layer_workspace(int64_t tokens, int64_t top_k, int64_t H, int64_t I, int64_t N_out, int64_t num_experts, int elt);
+int moe_tiles_layer_block(int type13, int type2, int64_t pairs, int64_t num_experts, int64_t I, bool vec_sums);
+int64_t moe_tiles_layer_workspace(int64_t tokens, int64_t top_k, int64_t H, int64_t I, int64_t N_out, int64_t num_experts, int elt, int block);
 int moe_tiles_layer(const void* X, int xdtype, void* workspace, const void* W13, int type13, const void* W2, int type2, const int32_t* topk_ids,
                     const float* topk_w, void* out, int H, int I, int N_out, int top_k, int tokens, int act, int num_experts, bool vec_sums,
-                    hipStream_t s);
+                    int block, hipStream_t s);
 
 struct MoeUpArgs {
   const int32_t* topk_ids;
@@ -395,7 +395,7 @@ static int moe_layer_takes(int type13, int type2, int H, int I, int N_out, int t
   const int64_t pairs = (int64_t)tokens * top_k;
   const bool shared13 = num_experts > 0 && moe_share_pays(pairs, num_experts, (int64_t)2 * I * (H / qk13) * block_bytes(type13));
   const bool shared2 = num_experts > 0 && moe_share_pays(pairs, num_experts, (int64_t)N_out * (I / qk2) * block_bytes(type2));
-  if (shared13 || shared2) return shared13 && shared2 && moe_tiles_layer_ok(type13, type2, pairs, num_experts, I) ? 2 : 0;
+  if (shared13 || shared2) return shared13 && shared2 && moe_tiles_layer_block(type13, type2, pairs, num_experts, I, true) == 16 ? 2 : 0;
   bool up = false, down = false;
   switch (type13) {
 #define MOE_LAYER_CASE(ID, FMT) case ID: up = moe_up_plan<FMT>(H, I, (int)pairs).ok; break;
@@ -428,7 +428,10 @@ extern "C" int64_t gguf_moe_vec_layer_workspace_bytes(int64_t tokens, int64_t to
                                                       int xdtype) {
   if (tokens <= 0 || top_k <= 0 || H <= 0 || I <= 0 || N_out <= 0 || num_experts < 0) return 0;
   const int64_t pair_rows = tokens * top_k * gguf::q8_row_bytes(I);
-  const int64_t tiles = gguf::moe_tiles_layer_workspace(tokens, top_k, H, I, N_out, num_experts, xdtype == GGUF_DTYPE_F32 ? 4 : 2);
+  const int elt = xdtype == GGUF_DTYPE_F32 ? 4 : 2;
+  const int64_t t16 = gguf::moe_tiles_layer_workspace(tokens, top_k, H, I, N_out, num_experts, elt, 16);
+  const int64_t t32 = gguf::moe_tiles_layer_workspace(tokens, top_k, H, I, N_out, num_experts, elt, 32);
+  const int64_t tiles = t16 > t32 ? t16 : t32;
   return pair_rows > tiles ? pair_rows : tiles;
 }
 
@@ -448,9 +451,9 @@ extern "C" int gguf_moe_vec_layer(const void* X, int xdtype, const void* W13, in
   if (route == 0) return GGUF_ERR_SHAPE;
   hipStream_t s = (hipStream_t)stream;
   if (route == 2) {
-    if (workspace_bytes < moe_tiles_layer_workspace(tokens, top_k, H, I, N_out, ne, xdtype == GGUF_DTYPE_F32 ? 4 : 2)) return GGUF_ERR_WORKSPACE;
+    if (workspace_bytes < moe_tiles_layer_workspace(tokens, top_k, H, I, N_out, ne, xdtype == GGUF_DTYPE_F32 ? 4 : 2, 16)) return GGUF_ERR_WORKSPACE;
     return moe_tiles_layer(X, xdtype, workspace, W13, type13, W2, type2, topk_ids, topk_weights, out, (int)H, (int)I, (int)N_out, (int)top_k,
-                           (int)tokens, act, ne, true, s);
+                           (int)tokens, act, ne, true, 16, s);
   }
   if (workspace_bytes < tokens * top_k * q8_row_bytes(I)) return GGUF_ERR_WORKSPACE;
   int rc = GGUF_ERR_TYPE;
@@ -470,15 +473,18 @@ extern "C" int gguf_moe_vec_layer(const void* X, int xdtype, const void* W13, in
   return GGUF_ERR_TYPE;
 }
 
-// The same four launches with the grouped operator's arithmetic (gguf_moe_mmq_block on blocks of 16 slots, twice, and the
-// weighted sum): what a layer with more than 64 tokens takes while its experts still see at most 16 pairs each on average.
+// The same four launches with the grouped operator's arithmetic (gguf_moe_mmq_block twice and the weighted sum): what a
+// layer with more than 64 tokens takes -- on blocks of 16 slots while its experts see at most 16 pairs each on average and
+// both formats have such tiles (returns 1), else on the reference's blocks of 32 (returns 2).
 extern "C" int gguf_moe_mmq_layer_takes(int type13, int type2, int64_t H, int64_t I, int64_t N_out, int64_t top_k, int64_t tokens,
                                         int64_t num_experts) {
   using namespace gguf;
-  if (!moe_layer_sizes_ok(H, I, N_out, top_k, tokens)) return 0;
+  if (!(H > 0 && I > 0 && N_out > 0 && top_k > 0 && tokens > 0 && H <= 0x7FFFFFF0LL && 2 * I <= 0x7FFFFFF0LL && N_out <= 0x7FFFFFF0LL)) return 0;
+  if (num_experts <= 0 || num_experts > 256 || tokens > 0x7FFFFFF0LL / top_k || tokens * top_k + 31 * num_experts > 65535 * 32) return 0;   // (a grid row per block)
   const int qk13 = block_elems(type13), qk2 = block_elems(type2);
   if (qk13 == 0 || qk2 == 0 || H % qk13 != 0 || I % qk2 != 0) return 0;
-  return moe_tiles_layer_ok(type13, type2, tokens * top_k, num_experts, I) ? 1 : 0;
+  const int block = moe_tiles_layer_block(type13, type2, tokens * top_k, num_experts, I, false);
+  return block == 16 ? 1 : block == 32 ? 2 : 0;
 }
 
 extern "C" int gguf_moe_mmq_layer(const void* X, int xdtype, const void* W13, int type13, const void* W2, int type2, const int32_t* topk_ids,
@@ -489,11 +495,13 @@ extern "C" int gguf_moe_mmq_layer(const void* X, int xdtype, const void* W13, in
   if (block_elems(type13) == 0 || block_elems(type2) == 0) return GGUF_ERR_TYPE;
   if (xdtype < 0 || xdtype > 2) return GGUF_ERR_DTYPE;
   if (tokens == 0) return GGUF_OK;
-  if (!gguf_moe_mmq_layer_takes(type13, type2, H, I, N_out, top_k, tokens, num_experts)) return GGUF_ERR_SHAPE;
+  const int route = gguf_moe_mmq_layer_takes(type13, type2, H, I, N_out, top_k, tokens, num_experts);
+  if (!route) return GGUF_ERR_SHAPE;
   if (!X || !W13 || !W2 || !topk_ids || !topk_weights || !workspace || !out) return GGUF_ERR_NULL;
   if (((uintptr_t)W13 | (uintptr_t)W2) & 1) return GGUF_ERR_SHAPE;   // packed blocks sit at even addresses
-  if (workspace_bytes < moe_tiles_layer_workspace(tokens, top_k, H, I, N_out, num_experts, xdtype == GGUF_DTYPE_F32 ? 4 : 2))
+  const int block = route == 1 ? 16 : 32;
+  if (workspace_bytes < moe_tiles_layer_workspace(tokens, top_k, H, I, N_out, num_experts, xdtype == GGUF_DTYPE_F32 ? 4 : 2, block))
     return GGUF_ERR_WORKSPACE;
   return moe_tiles_layer(X, xdtype, workspace, W13, type13, W2, type2, topk_ids, topk_weights, out, (int)H, (int)I, (int)N_out, (int)top_k,
-                         (int)tokens, act, (int)num_experts, false, (hipStream_t)stream);
+                         (int)tokens, act, (int)num_experts, false, block, (hipStream_t)stream);
 }

@@ -30,15 +30,8 @@ struct Dense16 {
   float* partial;
 };
 
-// GATE (with MOE): the first expert GEMM of a layer with its seam.  The weight rows are [gate | up], inner features
-// each, and a tile's 128 columns are the SAME 64 features of both halves; the workgroup that has both finishes them --
-// y = T(sum), h = T(T(act(gate)) up), the q8_1 blocks of h -- and writes them into the pair's row of a second
-// activation workspace, which the second expert GEMM reads as it is (no [pairs][2 inner] tensor, no quantize launch).
-struct Gate16 {
-  char* rows;             // q8_1 rows of h, one per pair
-  int64_t row_bytes;
-  int inner, kp, act;     // features of each half; q8_kp(inner); ACT_SILU / ACT_GELU
-};
+// GATE (with MOE): the first expert GEMM of a layer with its seam (Gate16, mmq_formats.h): a tile's 128 columns are the
+// SAME 64 features of the gate and the up half.
 
 template <class F, typename T, int NW, int OCC, bool MOE = true, bool GATE = false>
 __global__ __launch_bounds__(64 * NW, OCC) void moe16_kernel(const uint8_t* __restrict__ W, const char* __restrict__ ws, int64_t ws_row_bytes,

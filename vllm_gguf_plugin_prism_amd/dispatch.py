@@ -192,8 +192,8 @@ def fused_moe_gguf(x, w1, w2, topk_weights, topk_ids, weight_type: int, weight_t
         experts, rows, _ = w1.shape
         if activation in ("silu", "gelu") and w2.shape[0] == experts and ops.moe_mmq_layer_takes(
                 weight_type, weight_type2, x.shape[1], rows // 2, w2.shape[1], top_k, tokens, experts):
-            # experts that see at most 16 pairs each: the layer in one call of four launches on 16-slot tiles (one sort for
-            # both GEMMs, the activation and the quantisation of its result in the first one's epilogue)
+            # the layer in one call of four launches (one sort for both GEMMs, the activation and the quantisation of its
+            # result in the first one's epilogue): on 16-slot tiles while experts see at most 16 pairs each, else on 32
             return ops.moe_mmq_layer(x, w1, w2, topk_weights, topk_ids, weight_type, weight_type2, activation, out_hidden)
         # the reference sorts with ggml_moe_get_block_size(type); here a layer whose experts see few pairs each (65 .. 128
         # tokens of a 64-expert top-8 layer) sorts with blocks of 16 slots where both formats have such tiles, so that the

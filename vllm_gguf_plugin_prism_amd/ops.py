@@ -349,8 +349,8 @@ def moe_vec_layer_takes(quant_type: int, quant_type2: int, hidden: int, inner: i
 
 def moe_mmq_layer_takes(quant_type: int, quant_type2: int, hidden: int, inner: int, out_features: int, top_k: int, tokens: int,
                         num_experts: int) -> bool:
-    """Whether :func:`moe_mmq_layer` serves a layer of this shape: experts that see at most 16 pairs each on average,
-    both formats with 16-slot tiles, at most 256 experts."""
+    """Whether :func:`moe_mmq_layer` serves a layer of this shape: two tile formats (the twelve of ``ggml_moe_a8``), at
+    most 256 experts, an inner size in whole blocks."""
     return bool(_lib.lib().gguf_moe_mmq_layer_takes(int(quant_type), int(quant_type2), int(hidden), int(inner), int(out_features),
                                                     int(top_k), int(tokens), int(num_experts)))
 
@@ -358,7 +358,7 @@ def moe_mmq_layer_takes(quant_type: int, quant_type2: int, hidden: int, inner: i
 def moe_mmq_layer(X, W13, W2, topk_weights, topk_ids, quant_type: int, quant_type2: int, activation: str,
                   output: torch.Tensor | None = None) -> torch.Tensor:
     """The reference's MoE layer on its grouped operator (quantization/fused_moe.py:62-95) in one call of four launches:
-    one routing sort on blocks of 16 slots for both ``ggml_moe_a8`` GEMMs, ``act`` and the q8_1 quantisation of its
+    one routing sort (on blocks of 16 slots while experts see at most 16 pairs each, else 32) for both ``ggml_moe_a8`` GEMMs, ``act`` and the q8_1 quantisation of its
     result in the first one's epilogue, ``mul_`` by the routing weights and ``moe_sum`` -> ``[tokens, W2.shape[1]]``.
     Same roundings as those steps run one by one; raises ``ValueError`` for shapes :func:`moe_mmq_layer_takes` declines."""
     return _moe_layer("gguf_moe_mmq_layer", X, W13, W2, topk_weights, topk_ids, quant_type, quant_type2, activation, output)
