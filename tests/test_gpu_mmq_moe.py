@@ -660,6 +660,13 @@ def test_moe_layer_on_grouped_tiles_matches_the_separate_steps(qtype, dt):
             assert err <= {"f32": 5e-4, "f16": 1e-3, "bf16": 4e-3}[dt], f"{o.TYPE_NAMES[qtype]} {o.TYPE_NAMES[qt2]} {dt} case {case} rel-L2 {err}"
             if t > 64:   # the layer through the dispatcher takes the same call
                 assert torch.equal(dispatch.fused_moe_gguf(x, w13d, w2d, _dev(wts), _dev(ids), qtype, qt2, "silu"), got)
+            if dt == "f16" and qt2 == qtype and case in (0, 2):   # the other activation the reference's MoE models use
+                h = ops.ggml_moe_a8(x, w13d, sorted_ids, expert_ids, post, qtype, 2 * inner, top_k, t, block_size=block)
+                y = ops.ggml_moe_a8(h, w2d, sorted_ids, expert_ids, post, qt2, hid, 1, pairs, activation="gelu", block_size=block)
+                want_g = torch.empty((t, hid), dtype=x.dtype, device="cuda")
+                ops.moe_weighted_sum(y.reshape(t, top_k, hid), _dev(wts), want_g)
+                got_g = ops.moe_mmq_layer(x, w13d, w2d, _dev(wts), _dev(ids), qtype, qt2, "gelu")
+                assert o.rel_l2(got_g.float().cpu().numpy(), want_g.float().cpu().numpy()) <= 1e-3
     with pytest.raises(ValueError):     # more experts than the tile kernels' guard on expert ids admits
         row = 256 // qk * o.QUANT_SIZES[qtype][1]
         ops.moe_mmq_layer(torch.zeros(70, 256, device="cuda", dtype=TORCH_DT[dt]), _dev(np.zeros((300, 512, row), dtype=np.uint8)),
