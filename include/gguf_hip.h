@@ -241,8 +241,11 @@ int gguf_moe_weighted_sum(const void* Y, const float* topk_weights, void* out, i
  *      launches on the tile kernels -- one that quantizes X and sorts the routing for both GEMMs, first GEMM with the
  *      activation and the quantisation of its result in the epilogue, second GEMM from those rows, weighted sum -- where
  *      the separate operators take seven.
+ *   3  the same four launches on blocks of 32 slots: shared experts in the other tile formats (Q4_1, Q5_1, Q2_K) or with
+ *      more than 16 pairs each.
  *   0  not served (I no multiple of 32 or of type2's block, top_k times the waves a row of W2 takes beyond a workgroup,
- *      more than 65535 pairs, experts shared by more pairs than that): gguf_moe_vec_layer returns GGUF_ERR_SHAPE.
+ *      more than 65535 pairs, shared experts in a format without tiles or in Q5_0, whose tile arithmetic is not its
+ *      GEMV's, or more than 256 of them): gguf_moe_vec_layer returns GGUF_ERR_SHAPE.
  * workspace: gguf_moe_vec_layer_workspace_bytes(...) bytes, layout private; GGUF_ERR_WORKSPACE if workspace_bytes is less
  * than the route needs.  act: 1 = SiLU, 2 = GELU.  A pair whose expert id is outside [0, num_experts) (num_experts > 0)
  * adds nothing on route 1. */

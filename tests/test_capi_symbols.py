@@ -155,8 +155,11 @@ def test_two_launch_moe_layer_states_which_shapes_it_serves():
     assert h.gguf_moe_vec_layer_takes(12, 14, 4096, 14336, 4096, 2, 1, 8) == 1
     assert h.gguf_moe_vec_layer_takes(2, 2, 2048, 8192, 2048, 8, 1, 64) == 0
     assert h.gguf_moe_vec_layer_takes(2, 2, 2048, 1024, 2048, 8, 64, 64) == 2      # 8 pairs per expert: the tile route
-    assert h.gguf_moe_vec_layer_takes(2, 2, 2048, 1024, 2048, 8, 200, 64) == 0     # 25 pairs per expert: blocks of 32, not served
-    assert h.gguf_moe_vec_layer_takes(6, 6, 2048, 1024, 2048, 8, 64, 64) == 0       # Q5_0 has no 16-slot tiles with the GEMV's sums
+    assert h.gguf_moe_vec_layer_takes(2, 2, 2048, 1024, 2048, 8, 200, 64) == 3     # 25 pairs per expert: blocks of 32
+    assert h.gguf_moe_vec_layer_takes(3, 3, 2048, 1024, 2048, 8, 64, 64) == 3       # Q4_1: blocks of 32 only
+    assert h.gguf_moe_vec_layer_takes(6, 6, 2048, 1024, 2048, 8, 64, 64) == 0       # Q5_0: its tile arithmetic is not its GEMV's
+    assert h.gguf_moe_vec_layer_takes(20, 20, 2048, 1024, 2048, 8, 64, 64) == 0     # IQ4_NL: shared experts, no tiles
+    assert h.gguf_moe_vec_layer_takes(2, 2, 2048, 1024, 2048, 8, 200, 300) == 0     # more experts than the tiles' id guard admits
     assert h.gguf_moe_vec_layer_takes(1, 2, 2048, 1024, 2048, 8, 1, 64) == 0
     assert h.gguf_moe_vec_layer_takes(2, 12, 2048, 1120, 2048, 8, 1, 64) == 0
     assert h.gguf_moe_vec_layer_workspace_bytes(3, 8, 2048, 1024, 2048, 64, 1) >= 24 * h.gguf_q8_1_row_bytes(1024) + 3 * h.gguf_q8_1_row_bytes(2048)

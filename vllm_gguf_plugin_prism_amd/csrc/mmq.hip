@@ -663,11 +663,13 @@ namespace gguf {
 static inline int64_t up16(int64_t v) { return (v + 15) / 16 * 16; }
 
 // 16: both formats have 16-slot tiles and the experts see at most 16 pairs each on average; 32: the layer runs on blocks of
-// 32 slots (grouped arithmetic only: the per-pair operator's differs there for Q5_0); 0: not on the tile kernels
+// 32 slots; 0: not on the tile kernels (a format without tiles; with the per-pair operator's arithmetic also Q5_0, the
+// one format whose tile arithmetic differs from its GEMV's)
 int moe_tiles_layer_block(int type13, int type2, int64_t pairs, int64_t num_experts, int64_t I, bool vec_sums) {
   if (num_experts <= 0 || num_experts > 256 || I % 32 != 0) return 0;
+  if (vec_sums && (type13 == T_Q5_0 || type2 == T_Q5_0)) return 0;
   if (moe_tiles16_ok(type13) && moe_tiles16_ok(type2) && type13 != T_Q5_0 && type2 != T_Q5_0 && pairs <= 16 * num_experts) return 16;
-  return !vec_sums && mmq_type_ok(type13) && mmq_type_ok(type2) ? 32 : 0;
+  return mmq_type_ok(type13) && mmq_type_ok(type2) ? 32 : 0;
 }
 
 // [q8_1 rows of X][q8_1 rows of h][second GEMM's result, pairs x N_out][sorted ids, expert ids, padded total]

@@ -387,7 +387,8 @@ static int moe_sum_fmt(int dtype, const void* W, const void* ws, const int32_t* 
   CASE(T_IQ2_XXS, FmtIQ2_XXS) CASE(T_IQ2_XS, FmtIQ2_XS) CASE(T_IQ2_S, FmtIQ2_S) CASE(T_IQ3_XXS, FmtIQ3_XXS) CASE(T_IQ3_S, FmtIQ3_S) \
   CASE(T_IQ1_S, FmtIQ1_S) CASE(T_IQ1_M, FmtIQ1_M)
 
-// 0: not served; 1: the two launches above; 2: four launches on the tile kernels (experts shared by a few pairs each)
+// 0: not served; 1: the two launches above; 2 / 3: four launches on the tile kernels with blocks of 16 / 32 slots (experts
+// shared by a few pairs each)
 static int moe_layer_takes(int type13, int type2, int H, int I, int N_out, int top_k, int tokens, int num_experts) {
   const int qk13 = block_elems(type13), qk2 = block_elems(type2);
   if (qk13 == 0 || qk2 == 0 || H % qk13 != 0 || I % qk2 != 0 || I % 32 != 0) return 0;
@@ -395,7 +396,10 @@ static int moe_layer_takes(int type13, int type2, int H, int I, int N_out, int t
   const int64_t pairs = (int64_t)tokens * top_k;
   const bool shared13 = num_experts > 0 && moe_share_pays(pairs, num_experts, (int64_t)2 * I * (H / qk13) * block_bytes(type13));
   const bool shared2 = num_experts > 0 && moe_share_pays(pairs, num_experts, (int64_t)N_out * (I / qk2) * block_bytes(type2));
-  if (shared13 || shared2) return shared13 && shared2 && moe_tiles_layer_block(type13, type2, pairs, num_experts, I, true) == 16 ? 2 : 0;
+  if (shared13 || shared2) {
+    const int block = shared13 && shared2 ? moe_tiles_layer_block(type13, type2, pairs, num_experts, I, true) : 0;
+    return block == 16 ? 2 : block == 32 ? 3 : 0;
+  }
   bool up = false, down = false;
   switch (type13) {
 #define MOE_LAYER_CASE(ID, FMT) case ID: up = moe_up_plan<FMT>(H, I, (int)pairs).ok; break;
@@ -450,10 +454,11 @@ extern "C" int gguf_moe_vec_layer(const void* X, int xdtype, const void* W13, in
   const int route = moe_layer_takes(type13, type2, (int)H, (int)I, (int)N_out, (int)top_k, (int)tokens, ne);
   if (route == 0) return GGUF_ERR_SHAPE;
   hipStream_t s = (hipStream_t)stream;
-  if (route == 2) {
-    if (workspace_bytes < moe_tiles_layer_workspace(tokens, top_k, H, I, N_out, ne, xdtype == GGUF_DTYPE_F32 ? 4 : 2, 16)) return GGUF_ERR_WORKSPACE;
+  if (route >= 2) {
+    const int block = route == 2 ? 16 : 32;
+    if (workspace_bytes < moe_tiles_layer_workspace(tokens, top_k, H, I, N_out, ne, xdtype == GGUF_DTYPE_F32 ? 4 : 2, block)) return GGUF_ERR_WORKSPACE;
     return moe_tiles_layer(X, xdtype, workspace, W13, type13, W2, type2, topk_ids, topk_weights, out, (int)H, (int)I, (int)N_out, (int)top_k,
-                           (int)tokens, act, ne, true, 16, s);
+                           (int)tokens, act, ne, true, block, s);
   }
   if (workspace_bytes < tokens * top_k * q8_row_bytes(I)) return GGUF_ERR_WORKSPACE;
   int rc = GGUF_ERR_TYPE;
