@@ -675,6 +675,39 @@ def test_moe_layer_on_grouped_tiles_matches_the_separate_steps(qtype, dt):
                           _dev(np.zeros((70, 2), dtype=np.int32)), qtype, qtype, "silu")
 
 
+def test_moe_layers_of_a_wide_model_match_the_separate_steps():
+    """A layer the size of an 8-expert top-2 model's (hidden 4096, inner 14336, Q4_K gate / up and Q6_K down projections:
+    224 tiles of features per block, a second format of another group size): the layer entry points against the
+    operators called one by one, below 64 tokens on 16-slot blocks, above on 16 and on 32."""
+    ops = _ops()
+    from vllm_gguf_plugin_prism_amd import _lib, dispatch, synth
+    rng = np.random.default_rng(77)
+    e, hid, inner, top_k, qt1, qt2 = 8, 4096, 14336, 2, o.Q4_K, o.Q6_K
+    w13d = _dev(np.stack([synth.random_blocks(rng, qt1, 2 * inner, hid) for _ in range(e)]))
+    w2d = _dev(np.stack([synth.random_blocks(rng, qt2, hid, inner, 1e-5, 1e-4) for _ in range(e)]))
+    for t, want_route in ((48, "vec 2"), (64, "vec 2"), (96, "mmq 2"), (33, "vec 2")):
+        ids, wts = _routing(rng, t, e, top_k)
+        pairs = t * top_k
+        x = torch.randn(t, hid, device="cuda")
+        x = x * (4.0 / ops.ggml_moe_a8_vec(x, w13d, _dev(ids), top_k, qt1, 2 * inner, t).abs().max())   # (random blocks: keep h small)
+        L = _lib.lib()
+        if t <= 64:
+            assert L.gguf_moe_vec_layer_takes(qt1, qt2, hid, inner, hid, top_k, t, e) == 2
+            h = ops.ggml_moe_a8_vec(x, w13d, _dev(ids), top_k, qt1, 2 * inner, t)
+            y = ops.ggml_moe_a8_vec(h, w2d, _dev(ids.reshape(pairs, 1)), 1, qt2, hid, pairs, activation="silu")
+        else:
+            assert L.gguf_moe_mmq_layer_takes(qt1, qt2, hid, inner, hid, top_k, t, e) == 2    # 24 pairs per expert: blocks of 32
+            s_ids, e_ids, post = ops.moe_align_block_size(_dev(ids), 32, e)
+            h = ops.ggml_moe_a8(x, w13d, s_ids, e_ids, post, qt1, 2 * inner, top_k, t)
+            y = ops.ggml_moe_a8(h, w2d, s_ids, e_ids, post, qt2, hid, 1, pairs, activation="silu")
+        want = torch.empty((t, hid), dtype=x.dtype, device="cuda")
+        ops.moe_weighted_sum(y.reshape(t, top_k, hid), _dev(wts), want)
+        got = dispatch.fused_moe_gguf(x, w13d, w2d, _dev(wts), _dev(ids), qt1, qt2, "silu")
+        assert not torch.isnan(want).any() and not torch.isinf(want).any()
+        err = o.rel_l2(got.float().cpu().numpy(), want.float().cpu().numpy())
+        assert err <= 5e-4, f"t={t} ({want_route}) rel-L2 {err}"
+
+
 def _lib_takes(ops, *args):
     from vllm_gguf_plugin_prism_amd import _lib
     return _lib.lib().gguf_moe_vec_layer_takes(*[int(a) for a in args])
