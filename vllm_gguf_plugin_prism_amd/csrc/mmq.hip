@@ -531,7 +531,12 @@ static void launch_mmq(const void* W, const void* ws, void* Y, int M, int N, int
 template <class F, typename T>
 static int moe_typed(const void* W, const void* ws, void* Y, int N, int K, int num_sorted, const MoeArgs& moe,
                      hipStream_t stream) {
-  launch_mmq<F, 1, 4, 1, 2, 128, 2, MODE_PREFETCH, T, true>(W, ws, Y, 0, N, K, num_sorted / 32, moe, stream);  // 32 slots x 256
+  // 32 slots x 256 features; x 128 where the blocks that hold pairs (estimated) times the feature tiles would leave CUs
+  // idle (12 blocks of an 8-expert layer at 128 tokens x 16 tiles of [4096,14336]: 192 workgroups for 512 places)
+  if (moe_blocks_estimate(num_sorted, moe.num_pairs, 32) * ((N + 255) / 256) < 2.0 * num_cus())
+    launch_mmq<F, 1, 4, 1, 1, 128, 2, MODE_PREFETCH, T, true>(W, ws, Y, 0, N, K, num_sorted / 32, moe, stream);
+  else
+    launch_mmq<F, 1, 4, 1, 2, 128, 2, MODE_PREFETCH, T, true>(W, ws, Y, 0, N, K, num_sorted / 32, moe, stream);
   return launch_status();
 }
 

@@ -18,6 +18,23 @@ struct MoeArgs {
                           // vecdotq.cuh:369-372), 1 = times d8 * (sum of the quants) (its GEMV, vecdotq.cuh:328-351)
 };
 
+// Expected number of blocks of `block` slots that hold pairs, for pairs spread over the experts at random (the sorted array
+// has room for block - 1 padding slots per expert, which gives the expert count).  How many there are is known on the
+// device only; launch plans that depend on it take this estimate.
+static inline double moe_blocks_estimate(int num_sorted, int num_pairs, int block) {
+  const double experts = (double)(num_sorted - num_pairs) / (double)(block - 1);
+  if (experts < 1.0) return (double)(num_sorted / block);
+  const double lam = (double)num_pairs / experts;
+  if (lam > 256.0) return (lam / block + 0.5) * experts;
+  double blocks = 0.0, term = exp(-lam), cdf = 0.0;   // sum over j >= 0 of P(pairs of an expert > block * j)
+  for (int c = 0; c <= 2048 && cdf < 1.0 - 1e-12; ++c) {
+    cdf += term;
+    if (c % block == 0) blocks += 1.0 - cdf;
+    term *= lam / (c + 1);
+  }
+  return blocks * experts;
+}
+
 // The first expert GEMM of a layer with its seam.  The weight rows are [gate | up], inner features each, and a tile's
 // columns are the SAME features of both halves (the first half of the columns gate, the second up); the workgroup that
 // has both finishes them -- y = T(sum), h = T(T(act(gate)) up), the q8_1 blocks of h -- and writes them into the pair's

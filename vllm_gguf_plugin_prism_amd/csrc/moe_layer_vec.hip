@@ -397,7 +397,9 @@ static int moe_layer_takes(int type13, int type2, int H, int I, int N_out, int t
   const bool shared13 = num_experts > 0 && moe_share_pays(pairs, num_experts, (int64_t)2 * I * (H / qk13) * block_bytes(type13));
   const bool shared2 = num_experts > 0 && moe_share_pays(pairs, num_experts, (int64_t)N_out * (I / qk2) * block_bytes(type2));
   if (shared13 || shared2) {
-    const int block = shared13 && shared2 ? moe_tiles_layer_block(type13, type2, pairs, num_experts, I, true) : 0;
+    // (where only one of the two says so -- the thresholds differ by half a pair per expert between experts that fit the
+    //  last-level cache together and experts that do not -- the other is near its own break-even: both go to the tiles)
+    const int block = moe_tiles_layer_block(type13, type2, pairs, num_experts, I, true);
     return block == 16 ? 2 : block == 32 ? 3 : 0;
   }
   bool up = false, down = false;

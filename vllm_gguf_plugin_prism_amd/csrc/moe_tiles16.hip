@@ -33,14 +33,14 @@ struct Dense16 {
 // GATE (with MOE): the first expert GEMM of a layer with its seam (Gate16, mmq_formats.h): a tile's 128 columns are the
 // SAME 64 features of the gate and the up half.
 
-template <class F, typename T, int NW, int OCC, bool MOE = true, bool GATE = false>
+template <class F, typename T, int NW, int OCC, bool MOE = true, bool GATE = false, int CT = 2>
 __global__ __launch_bounds__(64 * NW, OCC) void moe16_kernel(const uint8_t* __restrict__ W, const char* __restrict__ ws, int64_t ws_row_bytes,
                                                         T* __restrict__ Y, int N, int K, int Kp, int tiles_m, int tiles, MoeArgs moe,
                                                         Dense16 dn, const T* __restrict__ bias, Gate16 gate) {
-  static_assert(!GATE || (MOE && NW == 4), "the gated epilogue pairs the halves of a 128-column tile");
+  static_assert(!GATE || (MOE && NW == 4 && CT == 2), "the gated epilogue pairs the halves of a 128-column tile");
   static_assert(!(F::G == 16 && F::HAS_MIN), "16-deep formats with per-group offsets keep the 32-row kernel");
   constexpr int NT = 64 * NW, KS = MMQI_KS, KB = KS / 32, GR = KS / 16, LDK = Pitch<32, KS>::value;
-  constexpr int M_T = 16, CT = 2, N_T = 16 * CT * NW;   // two 16-feature tiles per wave
+  constexpr int M_T = 16, N_T = 16 * CT * NW;   // CT 16-feature tiles per wave: two, or one where the output has few tiles
   constexpr int PAIRS = N_T * KB, WP = PAIRS / NT;  // (weight row, 32-block) pairs per step, per thread
   constexpr int DEPTH = F::G == 16 ? 1 : 2;          // (two stages of the large Q6_K / Q3_K blocks do not fit the registers)
   constexpr size_t BUF = (size_t)(M_T + N_T) * LDK + (size_t)KB * M_T * 4 * (F::HAS_MIN ? 2 : 1) + (size_t)KB * N_T * 8;
@@ -157,7 +157,7 @@ __global__ __launch_bounds__(64 * NW, OCC) void moe16_kernel(const uint8_t* __re
         const long a = *(const long*)(xq + lcol * LDK + 32 * kb + 8 * lgrp);
 #pragma unroll
         for (int c = 0; c < CT; ++c) {
-          const int col = 32 * wave + 16 * c + lcol;
+          const int col = 16 * CT * wave + 16 * c + lcol;
           const long b = *(const long*)(wq + col * LDK + 32 * kb + 8 * lgrp);
           const f32x2 sc = wsc[kb * N_T + col];
           const v4i_t s = __builtin_amdgcn_mfma_i32_16x16x32_i8(a, b, seed, 0, 0, 0);
@@ -176,7 +176,7 @@ __global__ __launch_bounds__(64 * NW, OCC) void moe16_kernel(const uint8_t* __re
         const long a0 = lgrp < 2 ? a : 0L, a1 = lgrp < 2 ? 0L : a;
 #pragma unroll
         for (int c = 0; c < CT; ++c) {
-          const int col = 32 * wave + 16 * c + lcol;
+          const int col = 16 * CT * wave + 16 * c + lcol;
           const long b = *(const long*)(wq + col * LDK + 32 * kb + 8 * lgrp);
           const f32x2 sc = wsc[kb * N_T + col];
           const v4i_t sa = __builtin_amdgcn_mfma_i32_16x16x32_i8(a0, b, seed, 0, 0, 0);
@@ -228,7 +228,7 @@ __global__ __launch_bounds__(64 * NW, OCC) void moe16_kernel(const uint8_t* __re
 #pragma unroll
     for (int r = 0; r < 4; ++r)
 #pragma unroll
-      for (int c = 0; c < CT; ++c) yt[(4 * lgrp + r) * N_T + 32 * wave + 16 * c + lcol] = to_f32<T>(from_f32<T>(acc[c][r]));
+      for (int c = 0; c < CT; ++c) yt[(4 * lgrp + r) * N_T + 16 * CT * wave + 16 * c + lcol] = to_f32<T>(from_f32<T>(acc[c][r]));
     __syncthreads();
     if (tid < 16 * 8) {
       const int slot = tid >> 3, part = tid & 7;
@@ -259,7 +259,7 @@ __global__ __launch_bounds__(64 * NW, OCC) void moe16_kernel(const uint8_t* __re
 #pragma unroll
       for (int r = 0; r < 4; ++r)
 #pragma unroll
-        for (int c = 0; c < CT; ++c) mine[(4 * lgrp + r) * N_T + 32 * wave + 16 * c + lcol] = acc[c][r];
+        for (int c = 0; c < CT; ++c) mine[(4 * lgrp + r) * N_T + 16 * CT * wave + 16 * c + lcol] = acc[c][r];
       return;
     }
   }
@@ -276,7 +276,7 @@ __global__ __launch_bounds__(64 * NW, OCC) void moe16_kernel(const uint8_t* __re
     }
 #pragma unroll
     for (int c = 0; c < CT; ++c) {
-      const int nn = n_base + 32 * wave + 16 * c + lcol;
+      const int nn = n_base + 16 * CT * wave + 16 * c + lcol;
       if (nn < N) Y[row + nn] = finish<T>(acc[c][r], MOE ? (const T*)nullptr : bias, nn);
     }
   }
@@ -306,6 +306,22 @@ static inline size_t moe16_lds_request(size_t lds, int num_sorted, int num_pairs
   return est > 3.0 * cus && est <= 4.0 * cus && !four_each && lds < 54 * 1024 ? (size_t)54 * 1024 : lds;
 }
 
+// The same contraction on tiles of 64 features (one 16-feature tile per wave, four or five workgroups per CU): what a GEMM
+// with few blocks and a narrow output takes, whose 128-feature tiles would leave CUs idle (8 experts x [4096,14336] at 64
+// tokens: 256 .. 512 tiles of 112 steps each for 768 places).
+template <class F, typename T>
+static int moe16_narrow_typed(const void* W, const void* ws, void* Y, int N, int K, int num_sorted, const MoeArgs& moe, hipStream_t stream) {
+  constexpr int NW = 4, N_T = 16 * NW, OCC = 4;
+  constexpr size_t BUF = (size_t)(16 + N_T) * Pitch<32, MMQI_KS>::value + (size_t)4 * 16 * 4 * (F::HAS_MIN ? 2 : 1) + (size_t)4 * N_T * 8;
+  constexpr size_t lds = 2 * BUF;
+  auto kern = moe16_kernel<F, T, NW, OCC, true, false, 1>;
+  const int tiles_n = (N + N_T - 1) / N_T, tiles_m = num_sorted / 16, tiles = tiles_m * tiles_n;
+  if (tiles == 0) return GGUF_OK;
+  hipLaunchKernelGGL(kern, dim3(tiles), dim3(64 * NW), lds, stream, (const uint8_t*)W, (const char*)ws, q8_row_bytes(K), (T*)Y, N, K,
+                     (int)q8_kp(K), tiles_m, tiles, moe, Dense16{}, (const T*)nullptr, Gate16{});
+  return launch_status();
+}
+
 template <class F, typename T>
 static int moe16_typed(const void* W, const void* ws, void* Y, int N, int K, int num_sorted, const MoeArgs& moe, hipStream_t stream) {
   // four waves, three workgroups per CU (two for Q5_K, whose packed block needs the registers); eight waves with one
@@ -320,6 +336,9 @@ static int moe16_typed(const void* W, const void* ws, void* Y, int N, int K, int
   }
   const int tiles_n = (N + N_T - 1) / N_T, tiles_m = num_sorted / 16, tiles = tiles_m * tiles_n;
   if (tiles == 0) return GGUF_OK;
+  // (the blocks that hold pairs, estimated: fewer tiles than the chip has places -> tiles of 64 features)
+  if (moe_blocks_estimate(num_sorted, moe.num_pairs, 16) * tiles_n < (double)(OCC * num_cus()))
+    return moe16_narrow_typed<F, T>(W, ws, Y, N, K, num_sorted, moe, stream);
   const size_t lds_req = OCC == 3 ? moe16_lds_request(lds, num_sorted, moe.num_pairs, tiles_n) : lds;
   hipLaunchKernelGGL(kern, dim3(tiles), dim3(64 * NW), lds_req, stream, (const uint8_t*)W, (const char*)ws, q8_row_bytes(K), (T*)Y, N, K,
                      (int)q8_kp(K), tiles_m, tiles, moe, Dense16{}, (const T*)nullptr, Gate16{});
