@@ -268,10 +268,17 @@ int gguf_moe_vec_layer(const void* X, int xdtype, const void* W13, int type13, c
  *   2  the reference's blocks of 32 slots: every other layer of two tile formats (the twelve of ggml_moe_a8);
  *   0  not served (num_experts outside 1..256, I no multiple of 32 or of type2's block, a format without tiles, more
  *      than about two million pairs): gguf_moe_mmq_layer returns GGUF_ERR_SHAPE.
+ *   3  experts that see 96 pairs or more each on average: six launches on the pipelined integer engine of gguf_mmq
+ *      with blocks of 128 slots -- the routing sort with its inverse, the rows of X quantized into slot order, the
+ *      first GEMM as a dense product over runs of rows (only the weight matrix changes from block to block), its
+ *      result quantized with the activation, the second GEMM, and the weighted sum gathering its rows through the
+ *      inverse of the sort.
  * A pair whose expert id is outside [0, num_experts) adds nothing, like the rows the grouped operator leaves at zero.
- * Workspace: gguf_moe_vec_layer_workspace_bytes(...), which covers both entry points and every route. */
+ * Workspace: gguf_moe_mmq_layer_workspace_bytes(...) bytes for the route the same arguments take (0 where none does). */
 int gguf_moe_mmq_layer_takes(int type13, int type2, int64_t H, int64_t I, int64_t N_out, int64_t top_k, int64_t tokens,
                              int64_t num_experts);
+int64_t gguf_moe_mmq_layer_workspace_bytes(int type13, int type2, int64_t tokens, int64_t top_k, int64_t H, int64_t I,
+                                           int64_t N_out, int64_t num_experts, int xdtype);
 int gguf_moe_mmq_layer(const void* X, int xdtype, const void* W13, int type13, const void* W2, int type2,
                        const int32_t* topk_ids, const float* topk_weights, void* workspace, int64_t workspace_bytes,
                        void* out, int64_t H, int64_t I, int64_t N_out, int64_t top_k, int64_t tokens, int act,

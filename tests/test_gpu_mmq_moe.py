@@ -619,7 +619,7 @@ def test_moe_layer_on_grouped_tiles_matches_the_separate_steps(qtype, dt):
     """moe_mmq_layer (the four launches of the tile route with the grouped operator's arithmetic) against
     moe_align_block_size, ggml_moe_a8 twice (the second with the activation) and moe_weighted_sum on the same block
     size: blocks of 16 slots where the experts see few pairs and the format has such tiles, else the reference's blocks
-    of 32.  More than 64 tokens, inner sizes that end inside a tile of features, an expert without pairs, a second
+    of 32; from 96 pairs per expert on the layer runs in slot order on the dense engine with blocks of 128.  More than 64 tokens, inner sizes that end inside a tile of features, an expert without pairs, a second
     format, and a pair whose expert id names no expert (it adds nothing in both)."""
     ops = _ops()
     from vllm_gguf_plugin_prism_amd import _lib, dispatch
@@ -627,25 +627,29 @@ def test_moe_layer_on_grouped_tiles_matches_the_separate_steps(qtype, dt):
     qk = o.QUANT_SIZES[qtype][0]
     other = o.Q8_0 if qtype != o.Q8_0 else o.Q4_0
     cases = [(70, 2, 12, 512, 768, 16), (24, 4, 8, 256, 1280 if qk == 32 else 1024, 16),
-             (70, 4, 8, 512, 768, 32), (40, 2, 3, 256, 1312 if qk == 32 else 1280, 32)]
+             (70, 4, 8, 512, 768, 32), (40, 2, 3, 256, 1312 if qk == 32 else 1280, 32),
+             (300, 2, 5, 512, 768, 128), (300, 1, 3, 256, 1312 if qk == 32 else 1280, 128)]
     for case, (t, top_k, e, hid, inner, block) in enumerate(cases):
         if block == 16 and qtype not in TILE16_TYPES:
             continue
-        for qt2 in (qtype, other) if case in (0, 2) else (qtype,):
+        for qt2 in (qtype, other) if case in (0, 2, 4) else (qtype,):
             w13 = np.stack([o.make_weights(rng, qtype, 2 * inner, hid) for _ in range(e)])
             w2 = np.stack([o.make_weights(rng, qt2, hid, inner) for _ in range(e)])
             w13d, w2d = _dev(w13), _dev(w2)
             ids, wts = _routing(rng, t, e - 1, top_k)            # the last expert has no pairs
             if case % 2 == 1:
-                ids[5, 1] = e + 3
+                ids[5, top_k - 1] = e + 3
             pairs = t * top_k
             route = _lib.lib().gguf_moe_mmq_layer_takes(int(qtype), int(qt2), hid, inner, hid, top_k, t, e)
-            assert route == (1 if block == 16 else 2), (case, route)
-            sorted_ids, expert_ids, post = ops.moe_align_block_size(_dev(ids), block, e)
+            deep16 = bool({int(qtype), int(qt2)} & {o.Q2_K, o.Q3_K, o.Q6_K})   # the dense engine takes layers with a 16-deep format
+            assert route == {16: 1, 32: 2, 128: 3 if deep16 else 2}[block], (case, route)
+            # (the route on blocks of 128 slots is compared with the operators on the reference's blocks of 32)
+            sort_block = min(block, 32)
+            sorted_ids, expert_ids, post = ops.moe_align_block_size(_dev(ids), sort_block, e)
 
             def separate(x):
-                h = ops.ggml_moe_a8(x, w13d, sorted_ids, expert_ids, post, qtype, 2 * inner, top_k, t, block_size=block)
-                y = ops.ggml_moe_a8(h, w2d, sorted_ids, expert_ids, post, qt2, hid, 1, pairs, activation="silu", block_size=block)
+                h = ops.ggml_moe_a8(x, w13d, sorted_ids, expert_ids, post, qtype, 2 * inner, top_k, t, block_size=sort_block)
+                y = ops.ggml_moe_a8(h, w2d, sorted_ids, expert_ids, post, qt2, hid, 1, pairs, activation="silu", block_size=sort_block)
                 want = torch.empty((t, hid), dtype=x.dtype, device="cuda")
                 ops.moe_weighted_sum(y.reshape(t, top_k, hid), _dev(wts), want)
                 return h, want
@@ -659,11 +663,11 @@ def test_moe_layer_on_grouped_tiles_matches_the_separate_steps(qtype, dt):
             #  differently in the two kernels)
             err = o.rel_l2(got.float().cpu().numpy(), want.float().cpu().numpy())
             assert err <= {"f32": 5e-4, "f16": 1e-3, "bf16": 4e-3}[dt], f"{o.TYPE_NAMES[qtype]} {o.TYPE_NAMES[qt2]} {dt} case {case} rel-L2 {err}"
-            if t > 64:   # the layer through the dispatcher takes the same call
+            if dispatch.select_moe_path(int(qtype), int(qt2), t) == "grouped":   # the layer through the dispatcher takes the same call
                 assert torch.equal(dispatch.fused_moe_gguf(x, w13d, w2d, _dev(wts), _dev(ids), qtype, qt2, "silu"), got)
-            if dt == "f16" and qt2 == qtype and case in (0, 2):   # the other activation the reference's MoE models use
-                h = ops.ggml_moe_a8(x, w13d, sorted_ids, expert_ids, post, qtype, 2 * inner, top_k, t, block_size=block)
-                y = ops.ggml_moe_a8(h, w2d, sorted_ids, expert_ids, post, qt2, hid, 1, pairs, activation="gelu", block_size=block)
+            if dt == "f16" and qt2 == qtype and case in (0, 2, 4):   # the other activation the reference's MoE models use
+                h = ops.ggml_moe_a8(x, w13d, sorted_ids, expert_ids, post, qtype, 2 * inner, top_k, t, block_size=sort_block)
+                y = ops.ggml_moe_a8(h, w2d, sorted_ids, expert_ids, post, qt2, hid, 1, pairs, activation="gelu", block_size=sort_block)
                 want_g = torch.empty((t, hid), dtype=x.dtype, device="cuda")
                 ops.moe_weighted_sum(y.reshape(t, top_k, hid), _dev(wts), want_g)
                 got_g = ops.moe_mmq_layer(x, w13d, w2d, _dev(wts), _dev(ids), qtype, qt2, "gelu")

@@ -74,6 +74,8 @@ _SIGNATURES = {
                                       _c.c_void_p, _c.c_int64, _c.c_void_p, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64,
                                       _c.c_int, _c.c_int64, _c.c_void_p]),
     "gguf_moe_mmq_layer_takes": (_c.c_int, [_c.c_int, _c.c_int, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64]),
+    "gguf_moe_mmq_layer_workspace_bytes": (_c.c_int64, [_c.c_int, _c.c_int, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64,
+                                                        _c.c_int]),
     "gguf_moe_mmq_layer": (_c.c_int, [_c.c_void_p, _c.c_int, _c.c_void_p, _c.c_int, _c.c_void_p, _c.c_int, _c.c_void_p, _c.c_void_p,
                                       _c.c_void_p, _c.c_int64, _c.c_void_p, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64, _c.c_int64,
                                       _c.c_int, _c.c_int64, _c.c_void_p]),

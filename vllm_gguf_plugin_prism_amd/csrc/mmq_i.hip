@@ -96,5 +96,20 @@ int mmq_int(const void* W, const void* ws, void* Y, int dtype, int type, int M, 
   return GGUF_NOT_TAKEN;
 }
 
+// The grouped MoE contraction on the integer engine, rows in slot order (mmq_i_core.h, MmqiMoe); block = 128 slots.
+int mmq_int_moe(const void* W, const void* ws, void* Y, int dtype, int type, int slots, int N, int K, const int32_t* expert_ids,
+                const int32_t* num_tokens_post_padded, int64_t expert_stride, hipStream_t s) {
+  const MmqiMoe moe = {expert_ids, num_tokens_post_padded, expert_stride, 128};
+  switch (type) {
+#define MMQI_MOE_CASE(ID, FMT) \
+  case ID: GGUF_DISPATCH_DTYPE(dtype, return (mmqi_moe_typed<FMT, scalar_t>(W, ws, Y, slots, N, K, moe, s))); return GGUF_ERR_DTYPE;
+    MMQI_MOE_CASE(T_Q4_0, MQ4_0) MMQI_MOE_CASE(T_Q4_1, MQ4_1) MMQI_MOE_CASE(T_Q5_0, MQ5_0) MMQI_MOE_CASE(T_Q5_1, MQ5_1)
+    MMQI_MOE_CASE(T_Q8_0, MQ8_0) MMQI_MOE_CASE(T_Q2_K, MQ2_K) MMQI_MOE_CASE(T_Q3_K, MQ3_K) MMQI_MOE_CASE(T_Q4_K, MQ4_K)
+    MMQI_MOE_CASE(T_Q5_K, MQ5_K) MMQI_MOE_CASE(T_Q6_K, MQ6_K) MMQI_MOE_CASE(T_IQ4_XS, MIQ4_XS) MMQI_MOE_CASE(T_IQ2_XXS, MIQ2_XXS)
+#undef MMQI_MOE_CASE
+  }
+  return GGUF_NOT_TAKEN;
+}
+
 }  // namespace gguf
 

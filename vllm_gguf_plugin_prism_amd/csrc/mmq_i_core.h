@@ -66,12 +66,22 @@ __host__ __device__ constexpr size_t mmqi_buffer_bytes() {
   return (size_t)(M_T + N_T) * Pitch<F::G, MMQI_KS>::value + (size_t)KB * M_T * 4 * XP + (size_t)KB * N_T * 8 * WPL;
 }
 
+// The grouped MoE contraction on this kernel: the rows of the workspace are the slots of the routing sort in order (slot s
+// holds the quantized activations of the pair sorted_token_ids[s], zeros in padding), so a block of `block` slots is a
+// run of rows like any other and only the weight matrix changes with it; the results are rows in slot order too.
+struct MmqiMoe {
+  const int32_t* expert_ids;              // expert of each block of slots; null = an ordinary product
+  const int32_t* num_tokens_post_padded;  // slots in use: tiles past them leave
+  int64_t expert_stride;                  // bytes between the matrices of two experts
+  int block;                              // slots per block, a multiple of the tile's rows
+};
+
 template <class F, int WM, int WN, int TN, typename T>
 __global__ __launch_bounds__(64 * WM * WN, 2) void mmqi_kernel(const uint8_t* __restrict__ W, const char* __restrict__ ws,
                                                                 int64_t ws_row_bytes, T* __restrict__ Y, float* __restrict__ partial,
                                                                 int M, int N, int K, int Kp, int tiles_m, int whole_tiles,
                                                                 int shared_tiles, int splits, int64_t w_pitch, int64_t ldy,
-                                                                const T* __restrict__ bias) {
+                                                                const T* __restrict__ bias, MmqiMoe moe) {
   constexpr int NT = 64 * WM * WN;
   constexpr int KS = MMQI_KS, KB = KS / 32, GR = KS / 16;
   constexpr int LDK = Pitch<F::G, KS>::value;
@@ -102,6 +112,12 @@ __global__ __launch_bounds__(64 * WM * WN, 2) void mmqi_kernel(const uint8_t* __
   const int split = wg < whole_tiles ? 0 : sw / shared_tiles;
   const int nsplit = wg < whole_tiles ? 1 : splits;
   const int m_base = (tile % tiles_m) * M_T, n_base = (tile / tiles_m) * N_T;
+  if (moe.expert_ids) {
+    if (m_base >= moe.num_tokens_post_padded[0]) return;
+    const int e = moe.expert_ids[m_base / moe.block];
+    if (e < 0 || e > 255) return;                    // the reference's guard on expert ids (moe.cuh:33)
+    W += (int64_t)e * moe.expert_stride;
+  }
   const int nkb_total = K >> 5;
   const int nsteps = (K + KS - 1) / KS;
   const int per_split = (nsteps + nsplit - 1) / nsplit;
@@ -373,7 +389,7 @@ MmqiPlan mmq_int_plan(int M, int N, int K, int64_t partial_bytes_available, bool
 
 template <class F, int WM, int WN, int TN, typename T>
 static void launch_mmqi(const void* W, const void* ws, void* Y, int M, int N, int K, hipStream_t stream, const MmqiPlan& p, float* partial,
-                        const LinearArgs& la) {
+                        const LinearArgs& la, const MmqiMoe& moe = MmqiMoe{nullptr, nullptr, 0, 0}) {
   const int64_t w_pitch = la.w_pitch ? la.w_pitch : (int64_t)(K / F::QK) * F::BS, ldy = la.ldy ? la.ldy : (int64_t)N;
   constexpr int M_T = 32 * WM, N_T = 32 * WN * TN;
   constexpr size_t lds = 2 * mmqi_buffer_bytes<F, M_T, N_T>();
@@ -385,7 +401,7 @@ static void launch_mmqi(const void* W, const void* ws, void* Y, int M, int N, in
   const int tiles_m = (M + M_T - 1) / M_T;
   hipLaunchKernelGGL(kern, dim3(p.whole + p.shared * p.splits), dim3(64 * WM * WN), lds, stream, (const uint8_t*)W, (const char*)ws,
                      q8_row_bytes(K), (T*)Y, partial, M, N, K, (int)q8_kp(K), tiles_m, p.whole, p.shared > 0 ? p.shared : 1, p.splits, w_pitch,
-                     ldy, (const T*)la.bias);
+                     ldy, (const T*)la.bias, moe);
   if (p.shared > 0)
     hipLaunchKernelGGL((mmqi_reduce_kernel<M_T, N_T, T>), dim3(p.shared, M_T * N_T / 1024), dim3(256), 0, stream, partial, (T*)Y, M, N,
                        tiles_m, p.whole, p.splits, ldy, (const T*)la.bias);
@@ -406,6 +422,16 @@ static int mmqi_typed(const void* W, const void* ws, void* Y, int M, int N, int 
   else if (p.cfg == 1) launch_mmqi<F, 2, 2, 2, T>(W, ws, Y, M, N, K, stream, p, partial, la);   // 64 x 128
   else if (p.cfg == 3) launch_mmqi<F, 4, 2, 1, T>(W, ws, Y, M, N, K, stream, p, partial, la);   // 128 x 64, eight waves
   else if constexpr (MmqiWide<F>::ok) launch_mmqi<F, 8, 1, 4, T>(W, ws, Y, M, N, K, stream, p, partial, la);   // 256 x 128
+  return launch_status();
+}
+
+// The grouped contraction over `slots` rows in slot order (see MmqiMoe): 128 x 64 tiles, one block of 128 slots per row
+// of tiles, every tile whole (the tiles of blocks past the padded total leave at once).
+template <class F, typename T>
+static int mmqi_moe_typed(const void* W, const void* ws, void* Y, int slots, int N, int K, const MmqiMoe& moe, hipStream_t stream) {
+  const MmqiPlan p = {0, (slots / 128) * ((N + 63) / 64), 0, 1};
+  if (p.whole == 0) return GGUF_OK;
+  launch_mmqi<F, 4, 1, 2, T>(W, ws, Y, slots / 128 * 128, N, K, stream, p, nullptr, LinearArgs(), moe);
   return launch_status();
 }
 

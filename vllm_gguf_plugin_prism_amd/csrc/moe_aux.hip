@@ -25,7 +25,8 @@ constexpr int ALIGN_MAX_EXPERTS = 1024;
 __device__ __forceinline__ void moe_align_body(const int32_t* __restrict__ topk_ids, int numel, int num_experts, int block,
                                                int32_t* __restrict__ sorted_ids, int sorted_capacity,
                                                int32_t* __restrict__ expert_ids, int expert_capacity,
-                                               int32_t* __restrict__ num_post_padded, int* lds) {
+                                               int32_t* __restrict__ num_post_padded, int* lds,
+                                               int32_t* __restrict__ slot_of_pair = nullptr) {
   int* start = lds;                          // [E] pairs of the expert, then the first slot of its run
   int* cursor = lds + num_experts;           // [ALIGN_WAVES][E] per-wave counts, then per-wave cursors
   __shared__ int total_padded;
@@ -35,6 +36,8 @@ __device__ __forceinline__ void moe_align_body(const int32_t* __restrict__ topk_
   int* mine = cursor + wave * num_experts;
 
   for (int i = tid; i < sorted_capacity; i += ALIGN_THREADS) sorted_ids[i] = numel;
+  if (slot_of_pair)   // the inverse of the sort: -1 for a pair whose expert id names no expert
+    for (int i = tid; i < numel; i += ALIGN_THREADS) slot_of_pair[i] = -1;
   for (int e = lane; e < num_experts; e += 64) mine[e] = 0;
   for (int i = w_begin + lane; i < w_end; i += 64) {
     const int e = topk_ids[i];
@@ -95,6 +98,7 @@ __device__ __forceinline__ void moe_align_body(const int32_t* __restrict__ topk_
       const int below = __popcll(same & ((1ull << lane) - 1));
       const int pos = mine[e] + below;
       if (pos < sorted_capacity) sorted_ids[pos] = i;
+      if (slot_of_pair && pos < sorted_capacity) slot_of_pair[i] = pos;
       if (below == 0) mine[e] = pos + __popcll(same);   // one lane per expert moves the cursor; read above, written here
     }
   }
@@ -107,6 +111,39 @@ __global__ __launch_bounds__(ALIGN_THREADS) void moe_align_kernel(const int32_t*
                                                                   int32_t* __restrict__ num_post_padded) {
   extern __shared__ int lds[];
   moe_align_body(topk_ids, numel, num_experts, block, sorted_ids, sorted_capacity, expert_ids, expert_capacity, num_post_padded, lds);
+}
+
+__global__ __launch_bounds__(ALIGN_THREADS) void moe_align_inverse_kernel(const int32_t* __restrict__ topk_ids, int numel, int num_experts,
+                                                                          int block, int32_t* __restrict__ sorted_ids, int sorted_capacity,
+                                                                          int32_t* __restrict__ expert_ids, int expert_capacity,
+                                                                          int32_t* __restrict__ num_post_padded,
+                                                                          int32_t* __restrict__ slot_of_pair) {
+  extern __shared__ int lds[];
+  moe_align_body(topk_ids, numel, num_experts, block, sorted_ids, sorted_capacity, expert_ids, expert_capacity, num_post_padded, lds,
+                 slot_of_pair);
+}
+
+// Row s of the workspace = the q8_1 quantisation of the token row behind slot s of the sort (zeros in padding slots; slots
+// past the padded total are left alone): the activations in the order in which the grouped contraction walks them.
+template <typename T>
+__global__ __launch_bounds__(256) void moe_gather_quantize_kernel(const T* __restrict__ x, char* __restrict__ ws, int K, int Kp,
+                                                                  int64_t row_bytes, const int32_t* __restrict__ sorted_ids,
+                                                                  const int32_t* __restrict__ num_post_padded, int numel, int top_k) {
+  const int t = blockIdx.x * 256 + threadIdx.x;   // one thread per 8 values of the padded row
+  const int s = blockIdx.y;
+  if (t * 8 >= Kp || s >= num_post_padded[0]) return;
+  const int pair = sorted_ids[s];
+  if (pair < numel) {
+    q8_1_quantize_thread<T>(x + (int64_t)(pair / top_k) * K, ws + (int64_t)s * row_bytes, K, Kp, row_bytes, ACT_NONE, 0, t, nullptr);
+  } else {
+    char* row = ws + (int64_t)s * row_bytes;
+    *(uint2*)(row + 8 * t) = make_uint2(0, 0);
+    if ((t & 3) == 0) {
+      float* fd = (float*)(row + Kp);
+      const int b = t >> 2, nb = Kp / 32;
+      fd[b] = 0.0f; fd[nb + b] = 0.0f; fd[2 * nb + b] = 0.0f;
+    }
+  }
 }
 
 // The two preparations of a MoE layer on tiles in one launch: workgroup 0 sorts the routing, the others quantize the
@@ -135,14 +172,17 @@ __global__ __launch_bounds__(ALIGN_THREADS) void moe_prepare_kernel(const T* __r
 template <typename T>
 __global__ __launch_bounds__(256) void moe_weighted_sum_kernel(const T* __restrict__ Y, const float* __restrict__ w,
                                                                T* __restrict__ out, int top_k, int64_t N,
-                                                               const int32_t* __restrict__ ids, int num_experts) {
+                                                               const int32_t* __restrict__ ids, int num_experts,
+                                                               const int32_t* __restrict__ slot_of_pair) {
   const int64_t t = blockIdx.y;
   for (int64_t n = (int64_t)blockIdx.x * 256 + threadIdx.x; n < N; n += (int64_t)gridDim.x * 256) {
     float acc = 0.0f;
     for (int k = 0; k < top_k; ++k) {
       // (ids given: a pair whose id names no expert has a row of zeros, whatever Y holds there)
-      const bool live = !ids || (unsigned)ids[t * top_k + k] < (unsigned)num_experts;
-      const T p = from_f32<T>((live ? to_f32<T>(Y[(t * top_k + k) * N + n]) : 0.0f) * w[t * top_k + k]);
+      // (slot_of_pair given: the rows of Y are in the order of the routing sort; -1 = the pair was dropped)
+      const int64_t row = slot_of_pair ? (int64_t)slot_of_pair[t * top_k + k] : t * top_k + k;
+      const bool live = row >= 0 && (!ids || (unsigned)ids[t * top_k + k] < (unsigned)num_experts);
+      const T p = from_f32<T>((live ? to_f32<T>(Y[row * N + n]) : 0.0f) * w[t * top_k + k]);
       acc += to_f32<T>(p);
     }
     out[t * N + n] = from_f32<T>(acc);
@@ -150,14 +190,14 @@ __global__ __launch_bounds__(256) void moe_weighted_sum_kernel(const T* __restri
 }
 
 int moe_weighted_sum_live(const void* Y, const float* topk_weights, const int32_t* topk_ids, int num_experts, void* out, int dtype,
-                          int64_t tokens, int64_t top_k, int64_t N, hipStream_t s) {
+                          int64_t tokens, int64_t top_k, int64_t N, hipStream_t s, const int32_t* slot_of_pair) {
   const unsigned gx = (unsigned)((N + 255) / 256 < 64 ? (N + 255) / 256 : 64);
   for (int64_t t0 = 0; t0 < tokens; t0 += 65535) {
     const unsigned gy = (unsigned)(tokens - t0 < 65535 ? tokens - t0 : 65535);
     GGUF_DISPATCH_DTYPE(dtype, hipLaunchKernelGGL((moe_weighted_sum_kernel<scalar_t>), dim3(gx, gy), dim3(256), 0, s,
-                                                  (const scalar_t*)Y + t0 * top_k * N, topk_weights + t0 * top_k,
+                                                  (const scalar_t*)Y + (slot_of_pair ? 0 : t0 * top_k * N), topk_weights + t0 * top_k,
                                                   (scalar_t*)out + t0 * N, (int)top_k, N, topk_ids ? topk_ids + t0 * top_k : nullptr,
-                                                  num_experts));
+                                                  num_experts, slot_of_pair ? slot_of_pair + t0 * top_k : nullptr));
   }
   return launch_status();
 }
@@ -174,6 +214,23 @@ int moe_prepare(const void* X, int xdtype, void* q8x, int tokens, int K, const i
   GGUF_DISPATCH_DTYPE(xdtype, hipLaunchKernelGGL(moe_prepare_kernel<scalar_t>, dim3(grid), dim3(ALIGN_THREADS), lds, s, (const scalar_t*)X,
                                                  (char*)q8x, K, Kp, q8_row_bytes(K), tokens, topk_ids, numel, num_experts, block, sorted_ids,
                                                  sorted_capacity, expert_ids, expert_capacity, num_post_padded));
+  return launch_status();
+}
+
+// The routing sort with its inverse, then the rows of X quantized into slot order (two launches; sizes checked by the caller)
+int moe_prepare_sorted(const void* X, int xdtype, void* q8x_sorted, int K, const int32_t* topk_ids, int numel, int top_k, int num_experts,
+                       int block, int32_t* sorted_ids, int sorted_capacity, int32_t* expert_ids, int expert_capacity,
+                       int32_t* num_post_padded, int32_t* slot_of_pair, hipStream_t s) {
+  const size_t lds = (size_t)(1 + ALIGN_WAVES) * num_experts * sizeof(int);
+  if (lds > 65536) return GGUF_NOT_TAKEN;
+  hipLaunchKernelGGL(moe_align_inverse_kernel, dim3(1), dim3(ALIGN_THREADS), lds, s, topk_ids, numel, num_experts, block, sorted_ids,
+                     sorted_capacity, expert_ids, expert_capacity, num_post_padded, slot_of_pair);
+  const int Kp = (int)q8_kp(K);
+  const int slots = sorted_capacity / block * block;
+  if (slots > 65535) return GGUF_ERR_SHAPE;
+  GGUF_DISPATCH_DTYPE(xdtype, hipLaunchKernelGGL(moe_gather_quantize_kernel<scalar_t>, dim3((Kp / 8 + 255) / 256, slots), dim3(256), 0, s,
+                                                 (const scalar_t*)X, (char*)q8x_sorted, K, Kp, q8_row_bytes(K), sorted_ids, num_post_padded,
+                                                 numel, top_k));
   return launch_status();
 }
 
@@ -208,5 +265,5 @@ extern "C" int gguf_moe_weighted_sum(const void* Y, const float* topk_weights, v
   if (dtype < 0 || dtype > 2) return GGUF_ERR_DTYPE;
   if (tokens == 0 || N == 0) return GGUF_OK;
   if (!Y || !topk_weights || !out) return GGUF_ERR_NULL;
-  return moe_weighted_sum_live(Y, topk_weights, nullptr, 0, out, dtype, tokens, top_k, N, (hipStream_t)stream);
+  return moe_weighted_sum_live(Y, topk_weights, nullptr, 0, out, dtype, tokens, top_k, N, (hipStream_t)stream, nullptr);
 }

@@ -30,6 +30,9 @@ int64_t moe_tiles_layer_workspace(int64_t tokens, int64_t top_k, int64_t H, int6
 int moe_tiles_layer(const void* X, int xdtype, void* workspace, const void* W13, int type13, const void* W2, int type2, const int32_t* topk_ids,
                     const float* topk_w, void* out, int H, int I, int N_out, int top_k, int tokens, int act, int num_experts, bool vec_sums,
                     int block, hipStream_t s);
+int64_t moe_sorted_layer_workspace(int64_t tokens, int64_t top_k, int64_t H, int64_t I, int64_t N_out, int64_t num_experts, int elt);
+int moe_sorted_layer(const void* X, int xdtype, void* workspace, const void* W13, int type13, const void* W2, int type2, const int32_t* topk_ids,
+                     const float* topk_w, void* out, int H, int I, int N_out, int top_k, int tokens, int act, int num_experts, hipStream_t s);
 
 struct MoeUpArgs {
   const int32_t* topk_ids;
@@ -482,7 +485,16 @@ extern "C" int gguf_moe_vec_layer(const void* X, int xdtype, const void* W13, in
 
 // The same four launches with the grouped operator's arithmetic (gguf_moe_mmq_block twice and the weighted sum): what a
 // layer with more than 64 tokens takes -- on blocks of 16 slots while its experts see at most 16 pairs each on average and
-// both formats have such tiles (returns 1), else on the reference's blocks of 32 (returns 2).
+// both formats have such tiles (returns 1), else on the reference's blocks of 32 (returns 2); from MOE_SORTED_MIN_PAIRS
+// pairs per expert on, where one of the formats changes its scale every 16 values (Q2_K, Q3_K, Q6_K: the 32-slot kernel
+// multiplies those at half rate), the layer in slot order on the pipelined integer engine with blocks of 128 slots
+// (returns 3).  Measured, 96 .. 512 pairs per expert: Q4_K / Q6_K layers of 8 experts [4096,14336] 22 - 26 % faster, of
+// 64 experts [2048,1024] -3 .. +17 %; Q4_0 layers of 8 experts 1 - 13 % faster but of 64 experts 6 - 25 % slower (half of
+// a 128-slot block is padding on average and the first GEMM's result makes a round trip), hence the condition.
+#ifndef MOE_SORTED_MIN_PAIRS_VALUE
+#define MOE_SORTED_MIN_PAIRS_VALUE 96
+#endif
+static constexpr int64_t MOE_SORTED_MIN_PAIRS = MOE_SORTED_MIN_PAIRS_VALUE;
 extern "C" int gguf_moe_mmq_layer_takes(int type13, int type2, int64_t H, int64_t I, int64_t N_out, int64_t top_k, int64_t tokens,
                                         int64_t num_experts) {
   using namespace gguf;
@@ -491,7 +503,20 @@ extern "C" int gguf_moe_mmq_layer_takes(int type13, int type2, int64_t H, int64_
   const int qk13 = block_elems(type13), qk2 = block_elems(type2);
   if (qk13 == 0 || qk2 == 0 || H % qk13 != 0 || I % qk2 != 0) return 0;
   const int block = moe_tiles_layer_block(type13, type2, tokens * top_k, num_experts, I, false);
+  const auto deep16 = [](int t) { return t == T_Q2_K || t == T_Q3_K || t == T_Q6_K; };
+  if (block != 0 && (deep16(type13) || deep16(type2)) && tokens * top_k >= MOE_SORTED_MIN_PAIRS * num_experts &&
+      tokens * top_k + 127 * num_experts <= 65535)   // (a grid row per slot)
+    return 3;
   return block == 16 ? 1 : block == 32 ? 2 : 0;
+}
+
+extern "C" int64_t gguf_moe_mmq_layer_workspace_bytes(int type13, int type2, int64_t tokens, int64_t top_k, int64_t H, int64_t I, int64_t N_out,
+                                                      int64_t num_experts, int xdtype) {
+  using namespace gguf;
+  const int route = gguf_moe_mmq_layer_takes(type13, type2, H, I, N_out, top_k, tokens, num_experts);
+  const int elt = xdtype == GGUF_DTYPE_F32 ? 4 : 2;
+  if (route == 3) return moe_sorted_layer_workspace(tokens, top_k, H, I, N_out, num_experts, elt);
+  return route ? moe_tiles_layer_workspace(tokens, top_k, H, I, N_out, num_experts, elt, route == 1 ? 16 : 32) : 0;
 }
 
 extern "C" int gguf_moe_mmq_layer(const void* X, int xdtype, const void* W13, int type13, const void* W2, int type2, const int32_t* topk_ids,
@@ -506,6 +531,11 @@ extern "C" int gguf_moe_mmq_layer(const void* X, int xdtype, const void* W13, in
   if (!route) return GGUF_ERR_SHAPE;
   if (!X || !W13 || !W2 || !topk_ids || !topk_weights || !workspace || !out) return GGUF_ERR_NULL;
   if (((uintptr_t)W13 | (uintptr_t)W2) & 1) return GGUF_ERR_SHAPE;   // packed blocks sit at even addresses
+  if (route == 3) {
+    if (workspace_bytes < moe_sorted_layer_workspace(tokens, top_k, H, I, N_out, num_experts, xdtype == GGUF_DTYPE_F32 ? 4 : 2)) return GGUF_ERR_WORKSPACE;
+    return moe_sorted_layer(X, xdtype, workspace, W13, type13, W2, type2, topk_ids, topk_weights, out, (int)H, (int)I, (int)N_out, (int)top_k,
+                            (int)tokens, act, (int)num_experts, (hipStream_t)stream);
+  }
   const int block = route == 1 ? 16 : 32;
   if (workspace_bytes < moe_tiles_layer_workspace(tokens, top_k, H, I, N_out, num_experts, xdtype == GGUF_DTYPE_F32 ? 4 : 2, block))
     return GGUF_ERR_WORKSPACE;

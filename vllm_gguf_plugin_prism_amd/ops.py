@@ -398,7 +398,12 @@ def _moe_layer(entry, X, W13, W2, topk_weights, topk_ids, quant_type, quant_type
     L = _lib.lib()
     with _on_device_of(X):
         out = output if output is not None else torch.empty((tokens, n_out), dtype=X.dtype, device=W2.device)
-        nbytes = max(16, L.gguf_moe_vec_layer_workspace_bytes(tokens, top_k, hidden, inner, n_out, W13.shape[0], _code(X.dtype)))
+        if entry == "gguf_moe_mmq_layer":
+            nbytes = L.gguf_moe_mmq_layer_workspace_bytes(int(quant_type), int(quant_type2), tokens, top_k, hidden, inner, n_out, W13.shape[0],
+                                                          _code(X.dtype))
+        else:
+            nbytes = L.gguf_moe_vec_layer_workspace_bytes(tokens, top_k, hidden, inner, n_out, W13.shape[0], _code(X.dtype))
+        nbytes = max(16, nbytes)
         ws = torch.empty(nbytes, dtype=torch.uint8, device=X.device)
         rc = getattr(L, entry)(X.data_ptr(), _code(X.dtype), W13.data_ptr(), int(quant_type), W2.data_ptr(), int(quant_type2),
                                topk_ids.data_ptr(), w.data_ptr(), ws.data_ptr(), nbytes, out.data_ptr(), hidden, inner, n_out, top_k,
