@@ -343,13 +343,16 @@ struct MQ5_K {  // vecdotq.cuh:415-441, 1325-1415: Q4_K with a fifth bit, bit j 
   static __device__ __forceinline__ void offs8(const uint8_t* row, int b8, int nkb, float (&cs)[8], float (&cm)[8]) { k4_offs8(row, BS, b8, nkb, 16.0f, cs, cm); }
 };
 
-__device__ __forceinline__ int lut16q(uint32_t idx) {  // kvalues_iq4nl lookup of four indices, one per byte
+// kvalues_iq4nl lookup of the four 4-bit indices that the bytes of w hold at bit SH (0 or 4): byte permutes pick out of
+// either half of the table by bits 0-2, a third takes byte i of the half that bit 3 of index i names
+template <int SH>
+__device__ __forceinline__ int lut16q(uint32_t w) {
   constexpr uint32_t T0 = 0xBFAD9881u, T1 = 0xF6EADDCFu, T2 = 0x26190D01u, T3 = 0x71594535u;
-  const uint32_t sel = idx & 0x07070707u;
+  const uint32_t sel = (SH ? w >> SH : w) & 0x07070707u;
   const uint32_t lo = __builtin_amdgcn_perm(T1, T0, sel);
   const uint32_t hi = __builtin_amdgcn_perm(T3, T2, sel);
-  const uint32_t m = ((idx >> 3) & 0x01010101u) * 0xFFu;
-  return (int)((hi & m) | (lo & ~m));
+  const uint32_t pick = ((w >> (SH + 1)) & 0x04040404u) | 0x03020100u;
+  return (int)__builtin_amdgcn_perm(hi, lo, pick);
 }
 
 struct MIQ4_XS {  // extension: the reference has no MMQ tiles for i-quants (gguf_kernel.cu:236-287)
@@ -367,7 +370,7 @@ struct MIQ4_XS {  // extension: the reference has no MMQ tiles for i-quants (ggu
     const int ib = kb & 7;
     const uint32_t w[4] = {r.v.x, r.v.y, r.v.z, r.v.w};
 #pragma unroll
-    for (int i = 0; i < 4; ++i) { q[i] = (uint32_t)lut16q(w[i] & 0x0F0F0F0Fu); q[4 + i] = (uint32_t)lut16q((w[i] >> 4) & 0x0F0F0F0Fu); }
+    for (int i = 0; i < 4; ++i) { q[i] = (uint32_t)lut16q<0>(w[i]); q[4 + i] = (uint32_t)lut16q<4>(w[i]); }
     const int ls = (int)(((r.hdr.y >> (4 * ib)) & 0xF) | ((((r.hdr.x >> 16) >> (2 * ib)) & 3) << 4));
     s0 = (float)__builtin_bit_cast(_Float16, (uint16_t)(r.hdr.x & 0xFFFF)) * (float)(ls - 32);
     s1 = s0; mn = 0.0f;

@@ -222,12 +222,16 @@ struct FmtQ6_K {
 };
 
 // 16-entry signed byte table lookup of four 4-bit indices held one per byte
-__device__ __forceinline__ int lut16(uint32_t idx, uint32_t t0, uint32_t t1, uint32_t t2, uint32_t t3) {
-  const uint32_t sel = idx & 0x07070707u;
+// Bytes of `w`, shifted right by SH (0 or 4), hold four 4-bit table indices; the 16 table bytes are t0..t3.  Bits 0-2 pick a
+// byte out of either half of the table, and a third byte permute takes byte i of the half that bit 3 of index i names:
+// its selector is i, or 4 + i, which is (w >> (SH + 1)) & 4 in every byte on top of 0x03020100.
+template <int SH>
+__device__ __forceinline__ int lut16(uint32_t w, uint32_t t0, uint32_t t1, uint32_t t2, uint32_t t3) {
+  const uint32_t sel = (SH ? w >> SH : w) & 0x07070707u;
   const uint32_t lo = __builtin_amdgcn_perm(t1, t0, sel);
   const uint32_t hi = __builtin_amdgcn_perm(t3, t2, sel);
-  const uint32_t m = ((idx >> 3) & 0x01010101u) * 0xFFu;
-  return (int)((hi & m) | (lo & ~m));
+  const uint32_t pick = ((w >> (SH + 1)) & 0x04040404u) | 0x03020100u;
+  return (int)__builtin_amdgcn_perm(hi, lo, pick);
 }
 
 // ------------------------------------------------------------------ IQ4_XS (vecdotq.cuh:1791-1811)
@@ -256,8 +260,8 @@ struct FmtIQ4_XS {
     int s = 0;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      s = dot4(lut16(qq[i] & 0x0F0F0F0Fu, T0, T1, T2, T3), al[i], s);
-      s = dot4(lut16((qq[i] >> 4) & 0x0F0F0F0Fu, T0, T1, T2, T3), ah[i], s);
+      s = dot4(lut16<0>(qq[i], T0, T1, T2, T3), al[i], s);
+      s = dot4(lut16<4>(qq[i], T0, T1, T2, T3), ah[i], s);
     }
     return dl * x.d * (float)s;
   }
@@ -496,8 +500,8 @@ struct FmtIQ4_NL {
     int s = 0;
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
-      s = dot4(lut16(qq[i] & 0x0F0F0F0Fu, T0, T1, T2, T3), al[i], s);
-      s = dot4(lut16((qq[i] >> 4) & 0x0F0F0F0Fu, T0, T1, T2, T3), ah[i], s);
+      s = dot4(lut16<0>(qq[i], T0, T1, T2, T3), al[i], s);
+      s = dot4(lut16<4>(qq[i], T0, T1, T2, T3), ah[i], s);
     }
     return h2f(r.d) * x.d * (float)s;
   }
