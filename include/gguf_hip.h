@@ -268,8 +268,8 @@ int gguf_moe_vec_layer(const void* X, int xdtype, const void* W13, int type13, c
  *   2  the reference's blocks of 32 slots: every other layer of two tile formats (the twelve of ggml_moe_a8);
  *   0  not served (num_experts outside 1..256, I no multiple of 32 or of type2's block, a format without tiles, more
  *      than about two million pairs): gguf_moe_mmq_layer returns GGUF_ERR_SHAPE.
- *   3  experts that see 96 pairs or more each on average: six launches on the pipelined integer engine of gguf_mmq
- *      with blocks of 128 slots -- the routing sort with its inverse, the rows of X quantized into slot order, the
+ *   3  experts that see 64 pairs or more each on average, one of the formats being Q2_K, Q3_K or Q6_K: six launches on
+ *      the pipelined integer engine of gguf_mmq with blocks of 64 slots -- the routing sort with its inverse, the rows of X quantized into slot order, the
  *      first GEMM as a dense product over runs of rows (only the weight matrix changes from block to block), its
  *      result quantized with the activation, the second GEMM, and the weighted sum gathering its rows through the
  *      inverse of the sort.

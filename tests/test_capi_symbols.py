@@ -164,13 +164,13 @@ def test_two_launch_moe_layer_states_which_shapes_it_serves():
     assert h.gguf_moe_vec_layer_takes(2, 12, 2048, 1120, 2048, 8, 1, 64) == 0
     assert h.gguf_moe_vec_layer_workspace_bytes(3, 8, 2048, 1024, 2048, 64, 1) >= 24 * h.gguf_q8_1_row_bytes(1024) + 3 * h.gguf_q8_1_row_bytes(2048)
     # the grouped operator's arithmetic: 1 = blocks of 16 slots (up to 16 pairs per expert on average, formats with such
-    # tiles), 2 = blocks of 32, 3 = blocks of 128 in slot order on the dense engine; at most 256 experts
+    # tiles), 2 = blocks of 32, 3 = blocks of 64 in slot order on the dense engine; at most 256 experts
     assert h.gguf_moe_mmq_layer_takes(2, 2, 2048, 1024, 2048, 8, 96, 64) == 1
     assert h.gguf_moe_mmq_layer_takes(2, 2, 2048, 1024, 2048, 8, 128, 64) == 1
     assert h.gguf_moe_mmq_layer_takes(2, 2, 2048, 1024, 2048, 8, 129, 64) == 2
     assert h.gguf_moe_mmq_layer_takes(2, 2, 2048, 1024, 2048, 8, 512, 64) == 2
     assert h.gguf_moe_mmq_layer_takes(2, 2, 2048, 1024, 2048, 8, 2048, 64) == 2
-    assert h.gguf_moe_mmq_layer_takes(2, 14, 2048, 1024, 2048, 8, 2048, 64) == 3     # 256 pairs per expert, a 16-deep format: blocks of 128 on the dense engine
+    assert h.gguf_moe_mmq_layer_takes(2, 14, 2048, 1024, 2048, 8, 2048, 64) == 3     # 256 pairs per expert, a 16-deep format: blocks of 64 on the dense engine
     assert h.gguf_moe_mmq_layer_takes(12, 14, 4096, 14336, 4096, 2, 512, 8) == 3
     assert h.gguf_moe_mmq_layer_workspace_bytes(2, 2, 96, 8, 2048, 1024, 2048, 64, 1) > 0
     assert h.gguf_moe_mmq_layer_workspace_bytes(2, 14, 2048, 8, 2048, 1024, 2048, 64, 1) > h.gguf_moe_mmq_layer_workspace_bytes(2, 2, 2048, 8, 2048, 1024, 2048, 64, 1)

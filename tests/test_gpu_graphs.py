@@ -126,22 +126,25 @@ def test_two_launch_moe_layer_replays_match_eager():
         assert torch.equal(out, eager)
 
 
-def test_tile_route_moe_layer_replays_match_eager():
+@pytest.mark.parametrize("e,t,qtype2,route", [(16, 70, o.Q4_K, 1), (4, 160, o.Q6_K, 3)])
+def test_tile_route_moe_layer_replays_match_eager(e, t, qtype2, route):
     """dispatch.fused_moe_gguf above 64 tokens with few pairs per expert (quantize, routing sort, both expert GEMMs on
     16-slot tiles and the weighted sum, all inside one call with a workspace allocated per call) captured and replayed
-    with eager work in between; the routing changes between replays as well."""
-    from vllm_gguf_plugin_prism_amd import dispatch, ops
+    with eager work in between; the routing changes between replays as well.  The second case is the layer in slot
+    order on the dense engine (80 pairs per expert, a Q6_K down projection): six launches, its padding slots and the
+    inverse of the sort rewritten by every replay."""
+    from vllm_gguf_plugin_prism_amd import _lib, dispatch, ops
     rng = np.random.default_rng(92)
-    e, hid, inner, t, top_k, qtype = 16, 512, 256, 70, 2, o.Q4_K
+    hid, inner, top_k, qtype = 512, 256, 2, o.Q4_K
     w13 = _dev(np.stack([o.make_weights(rng, qtype, 2 * inner, hid) for _ in range(e)]))
-    w2 = _dev(np.stack([o.make_weights(rng, qtype, hid, inner) for _ in range(e)]))
-    assert ops.moe_mmq_layer_takes(qtype, qtype, hid, inner, hid, top_k, t, e)
+    w2 = _dev(np.stack([o.make_weights(rng, qtype2, hid, inner) for _ in range(e)]))
+    assert _lib.lib().gguf_moe_mmq_layer_takes(int(qtype), int(qtype2), hid, inner, hid, top_k, t, e) == route
     routes = [_dev(np.stack([rng.choice(e, size=top_k, replace=False) for _ in range(t)]).astype(np.int32)) for _ in range(3)]
     ids = routes[0].clone()
     wts = torch.rand(t, top_k, device="cuda")
     xs = [torch.randn(t, hid, dtype=torch.float16, device="cuda") * 0.05 for _ in range(3)]
     x = xs[0].clone()
-    fn = lambda: dispatch.fused_moe_gguf(x, w13, w2, wts, ids, qtype, qtype, "silu")
+    fn = lambda: dispatch.fused_moe_gguf(x, w13, w2, wts, ids, qtype, qtype2, "silu")
     graph, out = _capture(fn)
     for xi, ri in zip(xs, routes):
         x.copy_(xi)

@@ -619,7 +619,7 @@ def test_moe_layer_on_grouped_tiles_matches_the_separate_steps(qtype, dt):
     """moe_mmq_layer (the four launches of the tile route with the grouped operator's arithmetic) against
     moe_align_block_size, ggml_moe_a8 twice (the second with the activation) and moe_weighted_sum on the same block
     size: blocks of 16 slots where the experts see few pairs and the format has such tiles, else the reference's blocks
-    of 32; from 96 pairs per expert on the layer runs in slot order on the dense engine with blocks of 128.  More than 64 tokens, inner sizes that end inside a tile of features, an expert without pairs, a second
+    of 32; from 64 pairs per expert on, layers with a 16-deep format run in slot order on the dense engine with blocks of 64 (cases 4, 5).  More than 64 tokens, inner sizes that end inside a tile of features, an expert without pairs, a second
     format, and a pair whose expert id names no expert (it adds nothing in both)."""
     ops = _ops()
     from vllm_gguf_plugin_prism_amd import _lib, dispatch
@@ -643,7 +643,7 @@ def test_moe_layer_on_grouped_tiles_matches_the_separate_steps(qtype, dt):
             route = _lib.lib().gguf_moe_mmq_layer_takes(int(qtype), int(qt2), hid, inner, hid, top_k, t, e)
             deep16 = bool({int(qtype), int(qt2)} & {o.Q2_K, o.Q3_K, o.Q6_K})   # the dense engine takes layers with a 16-deep format
             assert route == {16: 1, 32: 2, 128: 3 if deep16 else 2}[block], (case, route)
-            # (the route on blocks of 128 slots is compared with the operators on the reference's blocks of 32)
+            # (the route in slot order is compared with the operators on the reference's blocks of 32)
             sort_block = min(block, 32)
             sorted_ids, expert_ids, post = ops.moe_align_block_size(_dev(ids), sort_block, e)
 

@@ -692,7 +692,7 @@ int moe_prepare_sorted(const void* X, int xdtype, void* q8x_sorted, int K, const
                        int block, int32_t* sorted_ids, int sorted_capacity, int32_t* expert_ids, int expert_capacity,
                        int32_t* num_post_padded, int32_t* slot_of_pair, hipStream_t s);   // moe_aux.hip
 int mmq_int_moe(const void* W, const void* ws, void* Y, int dtype, int type, int slots, int N, int K, const int32_t* expert_ids,
-                const int32_t* num_tokens_post_padded, int64_t expert_stride, hipStream_t s);   // mmq_i.hip
+                const int32_t* num_tokens_post_padded, int64_t expert_stride, int block, hipStream_t s);   // mmq_i.hip
 
 int moe_tiles_layer(const void* X, int xdtype, void* workspace, const void* W13, int type13, const void* W2, int type2, const int32_t* topk_ids,
                     const float* topk_w, void* out, int H, int I, int N_out, int top_k, int tokens, int act, int num_experts, bool vec_sums,
@@ -730,22 +730,24 @@ int moe_tiles_layer(const void* X, int xdtype, void* workspace, const void* W13,
 }
 
 // ---- A MoE layer whose experts see many pairs each, on the pipelined integer engine: the routing is sorted into blocks of
-// 128 slots, the rows of X are quantized into slot order, and both expert GEMMs run as the dense product does, a block
+// `block` slots (64), the rows of X are quantized into slot order, and both expert GEMMs run as the dense product does, a block
 // of slots being a run of rows like any other (mmq_i_core.h, MmqiMoe); the intermediate and the result stay in slot
 // order and the weighted sum gathers its rows through the inverse of the sort.  Six launches: sort, quantize, GEMM,
 // quantize with the activation, GEMM, weighted sum.
 // [q8_1 rows of X, slot order][first GEMM's result, slots x 2 I][q8_1 rows of h][second GEMM's result, slots x N_out]
 // [sorted ids, expert ids, padded total, slot of every pair]
-int64_t moe_sorted_layer_workspace(int64_t tokens, int64_t top_k, int64_t H, int64_t I, int64_t N_out, int64_t num_experts, int elt) {
-  const int64_t pairs = tokens * top_k, cap = pairs + num_experts * 127, slots = cap / 128 * 128;
+int64_t moe_sorted_layer_workspace(int64_t tokens, int64_t top_k, int64_t H, int64_t I, int64_t N_out, int64_t num_experts, int elt,
+                                   int block) {
+  const int64_t pairs = tokens * top_k, cap = pairs + num_experts * (block - 1), slots = cap / block * block;
   return up16(slots * q8_row_bytes(H)) + up16(slots * 2 * I * elt) + up16(slots * q8_row_bytes(I)) + up16(slots * N_out * elt) +
-         (cap + cap / 128 + 2 + pairs) * 4;
+         (cap + cap / block + 2 + pairs) * 4;
 }
 
 int moe_sorted_layer(const void* X, int xdtype, void* workspace, const void* W13, int type13, const void* W2, int type2, const int32_t* topk_ids,
-                     const float* topk_w, void* out, int H, int I, int N_out, int top_k, int tokens, int act, int num_experts, hipStream_t s) {
+                     const float* topk_w, void* out, int H, int I, int N_out, int top_k, int tokens, int act, int num_experts, int block,
+                     hipStream_t s) {
   const int pairs = tokens * top_k, elt = xdtype == GGUF_DTYPE_F32 ? 4 : 2;
-  const int64_t cap = (int64_t)pairs + (int64_t)num_experts * 127, slots = cap / 128 * 128, block_cap = cap / 128 + 1;
+  const int64_t cap = (int64_t)pairs + (int64_t)num_experts * (block - 1), slots = cap / block * block, block_cap = cap / block + 1;
   char* q8x = (char*)workspace;
   char* y1 = q8x + up16(slots * q8_row_bytes(H));
   char* q8h = y1 + up16(slots * 2 * I * elt);
@@ -754,14 +756,14 @@ int moe_sorted_layer(const void* X, int xdtype, void* workspace, const void* W13
   int32_t* experts = sorted + cap;
   int32_t* post = experts + block_cap;
   int32_t* slot_of_pair = post + 1;
-  int rc = moe_prepare_sorted(X, xdtype, q8x, H, topk_ids, pairs, top_k, num_experts, 128, sorted, (int)cap, experts, (int)block_cap, post,
+  int rc = moe_prepare_sorted(X, xdtype, q8x, H, topk_ids, pairs, top_k, num_experts, block, sorted, (int)cap, experts, (int)block_cap, post,
                               slot_of_pair, s);
   if (rc != GGUF_OK) return rc;
-  rc = mmq_int_moe(W13, q8x, y1, xdtype, type13, (int)slots, 2 * I, H, experts, post, (int64_t)2 * I * (H / block_elems(type13)) * block_bytes(type13), s);
+  rc = mmq_int_moe(W13, q8x, y1, xdtype, type13, (int)slots, 2 * I, H, experts, post, (int64_t)2 * I * (H / block_elems(type13)) * block_bytes(type13), block, s);
   if (rc != GGUF_OK) return rc == GGUF_NOT_TAKEN ? GGUF_ERR_TYPE : rc;
   rc = quantize_q8_1(y1, xdtype, q8h, slots, I, s, act);     // rows of y1 are [gate | up]: h = T(T(act(gate)) up), quantized
   if (rc != GGUF_OK) return rc;
-  rc = mmq_int_moe(W2, q8h, y2, xdtype, type2, (int)slots, N_out, I, experts, post, (int64_t)N_out * (I / block_elems(type2)) * block_bytes(type2), s);
+  rc = mmq_int_moe(W2, q8h, y2, xdtype, type2, (int)slots, N_out, I, experts, post, (int64_t)N_out * (I / block_elems(type2)) * block_bytes(type2), block, s);
   if (rc != GGUF_OK) return rc == GGUF_NOT_TAKEN ? GGUF_ERR_TYPE : rc;
   return moe_weighted_sum_live(y2, topk_w, nullptr, 0, out, xdtype, tokens, top_k, N_out, s, slot_of_pair);
 }

@@ -96,10 +96,11 @@ int mmq_int(const void* W, const void* ws, void* Y, int dtype, int type, int M, 
   return GGUF_NOT_TAKEN;
 }
 
-// The grouped MoE contraction on the integer engine, rows in slot order (mmq_i_core.h, MmqiMoe); block = 128 slots.
+// The grouped MoE contraction on the integer engine, rows in slot order (mmq_i_core.h, MmqiMoe); blocks of 64 slots.
 int mmq_int_moe(const void* W, const void* ws, void* Y, int dtype, int type, int slots, int N, int K, const int32_t* expert_ids,
-                const int32_t* num_tokens_post_padded, int64_t expert_stride, hipStream_t s) {
-  const MmqiMoe moe = {expert_ids, num_tokens_post_padded, expert_stride, 128};
+                const int32_t* num_tokens_post_padded, int64_t expert_stride, int block, hipStream_t s) {
+  if (block != 64) return GGUF_ERR_SHAPE;
+  const MmqiMoe moe = {expert_ids, num_tokens_post_padded, expert_stride, block};
   switch (type) {
 #define MMQI_MOE_CASE(ID, FMT) \
   case ID: GGUF_DISPATCH_DTYPE(dtype, return (mmqi_moe_typed<FMT, scalar_t>(W, ws, Y, slots, N, K, moe, s))); return GGUF_ERR_DTYPE;

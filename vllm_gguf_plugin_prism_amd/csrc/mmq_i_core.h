@@ -425,13 +425,14 @@ static int mmqi_typed(const void* W, const void* ws, void* Y, int M, int N, int 
   return launch_status();
 }
 
-// The grouped contraction over `slots` rows in slot order (see MmqiMoe): 128 x 64 tiles, one block of 128 slots per row
-// of tiles, every tile whole (the tiles of blocks past the padded total leave at once).
+// The grouped contraction over `slots` rows in slot order (see MmqiMoe): blocks of 64 slots on 64 x 128 tiles, one block
+// per row of tiles, every tile whole (the tiles of blocks past the padded total leave at once).
 template <class F, typename T>
 static int mmqi_moe_typed(const void* W, const void* ws, void* Y, int slots, int N, int K, const MmqiMoe& moe, hipStream_t stream) {
-  const MmqiPlan p = {0, (slots / 128) * ((N + 63) / 64), 0, 1};
+  const int rows = slots / 64 * 64;
+  const MmqiPlan p = {1, (rows / 64) * ((N + 127) / 128), 0, 1};
   if (p.whole == 0) return GGUF_OK;
-  launch_mmqi<F, 4, 1, 2, T>(W, ws, Y, slots / 128 * 128, N, K, stream, p, nullptr, LinearArgs(), moe);
+  launch_mmqi<F, 2, 2, 2, T>(W, ws, Y, rows, N, K, stream, p, nullptr, LinearArgs(), moe);
   return launch_status();
 }
 

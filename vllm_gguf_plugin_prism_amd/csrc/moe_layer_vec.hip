@@ -30,9 +30,10 @@ int64_t moe_tiles_layer_workspace(int64_t tokens, int64_t top_k, int64_t H, int6
 int moe_tiles_layer(const void* X, int xdtype, void* workspace, const void* W13, int type13, const void* W2, int type2, const int32_t* topk_ids,
                     const float* topk_w, void* out, int H, int I, int N_out, int top_k, int tokens, int act, int num_experts, bool vec_sums,
                     int block, hipStream_t s);
-int64_t moe_sorted_layer_workspace(int64_t tokens, int64_t top_k, int64_t H, int64_t I, int64_t N_out, int64_t num_experts, int elt);
+int64_t moe_sorted_layer_workspace(int64_t tokens, int64_t top_k, int64_t H, int64_t I, int64_t N_out, int64_t num_experts, int elt, int block);
 int moe_sorted_layer(const void* X, int xdtype, void* workspace, const void* W13, int type13, const void* W2, int type2, const int32_t* topk_ids,
-                     const float* topk_w, void* out, int H, int I, int N_out, int top_k, int tokens, int act, int num_experts, hipStream_t s);
+                     const float* topk_w, void* out, int H, int I, int N_out, int top_k, int tokens, int act, int num_experts, int block,
+                     hipStream_t s);
 
 struct MoeUpArgs {
   const int32_t* topk_ids;
@@ -487,14 +488,21 @@ extern "C" int gguf_moe_vec_layer(const void* X, int xdtype, const void* W13, in
 // layer with more than 64 tokens takes -- on blocks of 16 slots while its experts see at most 16 pairs each on average and
 // both formats have such tiles (returns 1), else on the reference's blocks of 32 (returns 2); from MOE_SORTED_MIN_PAIRS
 // pairs per expert on, where one of the formats changes its scale every 16 values (Q2_K, Q3_K, Q6_K: the 32-slot kernel
-// multiplies those at half rate), the layer in slot order on the pipelined integer engine with blocks of 128 slots
-// (returns 3).  Measured, 96 .. 512 pairs per expert: Q4_K / Q6_K layers of 8 experts [4096,14336] 22 - 26 % faster, of
-// 64 experts [2048,1024] -3 .. +17 %; Q4_0 layers of 8 experts 1 - 13 % faster but of 64 experts 6 - 25 % slower (half of
-// a 128-slot block is padding on average and the first GEMM's result makes a round trip), hence the condition.
-#ifndef MOE_SORTED_MIN_PAIRS_VALUE
-#define MOE_SORTED_MIN_PAIRS_VALUE 96
-#endif
-static constexpr int64_t MOE_SORTED_MIN_PAIRS = MOE_SORTED_MIN_PAIRS_VALUE;
+// multiplies those at half rate), the layer in slot order on the pipelined integer engine with blocks of 64 slots
+// (returns 3).  Measured with Q4_K gate / up and a Q6_K down projection, against the 32-slot blocks at 64 pairs per
+// expert: 8 experts [4096,14336] 12 % faster, 64 experts [2048,1024] 7 %, 128 experts [2048,768] 2 % slower; at 32 pairs
+// per expert 4 - 6 % slower, at 128 pairs the 8-expert layer 26 % faster.  Blocks of 128 slots (128 x 64 tiles) were
+// 1 - 13 % slower than blocks of 64 from 128 to 512 pairs per expert: half a block of padding per expert costs more than
+// decoding each weight for 64 rows instead of 128.  Q4_0 layers gain nothing on either (64 experts: 0 - 22 % slower),
+// hence the condition on the format.
+static constexpr int64_t MOE_SORTED_MIN_PAIRS = 64, MOE_SORTED_BLOCK = 64;
+// whether the layer runs in slot order
+static bool moe_sorted_pays(int type13, int type2, int64_t pairs, int64_t num_experts) {
+  using namespace gguf;
+  const auto deep16 = [](int t) { return t == T_Q2_K || t == T_Q3_K || t == T_Q6_K; };
+  return (deep16(type13) || deep16(type2)) && pairs >= MOE_SORTED_MIN_PAIRS * num_experts &&
+         pairs + (MOE_SORTED_BLOCK - 1) * num_experts <= 65535;   // (a grid row per slot)
+}
 extern "C" int gguf_moe_mmq_layer_takes(int type13, int type2, int64_t H, int64_t I, int64_t N_out, int64_t top_k, int64_t tokens,
                                         int64_t num_experts) {
   using namespace gguf;
@@ -503,10 +511,7 @@ extern "C" int gguf_moe_mmq_layer_takes(int type13, int type2, int64_t H, int64_
   const int qk13 = block_elems(type13), qk2 = block_elems(type2);
   if (qk13 == 0 || qk2 == 0 || H % qk13 != 0 || I % qk2 != 0) return 0;
   const int block = moe_tiles_layer_block(type13, type2, tokens * top_k, num_experts, I, false);
-  const auto deep16 = [](int t) { return t == T_Q2_K || t == T_Q3_K || t == T_Q6_K; };
-  if (block != 0 && (deep16(type13) || deep16(type2)) && tokens * top_k >= MOE_SORTED_MIN_PAIRS * num_experts &&
-      tokens * top_k + 127 * num_experts <= 65535)   // (a grid row per slot)
-    return 3;
+  if (block != 0 && moe_sorted_pays(type13, type2, tokens * top_k, num_experts)) return 3;
   return block == 16 ? 1 : block == 32 ? 2 : 0;
 }
 
@@ -515,7 +520,7 @@ extern "C" int64_t gguf_moe_mmq_layer_workspace_bytes(int type13, int type2, int
   using namespace gguf;
   const int route = gguf_moe_mmq_layer_takes(type13, type2, H, I, N_out, top_k, tokens, num_experts);
   const int elt = xdtype == GGUF_DTYPE_F32 ? 4 : 2;
-  if (route == 3) return moe_sorted_layer_workspace(tokens, top_k, H, I, N_out, num_experts, elt);
+  if (route == 3) return moe_sorted_layer_workspace(tokens, top_k, H, I, N_out, num_experts, elt, (int)MOE_SORTED_BLOCK);
   return route ? moe_tiles_layer_workspace(tokens, top_k, H, I, N_out, num_experts, elt, route == 1 ? 16 : 32) : 0;
 }
 
@@ -532,9 +537,11 @@ extern "C" int gguf_moe_mmq_layer(const void* X, int xdtype, const void* W13, in
   if (!X || !W13 || !W2 || !topk_ids || !topk_weights || !workspace || !out) return GGUF_ERR_NULL;
   if (((uintptr_t)W13 | (uintptr_t)W2) & 1) return GGUF_ERR_SHAPE;   // packed blocks sit at even addresses
   if (route == 3) {
-    if (workspace_bytes < moe_sorted_layer_workspace(tokens, top_k, H, I, N_out, num_experts, xdtype == GGUF_DTYPE_F32 ? 4 : 2)) return GGUF_ERR_WORKSPACE;
+    const int sorted_block = (int)MOE_SORTED_BLOCK;
+    if (workspace_bytes < moe_sorted_layer_workspace(tokens, top_k, H, I, N_out, num_experts, xdtype == GGUF_DTYPE_F32 ? 4 : 2, sorted_block))
+      return GGUF_ERR_WORKSPACE;
     return moe_sorted_layer(X, xdtype, workspace, W13, type13, W2, type2, topk_ids, topk_weights, out, (int)H, (int)I, (int)N_out, (int)top_k,
-                            (int)tokens, act, (int)num_experts, (hipStream_t)stream);
+                            (int)tokens, act, (int)num_experts, sorted_block, (hipStream_t)stream);
   }
   const int block = route == 1 ? 16 : 32;
   if (workspace_bytes < moe_tiles_layer_workspace(tokens, top_k, H, I, N_out, num_experts, xdtype == GGUF_DTYPE_F32 ? 4 : 2, block))
