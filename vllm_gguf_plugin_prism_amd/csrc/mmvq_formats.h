@@ -151,6 +151,10 @@ struct FmtQ4_K {
   }
 };
 
+// Selector of the byte permute that gathers bytes h, 2 + h, 4 + h, 6 + h of eight, h = bit 1 of the unit's column group:
+// the per-group scale bytes of unit u in the Q6_K arrangement of units (also Q2_K's and Q3_K's)
+__device__ __forceinline__ uint32_t k8_group_bytes(int u) { return (u & 2) ? 0x07050301u : 0x06040200u; }
+
 // ------------------------------------------------------------------ Q6_K (vecdotq.cuh:447-465,1417-1441)
 // unit c of a super-block: half h = c>>2, columns l in [8*(c&3), +8) of that half; covers elements
 // 128h + 32t + l for t = 0..3, i.e. eight values in each of four q8_1 blocks.
@@ -186,8 +190,10 @@ struct FmtQ6_K {
     r.d = (uint16_t)(w[0] >> sh);
     return r;
   }
-  struct ActRegs { int2 a[4]; float d8[4]; int ones[4]; };
-  static __device__ __forceinline__ ActRegs load_act(const Act& x, int u) {
+  // `off`: the sum of the lane's eight quants of block t times the offset of the format's codes (32 here)
+  struct ActRegs { int2 a[4]; float d8[4]; int off[4]; };
+  template <int OFFSET>
+  static __device__ __forceinline__ ActRegs load_act_off(const Act& x, int u) {
     const int sb = u >> 3, c = u & 7, h = c >> 2, cc = c & 3;
     const int8_t* qa = x.q + 256 * sb + 128 * h + 8 * cc;
     ActRegs a;
@@ -195,14 +201,15 @@ struct FmtQ6_K {
     for (int t = 0; t < 4; ++t) {
       a.a[t] = *(const int2*)(qa + 32 * t);
       a.d8[t] = x.d[8 * sb + 4 * h + t];
-      a.ones[t] = dot4(0x01010101, a.a[t].x, dot4(0x01010101, a.a[t].y, 0));  // for the -32 offset of the codes
+      a.off[t] = OFFSET * dot4(0x01010101, a.a[t].x, dot4(0x01010101, a.a[t].y, 0));
     }
     return a;
   }
+  static __device__ __forceinline__ ActRegs load_act(const Act& x, int u) { return load_act_off<32>(x, u); }
   static __device__ __forceinline__ float dot(const Regs& r, const ActRegs& x, int u) {
-    const int cc = u & 3;
-    const uint64_t sw = ((uint64_t)r.sc.y << 32) | r.sc.x;
-    const int so = 8 * (cc >> 1);
+    // the signed scales of the lane's four 16-value groups are bytes h, 2 + h, 4 + h, 6 + h of the eight it holds:
+    // one byte permute gathers them (a 64-bit shift per group took three instructions each)
+    const uint32_t sc4 = __builtin_amdgcn_perm(r.sc.y, r.sc.x, k8_group_bytes(u));
     float acc = 0.0f;
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
@@ -210,9 +217,11 @@ struct FmtQ6_K {
       const int shl = (t >> 1) ? 4 : 0;
       const int vx = (int)(((ql.x >> shl) & 0x0F0F0F0Fu) | (((r.qh.x >> (2 * t)) & 0x03030303u) << 4));
       const int vy = (int)(((ql.y >> shl) & 0x0F0F0F0Fu) | (((r.qh.y >> (2 * t)) & 0x03030303u) << 4));
-      const int s = dot4(vx, x.a[t].x, dot4(vy, x.a[t].y, 0));
-      const int sc = (int)(int8_t)(sw >> (16 * t + so));
-      acc += x.d8[t] * (float)(sc * (s - 32 * x.ones[t]));
+      const int s = dot4(vx, x.a[t].x, dot4(vy, x.a[t].y, 0)) - x.off[t];
+      const int sc = (int)(int8_t)(sc4 >> (8 * t));
+      // (|sc * s| < 2^23: the product of the converted factors is the converted integer product, bit for bit, and a
+      //  float multiply issues at four times the rate of a 32-bit integer one)
+      acc += x.d8[t] * ((float)sc * (float)s);
     }
     return h2f(r.d) * acc;
   }
@@ -528,19 +537,27 @@ struct FmtQ2_K {
     r.q = make_uint2(w[4 + 8 * n + 2 * cc], w[5 + 8 * n + 2 * cc]); r.sc = make_uint2(w[2 * n], w[2 * n + 1]); r.dm = w[20];
     return r;
   }
-  typedef FmtQ6_K::ActRegs ActRegs;
-  static __device__ __forceinline__ ActRegs load_act(const Act& x, int u) { return FmtQ6_K::load_act(x, u); }
+  // `du8`: d8 times the sum of the lane's eight quants of block t, what the group's min multiplies
+  struct ActRegs { int2 a[4]; float d8[4]; float du8[4]; };
+  static __device__ __forceinline__ ActRegs load_act(const Act& x, int u) {
+    const FmtQ6_K::ActRegs b = FmtQ6_K::load_act_off<1>(x, u);
+    ActRegs a;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) { a.a[t] = b.a[t]; a.d8[t] = b.d8[t]; a.du8[t] = b.d8[t] * (float)b.off[t]; }
+    return a;
+  }
   static __device__ __forceinline__ float dot(const Regs& r, const ActRegs& x, int u) {
-    const int cc = u & 3;
-    const uint64_t sw = ((uint64_t)r.sc.y << 32) | r.sc.x;
+    // scale (low nibble) and min (high nibble) of the lane's four 16-value groups, gathered into one register
+    const uint32_t scm = __builtin_amdgcn_perm(r.sc.y, r.sc.x, k8_group_bytes(u));
+    const uint32_t sc4 = scm & 0x0F0F0F0Fu, mn4 = (scm >> 4) & 0x0F0F0F0Fu;
     float pos = 0.0f, neg = 0.0f;
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
       const int vx = (int)((r.q.x >> (2 * t)) & 0x03030303u), vy = (int)((r.q.y >> (2 * t)) & 0x03030303u);
       const int s = dot4(vx, x.a[t].x, dot4(vy, x.a[t].y, 0));
-      const uint32_t scm = (uint32_t)(sw >> (8 * (2 * t + (cc >> 1)))) & 0xFF;  // scale and min of this 16-element group
-      pos += x.d8[t] * (float)(s * (int)(scm & 0xF));
-      neg += x.d8[t] * (float)((int)(scm >> 4) * x.ones[t]);
+      // (the integer products s * scale and min * sum are exact as products of the converted factors)
+      pos += x.d8[t] * ((float)s * (float)((sc4 >> (8 * t)) & 0xFF));
+      neg += x.du8[t] * (float)((mn4 >> (8 * t)) & 0xFF);
     }
     return h2f(r.dm & 0xFFFF) * pos - h2f(r.dm >> 16) * neg;
   }
@@ -574,20 +591,25 @@ struct FmtQ3_K {
     return r;
   }
   typedef FmtQ6_K::ActRegs ActRegs;
-  static __device__ __forceinline__ ActRegs load_act(const Act& x, int u) { return FmtQ6_K::load_act(x, u); }
+  static __device__ __forceinline__ ActRegs load_act(const Act& x, int u) { return FmtQ6_K::load_act_off<4>(x, u); }
   static __device__ __forceinline__ float dot(const Regs& r, const ActRegs& x, int u) {
-    const int n = (u & 7) >> 2, cc = u & 3;
-    const uint64_t lo64 = ((uint64_t)r.sc01.y << 32) | r.sc01.x;
+    const int n4 = (u & 4);   // 4 n: the super-block's second half takes the high nibbles and the upper bit pairs
+    // The 6-bit scale of group is = 8 n + g, g = 2 t + h: low nibble from nibble n of byte g of the first eight scale
+    // bytes, two high bits from bits 4 n + 2 (t / 2) of byte g mod 4 of the last four.  Byte permutes gather the four
+    // bytes of either kind, so that the four scales are formed together in one register.
+    const uint32_t h = (u >> 1) & 1;
+    const uint32_t lo4 = (__builtin_amdgcn_perm(r.sc01.y, r.sc01.x, k8_group_bytes(u)) >> n4) & 0x0F0F0F0Fu;
+    const uint32_t p2 = __builtin_amdgcn_perm(r.sc2, r.sc2, h ? 0x03010301u : 0x02000200u) >> n4;
+    const uint32_t us4 = lo4 | (((p2 & 0x00000303u) | ((p2 >> 2) & 0x03030000u)) << 4);
+    const uint32_t hmx = r.hm.x >> n4, hmy = r.hm.y >> n4;
     float acc = 0.0f;
 #pragma unroll
     for (int t = 0; t < 4; ++t) {
-      // 6-bit scale of group is = 8n + 2t + (cc>>1): low nibble from bytes 0..7, two high bits from bytes 8..11
-      const int g = 2 * t + (cc >> 1), is = 8 * n + g;
-      const int us = (int)((lo64 >> (8 * g + 4 * n)) & 0xF) | (int)(((r.sc2 >> (8 * (is & 3) + 2 * (is >> 2))) & 3) << 4);
-      const uint32_t hx = (r.hm.x >> (4 * n + t)) & 0x01010101u, hy = (r.hm.y >> (4 * n + t)) & 0x01010101u;
+      const uint32_t hx = (hmx >> t) & 0x01010101u, hy = (hmy >> t) & 0x01010101u;
       const int vx = (int)(((r.q.x >> (2 * t)) & 0x03030303u) | (hx << 2)), vy = (int)(((r.q.y >> (2 * t)) & 0x03030303u) | (hy << 2));
-      const int s = dot4(vx, x.a[t].x, dot4(vy, x.a[t].y, 0)) - 4 * x.ones[t];
-      acc += x.d8[t] * (float)((us - 32) * s);
+      const int s = dot4(vx, x.a[t].x, dot4(vy, x.a[t].y, 0)) - x.off[t];
+      // ((scale - 32) * s is exact as a product of the converted factors: |.| < 2^19)
+      acc += x.d8[t] * (((float)((us4 >> (8 * t)) & 0xFF) - 32.0f) * (float)s);
     }
     return h2f(r.d) * acc;
   }
