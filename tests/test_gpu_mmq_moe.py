@@ -46,6 +46,47 @@ def test_mmq_matches_a8_oracle_fp32(qtype, m):
         assert err <= 1e-5, (o.TYPE_NAMES[qtype], m, n, k, err)
 
 
+@pytest.mark.parametrize("kind", ["offset", "positive"])
+@pytest.mark.parametrize("qtype", [o.Q4_0, o.Q4_1, o.Q5_0, o.Q5_1, o.Q2_K, o.Q4_K, o.Q5_K])
+def test_tile_operators_with_activations_of_one_sign(qtype, kind):
+    """The formats with an offset term on activations that share a sign: their q8_1 block sums are far from zero (up to
+    32 * 127 in magnitude), so the offset term is as large as the product term and partly cancels it -- the case in which
+    a block sum carried with too few bits shows.  The tile operator at the row counts of each of its kernels (streaming
+    GEMV with tile sums, packed-block rows, 16-row tiles, the pipelined engine on 64-, 128- and 256-row tiles) and the
+    grouped MoE operator on 16- and 32-slot blocks, fp32 results within 1e-5 of the a8 oracle as for centred activations."""
+    ops = _ops()
+    rng = np.random.default_rng(4300 + qtype)
+    n, k = 384, 2048
+
+    def draw(rows):
+        base = rng.standard_normal((rows, k)).astype(np.float32)
+        return ((1.0 + 0.3 * base) if kind == "offset" else (np.abs(base) + 0.5)).astype(np.float32)
+
+    w = o.make_weights(rng, qtype, n, k)
+    wd = _dev(w)
+    for m in (3, 8, 16, 32, 64, 128, 300, 512):
+        x32 = draw(m)
+        if m == 3:
+            sums = np.abs(np.asarray(o.quantize_q8_1(x32)[0], dtype=np.int64).reshape(m, -1, 32).sum(-1))
+            assert (sums > 2048).any()
+        y = ops.ggml_mul_mat_a8(wd, torch.from_numpy(x32).cuda(), qtype, n)
+        err = o.rel_l2(y.cpu().numpy(), o.mul_mat_a8(w, x32, qtype, n, "mmq"))
+        assert err <= 1e-5, (o.TYPE_NAMES[qtype], kind, m, err)
+    e, top_k = 6, 2
+    we = np.stack([o.make_weights(rng, qtype, 160, k) for _ in range(e)])
+    for t in (20, 150):                       # about 7 and 50 pairs per expert: 16-slot blocks where the format has them, else 32
+        x32 = draw(t)
+        ids, _ = _routing(rng, t, e, top_k)
+        blk = ops.moe_block_size_for(qtype, t * top_k, e)
+        s_, eids, npost = o.moe_align_block_size(ids, blk, e)
+        y = ops.ggml_moe_a8(torch.from_numpy(x32).cuda(), _dev(we), _dev(s_), _dev(eids), _dev(npost), qtype, 160, top_k, t, block_size=blk)
+        err = o.rel_l2(y.cpu().numpy(), o.moe_a8(x32, we, s_, eids, npost, qtype, 160, top_k, t, blk))
+        assert err <= 1e-5, (o.TYPE_NAMES[qtype], kind, "moe", t, blk, err)
+        yv = ops.ggml_moe_a8_vec(torch.from_numpy(x32).cuda(), _dev(we), _dev(ids), top_k, qtype, 160, t)
+        err = o.rel_l2(yv.cpu().numpy(), o.moe_a8_vec(x32, we, ids, top_k, qtype, 160, t))
+        assert err <= 1e-5, (o.TYPE_NAMES[qtype], kind, "moe vec", t, err)
+
+
 @pytest.mark.parametrize("qtype", [o.Q4_0, o.Q5_0, o.Q5_1, o.Q8_0, o.Q2_K, o.Q3_K, o.Q4_K, o.Q5_K, o.Q6_K])
 def test_mmq_2048_tokens_as_the_reference_tests_them(qtype):
     """The largest batch of the reference's test_mmq (tests/test_kernels.py:150-196: 7, 83, 128, 2048 tokens on
