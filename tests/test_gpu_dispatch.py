@@ -52,6 +52,55 @@ def test_fused_moe_pipeline_q4_0(tokens, expected_path):
     assert o.rel_l2(got.float().cpu().numpy(), want) <= 1e-2
 
 
+@pytest.mark.parametrize("qt,qt2", [(o.Q4_0, o.Q4_0), (o.Q4_K, o.Q6_K)])
+@pytest.mark.parametrize("tokens", [2, 30, 100, 400])
+def test_fused_moe_with_activations_of_one_sign(tokens, qt, qt2):
+    """The MoE layer on token rows whose values share a sign (block sums of the quantized rows far from zero, the offset
+    terms of Q4_0 / Q4_K as large as their product terms), through every route of the layer: two launches (2 tokens),
+    16-slot tiles (30), 32-slot tiles (100) and, for the Q6_K down projection, the slot order on the dense engine (400
+    tokens, 200 pairs per expert).  Two links: each separate operator against the a8 oracle on the inputs it was given,
+    and the layer against the separate operators chained with the reference's roundings between them
+    (fused_moe.py:62-95).  (The layer is not held to an oracle that forms its own intermediate: on these inputs one
+    intermediate value in a hundred moved by a half-precision step flips the roundings of the half-precision block sums
+    that Q4_0's offset term multiplies (vecdotq.cuh:46-66) and moves the oracle's own result by 8e-4 while one q8_1 code
+    in 30000 changes, so such a comparison measures the conditioning of the reference's arithmetic, not the kernels.)"""
+    from vllm_gguf_plugin_prism_amd import ops
+    rng = np.random.default_rng(7000 + tokens + qt)
+    E, H, I, top_k = 4, 512, 256, 2
+    w1 = np.stack([synth.make_weights(rng, qt, 2 * I, H) for _ in range(E)])
+    w2 = np.stack([synth.make_weights(rng, qt2, H, I) for _ in range(E)])
+    x = (4.0 * (1.0 + 0.3 * rng.standard_normal((tokens, H)))).astype(np.float16)
+    logits = rng.standard_normal((tokens, E))
+    ids = np.argsort(-logits, axis=1)[:, :top_k].astype(np.int32)
+    sel = np.take_along_axis(logits, ids, 1)
+    tw = (np.exp(sel) / np.exp(sel).sum(1, keepdims=True)).astype(np.float32)
+    xd, w1d, w2d, idd = torch.from_numpy(x).cuda(), torch.from_numpy(w1).cuda(), torch.from_numpy(w2).cuda(), torch.from_numpy(ids).cuda()
+    got = D.fused_moe_gguf(xd, w1d, w2d, torch.from_numpy(tw).cuda().half(), idd, qt, qt2, "silu")
+    torch.cuda.synchronize()
+    assert got.shape == (tokens, H) and torch.isfinite(got).all()
+    pairs, flat = tokens * top_k, ids.reshape(-1)
+    if D.select_moe_path(qt, qt2, tokens) == "vec":
+        h = ops.ggml_moe_a8_vec(xd, w1d, idd, top_k, qt, 2 * I, tokens)
+        h_or = o.moe_a8_vec(x.astype(np.float32), w1, flat, top_k, qt, 2 * I, tokens)
+        a = o.silu_and_mul(h.cpu().numpy(), stored=np.float16)
+        y = ops.ggml_moe_a8_vec(torch.from_numpy(a).cuda(), w2d, idd.reshape(-1, 1).contiguous(), 1, qt2, H, pairs)
+        y_or = o.moe_a8_vec(a.astype(np.float32), w2, flat, 1, qt2, H, pairs)
+    else:
+        blk = ops.ggml_moe_get_block_size(qt)
+        s_, eids, npost = o.moe_align_block_size(ids, blk, E)
+        sd, ed, nd = (torch.from_numpy(np.ascontiguousarray(v)).cuda() for v in (s_, eids, npost))
+        h = ops.ggml_moe_a8(xd, w1d, sd, ed, nd, qt, 2 * I, top_k, tokens)
+        h_or = o.moe_a8(x.astype(np.float32), w1, s_, eids, npost, qt, 2 * I, top_k, tokens, blk)
+        a = o.silu_and_mul(h.cpu().numpy(), stored=np.float16)
+        y = ops.ggml_moe_a8(torch.from_numpy(a).cuda(), w2d, sd, ed, nd, qt2, H, 1, pairs)
+        y_or = o.moe_a8(a.astype(np.float32), w2, s_, eids, npost, qt2, H, 1, pairs, blk)
+    assert o.rel_l2(h.float().cpu().numpy(), h_or) <= 1e-3 and o.rel_l2(y.float().cpu().numpy(), y_or) <= 1e-3
+    yy = y.cpu().numpy().astype(np.float64).reshape(tokens, top_k, H)
+    want = (yy * tw.astype(np.float16).astype(np.float64)[:, :, None]).astype(np.float16).astype(np.float64).sum(1)
+    err = o.rel_l2(got.float().cpu().numpy(), want)
+    assert err <= 5e-4, (tokens, o.TYPE_NAMES[qt], o.TYPE_NAMES[qt2], err)    # (the result's own rounding to half: 2.2e-4)
+
+
 @pytest.mark.parametrize("qt,batch,rows,path", [(o.Q4_K, 2, 64, "mmvq"), (o.Q4_K, 7, 64, "mmq"),
                                                 (o.IQ4_XS, 3, 64, "mmvq"), (o.IQ4_XS, 40, 64, "dequant")])
 def test_fused_mul_mat_routes(qt, batch, rows, path):
