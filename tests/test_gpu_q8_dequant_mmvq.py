@@ -261,6 +261,33 @@ def test_mmvq_tile_route_keeps_large_block_sums_exact(qtype, kind):
         assert o.rel_l2(y.cpu().numpy(), want) <= 1e-5, (o.TYPE_NAMES[qtype], kind, m)
 
 
+def test_empty_batches_single_rows_and_rows_beyond_the_streaming_kernel():
+    """The corners of the two dense operators: no rows of X at all (the reference's callers answer an empty batch
+    themselves, linear.py:36-37; the operators return an empty result), a matrix of one, three and seven rows, and
+    rows of 33792 to 65536 values, longer than the streaming kernel takes -- for both offset-term semantics."""
+    ops = _ops()
+    rng = np.random.default_rng(2900)
+    w = _to_dev(o.make_weights(rng, o.Q4_K, 64, 512))
+    for f in (ops.ggml_mul_mat_vec_a8, ops.ggml_mul_mat_a8):
+        y = f(w, torch.empty(0, 512, dtype=torch.float16, device="cuda"), o.Q4_K, 64)
+        assert y.shape == (0, 64) and y.dtype == torch.float16
+    we = _to_dev(np.stack([o.make_weights(rng, o.Q4_0, 64, 256) for _ in range(4)]))
+    y = ops.ggml_moe_a8_vec(torch.empty(0, 256, dtype=torch.float16, device="cuda"), we,
+                            torch.empty(0, 2, dtype=torch.int32, device="cuda"), 2, o.Q4_0, 64, 0)
+    assert y.shape == (0, 64)
+    for qtype in (o.Q4_K, o.Q8_0, o.Q6_K, o.IQ4_XS):
+        for n, k in [(1, 4096), (3, 40960), (7, 65536), (130, 33792)]:
+            wn = o.make_weights(rng, qtype, n, k)
+            wd = _to_dev(wn)
+            for m in (1, 2, 5):
+                x = rng.standard_normal((m, k)).astype(np.float32)
+                xd = torch.from_numpy(x).cuda()
+                err = o.rel_l2(ops.ggml_mul_mat_vec_a8(wd, xd, qtype, n).cpu().numpy(), o.mul_mat_a8(wn, x, qtype, n, "mmvq"))
+                assert err <= 1e-5, (o.TYPE_NAMES[qtype], n, k, m, err)
+                err = o.rel_l2(ops.ggml_mul_mat_a8(wd, xd, qtype, n).cpu().numpy(), o.mul_mat_a8(wn, x, qtype, n, "mmq"))
+                assert err <= 1e-5, (o.TYPE_NAMES[qtype], n, k, m, err)
+
+
 SPAN_TYPES = [o.Q4_0, o.Q4_1, o.Q5_0, o.Q5_1, o.Q8_0, o.Q2_K, o.Q3_K, o.Q4_K, o.Q5_K, o.Q6_K, o.IQ4_NL]
 
 
