@@ -288,6 +288,32 @@ def test_empty_batches_single_rows_and_rows_beyond_the_streaming_kernel():
                 assert err <= 1e-5, (o.TYPE_NAMES[qtype], n, k, m, err)
 
 
+@pytest.mark.parametrize("qtype", [o.Q4_K, o.Q4_0, o.Q6_K, o.Q8_0, o.IQ2_XXS])
+def test_rows_of_zeros_and_rows_at_the_bottom_of_the_float_range(qtype):
+    """Activation rows that are all zero (d = 0: every code 0, the result exactly 0, no NaN from 0 / 0), rows with whole
+    blocks of zeros, and a row scaled to 1e-30 (its q8_1 scales are subnormal as halves or flush to zero, as in the
+    reference), at the row counts of every kernel of both dense operators."""
+    ops = _ops()
+    rng = np.random.default_rng(3100 + qtype)
+    n, k = 96, 2048
+    wn = o.make_weights(rng, qtype, n, k)
+    wd = _to_dev(wn)
+    for m in (1, 3, 8, 40, 200):
+        x = rng.standard_normal((m, k)).astype(np.float32)
+        x[0] = 0.0
+        if m > 2:
+            x[2, :64] = 0.0
+            x[1] *= 1e-30
+        for f, mode in ((ops.ggml_mul_mat_vec_a8, "mmvq"), (ops.ggml_mul_mat_a8, "mmq")):
+            y = f(wd, torch.from_numpy(x).cuda(), qtype, n).cpu().numpy()
+            want = o.mul_mat_a8(wn, x, qtype, n, mode)
+            assert np.isfinite(y).all() and (y[0] == 0).all(), (o.TYPE_NAMES[qtype], m, mode)
+            rows = [i for i in range(m) if i != 1 or m <= 2]
+            assert o.rel_l2(y[rows], want[rows]) <= 1e-5, (o.TYPE_NAMES[qtype], m, mode)
+            if m > 2:
+                assert np.abs(y[1] - want[1]).max() <= 1e-5 * np.abs(want[1]).max() + 1e-38, (o.TYPE_NAMES[qtype], m, mode)
+
+
 SPAN_TYPES = [o.Q4_0, o.Q4_1, o.Q5_0, o.Q5_1, o.Q8_0, o.Q2_K, o.Q3_K, o.Q4_K, o.Q5_K, o.Q6_K, o.IQ4_NL]
 
 
